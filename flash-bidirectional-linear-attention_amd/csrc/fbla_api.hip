@@ -1,0 +1,218 @@
+// C-ABI layer of libfbla_hip.so: argument checks, kernel-family dispatch and
+// error reporting.  Declarations and the reference call sites each entry point
+// replaces are in include/flash_bla_hip.h.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/flash_bla_hip.h"
+#include "fbla_kernels.h"
+
+namespace fbla {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+static int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("%s: kernel launch failed: %s", what, hipGetErrorString(e));
+    return kErrLaunch;
+  }
+  return kOk;
+}
+
+static int check_dims(const char* what, int64_t N, int64_t H, int64_t L, int DK, int DV,
+                      int dtype, int flags) {
+  if (N < 0 || H <= 0 || L < 0) {
+    set_error("%s: bad sizes N=%lld H=%lld L=%lld", what, (long long)N, (long long)H, (long long)L);
+    return kErrBadArg;
+  }
+  if (DK < 1 || DK > 128 || DV < 1 || DV > 128) {
+    set_error("%s: head dims must be in [1,128], got DK=%d DV=%d", what, DK, DV);
+    return kErrUnsupported;
+  }
+  if (dtype != kF16 && dtype != kBF16 && dtype != kF32) {
+    set_error("%s: unknown dtype %d", what, dtype);
+    return kErrBadArg;
+  }
+  if ((flags & kDecoupled) && !(flags & kNormalize)) {
+    set_error("%s: FBLA_DECOUPLED requires FBLA_NORMALIZE", what);
+    return kErrBadArg;
+  }
+  if (N * H > 0x7fffffffLL / 4 || L > 0x7fffffffLL / 2) {
+    set_error("%s: problem too large for 32-bit grid indexing", what);
+    return kErrUnsupported;
+  }
+  return kOk;
+}
+
+static Prob make_prob(const int32_t* cu, int64_t N, int64_t H, int64_t L, int DK, int DV, int flags,
+                      float scale, float eps) {
+  Prob p;
+  p.cu = cu;
+  p.N = (int)N;
+  p.H = (int)H;
+  p.L = (int)L;
+  p.DK = DK;
+  p.DV = DV;
+  p.scale = scale;
+  p.eps = eps;
+  p.flags = flags;
+  return p;
+}
+
+static size_t workspace_bytes(const Prob& p, int dtype, int pass) {
+  (void)dtype;
+  return pass == 0 ? generic::fwd_workspace_bytes(p) : generic::bwd_workspace_bytes(p);
+}
+
+static int run_fwd(const char* what, const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
+  if ((int64_t)p.N * p.H == 0 || p.L == 0) return kOk;
+  const size_t need = workspace_bytes(p, dtype, 0);
+  if (a.workspace_bytes < need || (need && !a.workspace)) {
+    set_error("%s: workspace too small (%zu < %zu bytes)", what, a.workspace_bytes, need);
+    return kErrWorkspace;
+  }
+  int rc = generic::forward(p, dtype, a, st);
+  if (rc != kOk) return rc;
+  return check_launch(what);
+}
+
+static int run_bwd(const char* what, const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
+  if ((int64_t)p.N * p.H == 0 || p.L == 0) return kOk;
+  const size_t need = workspace_bytes(p, dtype, 1);
+  if (a.workspace_bytes < need || (need && !a.workspace)) {
+    set_error("%s: workspace too small (%zu < %zu bytes)", what, a.workspace_bytes, need);
+    return kErrWorkspace;
+  }
+  int rc = generic::backward(p, dtype, a, st);
+  if (rc != kOk) return rc;
+  return check_launch(what);
+}
+
+}  // namespace fbla
+
+using namespace fbla;
+
+extern "C" {
+
+int fbla_version(void) { return 100; }
+
+const char* fbla_last_error(void) { return g_err; }
+
+size_t fbla_la_workspace_bytes(int pass, int64_t B, int64_t H, int64_t L, int DK, int DV, int dtype,
+                               int flags) {
+  if (check_dims("fbla_la_workspace_bytes", B, H, L, DK, DV, dtype, flags) != kOk) return 0;
+  Prob p = make_prob(nullptr, B, H, L, DK, DV, flags, 1.f, 0.f);
+  return workspace_bytes(p, dtype, pass);
+}
+
+int fbla_la_fwd(const void* q, const void* k, const void* v, const void* q_rope,
+                const void* k_rope, void* o, float* s, float* km, void* workspace,
+                size_t workspace_bytes_, int64_t B, int64_t H, int64_t L, int DK, int DV, int dtype,
+                int flags, float scale, float eps, void* stream) {
+  const char* what = "fbla_la_fwd";
+  int rc = check_dims(what, B, H, L, DK, DV, dtype, flags);
+  if (rc != kOk) return rc;
+  if (flags & kDefaultScale) {
+    set_error("%s: FBLA_DEFAULT_SCALE is only valid for the packed entry points", what);
+    return kErrBadArg;
+  }
+  if (!q || !k || !v || !o || !s || ((flags & kNormalize) && !km) ||
+      ((flags & kDecoupled) && (!q_rope || !k_rope))) {
+    if (B * H * L != 0) {
+      set_error("%s: null tensor pointer", what);
+      return kErrBadArg;
+    }
+  }
+  Prob p = make_prob(nullptr, B, H, L, DK, DV, flags, scale, eps);
+  FwdArgs a{q, k, v, q_rope, k_rope, o, s, km, workspace, workspace_bytes_};
+  return run_fwd(what, p, dtype, a, (hipStream_t)stream);
+}
+
+int fbla_la_bwd(const void* q, const void* k, const void* v, const void* q_rope,
+                const void* k_rope, const void* dout, const float* s, const float* km, void* dq,
+                void* dk, void* dv, void* dq_rope, void* dk_rope, void* workspace,
+                size_t workspace_bytes_, int64_t B, int64_t H, int64_t L, int DK, int DV, int dtype,
+                int flags, float scale, float eps, void* stream) {
+  const char* what = "fbla_la_bwd";
+  int rc = check_dims(what, B, H, L, DK, DV, dtype, flags);
+  if (rc != kOk) return rc;
+  if (flags & kDefaultScale) {
+    set_error("%s: FBLA_DEFAULT_SCALE is only valid for the packed entry points", what);
+    return kErrBadArg;
+  }
+  const bool dec = flags & kDecoupled;
+  if (B * H * L != 0 &&
+      (!q || !v || !dout || !s || !dq || !dk || !dv || (!dec && !k) || ((flags & kNormalize) && !km) ||
+       (dec && (!q_rope || !k_rope || !dq_rope || !dk_rope)))) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  Prob p = make_prob(nullptr, B, H, L, DK, DV, flags, scale, eps);
+  BwdArgs a{q, k, v, q_rope, k_rope, dout, s, km, dq, dk, dv, dq_rope, dk_rope, workspace,
+            workspace_bytes_};
+  return run_bwd(what, p, dtype, a, (hipStream_t)stream);
+}
+
+size_t fbla_varlen_workspace_bytes(int pass, int64_t total_tokens, int64_t N, int64_t H,
+                                   int64_t max_seqlen, int DK, int DV, int dtype, int flags) {
+  (void)total_tokens;
+  if (check_dims("fbla_varlen_workspace_bytes", N, H, max_seqlen, DK, DV, dtype, flags) != kOk)
+    return 0;
+  static const int32_t dummy = 0;
+  Prob p = make_prob(&dummy, N, H, max_seqlen, DK, DV, flags, 1.f, 0.f);
+  return workspace_bytes(p, dtype, pass);
+}
+
+int fbla_varlen_fwd(const void* q, const void* k, const void* v, const int32_t* cu_seqlens,
+                    void* o, float* s, float* km, void* workspace, size_t workspace_bytes_,
+                    int64_t total_tokens, int64_t N, int64_t H, int64_t max_seqlen, int DK, int DV,
+                    int dtype, int flags, float scale, float eps, void* stream) {
+  const char* what = "fbla_varlen_fwd";
+  int rc = check_dims(what, N, H, max_seqlen, DK, DV, dtype, flags);
+  if (rc != kOk) return rc;
+  if ((flags & kDecoupled) || !(flags & kNormalize)) {
+    set_error("%s: only the normalised, non-decoupled operator has a packed form", what);
+    return kErrUnsupported;
+  }
+  if (total_tokens == 0 || N == 0) return kOk;
+  if (!q || !k || !v || !o || !s || !km || !cu_seqlens) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  Prob p = make_prob(cu_seqlens, N, H, max_seqlen, DK, DV, flags, scale, eps);
+  FwdArgs a{q, k, v, nullptr, nullptr, o, s, km, workspace, workspace_bytes_};
+  return run_fwd(what, p, dtype, a, (hipStream_t)stream);
+}
+
+int fbla_varlen_bwd(const void* q, const void* k, const void* v, const int32_t* cu_seqlens,
+                    const void* dout, const float* s, const float* km, void* dq, void* dk, void* dv,
+                    void* workspace, size_t workspace_bytes_, int64_t total_tokens, int64_t N,
+                    int64_t H, int64_t max_seqlen, int DK, int DV, int dtype, int flags,
+                    float scale, float eps, void* stream) {
+  const char* what = "fbla_varlen_bwd";
+  int rc = check_dims(what, N, H, max_seqlen, DK, DV, dtype, flags);
+  if (rc != kOk) return rc;
+  if ((flags & kDecoupled) || !(flags & kNormalize)) {
+    set_error("%s: only the normalised, non-decoupled operator has a packed form", what);
+    return kErrUnsupported;
+  }
+  if (total_tokens == 0 || N == 0) return kOk;
+  if (!q || !k || !v || !dout || !s || !km || !dq || !dk || !dv || !cu_seqlens) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  Prob p = make_prob(cu_seqlens, N, H, max_seqlen, DK, DV, flags, scale, eps);
+  BwdArgs a{q, k, v, nullptr, nullptr, dout, s, km, dq, dk, dv, nullptr, nullptr, workspace,
+            workspace_bytes_};
+  return run_bwd(what, p, dtype, a, (hipStream_t)stream);
+}
+
+}  // extern "C"

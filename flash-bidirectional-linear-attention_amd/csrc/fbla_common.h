@@ -1,0 +1,79 @@
+// Shared host/device definitions for the gfx950 bidirectional linear-attention kernels.
+//
+// Terminology (follows flash_bla): a *sequence* is one (batch) entry of a dense
+// [B,H,L,D] tensor or one [cu[i],cu[i+1]) range of a packed [T,H,D] tensor; the
+// *state* of a (sequence, head) is S = scale * K^T V (DK x DV, fp32) together
+// with km = mean_t k_t (DK, fp32).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fbla {
+
+enum DType : int { kF16 = 0, kBF16 = 1, kF32 = 2 };
+
+enum Flags : int {
+  kNormalize = 1,     // divide by z = q.km + eps (linear_attn); off = simple_la
+  kDecoupled = 2,     // numerator uses q_rope/k_rope, denominator q/k
+  kDefaultScale = 4,  // varlen only: scale = 1/len_i per sequence
+};
+
+// One problem instance.  Dense: cu == nullptr, N = batch, every sequence has L
+// tokens and tensors are [N,H,L,D].  Packed: cu = int32[N+1] on the device and
+// tensors are [T_total,H,D].
+struct Prob {
+  const int32_t* cu;
+  int N, H, L;  // L: dense length, or max_seqlen upper bound when packed
+  int DK, DV;
+  float scale;
+  float eps;
+  int flags;
+};
+
+// Token range of sequence n.
+__device__ __forceinline__ void seq_range(const Prob& p, int n, int64_t& bos, int& len) {
+  if (p.cu) {
+    int b = p.cu[n];
+    bos = b;
+    len = p.cu[n + 1] - b;
+  } else {
+    bos = 0;
+    len = p.L;
+  }
+}
+
+// Row index (units of D-element rows) of local token 0 of (n,h) and the row
+// stride between consecutive tokens.
+__device__ __forceinline__ void row_base(const Prob& p, int n, int h, int64_t bos,
+                                         int64_t& row0, int64_t& rstride) {
+  if (p.cu) {
+    row0 = bos * p.H + h;
+    rstride = p.H;
+  } else {
+    row0 = ((int64_t)n * p.H + h) * p.L;
+    rstride = 1;
+  }
+}
+
+__device__ __forceinline__ float seq_scale(const Prob& p, int len) {
+  return (p.flags & kDefaultScale) ? (len > 0 ? 1.0f / (float)len : 0.0f) : p.scale;
+}
+
+template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
+template <typename T> __device__ __forceinline__ T from_f32(float x) { return (T)x; }
+
+inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// Error reporting across the C ABI (thread-local message, integer codes).
+void set_error(const char* fmt, ...);
+
+enum Err : int {
+  kOk = 0,
+  kErrBadArg = -1,
+  kErrUnsupported = -2,
+  kErrWorkspace = -3,
+  kErrLaunch = -4,
+};
+
+}  // namespace fbla

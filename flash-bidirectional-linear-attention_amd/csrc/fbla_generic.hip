@@ -1,0 +1,570 @@
+// Shape-generic kernels: any DK, DV in [1,128], fp16 / bf16 / fp32 inputs, dense
+// [B,H,L,D] or packed [T,H,D] layout.  They stage token tiles through LDS as
+// fp32 and use plain FMA arithmetic; the MFMA kernels in fbla_mfma.hip take over
+// for the 16-bit head dims they cover.  All cross-workgroup reductions are
+// two-stage and fixed-order (no atomics), so results are run-to-run identical.
+//
+// Replaces the Triton kernels of flash_bla/ops/linear_attn/fused.py:26-347,
+// decoupled.py:27-408, varlen.py:30-332 and simple_la/fused.py:26-426.
+#include "fbla_kernels.h"
+
+namespace fbla {
+namespace generic {
+
+constexpr int kThreads = 256;
+constexpr int kTile = 32;   // tokens per LDS stage
+constexpr int kLd = 129;    // LDS row pitch in floats (128 + 1: conflict-free column walks)
+
+// ---------------------------------------------------------------------------
+// helpers
+// ---------------------------------------------------------------------------
+
+// Copy rows [t0, t0+nvalid) x [0,D) of X into dst[kTile][kLd] as fp32, zero-filling
+// the rest of the [kTile][Dpad] rectangle.
+template <typename T>
+__device__ __forceinline__ void load_tile(float* dst, const T* __restrict__ X, int64_t row0,
+                                          int64_t rstride, int D, int Dpad, int t0, int nvalid) {
+  for (int i = threadIdx.x; i < kTile * Dpad; i += kThreads) {
+    int t = i / Dpad, d = i - t * Dpad;
+    float x = 0.f;
+    if (t < nvalid && d < D) x = to_f32(X[(row0 + (int64_t)(t0 + t) * rstride) * D + d]);
+    dst[t * kLd + d] = x;
+  }
+}
+
+// acc[r][c] += sum_t Ls[t][ty+16r] * Rs[t][tx+16c]  (token-contracted outer products)
+template <int M>
+__device__ __forceinline__ void outer_accumulate(float (&acc)[M][M], const float* Ls,
+                                                 const float* Rs, int tx, int ty) {
+#pragma unroll 4
+  for (int t = 0; t < kTile; ++t) {
+    float a[M], b[M];
+#pragma unroll
+    for (int r = 0; r < M; ++r) a[r] = Ls[t * kLd + ty + 16 * r];
+#pragma unroll
+    for (int c = 0; c < M; ++c) b[c] = Rs[t * kLd + tx + 16 * c];
+#pragma unroll
+    for (int r = 0; r < M; ++r)
+#pragma unroll
+      for (int c = 0; c < M; ++c) acc[r][c] = fmaf(a[r], b[c], acc[r][c]);
+  }
+}
+
+// acc[i][j] = sum_r Xs[tg+8i][r] * Mat[r][lane+32j]   (token rows times a small matrix)
+__device__ __forceinline__ void rows_times_matrix(float (&acc)[4][4], const float* Xs,
+                                                  const float* __restrict__ Mat, int R, int C,
+                                                  int tg, int lane) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  for (int r = 0; r < R; ++r) {
+    float m[4], x[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int c = lane + 32 * j;
+      m[j] = c < C ? Mat[(int64_t)r * C + c] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) x[i] = Xs[(tg + 8 * i) * kLd + r];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(x[i], m[j], acc[i][j]);
+  }
+}
+
+template <int M>
+__device__ __forceinline__ void write_partial(float* dst, const float (&acc)[M][M], int DK, int DV,
+                                              int tx, int ty) {
+#pragma unroll
+  for (int r = 0; r < M; ++r)
+#pragma unroll
+    for (int c = 0; c < M; ++c) {
+      int dk = ty + 16 * r, dv = tx + 16 * c;
+      if (dk < DK && dv < DV) dst[dk * DV + dv] = acc[r][c];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// forward, stage 1: per (sequence, head, token chunk) partial K~^T V and sum_t k_t
+// ---------------------------------------------------------------------------
+template <typename T, int M>
+__global__ __launch_bounds__(kThreads) void state_partial_kernel(
+    Prob p, const T* __restrict__ kn, const T* __restrict__ v, const T* __restrict__ kd,
+    float* __restrict__ partial, int chunk, int nchunks) {
+  __shared__ float Ls[kTile * kLd];
+  __shared__ float Rs[kTile * kLd];
+  __shared__ float Cs[kTile * kLd];
+  const int nh = blockIdx.x / nchunks, c = blockIdx.x - nh * nchunks;
+  const int n = nh / p.H, h = nh - n * p.H;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t_begin = c * chunk;
+  if (t_begin >= len) return;
+  const int t_end = min(len, t_begin + chunk);
+  row_base(p, n, h, bos, row0, rstride);
+
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int DK = p.DK, DV = p.DV, Dpad = 16 * M;
+  const bool split = p.flags & kDecoupled;
+  float acc[M][M];
+#pragma unroll
+  for (int r = 0; r < M; ++r)
+#pragma unroll
+    for (int cc = 0; cc < M; ++cc) acc[r][cc] = 0.f;
+  float ksum = 0.f;
+
+  for (int t0 = t_begin; t0 < t_end; t0 += kTile) {
+    const int nvalid = min(kTile, t_end - t0);
+    load_tile(Ls, kn, row0, rstride, DK, Dpad, t0, nvalid);
+    load_tile(Rs, v, row0, rstride, DV, Dpad, t0, nvalid);
+    if (split) load_tile(Cs, kd, row0, rstride, DK, Dpad, t0, nvalid);
+    __syncthreads();
+    outer_accumulate<M>(acc, Ls, Rs, tx, ty);
+    if ((int)threadIdx.x < DK) {
+      const float* src = split ? Cs : Ls;
+      for (int t = 0; t < kTile; ++t) ksum += src[t * kLd + threadIdx.x];
+    }
+    __syncthreads();
+  }
+  float* dst = partial + (int64_t)blockIdx.x * (DK * DV + DK);
+  write_partial<M>(dst, acc, DK, DV, tx, ty);
+  if ((int)threadIdx.x < DK) dst[DK * DV + threadIdx.x] = ksum;
+}
+
+// ---------------------------------------------------------------------------
+// stage 2 (forward and backward): fixed-order sum of the chunk partials.
+//   mat[dk][dv] = scale_n * sum_c partial_c ;  mat_t = its transpose (optional)
+//   vec[dk]     = (1/len) * sum_c partial_vec_c
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void state_reduce_kernel(
+    Prob p, const float* __restrict__ partial, int chunk, int nchunks, float* __restrict__ mat,
+    float* __restrict__ mat_t, float* __restrict__ vec) {
+  const int nh = blockIdx.x;
+  const int n = nh / p.H;
+  int64_t bos;
+  int len;
+  seq_range(p, n, bos, len);
+  const int DK = p.DK, DV = p.DV, E = DK * DV, stride = E + DK;
+  const int nvalid = len > 0 ? (len + chunk - 1) / chunk : 0;
+  const float s = seq_scale(p, len);
+  const float inv_len = len > 0 ? 1.0f / (float)len : 0.f;
+  const float* src = partial + (int64_t)nh * nchunks * stride;
+  for (int e = threadIdx.x; e < stride; e += kThreads) {
+    float a = 0.f;
+    for (int c = 0; c < nvalid; ++c) a += src[(int64_t)c * stride + e];
+    if (e < E) {
+      a *= s;
+      mat[(int64_t)nh * E + e] = a;
+      if (mat_t) {
+        int dk = e / DV, dv = e - dk * DV;
+        mat_t[(int64_t)nh * E + dv * DK + dk] = a;
+      }
+    } else {
+      if (vec) vec[(int64_t)nh * DK + (e - E)] = a * inv_len;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void transpose_state_kernel(const float* __restrict__ mat,
+                                                                   float* __restrict__ mat_t,
+                                                                   int DK, int DV) {
+  const int64_t base = (int64_t)blockIdx.x * DK * DV;
+  for (int e = threadIdx.x; e < DK * DV; e += kThreads) {
+    int dk = e / DV, dv = e - dk * DV;
+    mat_t[base + dv * DK + dk] = mat[base + e];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// forward, stage 3: o_t = (q~_t S) / (q_t . km + eps)
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kThreads) void output_kernel(
+    Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const float* __restrict__ S,
+    const float* __restrict__ km, T* __restrict__ o, int ntiles) {
+  __shared__ float Xs[kTile * kLd];
+  __shared__ float Ds[kTile * kLd];
+  __shared__ float zs[kTile];
+  const int nh = blockIdx.x / ntiles, tile = blockIdx.x - nh * ntiles;
+  const int n = nh / p.H, h = nh - n * p.H;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t0 = tile * kTile;
+  if (t0 >= len) return;
+  const int nvalid = min(kTile, len - t0);
+  row_base(p, n, h, bos, row0, rstride);
+  const int DK = p.DK, DV = p.DV;
+  const bool normalize = p.flags & kNormalize;
+  const bool split = p.flags & kDecoupled;
+
+  load_tile(Xs, qn, row0, rstride, DK, DK, t0, nvalid);
+  if (split && normalize) load_tile(Ds, qd, row0, rstride, DK, DK, t0, nvalid);
+  __syncthreads();
+  if (threadIdx.x < kTile) {
+    float z = 1.f;
+    if (normalize) {
+      const float* src = split ? Ds : Xs;
+      const float* kmh = km + (int64_t)nh * DK;
+      z = 0.f;
+      for (int r = 0; r < DK; ++r) z = fmaf(src[threadIdx.x * kLd + r], kmh[r], z);
+      z += p.eps;
+    }
+    zs[threadIdx.x] = z;
+  }
+  __syncthreads();
+  const int tg = threadIdx.x >> 5, lane = threadIdx.x & 31;
+  float acc[4][4];
+  rows_times_matrix(acc, Xs, S + (int64_t)nh * DK * DV, DK, DV, tg, lane);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = tg + 8 * i;
+    if (t >= nvalid) continue;
+    const float rz = 1.0f / zs[t];
+    T* dst = o + (row0 + (int64_t)(t0 + t) * rstride) * DV;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = lane + 32 * j;
+      if (c < DV) dst[c] = from_f32<T>(acc[i][j] * rz);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// backward, pass A: reads q~, q, dO (+S, S^T, km); writes dq~ (and dq when
+// decoupled) and per-chunk partials of dS = sum_t (q~_t/z_t)^T dO_t and
+// dkm = sum_t dz_t q_t, with dz_t = -(o_t.dO_t)/z_t and o_t recomputed from q~_t S.
+// ---------------------------------------------------------------------------
+template <typename T, int M>
+__global__ __launch_bounds__(kThreads) void bwd_a_kernel(
+    Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const T* __restrict__ dout,
+    const float* __restrict__ S, const float* __restrict__ St, const float* __restrict__ km,
+    T* __restrict__ dqn, T* __restrict__ dqd, float* __restrict__ partial, int chunk,
+    int nchunks) {
+  __shared__ float Qn[kTile * kLd];
+  __shared__ float Qd[kTile * kLd];
+  __shared__ float Gs[kTile * kLd];
+  __shared__ float zs[kTile];
+  __shared__ float dzs[kTile];
+  __shared__ float Ps[kTile];
+  const int nh = blockIdx.x / nchunks, c = blockIdx.x - nh * nchunks;
+  const int n = nh / p.H, h = nh - n * p.H;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t_begin = c * chunk;
+  if (t_begin >= len) return;
+  const int t_end = min(len, t_begin + chunk);
+  row_base(p, n, h, bos, row0, rstride);
+
+  const int DK = p.DK, DV = p.DV, Dpad = 16 * M;
+  const bool normalize = p.flags & kNormalize;
+  const bool split = p.flags & kDecoupled;
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int tg = threadIdx.x >> 5, lane = threadIdx.x & 31;
+  const float* Sh = S + (int64_t)nh * DK * DV;
+  const float* Sth = St + (int64_t)nh * DK * DV;
+  const float* kmh = km + (int64_t)nh * DK;
+
+  float acc[M][M];
+#pragma unroll
+  for (int r = 0; r < M; ++r)
+#pragma unroll
+    for (int cc = 0; cc < M; ++cc) acc[r][cc] = 0.f;
+  float dkm = 0.f;
+
+  for (int t0 = t_begin; t0 < t_end; t0 += kTile) {
+    const int nvalid = min(kTile, t_end - t0);
+    load_tile(Qn, qn, row0, rstride, DK, Dpad, t0, nvalid);
+    load_tile(Gs, dout, row0, rstride, DV, Dpad, t0, nvalid);
+    if (split) load_tile(Qd, qd, row0, rstride, DK, Dpad, t0, nvalid);
+    __syncthreads();
+    const float* Qden = split ? Qd : Qn;
+    float u[4][4];
+    if (normalize) {
+      if (threadIdx.x < kTile) {
+        float z = 0.f;
+        for (int r = 0; r < DK; ++r) z = fmaf(Qden[threadIdx.x * kLd + r], kmh[r], z);
+        zs[threadIdx.x] = (int)threadIdx.x < nvalid ? z + p.eps : 1.0f;  // padding rows: dz = 0
+      }
+      // P_t = (q~_t S) . dO_t
+      rows_times_matrix(u, Qn, Sh, DK, DV, tg, lane);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int t = tg + 8 * i;
+        float part = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int cc = lane + 32 * j;
+          if (cc < DV) part = fmaf(u[i][j], Gs[t * kLd + cc], part);
+        }
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1) part += __shfl_xor(part, off, 32);
+        if (lane == 0) Ps[t] = part;
+      }
+      __syncthreads();
+      if (threadIdx.x < kTile) {
+        const float z = zs[threadIdx.x];
+        dzs[threadIdx.x] = -Ps[threadIdx.x] / (z * z);
+      }
+      __syncthreads();
+    }
+    // dq~_t = dO_t S^T / z_t (+ dz_t km when q~ == q)
+    rows_times_matrix(u, Gs, Sth, DV, DK, tg, lane);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int t = tg + 8 * i;
+      if (t >= nvalid) continue;
+      const float rz = normalize ? 1.0f / zs[t] : 1.0f;
+      const float dz = normalize ? dzs[t] : 0.f;
+      const int64_t roff = (row0 + (int64_t)(t0 + t) * rstride) * DK;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int cc = lane + 32 * j;
+        if (cc >= DK) continue;
+        float g = u[i][j] * rz;
+        const float den = normalize ? dz * kmh[cc] : 0.f;
+        if (split) {
+          dqd[roff + cc] = from_f32<T>(den);
+        } else {
+          g += den;
+        }
+        dqn[roff + cc] = from_f32<T>(g);
+      }
+    }
+    if (normalize) {
+      if ((int)threadIdx.x < DK) {
+        for (int t = 0; t < kTile; ++t) dkm = fmaf(dzs[t], Qden[t * kLd + threadIdx.x], dkm);
+      }
+      __syncthreads();
+      for (int i = threadIdx.x; i < kTile * Dpad; i += kThreads) {
+        int t = i / Dpad, d = i - t * Dpad;
+        Qn[t * kLd + d] *= 1.0f / zs[t];
+      }
+      __syncthreads();
+    }
+    outer_accumulate<M>(acc, Qn, Gs, tx, ty);
+    __syncthreads();
+  }
+  float* dst = partial + (int64_t)blockIdx.x * (DK * DV + DK);
+  write_partial<M>(dst, acc, DK, DV, tx, ty);
+  if ((int)threadIdx.x < DK) dst[DK * DV + threadIdx.x] = dkm;
+}
+
+// ---------------------------------------------------------------------------
+// backward, pass B: dk~_t = v_t (s dS)^T (+ dkm/L when k~ == k), dv_t = k~_t (s dS),
+// and dk_t = dkm/L for every row when decoupled.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kThreads) void bwd_b_kernel(
+    Prob p, const T* __restrict__ kn, const T* __restrict__ v, const float* __restrict__ dS,
+    const float* __restrict__ dSt, const float* __restrict__ dkm, T* __restrict__ dkn,
+    T* __restrict__ dkd, T* __restrict__ dv, int ntiles) {
+  __shared__ float Ks[kTile * kLd];
+  __shared__ float Vs[kTile * kLd];
+  const int nh = blockIdx.x / ntiles, tile = blockIdx.x - nh * ntiles;
+  const int n = nh / p.H, h = nh - n * p.H;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t0 = tile * kTile;
+  if (t0 >= len) return;
+  const int nvalid = min(kTile, len - t0);
+  row_base(p, n, h, bos, row0, rstride);
+  const int DK = p.DK, DV = p.DV;
+  const bool normalize = p.flags & kNormalize;
+  const bool split = p.flags & kDecoupled;
+  const float* dSh = dS + (int64_t)nh * DK * DV;
+  const float* dSth = dSt + (int64_t)nh * DK * DV;
+  const float* dkmh = dkm + (int64_t)nh * DK;
+
+  load_tile(Ks, kn, row0, rstride, DK, DK, t0, nvalid);
+  load_tile(Vs, v, row0, rstride, DV, DV, t0, nvalid);
+  __syncthreads();
+  const int tg = threadIdx.x >> 5, lane = threadIdx.x & 31;
+  float acc[4][4];
+  rows_times_matrix(acc, Vs, dSth, DV, DK, tg, lane);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = tg + 8 * i;
+    if (t >= nvalid) continue;
+    const int64_t roff = (row0 + (int64_t)(t0 + t) * rstride) * DK;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int cc = lane + 32 * j;
+      if (cc >= DK) continue;
+      float g = acc[i][j];
+      const float den = normalize ? dkmh[cc] : 0.f;
+      if (split) {
+        dkd[roff + cc] = from_f32<T>(den);
+      } else {
+        g += den;
+      }
+      dkn[roff + cc] = from_f32<T>(g);
+    }
+  }
+  rows_times_matrix(acc, Ks, dSh, DK, DV, tg, lane);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = tg + 8 * i;
+    if (t >= nvalid) continue;
+    const int64_t roff = (row0 + (int64_t)(t0 + t) * rstride) * DV;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int cc = lane + 32 * j;
+      if (cc < DV) dv[roff + cc] = from_f32<T>(acc[i][j]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+
+// Tokens per reduction chunk: enough chunks to give every CU several workgroups,
+// few enough that the partial buffer stays small.
+int pick_chunk(const Prob& p) {
+  const int64_t nh = (int64_t)p.N * p.H;
+  const int64_t target_wgs = 1024;
+  int64_t chunk = cdiv64((int64_t)p.L * nh, target_wgs);
+  chunk = cdiv64(chunk, kTile) * kTile;
+  if (chunk < 2 * kTile) chunk = 2 * kTile;
+  return (int)chunk;
+}
+
+size_t partial_bytes(const Prob& p) {
+  const int chunk = pick_chunk(p);
+  const int64_t nchunks = cdiv64(p.L, chunk);
+  return align_up((size_t)p.N * p.H * nchunks * ((size_t)p.DK * p.DV + p.DK) * sizeof(float), 256);
+}
+
+size_t state_bytes(const Prob& p) {
+  return align_up((size_t)p.N * p.H * p.DK * p.DV * sizeof(float), 256);
+}
+
+size_t vec_bytes(const Prob& p) { return align_up((size_t)p.N * p.H * p.DK * sizeof(float), 256); }
+
+size_t fwd_workspace_bytes(const Prob& p) { return partial_bytes(p); }
+
+// partials | S^T | s*dS | (s*dS)^T | dkm/L
+size_t bwd_workspace_bytes(const Prob& p) {
+  return partial_bytes(p) + 3 * state_bytes(p) + vec_bytes(p);
+}
+
+template <typename T, int M>
+static void launch_state_partial(const Prob& p, const T* kn, const T* v, const T* kd,
+                                 float* partial, int chunk, int nchunks, hipStream_t st) {
+  const int64_t grid = (int64_t)p.N * p.H * nchunks;
+  state_partial_kernel<T, M><<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial,
+                                                                             chunk, nchunks);
+}
+
+template <typename T, int M>
+static void launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, const float* S,
+                         const float* St, const float* km, T* dqn, T* dqd, float* partial,
+                         int chunk, int nchunks, hipStream_t st) {
+  const int64_t grid = (int64_t)p.N * p.H * nchunks;
+  bwd_a_kernel<T, M><<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(
+      p, qn, qd, dout, S, St, km, dqn, dqd, partial, chunk, nchunks);
+}
+
+static int micro(const Prob& p) {
+  const int d = p.DK > p.DV ? p.DK : p.DV;
+  return d <= 32 ? 2 : (d <= 64 ? 4 : 8);
+}
+
+template <typename T>
+static int forward_t(const Prob& p, const FwdArgs& a, hipStream_t st) {
+  const T* q = (const T*)a.q;
+  const T* k = (const T*)a.k;
+  const T* v = (const T*)a.v;
+  const bool dec = p.flags & kDecoupled;
+  const T* qn = dec ? (const T*)a.q_rope : q;
+  const T* kn = dec ? (const T*)a.k_rope : k;
+  const int chunk = pick_chunk(p);
+  const int nchunks = (int)cdiv64(p.L, chunk);
+  float* partial = (float*)a.workspace;
+  switch (micro(p)) {
+    case 2: launch_state_partial<T, 2>(p, kn, v, k, partial, chunk, nchunks, st); break;
+    case 4: launch_state_partial<T, 4>(p, kn, v, k, partial, chunk, nchunks, st); break;
+    default: launch_state_partial<T, 8>(p, kn, v, k, partial, chunk, nchunks, st); break;
+  }
+  const int64_t nh = (int64_t)p.N * p.H;
+  state_reduce_kernel<<<dim3((unsigned)nh), dim3(kThreads), 0, st>>>(p, partial, chunk, nchunks,
+                                                                    a.s, nullptr, a.km);
+  const int ntiles = (int)cdiv64(p.L, kTile);
+  output_kernel<T><<<dim3((unsigned)(nh * ntiles)), dim3(kThreads), 0, st>>>(
+      p, qn, q, a.s, a.km, (T*)a.o, ntiles);
+  return kOk;
+}
+
+template <typename T>
+static int backward_t(const Prob& p, const BwdArgs& a, hipStream_t st) {
+  const bool dec = p.flags & kDecoupled;
+  const T* q = (const T*)a.q;
+  const T* v = (const T*)a.v;
+  const T* qn = dec ? (const T*)a.q_rope : q;
+  const T* kn = dec ? (const T*)a.k_rope : (const T*)a.k;
+  T* dqn = dec ? (T*)a.dq_rope : (T*)a.dq;
+  T* dkn = dec ? (T*)a.dk_rope : (T*)a.dk;
+  T* dqd = dec ? (T*)a.dq : nullptr;
+  T* dkd = dec ? (T*)a.dk : nullptr;
+  const int chunk = pick_chunk(p);
+  const int nchunks = (int)cdiv64(p.L, chunk);
+  char* ws = (char*)a.workspace;
+  float* partial = (float*)ws;
+  ws += partial_bytes(p);
+  float* St = (float*)ws;
+  ws += state_bytes(p);
+  float* dS = (float*)ws;
+  ws += state_bytes(p);
+  float* dSt = (float*)ws;
+  ws += state_bytes(p);
+  float* dkm = (float*)ws;
+  const int64_t nh = (int64_t)p.N * p.H;
+  transpose_state_kernel<<<dim3((unsigned)nh), dim3(kThreads), 0, st>>>(a.s, St, p.DK, p.DV);
+  switch (micro(p)) {
+    case 2:
+      launch_bwd_a<T, 2>(p, qn, q, (const T*)a.dout, a.s, St, a.km, dqn, dqd, partial, chunk,
+                         nchunks, st);
+      break;
+    case 4:
+      launch_bwd_a<T, 4>(p, qn, q, (const T*)a.dout, a.s, St, a.km, dqn, dqd, partial, chunk,
+                         nchunks, st);
+      break;
+    default:
+      launch_bwd_a<T, 8>(p, qn, q, (const T*)a.dout, a.s, St, a.km, dqn, dqd, partial, chunk,
+                         nchunks, st);
+      break;
+  }
+  state_reduce_kernel<<<dim3((unsigned)nh), dim3(kThreads), 0, st>>>(p, partial, chunk, nchunks, dS,
+                                                                    dSt, dkm);
+  const int ntiles = (int)cdiv64(p.L, kTile);
+  bwd_b_kernel<T><<<dim3((unsigned)(nh * ntiles)), dim3(kThreads), 0, st>>>(
+      p, kn, v, dS, dSt, dkm, dkn, dkd, (T*)a.dv, ntiles);
+  return kOk;
+}
+
+int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
+  switch (dtype) {
+    case kF16: return forward_t<_Float16>(p, a, st);
+    case kBF16: return forward_t<__bf16>(p, a, st);
+    case kF32: return forward_t<float>(p, a, st);
+  }
+  return kErrUnsupported;
+}
+
+int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
+  switch (dtype) {
+    case kF16: return backward_t<_Float16>(p, a, st);
+    case kBF16: return backward_t<__bf16>(p, a, st);
+    case kF32: return backward_t<float>(p, a, st);
+  }
+  return kErrUnsupported;
+}
+
+}  // namespace generic
+}  // namespace fbla

@@ -1,0 +1,176 @@
+"""ctypes binding of libfbla_hip.so (declared in include/flash_bla_hip.h).
+
+PyTorch is used for device memory (outputs, state, workspace come from its
+caching allocator) and for the current stream; all arithmetic happens inside the
+library.  There is no fallback: a missing library or a non-GPU tensor raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "libfbla_hip.so")
+_lib = None
+
+F16, BF16, F32 = 0, 1, 2
+NORMALIZE, DECOUPLED, DEFAULT_SCALE = 1, 2, 4
+
+_DTYPES = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
+
+_vp, _i64, _i32, _f32, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float,
+                              ctypes.c_size_t)
+
+_SIGNATURES = {
+    "fbla_version": (ctypes.c_int, []),
+    "fbla_last_error": (ctypes.c_char_p, []),
+    "fbla_la_workspace_bytes": (_sz, [_i32, _i64, _i64, _i64, _i32, _i32, _i32, _i32]),
+    "fbla_la_fwd": (_i32, [_vp] * 9 + [_sz, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
+    "fbla_la_bwd": (_i32, [_vp] * 14 + [_sz, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
+    "fbla_varlen_workspace_bytes": (_sz, [_i32, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32]),
+    "fbla_varlen_fwd": (_i32, [_vp] * 8 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
+    "fbla_varlen_bwd": (_i32, [_vp] * 11 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
+}
+
+
+def lib_path():
+    return _LIB_PATH
+
+
+def exported_symbols():
+    """Names this binding expects the shared library to export."""
+    return sorted(_SIGNATURES)
+
+
+def lib():
+    """Load libfbla_hip.so once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                f"flash_bla: HIP library not found at {_LIB_PATH}; build it with "
+                "`make -C flash-bidirectional-linear-attention_amd/csrc` (there is no fallback path)")
+        handle = ctypes.CDLL(_LIB_PATH)
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = handle
+    return _lib
+
+
+def _check(rc, what):
+    if rc != 0:
+        msg = lib().fbla_last_error().decode("utf-8", "replace")
+        exc = ValueError if rc in (-1, -2) else RuntimeError
+        raise exc(f"{what} failed ({rc}): {msg}")
+
+
+def dtype_code(t):
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError("q, k, and v must have dtype float16, bfloat16, or float32") from None
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _workspace(nbytes, device):
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise ValueError("flash_bla HIP operators need GPU tensors (got a CPU tensor); "
+                             "use the naive_* functions for CPU math")
+
+
+def la_fwd(q, k, v, q_rope, k_rope, scale, eps, flags):
+    """Dense forward: returns (o, s, km).  Tensors must be contiguous [B,H,L,D]."""
+    _require_gpu(q, k, v, q_rope, k_rope)
+    L = lib()
+    B, H, T, DK = q.shape
+    DV = v.shape[-1]
+    code = dtype_code(q)
+    dev = q.device
+    o = torch.empty_like(v)
+    s = torch.empty(B, H, DK, DV, dtype=torch.float32, device=dev)
+    km = torch.empty(B, H, DK, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        ws = _workspace(L.fbla_la_workspace_bytes(0, B, H, T, DK, DV, code, flags), dev)
+        rc = L.fbla_la_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(q_rope), _ptr(k_rope), _ptr(o), _ptr(s),
+                           _ptr(km), _ptr(ws), ws.numel(), B, H, T, DK, DV, code, flags,
+                           float(scale), float(eps), _stream(dev))
+    _check(rc, "fbla_la_fwd")
+    return o, s, km
+
+
+def la_bwd(q, k, v, q_rope, k_rope, do, s, km, scale, eps, flags):
+    """Dense backward: returns (dq, dk, dv, dq_rope, dk_rope)."""
+    _require_gpu(q, k, v, do)
+    L = lib()
+    B, H, T, DK = q.shape
+    DV = v.shape[-1]
+    code = dtype_code(q)
+    dev = q.device
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dqr = torch.empty_like(q_rope) if flags & DECOUPLED else None
+    dkr = torch.empty_like(k_rope) if flags & DECOUPLED else None
+    with torch.cuda.device(dev):
+        ws = _workspace(L.fbla_la_workspace_bytes(1, B, H, T, DK, DV, code, flags), dev)
+        rc = L.fbla_la_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(q_rope), _ptr(k_rope), _ptr(do), _ptr(s),
+                           _ptr(km), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dqr), _ptr(dkr), _ptr(ws),
+                           ws.numel(), B, H, T, DK, DV, code, flags, float(scale), float(eps),
+                           _stream(dev))
+    _check(rc, "fbla_la_bwd")
+    return dq, dk, dv, dqr, dkr
+
+
+def varlen_fwd(q, k, v, cu_seqlens, max_seqlen, scale, eps):
+    """Packed forward: returns (o, s, km).  Tensors contiguous [T,H,D]."""
+    _require_gpu(q, k, v, cu_seqlens)
+    L = lib()
+    T, H, DK = q.shape
+    DV = v.shape[-1]
+    N = cu_seqlens.numel() - 1
+    code = dtype_code(q)
+    dev = q.device
+    flags = NORMALIZE | (DEFAULT_SCALE if scale is None else 0)
+    o = torch.empty_like(v)
+    s = torch.empty(N, H, DK, DV, dtype=torch.float32, device=dev)
+    km = torch.empty(N, H, DK, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        ws = _workspace(L.fbla_varlen_workspace_bytes(0, T, N, H, max_seqlen, DK, DV, code, flags), dev)
+        rc = L.fbla_varlen_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(cu_seqlens), _ptr(o), _ptr(s),
+                               _ptr(km), _ptr(ws), ws.numel(), T, N, H, max_seqlen, DK, DV, code,
+                               flags, 0.0 if scale is None else float(scale), float(eps),
+                               _stream(dev))
+    _check(rc, "fbla_varlen_fwd")
+    return o, s, km
+
+
+def varlen_bwd(q, k, v, cu_seqlens, max_seqlen, do, s, km, scale, eps):
+    """Packed backward: returns (dq, dk, dv)."""
+    _require_gpu(q, k, v, do, cu_seqlens)
+    L = lib()
+    T, H, DK = q.shape
+    DV = v.shape[-1]
+    N = cu_seqlens.numel() - 1
+    code = dtype_code(q)
+    dev = q.device
+    flags = NORMALIZE | (DEFAULT_SCALE if scale is None else 0)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    with torch.cuda.device(dev):
+        ws = _workspace(L.fbla_varlen_workspace_bytes(1, T, N, H, max_seqlen, DK, DV, code, flags), dev)
+        rc = L.fbla_varlen_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(cu_seqlens), _ptr(do), _ptr(s),
+                               _ptr(km), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws.numel(), T, N,
+                               H, max_seqlen, DK, DV, code, flags,
+                               0.0 if scale is None else float(scale), float(eps), _stream(dev))
+    _check(rc, "fbla_varlen_bwd")
+    return dq, dk, dv

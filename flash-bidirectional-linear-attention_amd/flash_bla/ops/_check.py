@@ -1,0 +1,26 @@
+"""Argument validation shared by the dense operators."""
+import torch
+
+
+def check_dense(name, q, k, v, extra=()):
+    """The reference's dense wrappers validate nothing (linear_attn/fused.py:456-480);
+    the HIP kernels index raw memory, so shapes, dtypes and devices are checked here."""
+    tensors = (q, k, v) + tuple(extra)
+    for t in tensors:
+        if not isinstance(t, torch.Tensor) or t.ndim != 4:
+            raise ValueError(f"{name}: tensors must have shape (B, H, L, D)")
+    if q.shape != k.shape or any(t.shape != q.shape for t in extra):
+        raise ValueError(f"{name}: q and k (and their rope versions) must have identical shapes, "
+                         f"got {[tuple(t.shape) for t in (q, k) + tuple(extra)]}")
+    if q.shape[:3] != v.shape[:3]:
+        raise ValueError(f"{name}: q, k, and v must have matching batch, head and token dimensions")
+    if any(t.device != q.device for t in tensors):
+        raise ValueError(f"{name}: all tensors must be on the same device")
+    if any(t.dtype != q.dtype for t in tensors):
+        raise ValueError(f"{name}: all tensors must have the same dtype")
+    if not q.is_cuda:
+        raise ValueError(f"{name}: tensors must be GPU tensors")
+    if q.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        raise TypeError(f"{name}: dtype must be float16, bfloat16, or float32")
+    if not (0 < q.shape[-1] <= 128 and 0 < v.shape[-1] <= 128):
+        raise ValueError(f"{name}: key_dim and value_dim must be between 1 and 128")

@@ -1,0 +1,60 @@
+"""Normalised bidirectional linear attention (drop-in for
+flash_bla/ops/linear_attn/fused.py:350-480).
+
+    S = scale * K^T V,  km = mean_t k_t,  o_t = (q_t S) / (q_t . km + eps)
+
+The forward and backward launch hand-written gfx950 kernels through
+libfbla_hip.so.  The state (S, km) is kept in fp32 and saved for the backward,
+which recomputes o.dO from q and S instead of re-reading o.
+"""
+from typing import Optional
+
+import torch
+
+from flash_bla import _hip
+from flash_bla.ops._check import check_dense
+from flash_bla.utils import contiguous
+
+
+class LinearAttnFunction(torch.autograd.Function):
+    """Counterpart of LinearAttnFunction (linear_attn/fused.py:350-453)."""
+
+    @staticmethod
+    @contiguous
+    def forward(ctx, q, k, v, scale, eps):
+        o, s, km = _hip.la_fwd(q, k, v, None, None, scale, eps, _hip.NORMALIZE)
+        ctx.save_for_backward(q, k, v, s, km)
+        ctx.scale = scale
+        ctx.eps = eps
+        return o
+
+    @staticmethod
+    @contiguous
+    def backward(ctx, do):
+        q, k, v, s, km = ctx.saved_tensors
+        dq, dk, dv, _, _ = _hip.la_bwd(q, k, v, None, None, do, s, km, ctx.scale, ctx.eps,
+                                       _hip.NORMALIZE)
+        return dq, dk, dv, None, None
+
+
+def linear_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    scale: Optional[float] = None,
+    eps: float = 1e-6
+) -> torch.Tensor:
+    r"""
+    Args:
+        q: queries of shape `(B, H, L, K)` (positive features, e.g. elu+1)
+        k: keys of shape `(B, H, L, K)`
+        v: values of shape `(B, H, L, V)`
+        scale: factor applied to the key-value state; defaults to `1 / L`
+            (linear_attn/fused.py:477-478).
+        eps: constant added to the denominator.
+    Returns the output of shape `(B, H, L, V)` with `v`'s dtype.
+    """
+    check_dense("linear_attention", q, k, v)
+    if scale is None:
+        scale = k.shape[-2] ** -1.0
+    return LinearAttnFunction.apply(q, k, v, scale, eps)

@@ -1,0 +1,50 @@
+"""Helpers shared by the operator wrappers (counterpart of flash_bla/utils.py:9-15,45-67)."""
+import functools
+import warnings
+
+import torch
+
+
+def contiguous(fn):
+    """Make every tensor argument of an autograd forward/backward contiguous
+    (flash_bla/utils.py:9-15)."""
+    @functools.wraps(fn)
+    def wrapper(ctx, *args, **kwargs):
+        args = tuple(a.contiguous() if isinstance(a, torch.Tensor) else a for a in args)
+        kwargs = {n: (a.contiguous() if isinstance(a, torch.Tensor) else a) for n, a in kwargs.items()}
+        return fn(ctx, *args, **kwargs)
+    return wrapper
+
+
+def get_abs_err(x, y):
+    """Largest absolute difference (flash_bla/utils.py:45-46)."""
+    return (x.detach() - y.detach()).flatten().abs().max().item()
+
+
+def get_err_ratio(x, y):
+    """RMS(x - y) / RMS(x) (flash_bla/utils.py:49-52)."""
+    err = (x.detach() - y.detach()).flatten().square().mean().sqrt().item()
+    base = x.detach().flatten().square().mean().sqrt().item()
+    return err / (base + 1e-8)
+
+
+def get_max_rel_err(ref, x):
+    """max|x - ref| / max|ref|: the parity figure used for the HIP kernels."""
+    ref = ref.detach().double()
+    x = x.detach().double()
+    return ((x - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item()
+
+
+def assert_close(prefix, ref, tri, ratio, warning=False, err_atol=1e-6):
+    """Same acceptance rule as flash_bla/utils.py:55-67."""
+    abs_atol = get_abs_err(ref, tri)
+    error_rate = get_err_ratio(ref, tri)
+    msg = f"{prefix:>8} diff: {abs_atol:.6f} ratio: {error_rate:.6f}"
+    if abs_atol <= err_atol:
+        return abs_atol
+    if warning or (error_rate < 0.01 or abs_atol <= 0.3):
+        if error_rate > ratio:
+            warnings.warn(msg)
+        return error_rate
+    assert error_rate < ratio, msg
+    return error_rate

@@ -1,0 +1,114 @@
+/*
+ * flash_bla_hip.h -- C ABI of libfbla_hip.so: bidirectional (non-causal) linear
+ * attention for AMD gfx950 (MI355X).
+ *
+ * The reference (fla-org/flash-bidirectional-linear-attention, `flash_bla`) has
+ * no native layer: its operators are torch.autograd.Function classes that launch
+ * Triton kernels.  Each entry point below replaces the kernel launches made by
+ * one of those Functions; the Python operator layer keeps the reference's
+ * signatures and binds these symbols with ctypes.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless stated otherwise; the library
+ *     never allocates, frees or retains device memory: outputs and the workspace
+ *     are provided by the caller (size from the *_workspace_bytes queries);
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*); no call
+ *     synchronises the device;
+ *   - return value 0 = success, negative = error (fbla_last_error() gives the
+ *     text for the calling thread); no C++ exception crosses the boundary;
+ *   - dense tensors are contiguous [B,H,L,D]; packed tensors are contiguous
+ *     [T_total,H,D] with int32 cu_seqlens[N+1] on the device;
+ *   - the state tensors s [B*H,DK,DV] (or [N*H,DK,DV]) and km [..,DK] are fp32.
+ *     s already includes `scale`; km is the mean key.  Forward writes them,
+ *     backward reads them (the reference saves the same two tensors in its
+ *     autograd context: linear_attn/fused.py:395);
+ *   - reductions over tokens are two-stage and fixed-order: results are
+ *     bit-identical from run to run.
+ */
+#ifndef FLASH_BLA_HIP_H
+#define FLASH_BLA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type of q/k/v/o and of the gradients */
+#define FBLA_F16 0
+#define FBLA_BF16 1
+#define FBLA_F32 2
+
+/* flags */
+#define FBLA_NORMALIZE 1     /* o = (q S)/(q.km + eps); clear = simple_la (no denominator) */
+#define FBLA_DECOUPLED 2     /* numerator from q_rope/k_rope, denominator from q/k */
+#define FBLA_DEFAULT_SCALE 4 /* packed layout only: scale = 1/len_i per sequence */
+
+/* error codes */
+#define FBLA_OK 0
+#define FBLA_ERR_BAD_ARG (-1)
+#define FBLA_ERR_UNSUPPORTED (-2)
+#define FBLA_ERR_WORKSPACE (-3)
+#define FBLA_ERR_LAUNCH (-4)
+
+/* Library version (major*10000 + minor*100 + patch). */
+int fbla_version(void);
+
+/* Message of the last error raised on the calling thread ("" if none). */
+const char* fbla_last_error(void);
+
+/* Workspace (bytes) needed by fbla_la_fwd (pass=0) / fbla_la_bwd (pass=1) for a
+ * dense problem.  Replaces the torch.empty temporaries of
+ * linear_attn/fused.py:362-363,422-423 (which grow with L/32; ours do not). */
+size_t fbla_la_workspace_bytes(int pass, int64_t B, int64_t H, int64_t L, int DK, int DV,
+                               int dtype, int flags);
+
+/* Dense forward.  Replaces the launches in
+ *   LinearAttnFunction.forward        flash_bla/ops/linear_attn/fused.py:352-398
+ *   SimpleLinearAttnFunction.forward  flash_bla/ops/simple_la/fused.py:495-535   (flags without FBLA_NORMALIZE)
+ *   DecoupledLAFunction.forward       flash_bla/ops/linear_attn/decoupled.py:413-460 (FBLA_DECOUPLED)
+ * q,k,(q_rope,k_rope): [B,H,L,DK]; v,o: [B,H,L,DV]; q_rope/k_rope NULL unless decoupled. */
+int fbla_la_fwd(const void* q, const void* k, const void* v, const void* q_rope,
+                const void* k_rope, void* o, float* s, float* km, void* workspace,
+                size_t workspace_bytes, int64_t B, int64_t H, int64_t L, int DK, int DV, int dtype,
+                int flags, float scale, float eps, void* stream);
+
+/* Dense backward.  Replaces the launches in
+ *   LinearAttnFunction.backward        flash_bla/ops/linear_attn/fused.py:400-453
+ *   SimpleLinearAttnFunction.backward  flash_bla/ops/simple_la/fused.py:537-626
+ *   DecoupledLAFunction.backward       flash_bla/ops/linear_attn/decoupled.py:462-509
+ * `o` is not an input: o.dO is recomputed from q and s.  dq_rope/dk_rope are
+ * written only when decoupled (then dq/dk receive the denominator gradients). */
+int fbla_la_bwd(const void* q, const void* k, const void* v, const void* q_rope,
+                const void* k_rope, const void* dout, const float* s, const float* km, void* dq,
+                void* dk, void* dv, void* dq_rope, void* dk_rope, void* workspace,
+                size_t workspace_bytes, int64_t B, int64_t H, int64_t L, int DK, int DV, int dtype,
+                int flags, float scale, float eps, void* stream);
+
+/* Workspace for the packed (variable-length) entry points. */
+size_t fbla_varlen_workspace_bytes(int pass, int64_t total_tokens, int64_t N, int64_t H,
+                                   int64_t max_seqlen, int DK, int DV, int dtype, int flags);
+
+/* Packed forward.  Replaces VarlenLinearAttnFunction.forward
+ * (flash_bla/ops/linear_attn/varlen.py:339-422).  max_seqlen is an upper bound on
+ * the sequence lengths and only sizes the launch; any value >= the true maximum
+ * gives the same result (tests/ops/test_varlen_linear_attn.py:45-55).  With
+ * FBLA_DEFAULT_SCALE each sequence uses 1/len_i (varlen.py:66) and `scale` is ignored.
+ * s: [N*H,DK,DV], km: [N*H,DK] fp32. */
+int fbla_varlen_fwd(const void* q, const void* k, const void* v, const int32_t* cu_seqlens,
+                    void* o, float* s, float* km, void* workspace, size_t workspace_bytes,
+                    int64_t total_tokens, int64_t N, int64_t H, int64_t max_seqlen, int DK, int DV,
+                    int dtype, int flags, float scale, float eps, void* stream);
+
+/* Packed backward.  Replaces VarlenLinearAttnFunction.backward (varlen.py:426-505). */
+int fbla_varlen_bwd(const void* q, const void* k, const void* v, const int32_t* cu_seqlens,
+                    const void* dout, const float* s, const float* km, void* dq, void* dk, void* dv,
+                    void* workspace, size_t workspace_bytes, int64_t total_tokens, int64_t N,
+                    int64_t H, int64_t max_seqlen, int DK, int DV, int dtype, int flags,
+                    float scale, float eps, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASH_BLA_HIP_H */

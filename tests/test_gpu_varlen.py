@@ -1,0 +1,144 @@
+"""GPU parity of varlen_linear_attention: the reference's own test matrix
+(tests/ops/test_varlen_linear_attn.py:11-55) plus layout equivalences."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import TOL, make_qkv, max_rel_err, np64
+from oracle import closed_form as cf
+from oracle import torch_ref as tr
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _cu(lengths, device="cuda"):
+    return torch.tensor([0] + list(np.cumsum(lengths)), dtype=torch.int32, device=device)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=str)
+@pytest.mark.parametrize("scale", [None, 0.02])
+@pytest.mark.parametrize("heads", [1, 8])
+@pytest.mark.parametrize(("key_dim", "value_dim"), [(8, 8), (17, 13), (64, 48), (128, 128)])
+def test_varlen_linear_attention(dtype, scale, heads, key_dim, value_dim):
+    """The reference's parametrised case, same seed, lengths, distributions and
+    assert_close tolerances; the oracle stands in for naive_varlen_linear_attn."""
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    torch.manual_seed(42)
+    lengths = [8, 17, 32]
+    total = sum(lengths)
+    cu = _cu(lengths)
+    q = (F.elu(torch.randn(total, heads, key_dim, dtype=dtype, device="cuda")) + 1).requires_grad_()
+    k = (F.elu(torch.randn(total, heads, key_dim, dtype=dtype, device="cuda")) + 1).requires_grad_()
+    v = torch.randn(total, heads, value_dim, dtype=dtype, device="cuda", requires_grad=True)
+    do = torch.randn_like(v)
+    q_ref, k_ref, v_ref = (x.detach().clone().requires_grad_() for x in (q, k, v))
+
+    out = varlen_linear_attention(q, k, v, cu, max(lengths), scale=scale)
+    out_ref = tr.naive_varlen_linear_attn(q_ref, k_ref, v_ref, cu, scale=scale)
+    out.backward(do)
+    out_ref.backward(do)
+    atol, rtol = (1e-5, 1e-4) if dtype == torch.float32 else (2e-2, 8e-2)
+    torch.testing.assert_close(out, out_ref, atol=atol, rtol=rtol)
+    torch.testing.assert_close(q.grad, q_ref.grad, atol=atol, rtol=rtol)
+    torch.testing.assert_close(k.grad, k_ref.grad, atol=atol, rtol=rtol)
+    torch.testing.assert_close(v.grad, v_ref.grad, atol=atol, rtol=rtol)
+    # and the stricter gate against the float64 closed form
+    g = cf.varlen_backward(np64(q), np64(k), np64(v), np64(do), cu.cpu().numpy(), scale)
+    assert max_rel_err(out, g["o"]) <= TOL[dtype]
+    for name, t in (("dq", q), ("dk", k), ("dv", v)):
+        assert max_rel_err(t.grad, g[name]) <= TOL[dtype], name
+
+
+def test_varlen_linear_attention_oversized_max_seqlen():
+    """tests/ops/test_varlen_linear_attn.py:45-55."""
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    lengths = [7, 11]
+    cu = _cu(lengths)
+    g = torch.Generator().manual_seed(0)
+    q = torch.rand(sum(lengths), 2, 16, generator=g).cuda()
+    k = torch.rand(sum(lengths), 2, 16, generator=g).cuda()
+    v = torch.randn(sum(lengths), 2, 16, generator=g).cuda()
+    expected = varlen_linear_attention(q, k, v, cu, max(lengths))
+    oversized = varlen_linear_attention(q, k, v, cu, q.shape[0])
+    torch.testing.assert_close(oversized, expected)
+    assert torch.equal(oversized, expected)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32], ids=str)
+@pytest.mark.parametrize("D", [64, 128])
+def test_varlen_ragged_batch(dtype, D):
+    """A scaled-down BASELINE config 3: ragged lengths, 16 heads, fwd + bwd."""
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    g = torch.Generator().manual_seed(42)
+    lengths = torch.randint(1, 300, (9,), generator=g).tolist() + [1, 513]
+    T = sum(lengths)
+    q, k, v, do = make_qkv((T, 16, D), (T, 16, D), dtype, 5)
+    cu = _cu(lengths)
+    leaves = [x.cuda().requires_grad_() for x in (q, k, v)]
+    o = varlen_linear_attention(*leaves, cu, max(lengths))
+    o.backward(do.cuda())
+    ref = cf.varlen_backward(np64(q), np64(k), np64(v), np64(do), cu.cpu().numpy())
+    assert max_rel_err(o, ref["o"]) <= TOL[dtype]
+    for name, t in zip(("dq", "dk", "dv"), leaves):
+        # gradients of different sequences differ in magnitude by their lengths:
+        # compare sequence by sequence
+        for b, e in zip(cu[:-1].tolist(), cu[1:].tolist()):
+            assert max_rel_err(t.grad[b:e], ref[name][b:e]) <= TOL[dtype], (name, b, e)
+
+
+def test_varlen_single_sequence_equals_dense():
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    q, k, v, do = (x.cuda() for x in make_qkv((333, 4, 64), (333, 4, 64), torch.float16, 9))
+    cu = _cu([333])
+    o = varlen_linear_attention(q, k, v, cu, 333)
+    od = linear_attention(*(x.transpose(0, 1)[None] for x in (q, k, v)))
+    assert max_rel_err(o, od[0].transpose(0, 1)) < 1e-3
+
+
+def test_varlen_zero_length_sequence_is_skipped():
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    lengths = [5, 0, 9]
+    q, k, v, do = make_qkv((14, 2, 16), (14, 2, 16), torch.float32, 13)
+    cu = _cu(lengths)
+    leaves = [x.cuda().requires_grad_() for x in (q, k, v)]
+    o = varlen_linear_attention(*leaves, cu, 9)
+    o.backward(do.cuda())
+    ref = cf.varlen_backward(np64(q), np64(k), np64(v), np64(do), cu.cpu().numpy())
+    assert max_rel_err(o, ref["o"]) <= 1e-5
+    for name, t in zip(("dq", "dk", "dv"), leaves):
+        assert torch.isfinite(t.grad).all()
+        assert max_rel_err(t.grad, ref[name]) <= 1e-5
+
+
+def test_varlen_rejects_bad_cu_seqlens_on_gpu():
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    q = torch.rand(10, 2, 8, device="cuda")
+    with pytest.raises(ValueError, match="int32"):
+        varlen_linear_attention(q, q, q, torch.tensor([0, 10], device="cuda"), 10)
+    with pytest.raises(ValueError, match="positive integer"):
+        varlen_linear_attention(q, q, q, _cu([10]), 0)
+    with pytest.raises(TypeError):
+        varlen_linear_attention(q.double(), q.double(), q.double(), _cu([10]), 10)
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "varlen_*.npz"))), ids=os.path.basename)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32], ids=str)
+def test_varlen_golden_fixtures(path, dtype):
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    d = np.load(path)
+    scale = None if d["meta"][0] < 0 else float(d["meta"][0])
+    leaves = [torch.from_numpy(d[n]).to(dtype).cuda().requires_grad_() for n in ("q", "k", "v")]
+    cu = torch.from_numpy(d["cu_seqlens"]).cuda()
+    lens = np.diff(d["cu_seqlens"])
+    o = varlen_linear_attention(*leaves, cu, int(lens.max()), scale=scale, eps=float(d["meta"][1]))
+    o.backward(torch.from_numpy(d["do"]).to(dtype).cuda())
+    assert max_rel_err(o, d["ref_o"]) <= TOL[dtype]
+    for name, t in zip(("dq", "dk", "dv"), leaves):
+        for b, e in zip(d["cu_seqlens"][:-1], d["cu_seqlens"][1:]):
+            assert max_rel_err(t.grad[b:e], d["ref_" + name][b:e]) <= TOL[dtype], name

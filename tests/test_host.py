@@ -1,0 +1,101 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every
+declared symbol, host-only entry points answer, argument validation raises the
+reference's exception types, and the oracle reproduces the golden fixtures."""
+import ctypes
+import glob
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from flash_bla import _hip
+from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+from flash_bla.ops.linear_attn.fused import linear_attention
+from oracle import closed_form as cf
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+def _declared_symbols():
+    names = set()
+    for path in glob.glob(os.path.join(ROOT, "include", "*.h")):
+        text = re.sub(r"/\*.*?\*/", "", open(path).read(), flags=re.S)
+        names.update(re.findall(r"\b(fbla_\w+)\s*\(", text))
+    return sorted(names)
+
+
+def test_library_exports_every_declared_symbol():
+    declared = _declared_symbols()
+    assert len(declared) >= 8
+    handle = ctypes.CDLL(_hip.lib_path())
+    for name in declared:
+        assert hasattr(handle, name), f"{name} declared in include/ but not exported"
+    assert set(declared) == set(_hip.exported_symbols())
+
+
+def test_host_only_entry_points():
+    L = _hip.lib()
+    assert L.fbla_version() >= 100
+    fwd = L.fbla_la_workspace_bytes(0, 8, 16, 16384, 64, 64, _hip.F16, _hip.NORMALIZE)
+    bwd = L.fbla_la_workspace_bytes(1, 8, 16, 16384, 64, 64, _hip.F16, _hip.NORMALIZE)
+    assert 0 < fwd <= bwd < (1 << 30)
+    # workspace does not grow with L once the chunk count saturates
+    assert L.fbla_la_workspace_bytes(0, 8, 16, 32768, 64, 64, _hip.F16, _hip.NORMALIZE) <= 2 * fwd
+    assert L.fbla_varlen_workspace_bytes(0, 73000, 64, 16, 2048, 64, 64, _hip.BF16, 5) > 0
+
+
+def test_bad_arguments_return_error_codes_without_touching_the_gpu():
+    L = _hip.lib()
+    args = [None] * 9 + [0, 1, 1, 16, 0, 64, _hip.F16, _hip.NORMALIZE, 1.0, 1e-6, None]
+    assert L.fbla_la_fwd(*args) == -2          # DK = 0
+    assert b"head dims" in L.fbla_last_error()
+    args[13:15] = [64, 64]
+    args[15] = 7
+    assert L.fbla_la_fwd(*args) == -1          # unknown dtype
+    args[15], args[16] = _hip.F16, _hip.DECOUPLED
+    assert L.fbla_la_fwd(*args) == -1          # decoupled without normalize
+    args[16] = _hip.NORMALIZE
+    assert L.fbla_la_fwd(*args) == -1          # null pointers with a non-empty problem
+    assert b"null" in L.fbla_last_error()
+    assert L.fbla_la_workspace_bytes(0, 1, 1, 16, 129, 64, 0, 1) == 0
+
+
+def test_varlen_validation_matches_reference_exception_types():
+    q = torch.rand(10, 2, 8)
+    cu = torch.tensor([0, 4, 10], dtype=torch.int32)
+    with pytest.raises(ValueError, match="shape"):
+        varlen_linear_attention(q[0], q, q, cu, 6)
+    with pytest.raises(ValueError, match="identical shapes"):
+        varlen_linear_attention(q, q[:, :, :4], q, cu, 6)
+    with pytest.raises(ValueError, match="matching token"):
+        varlen_linear_attention(q, q, q[:5], cu, 6)
+    with pytest.raises(ValueError, match="same dtype"):
+        varlen_linear_attention(q, q, q.double(), cu, 6)
+    with pytest.raises(ValueError, match="CUDA"):
+        varlen_linear_attention(q, q, q, cu, 6)   # CPU tensors: no silent fallback
+
+
+def test_dense_ops_refuse_cpu_tensors():
+    q = torch.rand(1, 2, 8, 4)
+    with pytest.raises(ValueError, match="GPU"):
+        linear_attention(q, q, q)
+    with pytest.raises(ValueError, match="identical shapes"):
+        linear_attention(q, q[..., :2], q)
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "*.npz"))), ids=os.path.basename)
+def test_oracle_reproduces_golden_fixture(path):
+    d = np.load(path)
+    if "cu_seqlens" in d:
+        scale = None if d["meta"][0] < 0 else float(d["meta"][0])
+        g = cf.varlen_backward(d["q"], d["k"], d["v"], d["do"], d["cu_seqlens"], scale, float(d["meta"][1]))
+    else:
+        s, eps, normalize, dec = d["meta"]
+        kw = dict(q_rope=d["q_rope"], k_rope=d["k_rope"]) if dec else {}
+        g = cf.dense_backward(d["q"], d["k"], d["v"], d["do"], float(s), float(eps), bool(normalize), **kw)
+    for name, ref in d.items():
+        if name.startswith("ref_") and name[4:] in g:
+            np.testing.assert_allclose(g[name[4:]], ref, rtol=1e-12, atol=1e-14)

@@ -1,0 +1,221 @@
+"""Pins the CPU oracle (oracle/) without a GPU.
+
+The reference holds no golden vectors for these operators, so the oracle is
+pinned by (i) an O(L^2) brute-force evaluation in plain C that never forms the
+K^T V state, (ii) closed-form special cases and invariants, (iii) agreement of
+the three independent restatements (torch formulas, float64 closed forms, C),
+and (iv) torch.autograd / gradcheck for the hand-derived backward.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import make_qkv, np64
+from oracle import brute, closed_form as cf, piecewise as pw, torch_ref as tr
+
+
+def _dense_inputs(B=2, H=3, L=37, DK=16, DV=8, seed=0, n_extra=0):
+    return make_qkv((B, H, L, DK), (B, H, L, DV), torch.float64, seed, n_extra)
+
+
+@pytest.mark.parametrize("L,DK,DV", [(1, 4, 3), (37, 16, 8), (64, 8, 24)])
+@pytest.mark.parametrize("scale", [None, 0.37])
+def test_linear_attn_matches_brute_force(L, DK, DV, scale):
+    q, k, v, _ = _dense_inputs(1, 2, L, DK, DV)
+    s = 1.0 / L if scale is None else scale
+    o_cf = cf.dense_forward(np64(q), np64(k), np64(v), s)[0]
+    o_tr = np64(tr.naive_linear_attn(q, k, v, scale))
+    for h in range(2):
+        o_b = brute.brute_linear_attn(np64(q)[0, h], np64(k)[0, h], np64(v)[0, h], s)
+        np.testing.assert_allclose(o_cf[0, h], o_b, rtol=1e-12, atol=1e-13)
+        np.testing.assert_allclose(o_tr[0, h], o_b, rtol=1e-11, atol=1e-12)
+
+
+def test_simple_la_matches_brute_force():
+    q, k, v, _ = _dense_inputs(1, 2, 29, 12, 20)
+    o_tr = np64(tr.naive_simple_la(q, k, v))
+    o_cf = cf.dense_forward(np64(q), np64(k), np64(v), 12 ** -0.5, normalize=False)[0]
+    for h in range(2):
+        o_b = brute.brute_linear_attn(np64(q)[0, h], np64(k)[0, h], np64(v)[0, h], 12 ** -0.5,
+                                      normalize=False)
+        np.testing.assert_allclose(o_tr[0, h], o_b, rtol=1e-11, atol=1e-12)
+        np.testing.assert_allclose(o_cf[0, h], o_b, rtol=1e-12, atol=1e-13)
+    # associativity: scale * (q k^T) v
+    ref = (q @ k.transpose(-1, -2)) @ v * 12 ** -0.5
+    np.testing.assert_allclose(o_tr, np64(ref), rtol=1e-11, atol=1e-12)
+
+
+def test_decoupled_matches_brute_force_and_reduces_to_plain():
+    q, k, v, _, qr, kr = _dense_inputs(1, 2, 33, 8, 8, n_extra=2)
+    o_tr = np64(tr.naive_decoupled_la(q, k, qr, kr, v))
+    o_cf = cf.dense_forward(np64(q), np64(k), np64(v), 1 / 33, q_rope=np64(qr), k_rope=np64(kr))[0]
+    for h in range(2):
+        o_b = brute.brute_linear_attn(np64(q)[0, h], np64(k)[0, h], np64(v)[0, h], 1 / 33,
+                                      q_rope=np64(qr)[0, h], k_rope=np64(kr)[0, h])
+        np.testing.assert_allclose(o_tr[0, h], o_b, rtol=1e-11, atol=1e-12)
+        np.testing.assert_allclose(o_cf[0, h], o_b, rtol=1e-12, atol=1e-13)
+    same = tr.naive_decoupled_la(q, k, q, k, v)
+    np.testing.assert_allclose(np64(same), np64(tr.naive_linear_attn(q, k, v)), rtol=1e-13)
+
+
+def test_invariants():
+    q, k, v, _ = _dense_inputs(1, 1, 50, 8, 5)
+    L = 50
+    o = tr.naive_linear_attn(q, k, v)
+    # constant v = c  =>  o = c * z / (z + eps) with z = q.km  (default scale 1/L)
+    c = torch.full_like(v, 1.7)
+    z = (q @ k.mean(-2, keepdim=True).transpose(-1, -2))
+    np.testing.assert_allclose(np64(tr.naive_linear_attn(q, k, c)), np64(1.7 * z / (z + 1e-6)).repeat(5, -1),
+                               rtol=1e-12)
+    # joint permutation of (k, v) rows leaves o unchanged
+    perm = torch.randperm(L, generator=torch.Generator().manual_seed(1))
+    np.testing.assert_allclose(np64(tr.naive_linear_attn(q, k[..., perm, :], v[..., perm, :])), np64(o),
+                               rtol=1e-11, atol=1e-13)
+    # k -> a*k leaves o unchanged as eps -> 0
+    np.testing.assert_allclose(np64(tr.naive_linear_attn(q, 3 * k, v, eps=0.0)),
+                               np64(tr.naive_linear_attn(q, k, v, eps=0.0)), rtol=1e-11, atol=1e-13)
+    # linear in v
+    v2 = torch.randn(v.shape, dtype=v.dtype, generator=torch.Generator().manual_seed(2))
+    np.testing.assert_allclose(np64(tr.naive_linear_attn(q, k, 2 * v - 3 * v2)),
+                               np64(2 * o - 3 * tr.naive_linear_attn(q, k, v2)), rtol=1e-10, atol=1e-12)
+    # every output component lies inside the range of the values (positive features)
+    assert (o <= v.max(-2, keepdim=True).values + 1e-12).all()
+    assert (o >= v.min(-2, keepdim=True).values - 1e-12).all()
+    # L = 1, scale = 1:  o = v (q.k)/(q.k + eps)
+    q1, k1, v1 = q[..., :1, :], k[..., :1, :], v[..., :1, :]
+    qk = (q1 * k1).sum(-1, keepdim=True)
+    np.testing.assert_allclose(np64(tr.naive_linear_attn(q1, k1, v1, scale=1.0)), np64(v1 * qk / (qk + 1e-6)),
+                               rtol=1e-12)
+    # the LinFusion layer's torch formula is linear_attn with eps = 1e-4
+    np.testing.assert_allclose(np64(tr.linfusion_torch_mode(q, k, v)),
+                               np64(tr.naive_linear_attn(q, k, v, eps=1e-4)), rtol=1e-11)
+
+
+@pytest.mark.parametrize("variant", ["linear", "simple", "decoupled"])
+def test_closed_form_backward_matches_autograd(variant):
+    q, k, v, do, qr, kr = _dense_inputs(2, 2, 23, 8, 6, n_extra=2)
+    leaves = [t.clone().requires_grad_() for t in (q, k, v, qr, kr)]
+    ql, kl, vl, qrl, krl = leaves
+    if variant == "linear":
+        o = tr.naive_linear_attn(ql, kl, vl, 0.11)
+        g = cf.dense_backward(np64(q), np64(k), np64(v), np64(do), 0.11)
+    elif variant == "simple":
+        o = tr.naive_simple_la(ql, kl, vl, 0.11)
+        g = cf.dense_backward(np64(q), np64(k), np64(v), np64(do), 0.11, normalize=False)
+    else:
+        o = tr.naive_decoupled_la(ql, kl, qrl, krl, vl, 0.11)
+        g = cf.dense_backward(np64(q), np64(k), np64(v), np64(do), 0.11, q_rope=np64(qr),
+                              k_rope=np64(kr))
+    o.backward(do)
+    np.testing.assert_allclose(g["o"], np64(o), rtol=1e-11, atol=1e-13)
+    np.testing.assert_allclose(g["dq"], np64(ql.grad), rtol=1e-9, atol=1e-11)
+    np.testing.assert_allclose(g["dk"], np64(kl.grad), rtol=1e-9, atol=1e-11)
+    np.testing.assert_allclose(g["dv"], np64(vl.grad), rtol=1e-9, atol=1e-11)
+    if variant == "decoupled":
+        np.testing.assert_allclose(g["dq_rope"], np64(qrl.grad), rtol=1e-9, atol=1e-11)
+        np.testing.assert_allclose(g["dk_rope"], np64(krl.grad), rtol=1e-9, atol=1e-11)
+
+
+def test_gradcheck_torch_ref():
+    q, k, v, _ = _dense_inputs(1, 1, 7, 3, 2)
+    args = [t.clone().requires_grad_() for t in (q, k, v)]
+    assert torch.autograd.gradcheck(lambda a, b, c: tr.naive_linear_attn(a, b, c, 0.3), args)
+    assert torch.autograd.gradcheck(lambda a, b, c: tr.naive_simple_la(a, b, c, 0.3), args)
+
+
+def _varlen_inputs(lengths, H=2, DK=8, DV=5, seed=3):
+    T = int(sum(lengths))
+    q, k, v, do = make_qkv((T, H, DK), (T, H, DV), torch.float64, seed)
+    cu = torch.tensor([0] + list(np.cumsum(lengths)), dtype=torch.int32)
+    return q, k, v, do, cu
+
+
+@pytest.mark.parametrize("scale", [None, 0.02])
+def test_varlen_equals_dense_per_sequence(scale):
+    lengths = [8, 17, 32]
+    q, k, v, do, cu = _varlen_inputs(lengths)
+    o = tr.naive_varlen_linear_attn(q, k, v, cu, scale)
+    o_cf = cf.varlen_forward(np64(q), np64(k), np64(v), cu.numpy(), scale)
+    np.testing.assert_allclose(np64(o), o_cf, rtol=1e-11, atol=1e-13)
+    for b, e in zip(cu[:-1].tolist(), cu[1:].tolist()):
+        dense = tr.naive_linear_attn(q[b:e].transpose(0, 1)[None], k[b:e].transpose(0, 1)[None],
+                                     v[b:e].transpose(0, 1)[None], scale)
+        np.testing.assert_allclose(np64(o[b:e]), np64(dense[0].transpose(0, 1)), rtol=1e-11, atol=1e-13)
+    # backward
+    leaves = [t.clone().requires_grad_() for t in (q, k, v)]
+    tr.naive_varlen_linear_attn(*leaves, cu, scale).backward(do)
+    g = cf.varlen_backward(np64(q), np64(k), np64(v), np64(do), cu.numpy(), scale)
+    for name, leaf in zip(("dq", "dk", "dv"), leaves):
+        np.testing.assert_allclose(g[name], np64(leaf.grad), rtol=1e-9, atol=1e-11)
+
+
+def test_varlen_equal_lengths_is_dense_batch():
+    q, k, v, _, cu = _varlen_inputs([16, 16, 16])
+    o = tr.naive_varlen_linear_attn(q, k, v, cu)
+    qd, kd, vd = (t.view(3, 16, 2, -1).permute(0, 2, 1, 3) for t in (q, k, v))
+    od = tr.naive_linear_attn(qd, kd, vd)
+    np.testing.assert_allclose(np64(o), np64(od.permute(0, 2, 1, 3).reshape(48, 2, -1)), rtol=1e-12)
+
+
+# ---------------------------------------------------------------------------
+# piecewise (PISA) oracle: mathematical pins only (reference parity unpinned)
+# ---------------------------------------------------------------------------
+def _pw_inputs(T=200, K=16, V=8, seed=5):
+    g = torch.Generator().manual_seed(seed)
+    return tuple(torch.randn(T, d, generator=g, dtype=torch.float64).numpy() for d in (K, K, V))
+
+
+def test_piecewise_all_blocks_selected_is_softmax_attention():
+    q, k, v = _pw_inputs()
+    NT = -(-200 // 64)
+    idx = np.tile(np.arange(NT), (NT, 1))
+    o = pw.piecewise_forward(q, k, v, idx, 64)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        torch.from_numpy(q)[None], torch.from_numpy(k)[None], torch.from_numpy(v)[None])[0].numpy()
+    np.testing.assert_allclose(o, ref, rtol=1e-10, atol=1e-12)
+
+
+def test_piecewise_constant_keys_per_chunk_zeroth_order_exact():
+    # identical keys inside every chunk: block-mean scores are exact and H = 0,
+    # so ANY selection reproduces softmax attention.
+    q, k, v = _pw_inputs(T=192)
+    k = np.repeat(k[::64], 64, axis=0)
+    qc, kc, vc, hc, H, lens = pw.chunk_reduce(q, k, v, 64)
+    assert np.abs(H).max() < 1e-12
+    idx = np.array([[0], [2], [1]])
+    o = pw.piecewise_forward(q, k, v, idx, 64)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        torch.from_numpy(q)[None], torch.from_numpy(k)[None], torch.from_numpy(v)[None])[0].numpy()
+    np.testing.assert_allclose(o, ref, rtol=1e-10, atol=1e-12)
+
+
+def test_piecewise_chunk_reduce_and_selection():
+    q, k, v = _pw_inputs(T=200)
+    qc, kc, vc, hc, H, lens = pw.chunk_reduce(q, k, v, 64)
+    assert lens.tolist() == [64, 64, 64, 8]
+    np.testing.assert_allclose(kc[3], k[192:].mean(0))
+    np.testing.assert_allclose(vc[3], v[192:].sum(0))
+    np.testing.assert_allclose((kc * lens[:, None]).sum(0), k.sum(0), rtol=1e-12)
+    # H = K^T V - sum_c n_c kc_c vc_c^T / n_c
+    np.testing.assert_allclose(H, k.T @ v - np.einsum('ck,cv->kv', kc, vc), rtol=1e-10, atol=1e-11)
+    idx = pw.select_blocks(qc, kc, 16 ** -0.5, 0.5)
+    assert idx.shape == (4, 2)
+    score = torch.from_numpy(qc @ (kc * 16 ** -0.5).T)
+    assert (np.sort(idx, -1) == np.sort(torch.topk(score, 2, dim=-1).indices.numpy(), -1)).all()
+
+
+def test_piecewise_first_order_term_is_taylor_expansion():
+    # Small scores: exp(s_ij) ~ exp(sb_ic)(1 + s_ij - sb_ic); summed over a chunk the
+    # numerator correction is exp(sb_ic) scale q.(K_c - kc_c)^T V_c, which the kernel
+    # approximates with the global H weighted by G/T.  With one unselected chunk and
+    # the rest selected, G/T * H_total differs from exp(sb)*hc_c, so only check that
+    # the first-order term moves the result towards exact attention on average.
+    q, k, v = _pw_inputs(T=512, K=8, V=4, seed=9)
+    q, k = 0.3 * q, 0.3 * k
+    NT = 8
+    idx = np.stack([np.array([t]) for t in range(NT)])
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        torch.from_numpy(q)[None], torch.from_numpy(k)[None], torch.from_numpy(v)[None])[0].numpy()
+    e0 = np.abs(pw.piecewise_forward(q, k, v, idx, 64, first_order=False) - ref).mean()
+    e1 = np.abs(pw.piecewise_forward(q, k, v, idx, 64, first_order=True) - ref).mean()
+    assert e1 < 0.5 * e0
