@@ -41,7 +41,12 @@ def dense_backward(q, k, v, do, scale, eps=1e-6, normalize=True, q_rope=None, k_
     dq~_t = dO_t S^T / z_t, dq_t = dz_t km, dk~_t = scale v_t dS^T, dk_t = dkm/L,
     dv_t = scale k~_t dS   (linear_attn/fused.py:238-242,325-328;
     decoupled.py:274-283,375-380; simple_la/fused.py:198,394-397).
-    Returns a dict with dq, dk, dv (+ dq_rope, dk_rope when decoupled)."""
+    Returns a dict with dq, dk, dv (+ dq_rope, dk_rope when decoupled).
+
+    dq_mag / dk_mag give, element by element, the larger of the two terms that
+    are added to form dq / dk.  For very short sequences the terms cancel (with
+    L = 1 the output does not depend on q at all, up to eps), so a comparison of
+    dq or dk should use max(|ref|.max(), mag.max()) as its scale."""
     decoupled = q_rope is not None
     q, k, v, do = _f64(q), _f64(k), _f64(v), _f64(do)
     qn = q if not decoupled else _f64(q_rope)
@@ -63,7 +68,9 @@ def dense_backward(q, k, v, do, scale, eps=1e-6, normalize=True, q_rope=None, k_
         dk_den = np.zeros_like(k)
     if decoupled:
         return dict(dq=dq_den, dk=np.array(dk_den), dq_rope=dq_num, dk_rope=dk_num, dv=dv, o=o, S=S, km=km)
-    return dict(dq=dq_num + dq_den, dk=dk_num + dk_den, dv=dv, o=o, S=S, km=km)
+    return dict(dq=dq_num + dq_den, dk=dk_num + dk_den, dv=dv, o=o, S=S, km=km,
+                dq_mag=np.maximum(np.abs(dq_num), np.abs(dq_den)),
+                dk_mag=np.maximum(np.abs(dk_num), np.abs(dk_den)))
 
 
 def varlen_forward(q, k, v, cu_seqlens, scale=None, eps=1e-6):
@@ -85,7 +92,8 @@ def varlen_forward(q, k, v, cu_seqlens, scale=None, eps=1e-6):
 def varlen_backward(q, k, v, do, cu_seqlens, scale=None, eps=1e-6):
     """varlen.py:216-219,310-314: the dense gradients applied per sequence."""
     q, k, v, do = _f64(q), _f64(k), _f64(v), _f64(do)
-    out = dict(dq=np.zeros(q.shape), dk=np.zeros(k.shape), dv=np.zeros(v.shape), o=np.zeros(v.shape))
+    out = dict(dq=np.zeros(q.shape), dk=np.zeros(k.shape), dv=np.zeros(v.shape), o=np.zeros(v.shape),
+               dq_mag=np.zeros(q.shape), dk_mag=np.zeros(k.shape))
     cu = [int(x) for x in np.asarray(cu_seqlens).tolist()]
     for b, e in zip(cu[:-1], cu[1:]):
         if e <= b:
@@ -93,6 +101,6 @@ def varlen_backward(q, k, v, do, cu_seqlens, scale=None, eps=1e-6):
         s = 1.0 / (e - b) if scale is None else scale
         g = dense_backward(q[b:e].transpose(1, 0, 2), k[b:e].transpose(1, 0, 2),
                            v[b:e].transpose(1, 0, 2), do[b:e].transpose(1, 0, 2), s, eps)
-        for name in ('dq', 'dk', 'dv', 'o'):
+        for name in ('dq', 'dk', 'dv', 'o', 'dq_mag', 'dk_mag'):
             out[name][b:e] = g[name].transpose(1, 0, 2)
     return out

@@ -24,6 +24,11 @@ from oracle import closed_form as cf  # noqa: E402
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 
+def _slim(name, a):
+    """Term magnitudes are only used through their maximum: keep one value per token."""
+    return a.max(axis=-1, keepdims=True) if name.endswith("_mag") else a
+
+
 def dense_case(name, B, H, L, DK, DV, scale, eps, normalize, decoupled, seed):
     q, k, v, do, qr, kr = make_qkv((B, H, L, DK), (B, H, L, DV), torch.float16, seed, n_extra=2)
     arrs = {n: np64(t).astype(np.float32) for n, t in dict(q=q, k=k, v=v, do=do).items()}
@@ -34,7 +39,7 @@ def dense_case(name, B, H, L, DK, DV, scale, eps, normalize, decoupled, seed):
     s = (1.0 / L if normalize else DK ** -0.5) if scale is None else scale
     g = cf.dense_backward(arrs["q"], arrs["k"], arrs["v"], arrs["do"], s, eps, normalize, **kw)
     out = dict(arrs)
-    out.update({"ref_" + n: a for n, a in g.items()})
+    out.update({"ref_" + n: _slim(n, a) for n, a in g.items()})
     out["meta"] = np.array([s, eps, float(normalize), float(decoupled)])
     np.savez_compressed(os.path.join(HERE, name + ".npz"), **out)
 
@@ -46,7 +51,7 @@ def varlen_case(name, lengths, H, DK, DV, scale, eps, seed):
     cu = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
     g = cf.varlen_backward(arrs["q"], arrs["k"], arrs["v"], arrs["do"], cu, scale, eps)
     out = dict(arrs)
-    out.update({"ref_" + n: a for n, a in g.items()})
+    out.update({"ref_" + n: _slim(n, a) for n, a in g.items()})
     out["cu_seqlens"] = cu
     out["meta"] = np.array([-1.0 if scale is None else scale, eps])
     np.savez_compressed(os.path.join(HERE, name + ".npz"), **out)
