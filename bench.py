@@ -1,0 +1,263 @@
+#!/usr/bin/env python3
+"""Benchmark of the bidirectional linear-attention hot path on one MI355X.
+
+Default workload (BASELINE.json configs[1] at the headline length): linear_attn
+fused forward+backward, B=8, H=16, D=64, T=16384, fp16, eps=1e-6, scale=1/T,
+q,k = elu(N(0,1))+1, v,dO ~ N(0,1) (synthetic, seeded).  One step is
+`linear_attention(q, k, v).backward(dO)` (benchmarks/ops/benchmark_linear_attn.py:56).
+
+Prints ONE JSON line:  value = algorithmic HBM bytes of a step / time per step
+(GB/s), with `roofline` (dominant kernel, timed live with events on the launch
+stream) and `cpu_baseline` (the torch restatement of the reference's naive
+operator, on the host cores, on a bounded sample of the same workload).
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--T 16384] [--sweep]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "flash-bidirectional-linear-attention_amd"), os.path.join(ROOT, "tests")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+import torch  # noqa: E402
+import torch.nn.functional as F  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+
+PHASES = {  # name -> (phase bit, tensors read+written once, entry point)
+    "fwd_state": (1, 2, "fwd"),     # reads k, v
+    "fwd_output": (4, 2, "fwd"),    # reads q, writes o
+    "bwd_pass_a": (8, 3, "bwd"),    # reads q, dO, writes dq
+    "bwd_pass_b": (32, 4, "bwd"),   # reads k, v, writes dk, dv
+}
+
+
+def make_inputs(B, H, T, D, dtype, device, seed=42):
+    g = torch.Generator(device=device).manual_seed(seed)
+    shape = (B, H, T, D)
+    q = (F.elu(torch.randn(shape, generator=g, device=device)) + 1).to(dtype)
+    k = (F.elu(torch.randn(shape, generator=g, device=device)) + 1).to(dtype)
+    v = torch.randn(shape, generator=g, device=device).to(dtype)
+    do = torch.randn(shape, generator=g, device=device).to(dtype)
+    return q, k, v, do
+
+
+def timed_loop(fn, n):
+    """Average ms per call over n back-to-back calls, events on the current stream."""
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(n):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / n
+
+
+def do_bench(fn, flush, quantiles=(0.5, 0.2, 0.8)):
+    """Triton-free restatement of triton.testing.do_bench as used by
+    benchmarks/ops/benchmark_linear_attn.py:45-58: warm call, 5-call estimate,
+    ~25 ms warmup, ~100 ms of timed calls, cache-flush write before every call,
+    one event pair per call, quantiles of the per-call times."""
+    fn()
+    torch.cuda.synchronize()
+    est = timed_loop(lambda: (flush.zero_(), fn()), 5)
+    n_warmup, n_repeat = max(1, int(25 / est)), max(1, int(100 / est))
+    for _ in range(n_warmup):
+        fn()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(n_repeat)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(n_repeat)]
+    for i in range(n_repeat):
+        flush.zero_()
+        starts[i].record()
+        fn()
+        ends[i].record()
+    torch.cuda.synchronize()
+    times = torch.tensor([s.elapsed_time(e) for s, e in zip(starts, ends)], dtype=torch.float64)
+    return [float(x) for x in torch.quantile(times, torch.tensor(quantiles, dtype=torch.float64))]
+
+
+def cpu_baseline(T, D, H, sample_batches, reps=3):
+    """Reference torch path (oracle.torch_ref.naive_linear_attn + autograd) on the
+    host cores, fp32 math on fp16-valued inputs, for `sample_batches` of the 8
+    batches of the workload."""
+    from oracle import torch_ref
+    torch.set_num_threads(os.cpu_count() or 1)
+    g = torch.Generator().manual_seed(42)
+    shape = (sample_batches, H, T, D)
+    q = (F.elu(torch.randn(shape, generator=g)) + 1).half().float().requires_grad_()
+    k = (F.elu(torch.randn(shape, generator=g)) + 1).half().float().requires_grad_()
+    v = torch.randn(shape, generator=g).half().float().requires_grad_()
+    do = torch.randn(shape, generator=g).half().float()
+    times = []
+    for _ in range(reps + 1):
+        q.grad = k.grad = v.grad = None
+        t0 = time.perf_counter()
+        torch_ref.naive_linear_attn(q, k, v).backward(do)
+        times.append(time.perf_counter() - t0)
+    t = sorted(times[1:])[len(times[1:]) // 2]
+    bytes_fp16 = 11 * sample_batches * H * T * D * 2
+    return {
+        "value": round(bytes_fp16 / t / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"linear_attn fwd+bwd, {sample_batches} of 8 batches (B{sample_batches},H{H},T{T},D{D}), "
+                  f"fp32 math on the fp16-valued inputs, median of {reps} runs; "
+                  f"{t * 1e3:.1f} ms per run; bytes counted as the fp16 workload's 11 tensor passes",
+        "ms": round(t * 1e3, 3),
+    }
+
+
+def parity_spot_check(q, k, v, do, o, grads, heads=((0, 0), (7, 15))):
+    from helpers import np64, parity_errors
+    from oracle import closed_form as cf
+    out = {}
+    for b, h in heads:
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        ref = cf.dense_backward(np64(q[sl]), np64(k[sl]), np64(v[sl]), np64(do[sl]), 1.0 / q.shape[2])
+        for name, t in (("o", o), ("dq", grads[0]), ("dk", grads[1]), ("dv", grads[2])):
+            plain, excess, ok = parity_errors(t[sl], ref[name], q.dtype, ref.get(name + "_mag"))
+            prev = out.get(name, (0.0, 0.0, True))
+            out[name] = (max(prev[0], plain), max(prev[1], excess), prev[2] and ok)
+    return {n: {"max_rel": round(p, 7), "excess": round(e, 7), "ok": ok} for n, (p, e, ok) in out.items()}
+
+
+def kernel_times(q, k, v, do, n=20):
+    """Average duration of each large kernel, launched alone through the phase mask."""
+    from flash_bla import _hip
+    lib = _hip.lib()
+    T = q.shape[2]
+    scale, eps = 1.0 / T, 1e-6
+    o, s, km = _hip.la_fwd(q, k, v, None, None, scale, eps, _hip.NORMALIZE)
+    res = {}
+    for name, (bit, passes, entry) in PHASES.items():
+        lib.fbla_set_phase_mask(bit)
+        try:
+            if entry == "fwd":
+                fn = lambda: _hip.la_fwd(q, k, v, None, None, scale, eps, _hip.NORMALIZE)  # noqa: E731
+            else:
+                fn = lambda: _hip.la_bwd(q, k, v, None, None, do, s, km, scale, eps, _hip.NORMALIZE)  # noqa: E731
+            for _ in range(3):
+                fn()
+            ms = timed_loop(fn, n)
+        finally:
+            lib.fbla_set_phase_mask(0)
+        nbytes = passes * q.numel() * q.element_size()
+        res[name] = {"ms": round(ms, 5), "alg_bytes": nbytes, "gbps": round(nbytes / ms / 1e6, 1),
+                     "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--T", type=int, default=16384)
+    ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16", "fp32"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--sweep", action="store_true",
+                    help="also print a table over T in {1024,4096,16384,32768} to stderr")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path needs no collective: heads "
+              "are independent); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    dtype = {"fp16": torch.float16, "bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
+    B, H, D, T = 8, 16, 64, args.T
+    dev = torch.device("cuda:0")
+    q, k, v, do = make_inputs(B, H, T, D, dtype, dev)
+    q.requires_grad_(), k.requires_grad_(), v.requires_grad_()
+    tensor_bytes = q.numel() * q.element_size()
+    fwd_bytes, step_bytes = 4 * tensor_bytes, 11 * tensor_bytes
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        linear_attention(q, k, v).backward(do)
+
+    def fwd_only():
+        with torch.no_grad():
+            return linear_attention(q, k, v)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    o = fwd_only()
+    parity = parity_spot_check(q.detach(), k.detach(), v.detach(), do, o, (q.grad, k.grad, v.grad))
+
+    flush = torch.empty(256 << 20, dtype=torch.int8, device=dev)
+    fwd_q = do_bench(fwd_only, flush)
+    step_q = do_bench(step, flush)
+    kern = kernel_times(q.detach(), k.detach(), v.detach(), do)
+    dom = max(kern, key=lambda n: kern[n]["ms"])
+    roofline = {
+        "bound": "hbm", "kernel": dom, "achieved": kern[dom]["gbps"], "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s", "frac": kern[dom]["frac"], "traffic": None,
+        "alg_bytes_per_launch": kern[dom]["alg_bytes"], "avg_launch_ms": kern[dom]["ms"],
+    }
+    cpu = None if args.no_cpu else cpu_baseline(T, D, H, sample_batches=2)
+
+    line = {
+        "metric": "linear_attn fwd+bwd ms and achieved HBM GB/s, B8-H16-D64 T=16384 fp16",
+        "value": round(step_bytes / ms_per_step / 1e6, 2), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": f"linear_attn fused fwd+bwd B{B}-H{H}-D{D} T={T} {args.dtype} eps=1e-6 scale=1/T",
+                   "alg_bytes_per_step": step_bytes, "tensor_passes": 11},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "fwd_bwd": {"ms_p50_p20_p80_flushed": [round(x, 5) for x in step_q],
+                    "gbps_p50": round(step_bytes / step_q[0] / 1e6, 1),
+                    "frac_of_peak": round(step_bytes / ms_per_step / 1e6 / HBM_PEAK_GBPS, 4)},
+        "fwd": {"ms_p50_p20_p80_flushed": [round(x, 5) for x in fwd_q], "alg_bytes": fwd_bytes,
+                "gbps_p50": round(fwd_bytes / fwd_q[0] / 1e6, 1),
+                "frac_of_peak": round(fwd_bytes / fwd_q[0] / 1e6 / HBM_PEAK_GBPS, 4)},
+        "kernels": kern,
+        "parity": parity,
+    }
+    if args.sweep:
+        sweep(dtype, dev, flush)
+    print(json.dumps(line), flush=True)
+
+
+def sweep(dtype, dev, flush):
+    """Per-length table (forward and forward+backward, flushed medians) on stderr."""
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    for T in (1024, 4096, 16384, 32768):
+        q, k, v, do = make_inputs(8, 16, T, 64, dtype, dev)
+        q.requires_grad_(), k.requires_grad_(), v.requires_grad_()
+        nbytes = q.numel() * q.element_size()
+
+        def step():
+            q.grad = k.grad = v.grad = None
+            linear_attention(q, k, v).backward(do)
+
+        def fwd_only():
+            with torch.no_grad():
+                return linear_attention(q, k, v)
+
+        f = do_bench(fwd_only, flush)
+        s = do_bench(step, flush)
+        print(json.dumps({"T": T, "fwd_ms": round(f[0], 5), "fwd_gbps": round(4 * nbytes / f[0] / 1e6, 1),
+                          "fwd_bwd_ms": round(s[0], 5), "fwd_bwd_gbps": round(11 * nbytes / s[0] / 1e6, 1)}),
+              file=sys.stderr, flush=True)
+
+
+if __name__ == "__main__":
+    main()

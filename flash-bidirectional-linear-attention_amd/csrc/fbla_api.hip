@@ -18,6 +18,9 @@ void set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
+static thread_local unsigned g_phase_mask = kPhaseAll;
+unsigned phase_mask() { return g_phase_mask; }
+
 static int check_launch(const char* what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
@@ -103,6 +106,8 @@ using namespace fbla;
 extern "C" {
 
 int fbla_version(void) { return 100; }
+
+void fbla_set_phase_mask(unsigned mask) { g_phase_mask = mask ? mask : kPhaseAll; }
 
 const char* fbla_last_error(void) { return g_err; }
 

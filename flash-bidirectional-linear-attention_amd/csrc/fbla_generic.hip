@@ -487,17 +487,22 @@ static int forward_t(const Prob& p, const FwdArgs& a, hipStream_t st) {
   const int chunk = pick_chunk(p);
   const int nchunks = (int)cdiv64(p.L, chunk);
   float* partial = (float*)a.workspace;
-  switch (micro(p)) {
-    case 2: launch_state_partial<T, 2>(p, kn, v, k, partial, chunk, nchunks, st); break;
-    case 4: launch_state_partial<T, 4>(p, kn, v, k, partial, chunk, nchunks, st); break;
-    default: launch_state_partial<T, 8>(p, kn, v, k, partial, chunk, nchunks, st); break;
+  const unsigned phases = phase_mask();
+  if (phases & kPhaseFwdState) {
+    switch (micro(p)) {
+      case 2: launch_state_partial<T, 2>(p, kn, v, k, partial, chunk, nchunks, st); break;
+      case 4: launch_state_partial<T, 4>(p, kn, v, k, partial, chunk, nchunks, st); break;
+      default: launch_state_partial<T, 8>(p, kn, v, k, partial, chunk, nchunks, st); break;
+    }
   }
   const int64_t nh = (int64_t)p.N * p.H;
-  state_reduce_kernel<<<dim3((unsigned)nh), dim3(kThreads), 0, st>>>(p, partial, chunk, nchunks,
-                                                                    a.s, nullptr, a.km);
+  if (phases & kPhaseFwdReduce)
+    state_reduce_kernel<<<dim3((unsigned)nh), dim3(kThreads), 0, st>>>(p, partial, chunk, nchunks,
+                                                                      a.s, nullptr, a.km);
   const int ntiles = (int)cdiv64(p.L, kTile);
-  output_kernel<T><<<dim3((unsigned)(nh * ntiles)), dim3(kThreads), 0, st>>>(
-      p, qn, q, a.s, a.km, (T*)a.o, ntiles);
+  if (phases & kPhaseFwdOutput)
+    output_kernel<T><<<dim3((unsigned)(nh * ntiles)), dim3(kThreads), 0, st>>>(
+        p, qn, q, a.s, a.km, (T*)a.o, ntiles);
   return kOk;
 }
 
@@ -525,8 +530,10 @@ static int backward_t(const Prob& p, const BwdArgs& a, hipStream_t st) {
   ws += state_bytes(p);
   float* dkm = (float*)ws;
   const int64_t nh = (int64_t)p.N * p.H;
-  transpose_state_kernel<<<dim3((unsigned)nh), dim3(kThreads), 0, st>>>(a.s, St, p.DK, p.DV);
-  switch (micro(p)) {
+  const unsigned phases = phase_mask();
+  if (phases & kPhaseBwdA)
+    transpose_state_kernel<<<dim3((unsigned)nh), dim3(kThreads), 0, st>>>(a.s, St, p.DK, p.DV);
+  if (phases & kPhaseBwdA) switch (micro(p)) {
     case 2:
       launch_bwd_a<T, 2>(p, qn, q, (const T*)a.dout, a.s, St, a.km, dqn, dqd, partial, chunk,
                          nchunks, st);
@@ -540,10 +547,12 @@ static int backward_t(const Prob& p, const BwdArgs& a, hipStream_t st) {
                          nchunks, st);
       break;
   }
-  state_reduce_kernel<<<dim3((unsigned)nh), dim3(kThreads), 0, st>>>(p, partial, chunk, nchunks, dS,
-                                                                    dSt, dkm);
+  if (phases & kPhaseBwdReduce)
+    state_reduce_kernel<<<dim3((unsigned)nh), dim3(kThreads), 0, st>>>(p, partial, chunk, nchunks,
+                                                                      dS, dSt, dkm);
   const int ntiles = (int)cdiv64(p.L, kTile);
-  bwd_b_kernel<T><<<dim3((unsigned)(nh * ntiles)), dim3(kThreads), 0, st>>>(
+  if (phases & kPhaseBwdB)
+    bwd_b_kernel<T><<<dim3((unsigned)(nh * ntiles)), dim3(kThreads), 0, st>>>(
       p, kn, v, dS, dSt, dkm, dkn, dkd, (T*)a.dv, ntiles);
   return kOk;
 }

@@ -22,6 +22,19 @@ struct BwdArgs {
   size_t workspace_bytes;
 };
 
+// Kernel phases of one entry point, selectable for per-kernel timing
+// (fbla_set_phase_mask).  Default: all.
+enum Phase : unsigned {
+  kPhaseFwdState = 1u,    // per-chunk partial K^T V and sum k
+  kPhaseFwdReduce = 2u,   // fixed-order reduce of the partials
+  kPhaseFwdOutput = 4u,   // o = (q S)/z
+  kPhaseBwdA = 8u,        // dq + partial dS, dkm
+  kPhaseBwdReduce = 16u,  // reduce of the backward partials
+  kPhaseBwdB = 32u,       // dk, dv
+  kPhaseAll = 63u,
+};
+unsigned phase_mask();
+
 namespace generic {
 size_t fwd_workspace_bytes(const Prob& p);
 size_t bwd_workspace_bytes(const Prob& p);

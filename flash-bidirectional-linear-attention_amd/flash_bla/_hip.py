@@ -23,6 +23,7 @@ _vp, _i64, _i32, _f32, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, cty
 _SIGNATURES = {
     "fbla_version": (ctypes.c_int, []),
     "fbla_last_error": (ctypes.c_char_p, []),
+    "fbla_set_phase_mask": (None, [ctypes.c_uint]),
     "fbla_la_workspace_bytes": (_sz, [_i32, _i64, _i64, _i64, _i32, _i32, _i32, _i32]),
     "fbla_la_fwd": (_i32, [_vp] * 9 + [_sz, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_la_bwd": (_i32, [_vp] * 14 + [_sz, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),

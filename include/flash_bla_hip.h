@@ -55,6 +55,14 @@ extern "C" {
 /* Library version (major*10000 + minor*100 + patch). */
 int fbla_version(void);
 
+/* Profiling aid with no counterpart in the reference: restrict the entry points
+ * called from this thread to a subset of their kernels so that one kernel can be
+ * timed in isolation (bit 0 forward partial state, 1 forward state reduce,
+ * 2 forward output, 3 backward pass A, 4 backward reduce, 5 backward pass B).
+ * 0 restores the default (all kernels).  Skipped kernels leave their outputs
+ * untouched, so results are only meaningful with the default mask. */
+void fbla_set_phase_mask(unsigned mask);
+
 /* Message of the last error raised on the calling thread ("" if none). */
 const char* fbla_last_error(void);
 
