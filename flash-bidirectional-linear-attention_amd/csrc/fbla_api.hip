@@ -71,8 +71,7 @@ static Prob make_prob(const int32_t* cu, int64_t N, int64_t H, int64_t L, int DK
 }
 
 static size_t workspace_bytes(const Prob& p, int dtype, int pass) {
-  (void)dtype;
-  return pass == 0 ? generic::fwd_workspace_bytes(p) : generic::bwd_workspace_bytes(p);
+  return pass == 0 ? plan::fwd_workspace_bytes(p, dtype) : plan::bwd_workspace_bytes(p, dtype);
 }
 
 static int run_fwd(const char* what, const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
@@ -82,7 +81,7 @@ static int run_fwd(const char* what, const Prob& p, int dtype, const FwdArgs& a,
     set_error("%s: workspace too small (%zu < %zu bytes)", what, a.workspace_bytes, need);
     return kErrWorkspace;
   }
-  int rc = generic::forward(p, dtype, a, st);
+  int rc = plan::forward(p, dtype, a, st);
   if (rc != kOk) return rc;
   return check_launch(what);
 }
@@ -94,7 +93,7 @@ static int run_bwd(const char* what, const Prob& p, int dtype, const BwdArgs& a,
     set_error("%s: workspace too small (%zu < %zu bytes)", what, a.workspace_bytes, need);
     return kErrWorkspace;
   }
-  int rc = generic::backward(p, dtype, a, st);
+  int rc = plan::backward(p, dtype, a, st);
   if (rc != kOk) return rc;
   return check_launch(what);
 }

@@ -421,12 +421,12 @@ __global__ __launch_bounds__(kThreads) void bwd_b_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// host side
+// host side: one launcher per phase (the plan in fbla_plan.hip strings them together)
 // ---------------------------------------------------------------------------
 
 // Tokens per reduction chunk: enough chunks to give every CU several workgroups,
 // few enough that the partial buffer stays small.
-int pick_chunk(const Prob& p) {
+int state_chunk(const Prob& p) {
   const int64_t nh = (int64_t)p.N * p.H;
   const int64_t target_wgs = 1024;
   int64_t chunk = cdiv64((int64_t)p.L * nh, target_wgs);
@@ -435,144 +435,119 @@ int pick_chunk(const Prob& p) {
   return (int)chunk;
 }
 
-size_t partial_bytes(const Prob& p) {
-  const int chunk = pick_chunk(p);
-  const int64_t nchunks = cdiv64(p.L, chunk);
-  return align_up((size_t)p.N * p.H * nchunks * ((size_t)p.DK * p.DV + p.DK) * sizeof(float), 256);
-}
-
-size_t state_bytes(const Prob& p) {
-  return align_up((size_t)p.N * p.H * p.DK * p.DV * sizeof(float), 256);
-}
-
-size_t vec_bytes(const Prob& p) { return align_up((size_t)p.N * p.H * p.DK * sizeof(float), 256); }
-
-size_t fwd_workspace_bytes(const Prob& p) { return partial_bytes(p); }
-
-// partials | S^T | s*dS | (s*dS)^T | dkm/L
-size_t bwd_workspace_bytes(const Prob& p) {
-  return partial_bytes(p) + 3 * state_bytes(p) + vec_bytes(p);
-}
-
-template <typename T, int M>
-static void launch_state_partial(const Prob& p, const T* kn, const T* v, const T* kd,
-                                 float* partial, int chunk, int nchunks, hipStream_t st) {
-  const int64_t grid = (int64_t)p.N * p.H * nchunks;
-  state_partial_kernel<T, M><<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial,
-                                                                             chunk, nchunks);
-}
-
-template <typename T, int M>
-static void launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, const float* S,
-                         const float* St, const float* km, T* dqn, T* dqd, float* partial,
-                         int chunk, int nchunks, hipStream_t st) {
-  const int64_t grid = (int64_t)p.N * p.H * nchunks;
-  bwd_a_kernel<T, M><<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(
-      p, qn, qd, dout, S, St, km, dqn, dqd, partial, chunk, nchunks);
-}
-
 static int micro(const Prob& p) {
   const int d = p.DK > p.DV ? p.DK : p.DV;
   return d <= 32 ? 2 : (d <= 64 ? 4 : 8);
 }
 
 template <typename T>
-static int forward_t(const Prob& p, const FwdArgs& a, hipStream_t st) {
-  const T* q = (const T*)a.q;
-  const T* k = (const T*)a.k;
-  const T* v = (const T*)a.v;
-  const bool dec = p.flags & kDecoupled;
-  const T* qn = dec ? (const T*)a.q_rope : q;
-  const T* kn = dec ? (const T*)a.k_rope : k;
-  const int chunk = pick_chunk(p);
-  const int nchunks = (int)cdiv64(p.L, chunk);
-  float* partial = (float*)a.workspace;
-  const unsigned phases = phase_mask();
-  if (phases & kPhaseFwdState) {
-    switch (micro(p)) {
-      case 2: launch_state_partial<T, 2>(p, kn, v, k, partial, chunk, nchunks, st); break;
-      case 4: launch_state_partial<T, 4>(p, kn, v, k, partial, chunk, nchunks, st); break;
-      default: launch_state_partial<T, 8>(p, kn, v, k, partial, chunk, nchunks, st); break;
-    }
+static void state_partial_t(const Prob& p, const void* kn, const void* v, const void* kd,
+                            float* partial, int chunk, int nchunks, hipStream_t st) {
+  const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(kThreads);
+  const T *a = (const T*)kn, *b = (const T*)v, *c = (const T*)kd;
+  switch (micro(p)) {
+    case 2: state_partial_kernel<T, 2><<<grid, block, 0, st>>>(p, a, b, c, partial, chunk, nchunks); break;
+    case 4: state_partial_kernel<T, 4><<<grid, block, 0, st>>>(p, a, b, c, partial, chunk, nchunks); break;
+    default: state_partial_kernel<T, 8><<<grid, block, 0, st>>>(p, a, b, c, partial, chunk, nchunks); break;
   }
-  const int64_t nh = (int64_t)p.N * p.H;
-  if (phases & kPhaseFwdReduce)
-    state_reduce_kernel<<<dim3((unsigned)nh), dim3(kThreads), 0, st>>>(p, partial, chunk, nchunks,
-                                                                      a.s, nullptr, a.km);
-  const int ntiles = (int)cdiv64(p.L, kTile);
-  if (phases & kPhaseFwdOutput)
-    output_kernel<T><<<dim3((unsigned)(nh * ntiles)), dim3(kThreads), 0, st>>>(
-        p, qn, q, a.s, a.km, (T*)a.o, ntiles);
-  return kOk;
+}
+
+void state_partial(const Prob& p, int dtype, const void* kn, const void* v, const void* kd,
+                   float* partial, int chunk, int nchunks, hipStream_t st) {
+  if (dtype == kF16) state_partial_t<_Float16>(p, kn, v, kd, partial, chunk, nchunks, st);
+  else if (dtype == kBF16) state_partial_t<__bf16>(p, kn, v, kd, partial, chunk, nchunks, st);
+  else state_partial_t<float>(p, kn, v, kd, partial, chunk, nchunks, st);
+}
+
+void state_reduce(const Prob& p, const float* partial, int chunk, int nchunks, float* mat,
+                  float* mat_t, float* vec, hipStream_t st) {
+  state_reduce_kernel<<<dim3((unsigned)((int64_t)p.N * p.H)), dim3(kThreads), 0, st>>>(
+      p, partial, chunk, nchunks, mat, mat_t, vec);
+}
+
+void transpose_state(const Prob& p, const float* mat, float* mat_t, hipStream_t st) {
+  transpose_state_kernel<<<dim3((unsigned)((int64_t)p.N * p.H)), dim3(kThreads), 0, st>>>(
+      mat, mat_t, p.DK, p.DV);
 }
 
 template <typename T>
-static int backward_t(const Prob& p, const BwdArgs& a, hipStream_t st) {
-  const bool dec = p.flags & kDecoupled;
-  const T* q = (const T*)a.q;
-  const T* v = (const T*)a.v;
-  const T* qn = dec ? (const T*)a.q_rope : q;
-  const T* kn = dec ? (const T*)a.k_rope : (const T*)a.k;
-  T* dqn = dec ? (T*)a.dq_rope : (T*)a.dq;
-  T* dkn = dec ? (T*)a.dk_rope : (T*)a.dk;
-  T* dqd = dec ? (T*)a.dq : nullptr;
-  T* dkd = dec ? (T*)a.dk : nullptr;
-  const int chunk = pick_chunk(p);
-  const int nchunks = (int)cdiv64(p.L, chunk);
-  char* ws = (char*)a.workspace;
-  float* partial = (float*)ws;
-  ws += partial_bytes(p);
-  float* St = (float*)ws;
-  ws += state_bytes(p);
-  float* dS = (float*)ws;
-  ws += state_bytes(p);
-  float* dSt = (float*)ws;
-  ws += state_bytes(p);
-  float* dkm = (float*)ws;
-  const int64_t nh = (int64_t)p.N * p.H;
-  const unsigned phases = phase_mask();
-  if (phases & kPhaseBwdA)
-    transpose_state_kernel<<<dim3((unsigned)nh), dim3(kThreads), 0, st>>>(a.s, St, p.DK, p.DV);
-  if (phases & kPhaseBwdA) switch (micro(p)) {
-    case 2:
-      launch_bwd_a<T, 2>(p, qn, q, (const T*)a.dout, a.s, St, a.km, dqn, dqd, partial, chunk,
-                         nchunks, st);
-      break;
-    case 4:
-      launch_bwd_a<T, 4>(p, qn, q, (const T*)a.dout, a.s, St, a.km, dqn, dqd, partial, chunk,
-                         nchunks, st);
-      break;
-    default:
-      launch_bwd_a<T, 8>(p, qn, q, (const T*)a.dout, a.s, St, a.km, dqn, dqd, partial, chunk,
-                         nchunks, st);
-      break;
-  }
-  if (phases & kPhaseBwdReduce)
-    state_reduce_kernel<<<dim3((unsigned)nh), dim3(kThreads), 0, st>>>(p, partial, chunk, nchunks,
-                                                                      dS, dSt, dkm);
+static void output_t(const Prob& p, const void* qn, const void* qd, const float* S, const float* km,
+                     void* o, hipStream_t st) {
   const int ntiles = (int)cdiv64(p.L, kTile);
-  if (phases & kPhaseBwdB)
-    bwd_b_kernel<T><<<dim3((unsigned)(nh * ntiles)), dim3(kThreads), 0, st>>>(
-      p, kn, v, dS, dSt, dkm, dkn, dkd, (T*)a.dv, ntiles);
-  return kOk;
+  output_kernel<T><<<dim3((unsigned)((int64_t)p.N * p.H * ntiles)), dim3(kThreads), 0, st>>>(
+      p, (const T*)qn, (const T*)qd, S, km, (T*)o, ntiles);
 }
 
-int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
-  switch (dtype) {
-    case kF16: return forward_t<_Float16>(p, a, st);
-    case kBF16: return forward_t<__bf16>(p, a, st);
-    case kF32: return forward_t<float>(p, a, st);
-  }
-  return kErrUnsupported;
+void output(const Prob& p, int dtype, const void* qn, const void* qd, const float* S,
+            const float* km, void* o, hipStream_t st) {
+  if (dtype == kF16) output_t<_Float16>(p, qn, qd, S, km, o, st);
+  else if (dtype == kBF16) output_t<__bf16>(p, qn, qd, S, km, o, st);
+  else output_t<float>(p, qn, qd, S, km, o, st);
 }
 
-int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
-  switch (dtype) {
-    case kF16: return backward_t<_Float16>(p, a, st);
-    case kBF16: return backward_t<__bf16>(p, a, st);
-    case kF32: return backward_t<float>(p, a, st);
+template <typename T>
+static void bwd_a_t(const Prob& p, const void* qn, const void* qd, const void* dout, const float* S,
+                    const float* St, const float* km, void* dqn, void* dqd, float* partial,
+                    int chunk, int nchunks, hipStream_t st) {
+  const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(kThreads);
+  const T *a = (const T*)qn, *b = (const T*)qd, *c = (const T*)dout;
+  T *x = (T*)dqn, *y = (T*)dqd;
+  switch (micro(p)) {
+    case 2: bwd_a_kernel<T, 2><<<grid, block, 0, st>>>(p, a, b, c, S, St, km, x, y, partial, chunk, nchunks); break;
+    case 4: bwd_a_kernel<T, 4><<<grid, block, 0, st>>>(p, a, b, c, S, St, km, x, y, partial, chunk, nchunks); break;
+    default: bwd_a_kernel<T, 8><<<grid, block, 0, st>>>(p, a, b, c, S, St, km, x, y, partial, chunk, nchunks); break;
   }
-  return kErrUnsupported;
+}
+
+void bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout,
+           const float* S, const float* St, const float* km, void* dqn, void* dqd, float* partial,
+           int chunk, int nchunks, hipStream_t st) {
+  if (dtype == kF16) bwd_a_t<_Float16>(p, qn, qd, dout, S, St, km, dqn, dqd, partial, chunk, nchunks, st);
+  else if (dtype == kBF16) bwd_a_t<__bf16>(p, qn, qd, dout, S, St, km, dqn, dqd, partial, chunk, nchunks, st);
+  else bwd_a_t<float>(p, qn, qd, dout, S, St, km, dqn, dqd, partial, chunk, nchunks, st);
+}
+
+template <typename T>
+static void bwd_b_t(const Prob& p, const void* kn, const void* v, const float* dS, const float* dSt,
+                    const float* dkm, void* dkn, void* dkd, void* dv, hipStream_t st) {
+  const int ntiles = (int)cdiv64(p.L, kTile);
+  bwd_b_kernel<T><<<dim3((unsigned)((int64_t)p.N * p.H * ntiles)), dim3(kThreads), 0, st>>>(
+      p, (const T*)kn, (const T*)v, dS, dSt, dkm, (T*)dkn, (T*)dkd, (T*)dv, ntiles);
+}
+
+void bwd_b(const Prob& p, int dtype, const void* kn, const void* v, const float* dS,
+           const float* dSt, const float* dkm, void* dkn, void* dkd, void* dv, hipStream_t st) {
+  if (dtype == kF16) bwd_b_t<_Float16>(p, kn, v, dS, dSt, dkm, dkn, dkd, dv, st);
+  else if (dtype == kBF16) bwd_b_t<__bf16>(p, kn, v, dS, dSt, dkm, dkn, dkd, dv, st);
+  else bwd_b_t<float>(p, kn, v, dS, dSt, dkm, dkn, dkd, dv, st);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void broadcast_rows_kernel(Prob p, const float* __restrict__ vec,
+                                                                  T* __restrict__ out, int ntiles) {
+  const int nh = blockIdx.x / ntiles, tile = blockIdx.x - nh * ntiles;
+  const int n = nh / p.H, h = nh - n * p.H;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t0 = tile * kTile;
+  if (t0 >= len) return;
+  const int nvalid = min(kTile, len - t0);
+  row_base(p, n, h, bos, row0, rstride);
+  const int DK = p.DK;
+  for (int i = threadIdx.x; i < nvalid * DK; i += kThreads) {
+    const int t = i / DK, d = i - t * DK;
+    out[(row0 + (int64_t)(t0 + t) * rstride) * DK + d] = from_f32<T>(vec[(int64_t)nh * DK + d]);
+  }
+}
+
+// every row of out ([.., DK]) = vec of its (sequence, head): dk of the decoupled operator
+void broadcast_rows(const Prob& p, int dtype, const float* vec, void* out, hipStream_t st) {
+  const int ntiles = (int)cdiv64(p.L, kTile);
+  const dim3 grid((unsigned)((int64_t)p.N * p.H * ntiles)), block(kThreads);
+  if (dtype == kF16) broadcast_rows_kernel<_Float16><<<grid, block, 0, st>>>(p, vec, (_Float16*)out, ntiles);
+  else if (dtype == kBF16) broadcast_rows_kernel<__bf16><<<grid, block, 0, st>>>(p, vec, (__bf16*)out, ntiles);
+  else broadcast_rows_kernel<float><<<grid, block, 0, st>>>(p, vec, (float*)out, ntiles);
 }
 
 }  // namespace generic

@@ -1,4 +1,5 @@
-// Internal interface between the C-ABI layer (fbla_api.hip) and the kernel files.
+// Internal interface between the C-ABI layer (fbla_api.hip), the plan
+// (fbla_plan.hip) and the kernel files.
 #pragma once
 #include "fbla_common.h"
 
@@ -35,11 +36,49 @@ enum Phase : unsigned {
 };
 unsigned phase_mask();
 
-namespace generic {
-size_t fwd_workspace_bytes(const Prob& p);
-size_t bwd_workspace_bytes(const Prob& p);
+// The sequence of kernels behind each entry point.
+namespace plan {
+size_t fwd_workspace_bytes(const Prob& p, int dtype);
+size_t bwd_workspace_bytes(const Prob& p, int dtype);
 int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st);
 int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st);
+}  // namespace plan
+
+// Shape-generic FMA kernels (fbla_generic.hip).
+namespace generic {
+int state_chunk(const Prob& p);
+void state_partial(const Prob& p, int dtype, const void* kn, const void* v, const void* kd,
+                   float* partial, int chunk, int nchunks, hipStream_t st);
+void state_reduce(const Prob& p, const float* partial, int chunk, int nchunks, float* mat,
+                  float* mat_t, float* vec, hipStream_t st);
+void transpose_state(const Prob& p, const float* mat, float* mat_t, hipStream_t st);
+void output(const Prob& p, int dtype, const void* qn, const void* qd, const float* S,
+            const float* km, void* o, hipStream_t st);
+void bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout,
+           const float* S, const float* St, const float* km, void* dqn, void* dqd, float* partial,
+           int chunk, int nchunks, hipStream_t st);
+void bwd_b(const Prob& p, int dtype, const void* kn, const void* v, const float* dS,
+           const float* dSt, const float* dkm, void* dkn, void* dkd, void* dv, hipStream_t st);
+void broadcast_rows(const Prob& p, int dtype, const float* vec, void* out, hipStream_t st);
 }  // namespace generic
+
+// MFMA kernels for 16-bit inputs (fbla_mfma.hip).
+namespace mfma {
+struct RowsJob {
+  const void* x;        // [rows][DR] contracted operand
+  const void* xden;     // [rows][DR] rows dotted with km for z (== x unless decoupled); null: z = 1
+  const float* mat;     // per (sequence, head): element (r, c) at mat[r*ld_r + c*ld_c]
+  int ld_r, ld_c;
+  const float* km;      // per (sequence, head) [DR]; used when xden != null
+  const float* addvec;  // per (sequence, head) [DC] added to every row, or null
+  void* out;            // [rows][DC]
+};
+bool supported(const Prob& p, int dtype);
+int state_chunk(const Prob& p);
+void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
+           int chunk, int nchunks, hipStream_t st);
+// out_t = (x_t M) / (xden_t . km + eps) + addvec   with M of shape DR x DC
+void rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st);
+}  // namespace mfma
 
 }  // namespace fbla

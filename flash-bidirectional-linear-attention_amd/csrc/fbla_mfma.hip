@@ -1,0 +1,539 @@
+// MFMA kernels for 16-bit inputs (fp16 / bf16) with head dims in {64, 128}.
+//
+// Every wave is an independent worker: it streams its own 16- or 32-token
+// sub-tiles, keeps fp32 accumulators in registers and touches LDS only through
+// a wave-private staging area (plus one workgroup-shared, read-only matrix
+// operand).  The main loops contain no workgroup barrier.
+//
+//  state_kernel      S_part = K~^T V and sum_t k_t over a token chunk.  Rows are
+//                    read straight from global memory with one dword (2 features)
+//                    per lane, so a half-wave reads one full 128-byte row; the
+//                    token-major -> feature-major transposition MFMA needs is a
+//                    v_perm_b32 on pairs of rows (no LDS).
+//  rows_kernel       out_t = (x_t M) * rowscale_t + addvec: the forward output
+//                    (M = S, rowscale = 1/(q.km+eps)) and both products of backward
+//                    pass B (M = s dS and its transpose).  M is fp32 in memory and
+//                    is fed to MFMA as a hi+lo pair of 16-bit operands after a
+//                    power-of-two normalisation, so no precision is lost.
+//
+// MFMA used: v_mfma_f32_32x32x16_{f16,bf16}.  Operand layout (verified on
+// gfx950): A lane l holds A[m=l%32][k=8*(l/32)+i], B lane l holds
+// B[k=8*(l/32)+i][n=l%32], i=0..7; C register r of lane l is
+// C[8*(r/4)+4*(l/32)+r%4][l%32].
+#include "fbla_kernels.h"
+
+namespace fbla {
+namespace mfma {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+
+template <typename T> struct Ops;
+
+template <> struct Ops<_Float16> {
+  static __device__ __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c,
+                                  false);
+  }
+  static __device__ __forceinline__ float lo(uint32_t w) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+  }
+  static __device__ __forceinline__ float hi(uint32_t w) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+  }
+  static __device__ __forceinline__ uint32_t bits(float x) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)x);
+  }
+  static constexpr uint32_t kOnes = 0x3c003c00u;  // (1.0, 1.0)
+};
+
+template <> struct Ops<__bf16> {
+  static __device__ __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a),
+                                           __builtin_bit_cast(bf16x2, b), c, false);
+  }
+  static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+  static __device__ __forceinline__ float hi(uint32_t w) {
+    return __builtin_bit_cast(float, w & 0xffff0000u);
+  }
+  static __device__ __forceinline__ uint32_t bits(float x) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)x);
+  }
+  static constexpr uint32_t kOnes = 0x3f803f80u;
+};
+
+template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b) {
+  return Ops<T>::bits(a) | (Ops<T>::bits(b) << 16);
+}
+
+// Orders this wave's LDS traffic: everything written before is visible to every
+// lane of the wave after (LDS executes a wave's instructions in order; this keeps
+// the compiler from moving accesses across the point).
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// ===========================================================================
+// state kernel
+// ===========================================================================
+// Lane l = (p = l%32, kb = l/32) owns features CK*p .. CK*p+CK-1 (CK = D/32) of
+// eight tokens t0 + 8*kb + j.  A[c] / B[c] are the MFMA operands of feature
+// column c: 8 tokens of one feature = 4 dwords.
+template <int C> struct RowWords { uint32_t w[8][C / 2]; };
+
+template <typename T, int C>
+__device__ __forceinline__ void load_rows(RowWords<C>& dst, const T* __restrict__ base,
+                                          int64_t row0, int64_t rstride, int D, int tok0, int t_end,
+                                          int p) {
+  const T* ptr0 = base + (row0 + (int64_t)tok0 * rstride) * D + C * p;
+  const int64_t step = rstride * D;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int tok = tok0 + j;
+    if (tok < t_end) {
+      const T* ptr = ptr0 + j * step;
+      if constexpr (C == 2) {
+        dst.w[j][0] = *reinterpret_cast<const uint32_t*>(ptr);
+      } else {
+        u32x2 x = *reinterpret_cast<const u32x2*>(ptr);
+        dst.w[j][0] = x[0];
+        dst.w[j][1] = x[1];
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < C / 2; ++c) dst.w[j][c] = 0u;
+    }
+  }
+}
+
+// token-pair packing: operand c gets feature c of tokens (2i, 2i+1) in dword i
+template <int C>
+__device__ __forceinline__ void transpose_rows(const RowWords<C>& src, u32x4 (&op)[C]) {
+#pragma unroll
+  for (int c2 = 0; c2 < C / 2; ++c2)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t a = src.w[2 * i][c2], b = src.w[2 * i + 1][c2];
+      op[2 * c2][i] = __builtin_amdgcn_perm(b, a, 0x05040100u);      // low halves
+      op[2 * c2 + 1][i] = __builtin_amdgcn_perm(b, a, 0x07060302u);  // high halves
+    }
+}
+
+template <typename T, int DK, int DV, bool SPLIT_KD>
+__global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __restrict__ kn,
+                                                         const T* __restrict__ v,
+                                                         const T* __restrict__ kd,
+                                                         float* __restrict__ partial, int chunk,
+                                                         int nchunks) {
+  constexpr int CK = DK / 32, CV = DV / 32;
+  constexpr int kAcc = CK * CV * 16;          // accumulator floats per lane
+  __shared__ float red[64 * (kAcc + CK)];      // cross-wave reduction buffer, [value][lane]
+
+  const int nh = blockIdx.x / nchunks, c = blockIdx.x - nh * nchunks;
+  const int n = nh / p.H, h = nh - n * p.H;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t_begin = c * chunk;
+  if (t_begin >= len) return;
+  const int t_end = min(len, t_begin + chunk);
+  row_base(p, n, h, bos, row0, rstride);
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pp = lane & 31, kb = lane >> 5;
+
+  f32x16 acc[CK][CV];
+#pragma unroll
+  for (int a = 0; a < CK; ++a)
+#pragma unroll
+    for (int b = 0; b < CV; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  float ks[CK];
+#pragma unroll
+  for (int a = 0; a < CK; ++a) ks[a] = 0.f;
+
+  // 16-token tiles, interleaved over the 4 waves; next tile is in flight while
+  // the current one is multiplied.
+  int t0 = t_begin + 16 * wave;
+  RowWords<CK> kw, kw_n, kdw, kdw_n;
+  RowWords<CV> vw, vw_n;
+  if (t0 < t_end) {
+    load_rows<T, CK>(kw, kn, row0, rstride, DK, t0 + 8 * kb, t_end, pp);
+    load_rows<T, CV>(vw, v, row0, rstride, DV, t0 + 8 * kb, t_end, pp);
+    if constexpr (SPLIT_KD) load_rows<T, CK>(kdw, kd, row0, rstride, DK, t0 + 8 * kb, t_end, pp);
+  }
+  while (t0 < t_end) {
+    const int tn = t0 + 16 * kWaves;
+    if (tn < t_end) {
+      load_rows<T, CK>(kw_n, kn, row0, rstride, DK, tn + 8 * kb, t_end, pp);
+      load_rows<T, CV>(vw_n, v, row0, rstride, DV, tn + 8 * kb, t_end, pp);
+      if constexpr (SPLIT_KD) load_rows<T, CK>(kdw_n, kd, row0, rstride, DK, tn + 8 * kb, t_end, pp);
+    }
+    u32x4 A[CK], B[CV];
+    transpose_rows<CK>(kw, A);
+    transpose_rows<CV>(vw, B);
+#pragma unroll
+    for (int a = 0; a < CK; ++a)
+#pragma unroll
+      for (int b = 0; b < CV; ++b) acc[a][b] = Ops<T>::mma(A[a], B[b], acc[a][b]);
+    if constexpr (SPLIT_KD) {
+      u32x4 D[CK];
+      transpose_rows<CK>(kdw, D);
+#pragma unroll
+      for (int a = 0; a < CK; ++a)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ks[a] = Ops<T>::dot2(D[a][i], Ops<T>::kOnes, ks[a]);
+    } else {
+#pragma unroll
+      for (int a = 0; a < CK; ++a)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ks[a] = Ops<T>::dot2(A[a][i], Ops<T>::kOnes, ks[a]);
+    }
+    kw = kw_n;
+    vw = vw_n;
+    if constexpr (SPLIT_KD) kdw = kdw_n;
+    t0 = tn;
+  }
+
+  // fixed-order reduction over the 4 waves through one LDS buffer:
+  // 2 -> 0, 3 -> 1, 1 -> 0
+  auto spill = [&]() {
+#pragma unroll
+    for (int a = 0; a < CK; ++a)
+#pragma unroll
+      for (int b = 0; b < CV; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) red[((a * CV + b) * 16 + r) * 64 + lane] = acc[a][b][r];
+#pragma unroll
+    for (int a = 0; a < CK; ++a) red[(kAcc + a) * 64 + lane] = ks[a];
+  };
+  auto absorb = [&]() {
+#pragma unroll
+    for (int a = 0; a < CK; ++a)
+#pragma unroll
+      for (int b = 0; b < CV; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] += red[((a * CV + b) * 16 + r) * 64 + lane];
+#pragma unroll
+    for (int a = 0; a < CK; ++a) ks[a] += red[(kAcc + a) * 64 + lane];
+  };
+  if (wave == 2) spill();
+  __syncthreads();
+  if (wave == 0) absorb();
+  __syncthreads();
+  if (wave == 3) spill();
+  __syncthreads();
+  if (wave == 1) absorb();
+  __syncthreads();
+  if (wave == 1) spill();
+  __syncthreads();
+  if (wave != 0) return;
+  absorb();
+
+  // canonical [dk][dv] partial: register r of block (a,b) is dk = CK*m + a,
+  // dv = CV*pp + b with m = 8*(r/4) + 4*kb + r%4.
+  float* dst = partial + (int64_t)blockIdx.x * (DK * DV + DK);
+#pragma unroll
+  for (int a = 0; a < CK; ++a)
+#pragma unroll
+    for (int b = 0; b < CV; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = 8 * (r >> 2) + 4 * kb + (r & 3);
+        dst[(CK * m + a) * DV + CV * pp + b] = acc[a][b][r];
+      }
+#pragma unroll
+  for (int a = 0; a < CK; ++a) {
+    const float tot = ks[a] + __shfl_xor(ks[a], 32);
+    if (kb == 0) dst[DK * DV + CK * pp + a] = tot;
+  }
+}
+
+// ===========================================================================
+// rows kernel: out_t = (x_t M) * rowscale_t + addvec
+// ===========================================================================
+// byte offset of 16-byte chunk `chunk` of row `row` inside a swizzled tile
+template <int ROWB> __device__ __forceinline__ int swz(int row, int chunk) {
+  return row * ROWB + ((chunk ^ (row & 7)) << 4);
+}
+
+// LDS layout of the matrix operand: fragment f = (b*KS + s)*2 + hl holds, for
+// lane l = (m = l%32, kb = l/32), the 8 values  M[(DR/2)*kb + 8s + i][sigma(b,m)]
+// where sigma(b, m = 8g + 4kb' + j) = (DC/2)*kb' + 16b + 4g + j, so that after the
+// MFMA every lane (token, kb') owns DC/2 consecutive output features.
+template <typename T, int DR, int DC, bool NORM, bool DEN>
+__global__ __launch_bounds__(kThreads) void rows_kernel(Prob p, RowsJob job, int chunk,
+                                                        int nchunks) {
+  constexpr int KS = DR / 16;  // k-steps
+  constexpr int NB = DC / 32;  // output blocks
+  constexpr int XROWB = DR * 2, OROWB = DC * 2;
+  constexpr int XCH = XROWB / 16, OCH = OROWB / 16;  // 16-byte chunks per row
+  constexpr int kStage = 32 * (XROWB > OROWB ? XROWB : OROWB);
+  constexpr int kOpnd = NB * KS * 2 * 1024;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_opnd[kOpnd];
+  __shared__ __attribute__((aligned(16))) unsigned char lds_stage[kWaves][(DEN ? 2 : 1) * kStage];
+  __shared__ __attribute__((aligned(16))) uint32_t lds_km[2][DR / 2];
+  __shared__ __attribute__((aligned(16))) float lds_add[DC];
+  __shared__ float lds_max[kWaves];
+
+  const int nh = blockIdx.x / nchunks, c = blockIdx.x - nh * nchunks;
+  const int n = nh / p.H, h = nh - n * p.H;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t_begin = c * chunk;
+  if (t_begin >= len) return;
+  const int t_end = min(len, t_begin + chunk);
+  row_base(p, n, h, bos, row0, rstride);
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const T* x = (const T*)job.x;
+  const T* xden = (const T*)job.xden;
+  T* out = (T*)job.out;
+  const float* mat = job.mat + (int64_t)nh * DR * DC;
+
+  // ---- prologue: normalise M by a power of two, split hi/lo, store fragments ----
+  float mx = 0.f;
+  for (int e = tid; e < DR * DC; e += kThreads) mx = fmaxf(mx, fabsf(mat[e]));
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+  if (lane == 0) lds_max[wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(lds_max[0], lds_max[1]), fmaxf(lds_max[2], lds_max[3]));
+  // power of two that brings max|M| into [8,16); 1 when M is zero or not finite
+  float norm = 1.f;
+  if (mx > 0.f && mx < 3.0e38f) {
+    int e;
+    frexpf(mx, &e);
+    norm = ldexpf(1.f, 4 - e);
+  }
+  const float denorm = 1.f / norm;
+  {
+    uint16_t* op16 = reinterpret_cast<uint16_t*>(lds_opnd);
+    for (int e = tid; e < NB * KS * 64 * 8; e += kThreads) {
+      const int i = e & 7, l = (e >> 3) & 63, f = e >> 9;  // f = b*KS + s
+      const int s = f % KS, b = f / KS;
+      const int m = l & 31, kbA = l >> 5;
+      const int r = (DR / 2) * kbA + 8 * s + i;
+      const int cc = (DC / 2) * ((m >> 2) & 1) + 16 * b + 4 * (m >> 3) + (m & 3);
+      const float val = mat[(int64_t)r * job.ld_r + (int64_t)cc * job.ld_c] * norm;
+      const T hi = (T)val;
+      const T lo = (T)(val - (float)hi);
+      op16[((2 * f + 0) * 64 + l) * 8 + i] = __builtin_bit_cast(uint16_t, hi);
+      op16[((2 * f + 1) * 64 + l) * 8 + i] = __builtin_bit_cast(uint16_t, lo);
+    }
+    if constexpr (NORM) {
+      const float* kmh = job.km + (int64_t)nh * DR;
+      for (int e = tid; e < DR / 2; e += kThreads) {
+        const float a = kmh[2 * e], b = kmh[2 * e + 1];
+        const T ah = (T)a, bh = (T)b;
+        lds_km[0][e] = pack2<T>((float)ah, (float)bh);
+        lds_km[1][e] = pack2<T>(a - (float)ah, b - (float)bh);
+      }
+    }
+    for (int e = tid; e < DC; e += kThreads)
+      lds_add[e] = job.addvec ? job.addvec[(int64_t)nh * DC + e] : 0.f;
+  }
+  __syncthreads();
+
+  // ---- main loop: 32-token sub-tiles, interleaved over the waves ----
+  const int ntok = lane & 31, kb = lane >> 5;  // MFMA view: token column, k half
+  unsigned char* stage = lds_stage[wave];
+  unsigned char* stage_den = stage + kStage;
+  constexpr int XI = 32 * XCH / 64;  // flat 16-byte loads per lane per tile
+  constexpr int OI = 32 * OCH / 64;
+
+  auto load_tile = [&](u32x4(&dst)[XI], const T* src, int tok0) {
+#pragma unroll
+    for (int i = 0; i < XI; ++i) {
+      const int q = lane + 64 * i, row = q / XCH, ch = q % XCH;
+      const int tok = tok0 + row;
+      if (tok < t_end) {
+        dst[i] = *reinterpret_cast<const u32x4*>(src + (row0 + (int64_t)tok * rstride) * DR + ch * 8);
+      } else {
+        dst[i] = u32x4{0u, 0u, 0u, 0u};
+      }
+    }
+  };
+  auto stash_tile = [&](const u32x4(&src)[XI], unsigned char* dstb) {
+#pragma unroll
+    for (int i = 0; i < XI; ++i) {
+      const int q = lane + 64 * i, row = q / XCH, ch = q % XCH;
+      *reinterpret_cast<u32x4*>(dstb + swz<XROWB>(row, ch)) = src[i];
+    }
+  };
+
+  int t0 = t_begin + 32 * wave;
+  u32x4 xr[XI], xd[XI];
+  if (t0 < t_end) {
+    load_tile(xr, x, t0);
+    if constexpr (DEN) load_tile(xd, xden, t0);
+  }
+  while (t0 < t_end) {
+    wave_sync();  // previous tile's staging reads are done
+    stash_tile(xr, stage);
+    if constexpr (DEN) stash_tile(xd, stage_den);
+    const int tn = t0 + 32 * kWaves;
+    if (tn < t_end) {
+      load_tile(xr, x, tn);
+      if constexpr (DEN) load_tile(xd, xden, tn);
+    }
+    wave_sync();
+
+    f32x16 acc[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[b][r] = 0.f;
+    float z = 0.f;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const u32x4 bq = *reinterpret_cast<const u32x4*>(stage + swz<XROWB>(ntok, KS * kb + s));
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        const u32x4 ah = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * (b * KS + s) + 0) * 64 + lane) * 16);
+        const u32x4 al = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * (b * KS + s) + 1) * 64 + lane) * 16);
+        acc[b] = Ops<T>::mma(ah, bq, acc[b]);
+        acc[b] = Ops<T>::mma(al, bq, acc[b]);
+      }
+      if constexpr (NORM) {
+        u32x4 bd = bq;
+        if constexpr (DEN) bd = *reinterpret_cast<const u32x4*>(stage_den + swz<XROWB>(ntok, KS * kb + s));
+        const u32x4 kh = *reinterpret_cast<const u32x4*>(&lds_km[0][(DR / 4) * kb + 4 * s]);
+        const u32x4 kl = *reinterpret_cast<const u32x4*>(&lds_km[1][(DR / 4) * kb + 4 * s]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          z = Ops<T>::dot2(bd[i], kh[i], z);
+          z = Ops<T>::dot2(bd[i], kl[i], z);
+        }
+      }
+    }
+    float rs = denorm;
+    if constexpr (NORM) {
+      z += __shfl_xor(z, 32);
+      rs = denorm / (z + p.eps);
+    }
+    wave_sync();  // all lanes have read their x chunks; staging is reused for out
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      u32x4 w0, w1;
+      const float* av = &lds_add[(DC / 2) * kb + 16 * b];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        w0[i] = pack2<T>(fmaf(acc[b][2 * i], rs, av[2 * i]), fmaf(acc[b][2 * i + 1], rs, av[2 * i + 1]));
+        w1[i] = pack2<T>(fmaf(acc[b][8 + 2 * i], rs, av[8 + 2 * i]),
+                         fmaf(acc[b][8 + 2 * i + 1], rs, av[8 + 2 * i + 1]));
+      }
+      *reinterpret_cast<u32x4*>(stage + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b)) = w0;
+      *reinterpret_cast<u32x4*>(stage + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b + 1)) = w1;
+    }
+    wave_sync();
+#pragma unroll
+    for (int i = 0; i < OI; ++i) {
+      const int q = lane + 64 * i, row = q / OCH, ch = q % OCH;
+      const int tok = t0 + row;
+      if (tok < t_end) {
+        const u32x4 w = *reinterpret_cast<const u32x4*>(stage + swz<OROWB>(row, ch));
+        *reinterpret_cast<u32x4*>(out + (row0 + (int64_t)tok * rstride) * DC + ch * 8) = w;
+      }
+    }
+    t0 = tn;
+  }
+}
+
+// ===========================================================================
+// host side
+// ===========================================================================
+bool supported(const Prob& p, int dtype) {
+  if (dtype != kF16 && dtype != kBF16) return false;
+  return p.DK == 64 && p.DV == 64;
+}
+
+// Chunk (tokens per workgroup) of the reduction kernels: ~4 workgroups per CU.
+int state_chunk(const Prob& p) {
+  const int64_t nh = (int64_t)p.N * p.H;
+  int64_t chunk = cdiv64((int64_t)p.L * nh, 1024);
+  chunk = cdiv64(chunk, 64) * 64;
+  if (chunk < 256) chunk = 256;
+  return (int)chunk;
+}
+
+// Chunk of the row-parallel kernels: long enough to amortise the operand prologue.
+int rows_chunk(const Prob& p) {
+  const int64_t nh = (int64_t)p.N * p.H;
+  int64_t chunk = cdiv64((int64_t)p.L * nh, 2048);
+  chunk = cdiv64(chunk, 128) * 128;
+  if (chunk < 512) chunk = 512;
+  return (int)chunk;
+}
+
+template <typename T, int DK, int DV>
+static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, float* partial,
+                         int chunk, int nchunks, hipStream_t st) {
+  const unsigned grid = (unsigned)((int64_t)p.N * p.H * nchunks);
+  if (p.flags & kDecoupled)
+    state_kernel<T, DK, DV, true><<<dim3(grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
+  else
+    state_kernel<T, DK, DV, false><<<dim3(grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
+}
+
+template <typename T>
+void run_state(const Prob& p, const void* kn, const void* v, const void* kd, float* partial,
+               int chunk, int nchunks, hipStream_t st) {
+  launch_state<T, 64, 64>(p, (const T*)kn, (const T*)v, (const T*)kd, partial, chunk, nchunks, st);
+}
+
+template <typename T, int DR, int DC>
+static void launch_rows(const Prob& p, const RowsJob& job, hipStream_t st) {
+  const int chunk = rows_chunk(p);
+  const int nchunks = (int)cdiv64(p.L, chunk);
+  const unsigned grid = (unsigned)((int64_t)p.N * p.H * nchunks);
+  const bool norm = job.xden != nullptr;
+  const bool den = norm && job.xden != job.x;
+  if (!norm)
+    rows_kernel<T, DR, DC, false, false><<<dim3(grid), dim3(kThreads), 0, st>>>(p, job, chunk, nchunks);
+  else if (!den)
+    rows_kernel<T, DR, DC, true, false><<<dim3(grid), dim3(kThreads), 0, st>>>(p, job, chunk, nchunks);
+  else
+    rows_kernel<T, DR, DC, true, true><<<dim3(grid), dim3(kThreads), 0, st>>>(p, job, chunk, nchunks);
+}
+
+template <typename T>
+void run_rows(const Prob& p, const RowsJob& job, int DR, int DC, hipStream_t st) {
+  (void)DR;
+  (void)DC;
+  launch_rows<T, 64, 64>(p, job, st);
+}
+
+void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
+           int chunk, int nchunks, hipStream_t st) {
+  if (dtype == kF16) run_state<_Float16>(p, kn, v, kd, partial, chunk, nchunks, st);
+  else run_state<__bf16>(p, kn, v, kd, partial, chunk, nchunks, st);
+}
+
+void rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {
+  if (dtype == kF16) run_rows<_Float16>(p, job, DR, DC, st);
+  else run_rows<__bf16>(p, job, DR, DC, st);
+}
+
+}  // namespace mfma
+}  // namespace fbla

@@ -1,0 +1,111 @@
+// The plan: which kernels run, in which order, for each entry point, and how the
+// caller's workspace is carved up.  MFMA kernels are used for the shapes they
+// cover (16-bit inputs, head dims 64); everything else runs on the generic kernels.
+//
+// forward :  state partials -> fixed-order reduce (S, km) -> output rows
+// backward:  S^T -> pass A (dq, partial dS/dkm) -> reduce (s dS, its transpose, dkm/L)
+//            -> pass B (dk, dv)
+#include "fbla_kernels.h"
+
+namespace fbla {
+namespace plan {
+
+static size_t state_bytes(const Prob& p) {
+  return align_up((size_t)p.N * p.H * p.DK * p.DV * sizeof(float), 256);
+}
+static size_t vec_bytes(const Prob& p) {
+  return align_up((size_t)p.N * p.H * p.DK * sizeof(float), 256);
+}
+static size_t partial_bytes(const Prob& p, int chunk) {
+  const int64_t nchunks = cdiv64(p.L, chunk);
+  return align_up((size_t)p.N * p.H * nchunks * ((size_t)p.DK * p.DV + p.DK) * sizeof(float), 256);
+}
+static int fwd_chunk(const Prob& p, int dtype) {
+  return mfma::supported(p, dtype) ? mfma::state_chunk(p) : generic::state_chunk(p);
+}
+static int bwd_chunk(const Prob& p, int dtype) {
+  (void)dtype;
+  return generic::state_chunk(p);
+}
+
+size_t fwd_workspace_bytes(const Prob& p, int dtype) { return partial_bytes(p, fwd_chunk(p, dtype)); }
+
+// partials | S^T | s*dS | (s*dS)^T | dkm/L
+size_t bwd_workspace_bytes(const Prob& p, int dtype) {
+  return partial_bytes(p, bwd_chunk(p, dtype)) + 3 * state_bytes(p) + vec_bytes(p);
+}
+
+int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
+  const bool dec = p.flags & kDecoupled;
+  const bool normalize = p.flags & kNormalize;
+  const void* qn = dec ? a.q_rope : a.q;
+  const void* kn = dec ? a.k_rope : a.k;
+  const bool fast = mfma::supported(p, dtype);
+  const int chunk = fwd_chunk(p, dtype);
+  const int nchunks = (int)cdiv64(p.L, chunk);
+  float* partial = (float*)a.workspace;
+  const unsigned phases = phase_mask();
+  if (phases & kPhaseFwdState) {
+    if (fast) mfma::state(p, dtype, kn, a.v, a.k, partial, chunk, nchunks, st);
+    else generic::state_partial(p, dtype, kn, a.v, a.k, partial, chunk, nchunks, st);
+  }
+  if (phases & kPhaseFwdReduce)
+    generic::state_reduce(p, partial, chunk, nchunks, a.s, nullptr, a.km, st);
+  if (phases & kPhaseFwdOutput) {
+    if (fast) {
+      mfma::RowsJob job{qn, normalize ? a.q : nullptr, a.s, p.DV, 1, a.km, nullptr, a.o};
+      mfma::rows(p, dtype, job, p.DK, p.DV, st);
+    } else {
+      generic::output(p, dtype, qn, a.q, a.s, a.km, a.o, st);
+    }
+  }
+  return kOk;
+}
+
+int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
+  const bool dec = p.flags & kDecoupled;
+  const bool normalize = p.flags & kNormalize;
+  const void* qn = dec ? a.q_rope : a.q;
+  const void* kn = dec ? a.k_rope : a.k;
+  void* dqn = dec ? a.dq_rope : a.dq;
+  void* dkn = dec ? a.dk_rope : a.dk;
+  void* dqd = dec ? a.dq : nullptr;
+  void* dkd = dec ? a.dk : nullptr;
+  const bool fast = mfma::supported(p, dtype);
+  const int chunk = bwd_chunk(p, dtype);
+  const int nchunks = (int)cdiv64(p.L, chunk);
+  char* ws = (char*)a.workspace;
+  float* partial = (float*)ws;
+  ws += partial_bytes(p, chunk);
+  float* St = (float*)ws;
+  ws += state_bytes(p);
+  float* dS = (float*)ws;
+  ws += state_bytes(p);
+  float* dSt = (float*)ws;
+  ws += state_bytes(p);
+  float* dkm = (float*)ws;
+  const unsigned phases = phase_mask();
+  if (phases & kPhaseBwdA) {
+    generic::transpose_state(p, a.s, St, st);
+    generic::bwd_a(p, dtype, qn, a.q, a.dout, a.s, St, a.km, dqn, dqd, partial, chunk, nchunks, st);
+  }
+  if (phases & kPhaseBwdReduce)
+    generic::state_reduce(p, partial, chunk, nchunks, dS, dSt, dkm, st);
+  if (phases & kPhaseBwdB) {
+    if (fast) {
+      // dk~_t = v_t (s dS)^T (+ dkm/L): contraction over dv, M(r=dv, c=dk) = dS[c][r]
+      mfma::RowsJob jk{a.v, nullptr, dS, 1, p.DV, nullptr, (!dec && normalize) ? dkm : nullptr, dkn};
+      mfma::rows(p, dtype, jk, p.DV, p.DK, st);
+      // dv_t = k~_t (s dS): contraction over dk
+      mfma::RowsJob jv{kn, nullptr, dS, p.DV, 1, nullptr, nullptr, a.dv};
+      mfma::rows(p, dtype, jv, p.DK, p.DV, st);
+      if (dec) generic::broadcast_rows(p, dtype, dkm, dkd, st);
+    } else {
+      generic::bwd_b(p, dtype, kn, a.v, dS, dSt, dkm, dkn, dkd, a.dv, st);
+    }
+  }
+  return kOk;
+}
+
+}  // namespace plan
+}  // namespace fbla
