@@ -79,6 +79,10 @@ void state(const Prob& p, int dtype, const void* kn, const void* v, const void* 
            int chunk, int nchunks, hipStream_t st);
 // out_t = (x_t M) / (xden_t . km + eps) + addvec   with M of shape DR x DC
 void rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st);
+// backward pass A: dq~ (and dq when decoupled) + per-chunk partials of dS and dkm
+int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout, const float* S,
+          const float* km, void* dqn, void* dqd, float* partial, int chunk, int nchunks,
+          hipStream_t st);
 }  // namespace mfma
 
 }  // namespace fbla

@@ -137,6 +137,64 @@ __device__ __forceinline__ void transpose_rows(const RowWords<C>& src, u32x4 (&o
     }
 }
 
+// Fixed-order sum of the four waves' accumulators through one LDS buffer
+// (2 -> 0, 3 -> 1, 1 -> 0), then wave 0 writes the canonical [dk][dv] partial
+// followed by the [dk] vector.  Register r of block (a,b) is dk = CK*m + a,
+// dv = CV*pp + b with m = 8*(r/4) + 4*kb + r%4.  Must be reached by all waves.
+template <int CK, int CV>
+__device__ __forceinline__ void reduce_store_partial(f32x16 (&acc)[CK][CV], float (&ks)[CK],
+                                                     float* red, float* dst, int wave, int lane) {
+  constexpr int kAcc = CK * CV * 16;
+  constexpr int DK = 32 * CK, DV = 32 * CV;
+  const int pp = lane & 31, kb = lane >> 5;
+  auto spill = [&]() {
+#pragma unroll
+    for (int a = 0; a < CK; ++a)
+#pragma unroll
+      for (int b = 0; b < CV; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) red[((a * CV + b) * 16 + r) * 64 + lane] = acc[a][b][r];
+#pragma unroll
+    for (int a = 0; a < CK; ++a) red[(kAcc + a) * 64 + lane] = ks[a];
+  };
+  auto absorb = [&]() {
+#pragma unroll
+    for (int a = 0; a < CK; ++a)
+#pragma unroll
+      for (int b = 0; b < CV; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] += red[((a * CV + b) * 16 + r) * 64 + lane];
+#pragma unroll
+    for (int a = 0; a < CK; ++a) ks[a] += red[(kAcc + a) * 64 + lane];
+  };
+  if (wave == 2) spill();
+  __syncthreads();
+  if (wave == 0) absorb();
+  __syncthreads();
+  if (wave == 3) spill();
+  __syncthreads();
+  if (wave == 1) absorb();
+  __syncthreads();
+  if (wave == 1) spill();
+  __syncthreads();
+  if (wave != 0) return;
+  absorb();
+#pragma unroll
+  for (int a = 0; a < CK; ++a)
+#pragma unroll
+    for (int b = 0; b < CV; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = 8 * (r >> 2) + 4 * kb + (r & 3);
+        dst[(CK * m + a) * DV + CV * pp + b] = acc[a][b][r];
+      }
+#pragma unroll
+  for (int a = 0; a < CK; ++a) {
+    const float tot = ks[a] + __shfl_xor(ks[a], 32);
+    if (kb == 0) dst[DK * DV + CK * pp + a] = tot;
+  }
+}
+
 template <typename T, int DK, int DV, bool SPLIT_KD>
 __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __restrict__ kn,
                                                          const T* __restrict__ v,
@@ -214,58 +272,8 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
     t0 = tn;
   }
 
-  // fixed-order reduction over the 4 waves through one LDS buffer:
-  // 2 -> 0, 3 -> 1, 1 -> 0
-  auto spill = [&]() {
-#pragma unroll
-    for (int a = 0; a < CK; ++a)
-#pragma unroll
-      for (int b = 0; b < CV; ++b)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) red[((a * CV + b) * 16 + r) * 64 + lane] = acc[a][b][r];
-#pragma unroll
-    for (int a = 0; a < CK; ++a) red[(kAcc + a) * 64 + lane] = ks[a];
-  };
-  auto absorb = [&]() {
-#pragma unroll
-    for (int a = 0; a < CK; ++a)
-#pragma unroll
-      for (int b = 0; b < CV; ++b)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][b][r] += red[((a * CV + b) * 16 + r) * 64 + lane];
-#pragma unroll
-    for (int a = 0; a < CK; ++a) ks[a] += red[(kAcc + a) * 64 + lane];
-  };
-  if (wave == 2) spill();
-  __syncthreads();
-  if (wave == 0) absorb();
-  __syncthreads();
-  if (wave == 3) spill();
-  __syncthreads();
-  if (wave == 1) absorb();
-  __syncthreads();
-  if (wave == 1) spill();
-  __syncthreads();
-  if (wave != 0) return;
-  absorb();
-
-  // canonical [dk][dv] partial: register r of block (a,b) is dk = CK*m + a,
-  // dv = CV*pp + b with m = 8*(r/4) + 4*kb + r%4.
   float* dst = partial + (int64_t)blockIdx.x * (DK * DV + DK);
-#pragma unroll
-  for (int a = 0; a < CK; ++a)
-#pragma unroll
-    for (int b = 0; b < CV; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = 8 * (r >> 2) + 4 * kb + (r & 3);
-        dst[(CK * m + a) * DV + CV * pp + b] = acc[a][b][r];
-      }
-#pragma unroll
-  for (int a = 0; a < CK; ++a) {
-    const float tot = ks[a] + __shfl_xor(ks[a], 32);
-    if (kb == 0) dst[DK * DV + CK * pp + a] = tot;
-  }
+  reduce_store_partial<CK, CV>(acc, ks, red, dst, wave, lane);
 }
 
 // ===========================================================================
@@ -276,10 +284,59 @@ template <int ROWB> __device__ __forceinline__ int swz(int row, int chunk) {
   return row * ROWB + ((chunk ^ (row & 7)) << 4);
 }
 
-// LDS layout of the matrix operand: fragment f = (b*KS + s)*2 + hl holds, for
-// lane l = (m = l%32, kb = l/32), the 8 values  M[(DR/2)*kb + 8s + i][sigma(b,m)]
+// LDS layout of a DR x DC matrix operand M: fragment f = (b*KS + s)*2 + hl holds,
+// for lane l = (m = l%32, kb = l/32), the 8 values  M[(DR/2)*kb + 8s + i][sigma(b,m)]
 // where sigma(b, m = 8g + 4kb' + j) = (DC/2)*kb' + 16b + 4g + j, so that after the
-// MFMA every lane (token, kb') owns DC/2 consecutive output features.
+// MFMA every lane (token, kb') owns DC/2 consecutive output features.  M is first
+// multiplied by a power of two that brings max|M| into [8,16), then split into a
+// 16-bit hi part and a 16-bit lo remainder (two MFMAs recover ~fp32 accuracy).
+// Returns the factor that undoes the normalisation.  Contains workgroup barriers;
+// the caller must __syncthreads() before reading the fragments.
+template <typename T, int DR, int DC>
+__device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* lds_max,
+                                               const float* __restrict__ mat, int ld_r, int ld_c) {
+  constexpr int KS = DR / 16, NB = DC / 32;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  float mx = 0.f;
+  for (int e = tid; e < DR * DC; e += kThreads) mx = fmaxf(mx, fabsf(mat[e]));
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+  if (lane == 0) lds_max[wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(lds_max[0], lds_max[1]), fmaxf(lds_max[2], lds_max[3]));
+  float norm = 1.f;  // also when M is zero or not finite
+  if (mx > 0.f && mx < 3.0e38f) {
+    int e;
+    frexpf(mx, &e);
+    norm = ldexpf(1.f, 4 - e);
+  }
+  uint16_t* op16 = reinterpret_cast<uint16_t*>(lds_opnd);
+  for (int e = tid; e < NB * KS * 64 * 8; e += kThreads) {
+    const int i = e & 7, l = (e >> 3) & 63, f = e >> 9;  // f = b*KS + s
+    const int s = f % KS, b = f / KS;
+    const int m = l & 31, kbA = l >> 5;
+    const int r = (DR / 2) * kbA + 8 * s + i;
+    const int cc = (DC / 2) * ((m >> 2) & 1) + 16 * b + 4 * (m >> 3) + (m & 3);
+    const float val = mat[(int64_t)r * ld_r + (int64_t)cc * ld_c] * norm;
+    const T hi = (T)val;
+    const T lo = (T)(val - (float)hi);
+    op16[((2 * f + 0) * 64 + l) * 8 + i] = __builtin_bit_cast(uint16_t, hi);
+    op16[((2 * f + 1) * 64 + l) * 8 + i] = __builtin_bit_cast(uint16_t, lo);
+  }
+  return 1.f / norm;
+}
+
+// km as 16-bit hi/lo pairs (for v_dot2) : pairs[0][e] = hi(km[2e], km[2e+1]), pairs[1][e] = lo
+template <typename T>
+__device__ __forceinline__ void build_km_pairs(uint32_t* pairs, const float* __restrict__ kmh, int D) {
+  for (int e = threadIdx.x; e < D / 2; e += kThreads) {
+    const float a = kmh[2 * e], b = kmh[2 * e + 1];
+    const T ah = (T)a, bh = (T)b;
+    pairs[e] = pack2<T>((float)ah, (float)bh);
+    pairs[D / 2 + e] = pack2<T>(a - (float)ah, b - (float)bh);
+  }
+}
+
 template <typename T, int DR, int DC, bool NORM, bool DEN>
 __global__ __launch_bounds__(kThreads) void rows_kernel(Prob p, RowsJob job, int chunk,
                                                         int nchunks) {
@@ -311,45 +368,10 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(Prob p, RowsJob job, int
   T* out = (T*)job.out;
   const float* mat = job.mat + (int64_t)nh * DR * DC;
 
-  // ---- prologue: normalise M by a power of two, split hi/lo, store fragments ----
-  float mx = 0.f;
-  for (int e = tid; e < DR * DC; e += kThreads) mx = fmaxf(mx, fabsf(mat[e]));
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-  if (lane == 0) lds_max[wave] = mx;
-  __syncthreads();
-  mx = fmaxf(fmaxf(lds_max[0], lds_max[1]), fmaxf(lds_max[2], lds_max[3]));
-  // power of two that brings max|M| into [8,16); 1 when M is zero or not finite
-  float norm = 1.f;
-  if (mx > 0.f && mx < 3.0e38f) {
-    int e;
-    frexpf(mx, &e);
-    norm = ldexpf(1.f, 4 - e);
-  }
-  const float denorm = 1.f / norm;
+  // ---- prologue: matrix operand fragments, km pairs, addvec ----
+  const float denorm = build_operand<T, DR, DC>(lds_opnd, lds_max, mat, job.ld_r, job.ld_c);
   {
-    uint16_t* op16 = reinterpret_cast<uint16_t*>(lds_opnd);
-    for (int e = tid; e < NB * KS * 64 * 8; e += kThreads) {
-      const int i = e & 7, l = (e >> 3) & 63, f = e >> 9;  // f = b*KS + s
-      const int s = f % KS, b = f / KS;
-      const int m = l & 31, kbA = l >> 5;
-      const int r = (DR / 2) * kbA + 8 * s + i;
-      const int cc = (DC / 2) * ((m >> 2) & 1) + 16 * b + 4 * (m >> 3) + (m & 3);
-      const float val = mat[(int64_t)r * job.ld_r + (int64_t)cc * job.ld_c] * norm;
-      const T hi = (T)val;
-      const T lo = (T)(val - (float)hi);
-      op16[((2 * f + 0) * 64 + l) * 8 + i] = __builtin_bit_cast(uint16_t, hi);
-      op16[((2 * f + 1) * 64 + l) * 8 + i] = __builtin_bit_cast(uint16_t, lo);
-    }
-    if constexpr (NORM) {
-      const float* kmh = job.km + (int64_t)nh * DR;
-      for (int e = tid; e < DR / 2; e += kThreads) {
-        const float a = kmh[2 * e], b = kmh[2 * e + 1];
-        const T ah = (T)a, bh = (T)b;
-        lds_km[0][e] = pack2<T>((float)ah, (float)bh);
-        lds_km[1][e] = pack2<T>(a - (float)ah, b - (float)bh);
-      }
-    }
+    if constexpr (NORM) build_km_pairs<T>(&lds_km[0][0], job.km + (int64_t)nh * DR, DR);
     for (int e = tid; e < DC; e += kThreads)
       lds_add[e] = job.addvec ? job.addvec[(int64_t)nh * DC + e] : 0.f;
   }
@@ -461,6 +483,307 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(Prob p, RowsJob job, int
 }
 
 // ===========================================================================
+// backward pass A
+// ===========================================================================
+// Per 32-token sub-tile (one wave):
+//   token view (lane = token n, half kb):  g_t = dO_t S^T by MFMA, then in registers
+//     P_t = q~_t . g_t,  z_t = q_t . km + eps,  dz_t = -P_t / z_t^2,
+//     dq~_t = g_t / z_t (+ dz_t km),  and dO_t / z_t is written back to LDS as hi + lo;
+//   feature view (lane = feature pair, registers = tokens): dS += q~^T (dO / z) by MFMA
+//     with the same in-register transposition as the state kernel, dkm += dz_t q_t.
+// dS and dkm partials leave through the same reduction as the forward state.
+template <int C>
+__device__ __forceinline__ void lds_rows(RowWords<C>& dst, const unsigned char* tile, int tok0,
+                                         int pp) {
+  constexpr int ROWB = C * 64;  // bytes per row: 32 lanes x C features x 2 bytes
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int row = tok0 + j;
+    if constexpr (C == 2) {
+      dst.w[j][0] = *reinterpret_cast<const uint32_t*>(tile + swz<ROWB>(row, pp >> 2) + ((pp & 3) << 2));
+    } else {
+      const u32x2 x = *reinterpret_cast<const u32x2*>(tile + swz<ROWB>(row, pp >> 1) + ((pp & 1) << 3));
+      dst.w[j][0] = x[0];
+      dst.w[j][1] = x[1];
+    }
+  }
+}
+
+template <int DK, int DV, bool NORM, bool DEN> struct BwdALayout {
+  static constexpr int KS = DV / 16, NB = DK / 32;
+  static constexpr int kOpnd = NB * KS * 2 * 1024;
+  static constexpr int kQ = 32 * DK * 2, kG = 32 * DV * 2;
+  static constexpr int kWave = kQ + kG + (NORM ? kG : 0) + (DEN ? kQ : 0) + 128;  // + dz[32]
+  static constexpr int kKmPairs = kOpnd + kWaves * kWave;
+  static constexpr int kKmF = kKmPairs + DK * 4;
+  static constexpr int kMax = kKmF + DK * 4;
+  static constexpr int kTotal = kMax + 64;
+};
+
+template <typename T, int DK, int DV, bool NORM, bool DEN>
+__global__ __launch_bounds__(kThreads) void bwd_a_kernel(
+    Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const T* __restrict__ dout,
+    const float* __restrict__ S, const float* __restrict__ km, T* __restrict__ dqn,
+    T* __restrict__ dqd, float* __restrict__ partial, int chunk, int nchunks) {
+  using LY = BwdALayout<DK, DV, NORM, DEN>;
+  constexpr int KS = LY::KS, NB = LY::NB;
+  constexpr int CK = DK / 32, CV = DV / 32;
+  constexpr int QROWB = DK * 2, GROWB = DV * 2;
+  constexpr int QCH = QROWB / 16, GCH = GROWB / 16;
+  constexpr int QI = 32 * QCH / 64, GI = 32 * GCH / 64;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int nh = blockIdx.x / nchunks, c = blockIdx.x - nh * nchunks;
+  const int n = nh / p.H, h = nh - n * p.H;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t_begin = c * chunk;
+  if (t_begin >= len) return;
+  const int t_end = min(len, t_begin + chunk);
+  row_base(p, n, h, bos, row0, rstride);
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int ntok = lane & 31, kb = lane >> 5;
+
+  unsigned char* lds_opnd = smem;
+  unsigned char* qt = smem + LY::kOpnd + wave * LY::kWave;
+  unsigned char* gt = qt + LY::kQ;             // dO, later dO/z (hi part)
+  unsigned char* gl = gt + LY::kG;             // dO/z (lo part), NORM only
+  unsigned char* qdt = gl + (NORM ? LY::kG : 0);  // plain q, DEN only
+  float* dzs = reinterpret_cast<float*>(qdt + (DEN ? LY::kQ : 0));
+  uint32_t* km_pairs = reinterpret_cast<uint32_t*>(smem + LY::kKmPairs);
+  float* kmf = reinterpret_cast<float*>(smem + LY::kKmF);
+  float* lds_max = reinterpret_cast<float*>(smem + LY::kMax);
+
+  // g_t = dO_t S^T: contraction over dv, M(r = dv, c = dk) = S[c][r]
+  const float denorm = build_operand<T, DV, DK>(lds_opnd, lds_max, S + (int64_t)nh * DK * DV, 1, DV);
+  if constexpr (NORM) {
+    build_km_pairs<T>(km_pairs, km + (int64_t)nh * DK, DK);
+    for (int e = tid; e < DK; e += kThreads) kmf[e] = km[(int64_t)nh * DK + e];
+  }
+  __syncthreads();
+
+  f32x16 acc[CK][CV];
+#pragma unroll
+  for (int a = 0; a < CK; ++a)
+#pragma unroll
+    for (int b = 0; b < CV; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  float dkm[CK];
+#pragma unroll
+  for (int a = 0; a < CK; ++a) dkm[a] = 0.f;
+
+  auto load_q = [&](u32x4(&dst)[QI], const T* src, int tok0) {
+#pragma unroll
+    for (int i = 0; i < QI; ++i) {
+      const int q = lane + 64 * i, row = q / QCH, ch = q % QCH;
+      const int tok = tok0 + row;
+      dst[i] = tok < t_end
+                   ? *reinterpret_cast<const u32x4*>(src + (row0 + (int64_t)tok * rstride) * DK + ch * 8)
+                   : u32x4{0u, 0u, 0u, 0u};
+    }
+  };
+  auto load_g = [&](u32x4(&dst)[GI], const T* src, int tok0) {
+#pragma unroll
+    for (int i = 0; i < GI; ++i) {
+      const int q = lane + 64 * i, row = q / GCH, ch = q % GCH;
+      const int tok = tok0 + row;
+      dst[i] = tok < t_end
+                   ? *reinterpret_cast<const u32x4*>(src + (row0 + (int64_t)tok * rstride) * DV + ch * 8)
+                   : u32x4{0u, 0u, 0u, 0u};
+    }
+  };
+  auto stash_q = [&](const u32x4(&src)[QI], unsigned char* dstb) {
+#pragma unroll
+    for (int i = 0; i < QI; ++i) {
+      const int q = lane + 64 * i;
+      *reinterpret_cast<u32x4*>(dstb + swz<QROWB>(q / QCH, q % QCH)) = src[i];
+    }
+  };
+  auto stash_g = [&](const u32x4(&src)[GI], unsigned char* dstb) {
+#pragma unroll
+    for (int i = 0; i < GI; ++i) {
+      const int q = lane + 64 * i;
+      *reinterpret_cast<u32x4*>(dstb + swz<GROWB>(q / GCH, q % GCH)) = src[i];
+    }
+  };
+  auto store_q = [&](const unsigned char* srcb, T* dst, int tok0) {
+#pragma unroll
+    for (int i = 0; i < QI; ++i) {
+      const int q = lane + 64 * i, row = q / QCH, ch = q % QCH;
+      const int tok = tok0 + row;
+      if (tok < t_end)
+        *reinterpret_cast<u32x4*>(dst + (row0 + (int64_t)tok * rstride) * DK + ch * 8) =
+            *reinterpret_cast<const u32x4*>(srcb + swz<QROWB>(row, ch));
+    }
+  };
+
+  int t0 = t_begin + 32 * wave;
+  u32x4 rq[QI], rg[GI], rd[QI];
+  if (t0 < t_end) {
+    load_q(rq, qn, t0);
+    load_g(rg, dout, t0);
+    if constexpr (DEN) load_q(rd, qd, t0);
+  }
+  while (t0 < t_end) {
+    wave_sync();  // the previous sub-tile's staged dq has been read out
+    stash_q(rq, qt);
+    stash_g(rg, gt);
+    if constexpr (DEN) stash_q(rd, qdt);
+    const int tn = t0 + 32 * kWaves;
+    if (tn < t_end) {
+      load_q(rq, qn, tn);
+      load_g(rg, dout, tn);
+      if constexpr (DEN) load_q(rd, qd, tn);
+    }
+    wave_sync();
+
+    // ---- token view ----
+    f32x16 g[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) g[b][r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const u32x4 bq = *reinterpret_cast<const u32x4*>(gt + swz<GROWB>(ntok, KS * kb + s));
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        const u32x4 ah = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * (b * KS + s) + 0) * 64 + lane) * 16);
+        const u32x4 al = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * (b * KS + s) + 1) * 64 + lane) * 16);
+        g[b] = Ops<T>::mma(ah, bq, g[b]);
+        g[b] = Ops<T>::mma(al, bq, g[b]);
+      }
+    }
+    // this lane: g[token][c], c = (DK/2)*kb + 16b + r
+    float rz = 1.f, dz = 0.f;
+    if constexpr (NORM) {
+      float P = 0.f, z = 0.f;
+#pragma unroll
+      for (int ch = 0; ch < QCH / 2; ++ch) {
+        const u32x4 qw = *reinterpret_cast<const u32x4*>(qt + swz<QROWB>(ntok, (QCH / 2) * kb + ch));
+        u32x4 qz = qw;
+        if constexpr (DEN) qz = *reinterpret_cast<const u32x4*>(qdt + swz<QROWB>(ntok, (QCH / 2) * kb + ch));
+        const u32x4 kh = *reinterpret_cast<const u32x4*>(&km_pairs[(DK / 4) * kb + 4 * ch]);
+        const u32x4 kl = *reinterpret_cast<const u32x4*>(&km_pairs[DK / 2 + (DK / 4) * kb + 4 * ch]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int c0 = 8 * ch + 2 * i;
+          P = fmaf(Ops<T>::lo(qw[i]), g[c0 >> 4][c0 & 15], P);
+          P = fmaf(Ops<T>::hi(qw[i]), g[c0 >> 4][(c0 & 15) + 1], P);
+          z = Ops<T>::dot2(qz[i], kh[i], z);
+          z = Ops<T>::dot2(qz[i], kl[i], z);
+        }
+      }
+      P += __shfl_xor(P, 32);
+      z += __shfl_xor(z, 32);
+      if (t0 + ntok < t_end) {
+        rz = 1.f / (z + p.eps);
+        dz = -(P * denorm) * rz * rz;
+      } else {
+        rz = 0.f;  // padding rows contribute nothing
+      }
+      if (kb == 0) dzs[ntok] = dz;
+    }
+    // dq~ (and dq when decoupled), packed; staged after the feature view is done with qt
+    uint32_t dqp[DK / 4], dqdp[DEN ? DK / 4 : 1];
+    {
+      const float gs = denorm * rz;
+#pragma unroll
+      for (int c2 = 0; c2 < DK / 4; ++c2) {
+        const int c0 = 2 * c2;
+        float v0 = g[c0 >> 4][c0 & 15] * gs, v1 = g[c0 >> 4][(c0 & 15) + 1] * gs;
+        if constexpr (NORM) {
+          const float d0 = dz * kmf[(DK / 2) * kb + c0], d1 = dz * kmf[(DK / 2) * kb + c0 + 1];
+          if constexpr (DEN) {
+            dqdp[c2] = pack2<T>(d0, d1);
+          } else {
+            v0 += d0;
+            v1 += d1;
+          }
+        }
+        dqp[c2] = pack2<T>(v0, v1);
+      }
+    }
+    // dO / z as hi + lo, in place over this lane's own chunks of the dO tile
+    if constexpr (NORM) {
+#pragma unroll
+      for (int ch = 0; ch < GCH / 2; ++ch) {
+        const int off = swz<GROWB>(ntok, (GCH / 2) * kb + ch);
+        const u32x4 gw = *reinterpret_cast<const u32x4*>(gt + off);
+        u32x4 wh, wl;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float a = Ops<T>::lo(gw[i]) * rz, b = Ops<T>::hi(gw[i]) * rz;
+          const T ah = (T)a, bh = (T)b;
+          wh[i] = pack2<T>((float)ah, (float)bh);
+          wl[i] = pack2<T>(a - (float)ah, b - (float)bh);
+        }
+        *reinterpret_cast<u32x4*>(gt + off) = wh;
+        *reinterpret_cast<u32x4*>(gl + off) = wl;
+      }
+    }
+    wave_sync();
+
+    // ---- feature view: two k-steps of 16 tokens ----
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int tok0 = 16 * ks + 8 * kb;
+      RowWords<CK> qw;
+      RowWords<CV> gh;
+      lds_rows<CK>(qw, qt, tok0, ntok);
+      lds_rows<CV>(gh, gt, tok0, ntok);
+      u32x4 A[CK], Bh[CV];
+      transpose_rows<CK>(qw, A);
+      transpose_rows<CV>(gh, Bh);
+#pragma unroll
+      for (int a = 0; a < CK; ++a)
+#pragma unroll
+        for (int b = 0; b < CV; ++b) acc[a][b] = Ops<T>::mma(A[a], Bh[b], acc[a][b]);
+      if constexpr (NORM) {
+        RowWords<CV> glw;
+        lds_rows<CV>(glw, gl, tok0, ntok);
+        u32x4 Bl[CV];
+        transpose_rows<CV>(glw, Bl);
+#pragma unroll
+        for (int a = 0; a < CK; ++a)
+#pragma unroll
+          for (int b = 0; b < CV; ++b) acc[a][b] = Ops<T>::mma(A[a], Bl[b], acc[a][b]);
+        if constexpr (DEN) lds_rows<CK>(qw, qdt, tok0, ntok);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float dzj = dzs[tok0 + j];
+#pragma unroll
+          for (int c2 = 0; c2 < CK / 2; ++c2) {
+            dkm[2 * c2] = fmaf(dzj, Ops<T>::lo(qw.w[j][c2]), dkm[2 * c2]);
+            dkm[2 * c2 + 1] = fmaf(dzj, Ops<T>::hi(qw.w[j][c2]), dkm[2 * c2 + 1]);
+          }
+        }
+      }
+    }
+    wave_sync();  // qt (and qdt) are free: stage dq through them
+#pragma unroll
+    for (int ch = 0; ch < QCH / 2; ++ch) {
+      const int off = swz<QROWB>(ntok, (QCH / 2) * kb + ch);
+      *reinterpret_cast<u32x4*>(qt + off) = u32x4{dqp[4 * ch], dqp[4 * ch + 1], dqp[4 * ch + 2], dqp[4 * ch + 3]};
+      if constexpr (DEN)
+        *reinterpret_cast<u32x4*>(qdt + off) =
+            u32x4{dqdp[4 * ch], dqdp[4 * ch + 1], dqdp[4 * ch + 2], dqdp[4 * ch + 3]};
+    }
+    wave_sync();
+    store_q(qt, dqn, t0);
+    if constexpr (DEN) store_q(qdt, dqd, t0);
+    t0 = tn;
+  }
+
+  __syncthreads();  // every wave is done with its tiles: reuse them for the reduction
+  float* dst = partial + (int64_t)blockIdx.x * (DK * DV + DK);
+  reduce_store_partial<CK, CV>(acc, dkm, reinterpret_cast<float*>(smem + LY::kOpnd), dst, wave, lane);
+}
+
+// ===========================================================================
 // host side
 // ===========================================================================
 bool supported(const Prob& p, int dtype) {
@@ -533,6 +856,51 @@ void state(const Prob& p, int dtype, const void* kn, const void* v, const void* 
 void rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {
   if (dtype == kF16) run_rows<_Float16>(p, job, DR, DC, st);
   else run_rows<__bf16>(p, job, DR, DC, st);
+}
+
+template <typename T, int DK, int DV, bool NORM, bool DEN>
+static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, const float* S,
+                        const float* km, T* dqn, T* dqd, float* partial, int chunk, int nchunks,
+                        hipStream_t st) {
+  using LY = BwdALayout<DK, DV, NORM, DEN>;
+  static_assert(LY::kTotal - LY::kOpnd >= (int)sizeof(float) * 64 * ((DK / 32) * (DV / 32) * 16 + DK / 32),
+                "reduction buffer must fit in the tile area");
+  auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN>;
+  static thread_local bool configured = false;  // per instantiation
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, LY::kTotal);
+    if (e != hipSuccess) {
+      set_error("bwd_a: cannot reserve %d bytes of LDS: %s", LY::kTotal, hipGetErrorString(e));
+      return kErrLaunch;
+    }
+    configured = true;
+  }
+  const unsigned grid = (unsigned)((int64_t)p.N * p.H * nchunks);
+  kernel<<<dim3(grid), dim3(kThreads), LY::kTotal, st>>>(p, qn, qd, dout, S, km, dqn, dqd, partial,
+                                                         chunk, nchunks);
+  return kOk;
+}
+
+template <typename T>
+static int run_bwd_a(const Prob& p, const void* qn, const void* qd, const void* dout, const float* S,
+                     const float* km, void* dqn, void* dqd, float* partial, int chunk, int nchunks,
+                     hipStream_t st) {
+  const T *a = (const T*)qn, *b = (const T*)qd, *c = (const T*)dout;
+  T *x = (T*)dqn, *y = (T*)dqd;
+  if (!(p.flags & kNormalize))
+    return launch_bwd_a<T, 64, 64, false, false>(p, a, b, c, S, km, x, y, partial, chunk, nchunks, st);
+  if (p.flags & kDecoupled)
+    return launch_bwd_a<T, 64, 64, true, true>(p, a, b, c, S, km, x, y, partial, chunk, nchunks, st);
+  return launch_bwd_a<T, 64, 64, true, false>(p, a, b, c, S, km, x, y, partial, chunk, nchunks, st);
+}
+
+int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout, const float* S,
+          const float* km, void* dqn, void* dqd, float* partial, int chunk, int nchunks,
+          hipStream_t st) {
+  if (dtype == kF16)
+    return run_bwd_a<_Float16>(p, qn, qd, dout, S, km, dqn, dqd, partial, chunk, nchunks, st);
+  return run_bwd_a<__bf16>(p, qn, qd, dout, S, km, dqn, dqd, partial, chunk, nchunks, st);
 }
 
 }  // namespace mfma

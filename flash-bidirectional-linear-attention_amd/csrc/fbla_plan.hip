@@ -24,8 +24,7 @@ static int fwd_chunk(const Prob& p, int dtype) {
   return mfma::supported(p, dtype) ? mfma::state_chunk(p) : generic::state_chunk(p);
 }
 static int bwd_chunk(const Prob& p, int dtype) {
-  (void)dtype;
-  return generic::state_chunk(p);
+  return mfma::supported(p, dtype) ? mfma::state_chunk(p) : generic::state_chunk(p);
 }
 
 size_t fwd_workspace_bytes(const Prob& p, int dtype) { return partial_bytes(p, fwd_chunk(p, dtype)); }
@@ -86,8 +85,13 @@ int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
   float* dkm = (float*)ws;
   const unsigned phases = phase_mask();
   if (phases & kPhaseBwdA) {
-    generic::transpose_state(p, a.s, St, st);
-    generic::bwd_a(p, dtype, qn, a.q, a.dout, a.s, St, a.km, dqn, dqd, partial, chunk, nchunks, st);
+    if (fast) {
+      int rc = mfma::bwd_a(p, dtype, qn, a.q, a.dout, a.s, a.km, dqn, dqd, partial, chunk, nchunks, st);
+      if (rc != kOk) return rc;
+    } else {
+      generic::transpose_state(p, a.s, St, st);
+      generic::bwd_a(p, dtype, qn, a.q, a.dout, a.s, St, a.km, dqn, dqd, partial, chunk, nchunks, st);
+    }
   }
   if (phases & kPhaseBwdReduce)
     generic::state_reduce(p, partial, chunk, nchunks, dS, dSt, dkm, st);
