@@ -141,30 +141,35 @@ __global__ __launch_bounds__(kThreads) void state_partial_kernel(
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(kThreads) void state_reduce_kernel(
     Prob p, const float* __restrict__ partial, int chunk, int nchunks, float* __restrict__ mat,
-    float* __restrict__ mat_t, float* __restrict__ vec) {
-  const int nh = blockIdx.x;
+    float* __restrict__ mat_t, float* __restrict__ vec, int blocks_per_head) {
+  const int nh = blockIdx.x / blocks_per_head, blk = blockIdx.x - nh * blocks_per_head;
   const int n = nh / p.H;
   int64_t bos;
   int len;
   seq_range(p, n, bos, len);
   const int DK = p.DK, DV = p.DV, E = DK * DV, stride = E + DK;
+  const int e = blk * kThreads + threadIdx.x;
+  if (e >= stride) return;
   const int nvalid = len > 0 ? (len + chunk - 1) / chunk : 0;
-  const float s = seq_scale(p, len);
-  const float inv_len = len > 0 ? 1.0f / (float)len : 0.f;
-  const float* src = partial + (int64_t)nh * nchunks * stride;
-  for (int e = threadIdx.x; e < stride; e += kThreads) {
-    float a = 0.f;
-    for (int c = 0; c < nvalid; ++c) a += src[(int64_t)c * stride + e];
-    if (e < E) {
-      a *= s;
-      mat[(int64_t)nh * E + e] = a;
-      if (mat_t) {
-        int dk = e / DV, dv = e - dk * DV;
-        mat_t[(int64_t)nh * E + dv * DK + dk] = a;
-      }
-    } else {
-      if (vec) vec[(int64_t)nh * DK + (e - E)] = a * inv_len;
+  const float* src = partial + (int64_t)nh * nchunks * stride + e;
+  // fixed order: chunk 0, 1, 2, ... (four independent loads in flight at a time)
+  float a = 0.f;
+  int c = 0;
+  for (; c + 4 <= nvalid; c += 4) {
+    const float x0 = src[(int64_t)c * stride], x1 = src[(int64_t)(c + 1) * stride];
+    const float x2 = src[(int64_t)(c + 2) * stride], x3 = src[(int64_t)(c + 3) * stride];
+    a = (((a + x0) + x1) + x2) + x3;
+  }
+  for (; c < nvalid; ++c) a += src[(int64_t)c * stride];
+  if (e < E) {
+    a *= seq_scale(p, len);
+    mat[(int64_t)nh * E + e] = a;
+    if (mat_t) {
+      const int dk = e / DV, dv = e - dk * DV;
+      mat_t[(int64_t)nh * E + dv * DK + dk] = a;
     }
+  } else if (vec) {
+    vec[(int64_t)nh * DK + (e - E)] = len > 0 ? a / (float)len : 0.f;
   }
 }
 
@@ -461,8 +466,9 @@ void state_partial(const Prob& p, int dtype, const void* kn, const void* v, cons
 
 void state_reduce(const Prob& p, const float* partial, int chunk, int nchunks, float* mat,
                   float* mat_t, float* vec, hipStream_t st) {
-  state_reduce_kernel<<<dim3((unsigned)((int64_t)p.N * p.H)), dim3(kThreads), 0, st>>>(
-      p, partial, chunk, nchunks, mat, mat_t, vec);
+  const int blocks_per_head = (p.DK * p.DV + p.DK + kThreads - 1) / kThreads;
+  state_reduce_kernel<<<dim3((unsigned)((int64_t)p.N * p.H * blocks_per_head)), dim3(kThreads), 0, st>>>(
+      p, partial, chunk, nchunks, mat, mat_t, vec, blocks_per_head);
 }
 
 void transpose_state(const Prob& p, const float* mat, float* mat_t, hipStream_t st) {

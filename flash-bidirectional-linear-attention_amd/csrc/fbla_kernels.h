@@ -75,6 +75,7 @@ struct RowsJob {
 };
 bool supported(const Prob& p, int dtype);
 int state_chunk(const Prob& p);
+int bwd_a_chunk(const Prob& p);
 void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
            int chunk, int nchunks, hipStream_t st);
 // out_t = (x_t M) / (xden_t . km + eps) + addvec   with M of shape DR x DC

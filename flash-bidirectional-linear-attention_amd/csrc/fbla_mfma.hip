@@ -20,6 +20,8 @@
 // gfx950): A lane l holds A[m=l%32][k=8*(l/32)+i], B lane l holds
 // B[k=8*(l/32)+i][n=l%32], i=0..7; C register r of lane l is
 // C[8*(r/4)+4*(l/32)+r%4][l%32].
+#include <stdlib.h>
+
 #include "fbla_kernels.h"
 
 namespace fbla {
@@ -791,22 +793,57 @@ bool supported(const Prob& p, int dtype) {
   return p.DK == 64 && p.DV == 64;
 }
 
-// Chunk (tokens per workgroup) of the reduction kernels: ~4 workgroups per CU.
-int state_chunk(const Prob& p) {
+// Number of compute units of the current device (256 on MI355X; also the value
+// assumed when no device is visible, e.g. for a host-only workspace query).
+static int cu_count() {
+  static const int n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+      (void)hipGetLastError();
+      return 256;
+    }
+    return cus;
+  }();
+  return n;
+}
+
+// Integer tuning knob, overridable from the environment (FBLA_<NAME>) for sweeps.
+static int knob(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return v && atoi(v) > 0 ? atoi(v) : dflt;
+}
+
+// Tokens per workgroup for a kernel of which `wgs_per_cu` workgroups fit on a CU:
+// the grid is sized to at most `rounds` full rounds of resident workgroups, with
+// all workgroups doing the same amount of work (no ragged last round).
+static int chunk_for(const Prob& p, int wgs_per_cu, int rounds, int min_chunk, int align) {
   const int64_t nh = (int64_t)p.N * p.H;
-  int64_t chunk = cdiv64((int64_t)p.L * nh, 1024);
-  chunk = cdiv64(chunk, 64) * 64;
-  if (chunk < 256) chunk = 256;
+  const int64_t slots = (int64_t)cu_count() * wgs_per_cu * rounds;
+  int64_t nchunks = slots / (nh > 0 ? nh : 1);
+  if (nchunks < 1) nchunks = 1;
+  int64_t chunk = cdiv64(p.L, nchunks);
+  if (chunk < min_chunk) chunk = min_chunk;
+  chunk = cdiv64(chunk, align) * align;
   return (int)chunk;
 }
 
-// Chunk of the row-parallel kernels: long enough to amortise the operand prologue.
+// Reduction kernels (state, backward pass A): one round of resident workgroups.
+int state_chunk(const Prob& p) {
+  static const int per_cu = knob("FBLA_STATE_WGS_PER_CU", 2);
+  return chunk_for(p, per_cu, 1, 256, 64);
+}
+
+int bwd_a_chunk(const Prob& p) {
+  static const int per_cu = knob("FBLA_BWDA_WGS_PER_CU", 2);
+  return chunk_for(p, per_cu, 1, 256, 128);
+}
+
+// Row-parallel kernels: long enough chunks to amortise the operand prologue.
 int rows_chunk(const Prob& p) {
-  const int64_t nh = (int64_t)p.N * p.H;
-  int64_t chunk = cdiv64((int64_t)p.L * nh, 2048);
-  chunk = cdiv64(chunk, 128) * 128;
-  if (chunk < 512) chunk = 512;
-  return (int)chunk;
+  static const int per_cu = knob("FBLA_ROWS_WGS_PER_CU", 4);
+  static const int rounds = knob("FBLA_ROWS_ROUNDS", 1);
+  return chunk_for(p, per_cu, rounds, 512, 128);
 }
 
 template <typename T, int DK, int DV>

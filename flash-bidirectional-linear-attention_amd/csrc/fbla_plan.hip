@@ -24,7 +24,7 @@ static int fwd_chunk(const Prob& p, int dtype) {
   return mfma::supported(p, dtype) ? mfma::state_chunk(p) : generic::state_chunk(p);
 }
 static int bwd_chunk(const Prob& p, int dtype) {
-  return mfma::supported(p, dtype) ? mfma::state_chunk(p) : generic::state_chunk(p);
+  return mfma::supported(p, dtype) ? mfma::bwd_a_chunk(p) : generic::state_chunk(p);
 }
 
 size_t fwd_workspace_bytes(const Prob& p, int dtype) { return partial_bytes(p, fwd_chunk(p, dtype)); }
@@ -94,7 +94,7 @@ int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
     }
   }
   if (phases & kPhaseBwdReduce)
-    generic::state_reduce(p, partial, chunk, nchunks, dS, dSt, dkm, st);
+    generic::state_reduce(p, partial, chunk, nchunks, dS, fast ? nullptr : dSt, dkm, st);
   if (phases & kPhaseBwdB) {
     if (fast) {
       // dk~_t = v_t (s dS)^T (+ dkm/L): contraction over dv, M(r=dv, c=dk) = dS[c][r]
