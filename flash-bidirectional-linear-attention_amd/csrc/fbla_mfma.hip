@@ -197,7 +197,7 @@ __device__ __forceinline__ void reduce_store_partial(f32x16 (&acc)[CK][CV], floa
   }
 }
 
-template <typename T, int DK, int DV, bool SPLIT_KD>
+template <typename T, int DK, int DV, bool SPLIT_KD, int TILES>
 __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __restrict__ kn,
                                                          const T* __restrict__ v,
                                                          const T* __restrict__ kd,
@@ -231,46 +231,54 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
 #pragma unroll
   for (int a = 0; a < CK; ++a) ks[a] = 0.f;
 
-  // 16-token tiles, interleaved over the 4 waves; next tile is in flight while
-  // the current one is multiplied.
-  int t0 = t_begin + 16 * wave;
-  RowWords<CK> kw, kw_n, kdw, kdw_n;
-  RowWords<CV> vw, vw_n;
-  if (t0 < t_end) {
-    load_rows<T, CK>(kw, kn, row0, rstride, DK, t0 + 8 * kb, t_end, pp);
-    load_rows<T, CV>(vw, v, row0, rstride, DV, t0 + 8 * kb, t_end, pp);
-    if constexpr (SPLIT_KD) load_rows<T, CK>(kdw, kd, row0, rstride, DK, t0 + 8 * kb, t_end, pp);
-  }
+  // Each wave walks TILES consecutive 16-token tiles per step, the steps of the 4
+  // waves interleaved; the next step's rows are in flight while the current ones
+  // are multiplied.
+  constexpr int kStep = 16 * TILES;
+  int t0 = t_begin + kStep * wave;
+  RowWords<CK> kw[TILES], kw_n[TILES], kdw[TILES], kdw_n[TILES];
+  RowWords<CV> vw[TILES], vw_n[TILES];
+  auto fetch = [&](RowWords<CK>(&dk_)[TILES], RowWords<CV>(&dv_)[TILES], RowWords<CK>(&dd_)[TILES], int tok) {
+#pragma unroll
+    for (int u = 0; u < TILES; ++u) {
+      load_rows<T, CK>(dk_[u], kn, row0, rstride, DK, tok + 16 * u + 8 * kb, t_end, pp);
+      load_rows<T, CV>(dv_[u], v, row0, rstride, DV, tok + 16 * u + 8 * kb, t_end, pp);
+      if constexpr (SPLIT_KD) load_rows<T, CK>(dd_[u], kd, row0, rstride, DK, tok + 16 * u + 8 * kb, t_end, pp);
+    }
+  };
+  if (t0 < t_end) fetch(kw, vw, kdw, t0);
   while (t0 < t_end) {
-    const int tn = t0 + 16 * kWaves;
-    if (tn < t_end) {
-      load_rows<T, CK>(kw_n, kn, row0, rstride, DK, tn + 8 * kb, t_end, pp);
-      load_rows<T, CV>(vw_n, v, row0, rstride, DV, tn + 8 * kb, t_end, pp);
-      if constexpr (SPLIT_KD) load_rows<T, CK>(kdw_n, kd, row0, rstride, DK, tn + 8 * kb, t_end, pp);
-    }
-    u32x4 A[CK], B[CV];
-    transpose_rows<CK>(kw, A);
-    transpose_rows<CV>(vw, B);
+    const int tn = t0 + kStep * kWaves;
+    if (tn < t_end) fetch(kw_n, vw_n, kdw_n, tn);
 #pragma unroll
-    for (int a = 0; a < CK; ++a)
-#pragma unroll
-      for (int b = 0; b < CV; ++b) acc[a][b] = Ops<T>::mma(A[a], B[b], acc[a][b]);
-    if constexpr (SPLIT_KD) {
-      u32x4 D[CK];
-      transpose_rows<CK>(kdw, D);
+    for (int u = 0; u < TILES; ++u) {
+      u32x4 A[CK], B[CV];
+      transpose_rows<CK>(kw[u], A);
+      transpose_rows<CV>(vw[u], B);
 #pragma unroll
       for (int a = 0; a < CK; ++a)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ks[a] = Ops<T>::dot2(D[a][i], Ops<T>::kOnes, ks[a]);
-    } else {
+        for (int b = 0; b < CV; ++b) acc[a][b] = Ops<T>::mma(A[a], B[b], acc[a][b]);
+      if constexpr (SPLIT_KD) {
+        u32x4 D[CK];
+        transpose_rows<CK>(kdw[u], D);
 #pragma unroll
-      for (int a = 0; a < CK; ++a)
+        for (int a = 0; a < CK; ++a)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ks[a] = Ops<T>::dot2(A[a][i], Ops<T>::kOnes, ks[a]);
+          for (int i = 0; i < 4; ++i) ks[a] = Ops<T>::dot2(D[a][i], Ops<T>::kOnes, ks[a]);
+      } else {
+#pragma unroll
+        for (int a = 0; a < CK; ++a)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) ks[a] = Ops<T>::dot2(A[a][i], Ops<T>::kOnes, ks[a]);
+      }
     }
-    kw = kw_n;
-    vw = vw_n;
-    if constexpr (SPLIT_KD) kdw = kdw_n;
+#pragma unroll
+    for (int u = 0; u < TILES; ++u) {
+      kw[u] = kw_n[u];
+      vw[u] = vw_n[u];
+      if constexpr (SPLIT_KD) kdw[u] = kdw_n[u];
+    }
     t0 = tn;
   }
 
@@ -297,10 +305,19 @@ template <int ROWB> __device__ __forceinline__ int swz(int row, int chunk) {
 template <typename T, int DR, int DC>
 __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* lds_max,
                                                const float* __restrict__ mat, int ld_r, int ld_c) {
-  constexpr int KS = DR / 16, NB = DC / 32;
+  constexpr int KS = DR / 16;
+  constexpr int kPer = DR * DC / (4 * kThreads);  // float4 loads per thread
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  // one coalesced sweep over the matrix as it lies in memory; values stay in registers
+  f32x4 vals[kPer];
   float mx = 0.f;
-  for (int e = tid; e < DR * DC; e += kThreads) mx = fmaxf(mx, fabsf(mat[e]));
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    vals[i] = *reinterpret_cast<const f32x4*>(mat + 4 * (tid + kThreads * i));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) mx = fmaxf(mx, fabsf(vals[i][j]));
+  }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
   if (lane == 0) lds_max[wave] = mx;
@@ -313,18 +330,24 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
     norm = ldexpf(1.f, 4 - e);
   }
   uint16_t* op16 = reinterpret_cast<uint16_t*>(lds_opnd);
-  for (int e = tid; e < NB * KS * 64 * 8; e += kThreads) {
-    const int i = e & 7, l = (e >> 3) & 63, f = e >> 9;  // f = b*KS + s
-    const int s = f % KS, b = f / KS;
-    const int m = l & 31, kbA = l >> 5;
-    const int r = (DR / 2) * kbA + 8 * s + i;
-    const int cc = (DC / 2) * ((m >> 2) & 1) + 16 * b + 4 * (m >> 3) + (m & 3);
-    const float val = mat[(int64_t)r * ld_r + (int64_t)cc * ld_c] * norm;
-    const T hi = (T)val;
-    const T lo = (T)(val - (float)hi);
-    op16[((2 * f + 0) * 64 + l) * 8 + i] = __builtin_bit_cast(uint16_t, hi);
-    op16[((2 * f + 1) * 64 + l) * 8 + i] = __builtin_bit_cast(uint16_t, lo);
-  }
+  const bool c_fast = ld_c == 1;  // memory index = r*DC + c, else c*DR + r
+#pragma unroll
+  for (int i = 0; i < kPer; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = 4 * (tid + kThreads * i) + j;
+      const int r = c_fast ? e / DC : e % DR;
+      const int cc = c_fast ? e % DC : e / DR;
+      const int kbA = r / (DR / 2), s = (r % (DR / 2)) >> 3, i8 = r & 7;
+      const int kbC = cc / (DC / 2), rem = cc % (DC / 2);
+      const int b = rem >> 4, m = 8 * ((rem & 15) >> 2) + 4 * kbC + (rem & 3);
+      const int f = b * KS + s, l = m + 32 * kbA;
+      const float val = vals[i][j] * norm;
+      const T hi = (T)val;
+      const T lo = (T)(val - (float)hi);
+      op16[((2 * f + 0) * 64 + l) * 8 + i8] = __builtin_bit_cast(uint16_t, hi);
+      op16[((2 * f + 1) * 64 + l) * 8 + i8] = __builtin_bit_cast(uint16_t, lo);
+    }
   return 1.f / norm;
 }
 
@@ -370,16 +393,8 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(Prob p, RowsJob job, int
   T* out = (T*)job.out;
   const float* mat = job.mat + (int64_t)nh * DR * DC;
 
-  // ---- prologue: matrix operand fragments, km pairs, addvec ----
-  const float denorm = build_operand<T, DR, DC>(lds_opnd, lds_max, mat, job.ld_r, job.ld_c);
-  {
-    if constexpr (NORM) build_km_pairs<T>(&lds_km[0][0], job.km + (int64_t)nh * DR, DR);
-    for (int e = tid; e < DC; e += kThreads)
-      lds_add[e] = job.addvec ? job.addvec[(int64_t)nh * DC + e] : 0.f;
-  }
-  __syncthreads();
-
-  // ---- main loop: 32-token sub-tiles, interleaved over the waves ----
+  // 32-token sub-tiles, interleaved over the waves; the first one is requested
+  // before the prologue so that its latency overlaps the operand build.
   const int ntok = lane & 31, kb = lane >> 5;  // MFMA view: token column, k half
   unsigned char* stage = lds_stage[wave];
   unsigned char* stage_den = stage + kStage;
@@ -412,6 +427,17 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(Prob p, RowsJob job, int
     load_tile(xr, x, t0);
     if constexpr (DEN) load_tile(xd, xden, t0);
   }
+
+  // ---- prologue: matrix operand fragments, km pairs, addvec ----
+  const float denorm = build_operand<T, DR, DC>(lds_opnd, lds_max, mat, job.ld_r, job.ld_c);
+  {
+    if constexpr (NORM) build_km_pairs<T>(&lds_km[0][0], job.km + (int64_t)nh * DR, DR);
+    for (int e = tid; e < DC; e += kThreads)
+      lds_add[e] = job.addvec ? job.addvec[(int64_t)nh * DC + e] : 0.f;
+  }
+  __syncthreads();
+
+  // ---- main loop ----
   while (t0 < t_end) {
     wave_sync();  // previous tile's staging reads are done
     stash_tile(xr, stage);
@@ -558,14 +584,6 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
   float* kmf = reinterpret_cast<float*>(smem + LY::kKmF);
   float* lds_max = reinterpret_cast<float*>(smem + LY::kMax);
 
-  // g_t = dO_t S^T: contraction over dv, M(r = dv, c = dk) = S[c][r]
-  const float denorm = build_operand<T, DV, DK>(lds_opnd, lds_max, S + (int64_t)nh * DK * DV, 1, DV);
-  if constexpr (NORM) {
-    build_km_pairs<T>(km_pairs, km + (int64_t)nh * DK, DK);
-    for (int e = tid; e < DK; e += kThreads) kmf[e] = km[(int64_t)nh * DK + e];
-  }
-  __syncthreads();
-
   f32x16 acc[CK][CV];
 #pragma unroll
   for (int a = 0; a < CK; ++a)
@@ -629,6 +647,15 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
     load_g(rg, dout, t0);
     if constexpr (DEN) load_q(rd, qd, t0);
   }
+
+  // g_t = dO_t S^T: contraction over dv, M(r = dv, c = dk) = S[c][r]
+  const float denorm = build_operand<T, DV, DK>(lds_opnd, lds_max, S + (int64_t)nh * DK * DV, 1, DV);
+  if constexpr (NORM) {
+    build_km_pairs<T>(km_pairs, km + (int64_t)nh * DK, DK);
+    for (int e = tid; e < DK; e += kThreads) kmf[e] = km[(int64_t)nh * DK + e];
+  }
+  __syncthreads();
+
   while (t0 < t_end) {
     wave_sync();  // the previous sub-tile's staged dq has been read out
     stash_q(rq, qt);
@@ -850,10 +877,15 @@ template <typename T, int DK, int DV>
 static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, float* partial,
                          int chunk, int nchunks, hipStream_t st) {
   const unsigned grid = (unsigned)((int64_t)p.N * p.H * nchunks);
+  static const int tiles = knob("FBLA_STATE_TILES", 2);
   if (p.flags & kDecoupled)
-    state_kernel<T, DK, DV, true><<<dim3(grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
+    state_kernel<T, DK, DV, true, 1><<<dim3(grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
+  else if (tiles == 1)
+    state_kernel<T, DK, DV, false, 1><<<dim3(grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
+  else if (tiles == 2)
+    state_kernel<T, DK, DV, false, 2><<<dim3(grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
   else
-    state_kernel<T, DK, DV, false><<<dim3(grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
+    state_kernel<T, DK, DV, false, 4><<<dim3(grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
 }
 
 template <typename T>
