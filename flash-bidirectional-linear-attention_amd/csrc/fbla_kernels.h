@@ -74,12 +74,13 @@ struct RowsJob {
   void* out;            // [rows][DC]
 };
 bool supported(const Prob& p, int dtype);
+bool bwd_a_supported(const Prob& p, int dtype);
 int state_chunk(const Prob& p);
 int bwd_a_chunk(const Prob& p);
 void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
            int chunk, int nchunks, hipStream_t st);
 // out_t = (x_t M) / (xden_t . km + eps) + addvec   with M of shape DR x DC
-void rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st);
+int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st);
 // backward pass A: dq~ (and dq when decoupled) + per-chunk partials of dS and dkm
 int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout, const float* S,
           const float* km, void* dqn, void* dqd, float* partial, int chunk, int nchunks,

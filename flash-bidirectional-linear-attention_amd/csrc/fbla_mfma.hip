@@ -139,15 +139,17 @@ __device__ __forceinline__ void transpose_rows(const RowWords<C>& src, u32x4 (&o
     }
 }
 
-// Fixed-order sum of the four waves' accumulators through one LDS buffer
-// (2 -> 0, 3 -> 1, 1 -> 0), then wave 0 writes the canonical [dk][dv] partial
-// followed by the [dk] vector.  Register r of block (a,b) is dk = CK*m + a,
+// Fixed-order sum of the four waves' accumulators through one LDS buffer, then
+// the canonical [dk][dv] partial followed by the [dk] vector is written.
+// NS = 1: every wave holds the full DK x DV block (2 -> 0, 3 -> 1, 1 -> 0; wave 0 writes).
+// NS = 2: wave w holds value columns [(w%2)*32*CV, +32*CV) (2 -> 0, 3 -> 1; waves 0 and 1
+// write their halves, wave 0 the vector).  Register r of block (a,b) is dk = CK*m + a,
 // dv = CV*pp + b with m = 8*(r/4) + 4*kb + r%4.  Must be reached by all waves.
-template <int CK, int CV>
+template <int CK, int CV, int NS>
 __device__ __forceinline__ void reduce_store_partial(f32x16 (&acc)[CK][CV], float (&ks)[CK],
                                                      float* red, float* dst, int wave, int lane) {
   constexpr int kAcc = CK * CV * 16;
-  constexpr int DK = 32 * CK, DV = 32 * CV;
+  constexpr int DK = 32 * CK, DVW = 32 * CV, DV = DVW * NS;
   const int pp = lane & 31, kb = lane >> 5;
   auto spill = [&]() {
 #pragma unroll
@@ -176,11 +178,16 @@ __device__ __forceinline__ void reduce_store_partial(f32x16 (&acc)[CK][CV], floa
   if (wave == 3) spill();
   __syncthreads();
   if (wave == 1) absorb();
-  __syncthreads();
-  if (wave == 1) spill();
-  __syncthreads();
-  if (wave != 0) return;
-  absorb();
+  if constexpr (NS == 1) {
+    __syncthreads();
+    if (wave == 1) spill();
+    __syncthreads();
+    if (wave != 0) return;
+    absorb();
+  } else {
+    if (wave > 1) return;
+  }
+  const int dv_off = NS == 1 ? 0 : wave * DVW;
 #pragma unroll
   for (int a = 0; a < CK; ++a)
 #pragma unroll
@@ -188,12 +195,14 @@ __device__ __forceinline__ void reduce_store_partial(f32x16 (&acc)[CK][CV], floa
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = 8 * (r >> 2) + 4 * kb + (r & 3);
-        dst[(CK * m + a) * DV + CV * pp + b] = acc[a][b][r];
+        dst[(CK * m + a) * DV + dv_off + CV * pp + b] = acc[a][b][r];
       }
+  if (wave == 0) {
 #pragma unroll
-  for (int a = 0; a < CK; ++a) {
-    const float tot = ks[a] + __shfl_xor(ks[a], 32);
-    if (kb == 0) dst[DK * DV + CK * pp + a] = tot;
+    for (int a = 0; a < CK; ++a) {
+      const float tot = ks[a] + __shfl_xor(ks[a], 32);
+      if (kb == 0) dst[DK * DV + CK * pp + a] = tot;
+    }
   }
 }
 
@@ -203,7 +212,11 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
                                                          const T* __restrict__ kd,
                                                          float* __restrict__ partial, int chunk,
                                                          int nchunks) {
-  constexpr int CK = DK / 32, CV = DV / 32;
+  // 128 x 128 states are split by value columns over wave pairs (256 accumulator
+  // registers would not fit one wave): wave w owns columns [(w%NS)*DVW, +DVW).
+  constexpr int NS = (DK == 128 && DV == 128) ? 2 : 1;
+  constexpr int DVW = DV / NS, G = kWaves / NS;
+  constexpr int CK = DK / 32, CV = DVW / 32;
   constexpr int kAcc = CK * CV * 16;          // accumulator floats per lane
   __shared__ float red[64 * (kAcc + CK)];      // cross-wave reduction buffer, [value][lane]
 
@@ -235,20 +248,21 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
   // waves interleaved; the next step's rows are in flight while the current ones
   // are multiplied.
   constexpr int kStep = 16 * TILES;
-  int t0 = t_begin + kStep * wave;
+  const T* vcol = v + (wave % NS) * DVW;
+  int t0 = t_begin + kStep * (wave / NS);
   RowWords<CK> kw[TILES], kw_n[TILES], kdw[TILES], kdw_n[TILES];
   RowWords<CV> vw[TILES], vw_n[TILES];
   auto fetch = [&](RowWords<CK>(&dk_)[TILES], RowWords<CV>(&dv_)[TILES], RowWords<CK>(&dd_)[TILES], int tok) {
 #pragma unroll
     for (int u = 0; u < TILES; ++u) {
       load_rows<T, CK>(dk_[u], kn, row0, rstride, DK, tok + 16 * u + 8 * kb, t_end, pp);
-      load_rows<T, CV>(dv_[u], v, row0, rstride, DV, tok + 16 * u + 8 * kb, t_end, pp);
+      load_rows<T, CV>(dv_[u], vcol, row0, rstride, DV, tok + 16 * u + 8 * kb, t_end, pp);
       if constexpr (SPLIT_KD) load_rows<T, CK>(dd_[u], kd, row0, rstride, DK, tok + 16 * u + 8 * kb, t_end, pp);
     }
   };
   if (t0 < t_end) fetch(kw, vw, kdw, t0);
   while (t0 < t_end) {
-    const int tn = t0 + kStep * kWaves;
+    const int tn = t0 + kStep * G;
     if (tn < t_end) fetch(kw_n, vw_n, kdw_n, tn);
 #pragma unroll
     for (int u = 0; u < TILES; ++u) {
@@ -283,7 +297,7 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
   }
 
   float* dst = partial + (int64_t)blockIdx.x * (DK * DV + DK);
-  reduce_store_partial<CK, CV>(acc, ks, red, dst, wave, lane);
+  reduce_store_partial<CK, CV, NS>(acc, ks, red, dst, wave, lane);
 }
 
 // ===========================================================================
@@ -302,11 +316,11 @@ template <int ROWB> __device__ __forceinline__ int swz(int row, int chunk) {
 // 16-bit hi part and a 16-bit lo remainder (two MFMAs recover ~fp32 accuracy).
 // Returns the factor that undoes the normalisation.  Contains workgroup barriers;
 // the caller must __syncthreads() before reading the fragments.
-template <typename T, int DR, int DC>
+template <typename T, int DR, int DC, int NT = kThreads>
 __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* lds_max,
                                                const float* __restrict__ mat, int ld_r, int ld_c) {
   constexpr int KS = DR / 16;
-  constexpr int kPer = DR * DC / (4 * kThreads);  // float4 loads per thread
+  constexpr int kPer = DR * DC / (4 * NT);  // float4 loads per thread
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   // one coalesced sweep over the matrix as it lies in memory; values stay in registers
@@ -314,7 +328,7 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
   float mx = 0.f;
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
-    vals[i] = *reinterpret_cast<const f32x4*>(mat + 4 * (tid + kThreads * i));
+    vals[i] = *reinterpret_cast<const f32x4*>(mat + 4 * (tid + NT * i));
 #pragma unroll
     for (int j = 0; j < 4; ++j) mx = fmaxf(mx, fabsf(vals[i][j]));
   }
@@ -322,7 +336,9 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
   if (lane == 0) lds_max[wave] = mx;
   __syncthreads();
-  mx = fmaxf(fmaxf(lds_max[0], lds_max[1]), fmaxf(lds_max[2], lds_max[3]));
+  mx = lds_max[0];
+#pragma unroll
+  for (int w = 1; w < NT / 64; ++w) mx = fmaxf(mx, lds_max[w]);
   float norm = 1.f;  // also when M is zero or not finite
   if (mx > 0.f && mx < 3.0e38f) {
     int e;
@@ -335,7 +351,7 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
   for (int i = 0; i < kPer; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int e = 4 * (tid + kThreads * i) + j;
+      const int e = 4 * (tid + NT * i) + j;
       const int r = c_fast ? e / DC : e % DR;
       const int cc = c_fast ? e % DC : e / DR;
       const int kbA = r / (DR / 2), s = (r % (DR / 2)) >> 3, i8 = r & 7;
@@ -352,9 +368,9 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
 }
 
 // km as 16-bit hi/lo pairs (for v_dot2) : pairs[0][e] = hi(km[2e], km[2e+1]), pairs[1][e] = lo
-template <typename T>
+template <typename T, int NT = kThreads>
 __device__ __forceinline__ void build_km_pairs(uint32_t* pairs, const float* __restrict__ kmh, int D) {
-  for (int e = threadIdx.x; e < D / 2; e += kThreads) {
+  for (int e = threadIdx.x; e < D / 2; e += NT) {
     const float a = kmh[2 * e], b = kmh[2 * e + 1];
     const T ah = (T)a, bh = (T)b;
     pairs[e] = pack2<T>((float)ah, (float)bh);
@@ -362,20 +378,32 @@ __device__ __forceinline__ void build_km_pairs(uint32_t* pairs, const float* __r
   }
 }
 
-template <typename T, int DR, int DC, bool NORM, bool DEN>
-__global__ __launch_bounds__(kThreads) void rows_kernel(Prob p, RowsJob job, int chunk,
-                                                        int nchunks) {
+template <int DR, int DC, bool DEN, int WAVES> struct RowsLayout {
+  static constexpr int KS = DR / 16, NB = DC / 32;
+  static constexpr int kStage = 32 * 2 * (DR > DC ? DR : DC);  // one 32-token tile of the wider side
+  static constexpr int kOpnd = NB * KS * 2 * 1024;
+  static constexpr int kStages = kOpnd;
+  static constexpr int kKm = kStages + WAVES * (DEN ? 2 : 1) * kStage;
+  static constexpr int kAdd = kKm + DR * 4;
+  static constexpr int kMax = kAdd + DC * 4;
+  static constexpr int kTotal = kMax + 64;
+};
+
+template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job, int chunk,
+                                                          int nchunks) {
+  using LY = RowsLayout<DR, DC, DEN, WAVES>;
+  constexpr int NT = WAVES * 64;
   constexpr int KS = DR / 16;  // k-steps
   constexpr int NB = DC / 32;  // output blocks
   constexpr int XROWB = DR * 2, OROWB = DC * 2;
   constexpr int XCH = XROWB / 16, OCH = OROWB / 16;  // 16-byte chunks per row
-  constexpr int kStage = 32 * (XROWB > OROWB ? XROWB : OROWB);
-  constexpr int kOpnd = NB * KS * 2 * 1024;
-  __shared__ __attribute__((aligned(16))) unsigned char lds_opnd[kOpnd];
-  __shared__ __attribute__((aligned(16))) unsigned char lds_stage[kWaves][(DEN ? 2 : 1) * kStage];
-  __shared__ __attribute__((aligned(16))) uint32_t lds_km[2][DR / 2];
-  __shared__ __attribute__((aligned(16))) float lds_add[DC];
-  __shared__ float lds_max[kWaves];
+  constexpr int kStage = LY::kStage;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  unsigned char* lds_opnd = smem;
+  uint32_t* lds_km = reinterpret_cast<uint32_t*>(smem + LY::kKm);  // [2][DR/2]
+  float* lds_add = reinterpret_cast<float*>(smem + LY::kAdd);
+  float* lds_max = reinterpret_cast<float*>(smem + LY::kMax);
 
   const int nh = blockIdx.x / nchunks, c = blockIdx.x - nh * nchunks;
   const int n = nh / p.H, h = nh - n * p.H;
@@ -396,7 +424,7 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(Prob p, RowsJob job, int
   // 32-token sub-tiles, interleaved over the waves; the first one is requested
   // before the prologue so that its latency overlaps the operand build.
   const int ntok = lane & 31, kb = lane >> 5;  // MFMA view: token column, k half
-  unsigned char* stage = lds_stage[wave];
+  unsigned char* stage = smem + LY::kStages + wave * (DEN ? 2 : 1) * kStage;
   unsigned char* stage_den = stage + kStage;
   constexpr int XI = 32 * XCH / 64;  // flat 16-byte loads per lane per tile
   constexpr int OI = 32 * OCH / 64;
@@ -429,10 +457,10 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(Prob p, RowsJob job, int
   }
 
   // ---- prologue: matrix operand fragments, km pairs, addvec ----
-  const float denorm = build_operand<T, DR, DC>(lds_opnd, lds_max, mat, job.ld_r, job.ld_c);
+  const float denorm = build_operand<T, DR, DC, NT>(lds_opnd, lds_max, mat, job.ld_r, job.ld_c);
   {
-    if constexpr (NORM) build_km_pairs<T>(&lds_km[0][0], job.km + (int64_t)nh * DR, DR);
-    for (int e = tid; e < DC; e += kThreads)
+    if constexpr (NORM) build_km_pairs<T, NT>(lds_km, job.km + (int64_t)nh * DR, DR);
+    for (int e = tid; e < DC; e += NT)
       lds_add[e] = job.addvec ? job.addvec[(int64_t)nh * DC + e] : 0.f;
   }
   __syncthreads();
@@ -442,7 +470,7 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(Prob p, RowsJob job, int
     wave_sync();  // previous tile's staging reads are done
     stash_tile(xr, stage);
     if constexpr (DEN) stash_tile(xd, stage_den);
-    const int tn = t0 + 32 * kWaves;
+    const int tn = t0 + 32 * WAVES;
     if (tn < t_end) {
       load_tile(xr, x, tn);
       if constexpr (DEN) load_tile(xd, xden, tn);
@@ -468,8 +496,8 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(Prob p, RowsJob job, int
       if constexpr (NORM) {
         u32x4 bd = bq;
         if constexpr (DEN) bd = *reinterpret_cast<const u32x4*>(stage_den + swz<XROWB>(ntok, KS * kb + s));
-        const u32x4 kh = *reinterpret_cast<const u32x4*>(&lds_km[0][(DR / 4) * kb + 4 * s]);
-        const u32x4 kl = *reinterpret_cast<const u32x4*>(&lds_km[1][(DR / 4) * kb + 4 * s]);
+        const u32x4 kh = *reinterpret_cast<const u32x4*>(&lds_km[(DR / 4) * kb + 4 * s]);
+        const u32x4 kl = *reinterpret_cast<const u32x4*>(&lds_km[DR / 2 + (DR / 4) * kb + 4 * s]);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           z = Ops<T>::dot2(bd[i], kh[i], z);
@@ -809,15 +837,23 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
 
   __syncthreads();  // every wave is done with its tiles: reuse them for the reduction
   float* dst = partial + (int64_t)blockIdx.x * (DK * DV + DK);
-  reduce_store_partial<CK, CV>(acc, dkm, reinterpret_cast<float*>(smem + LY::kOpnd), dst, wave, lane);
+  reduce_store_partial<CK, CV, 1>(acc, dkm, reinterpret_cast<float*>(smem + LY::kOpnd), dst, wave, lane);
 }
 
 // ===========================================================================
 // host side
 // ===========================================================================
+// 16-bit inputs with head dims 64 or 128; the decoupled operator only at 64 x 64.
 bool supported(const Prob& p, int dtype) {
   if (dtype != kF16 && dtype != kBF16) return false;
-  return p.DK == 64 && p.DV == 64;
+  if (!((p.DK == 64 || p.DK == 128) && (p.DV == 64 || p.DV == 128))) return false;
+  if ((p.flags & kDecoupled) && !(p.DK == 64 && p.DV == 64)) return false;
+  return true;
+}
+
+// The fused backward pass A exists for 64 x 64 heads.
+bool bwd_a_supported(const Prob& p, int dtype) {
+  return supported(p, dtype) && p.DK == 64 && p.DV == 64;
 }
 
 // Number of compute units of the current device (256 on MI355X; also the value
@@ -867,53 +903,82 @@ int bwd_a_chunk(const Prob& p) {
 }
 
 // Row-parallel kernels: long enough chunks to amortise the operand prologue.
-int rows_chunk(const Prob& p) {
-  static const int per_cu = knob("FBLA_ROWS_WGS_PER_CU", 4);
+static int rows_chunk(const Prob& p, int DR, int DC) {
+  static const int per_cu_knob = knob("FBLA_ROWS_WGS_PER_CU", 4);
   static const int rounds = knob("FBLA_ROWS_ROUNDS", 1);
-  return chunk_for(p, per_cu, rounds, 512, 128);
+  const int big = (DR == 128) + (DC == 128);
+  const int per_cu = big == 0 ? per_cu_knob : (big == 1 ? 2 : 1);
+  return chunk_for(p, per_cu, rounds, 512, big == 2 ? 256 : 128);
 }
 
 template <typename T, int DK, int DV>
 static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, float* partial,
                          int chunk, int nchunks, hipStream_t st) {
-  const unsigned grid = (unsigned)((int64_t)p.N * p.H * nchunks);
-  static const int tiles = knob("FBLA_STATE_TILES", 2);
+  const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(kThreads);
   if (p.flags & kDecoupled)
-    state_kernel<T, DK, DV, true, 1><<<dim3(grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
-  else if (tiles == 1)
-    state_kernel<T, DK, DV, false, 1><<<dim3(grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
-  else if (tiles == 2)
-    state_kernel<T, DK, DV, false, 2><<<dim3(grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
+    state_kernel<T, DK, DV, true, 1><<<grid, block, 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
   else
-    state_kernel<T, DK, DV, false, 4><<<dim3(grid), dim3(kThreads), 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
+    state_kernel<T, DK, DV, false, 1><<<grid, block, 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
 }
 
 template <typename T>
-void run_state(const Prob& p, const void* kn, const void* v, const void* kd, float* partial,
-               int chunk, int nchunks, hipStream_t st) {
-  launch_state<T, 64, 64>(p, (const T*)kn, (const T*)v, (const T*)kd, partial, chunk, nchunks, st);
+static void run_state(const Prob& p, const void* kn, const void* v, const void* kd, float* partial,
+                      int chunk, int nchunks, hipStream_t st) {
+  const T *a = (const T*)kn, *b = (const T*)v, *c = (const T*)kd;
+  if (p.DK == 64 && p.DV == 64) launch_state<T, 64, 64>(p, a, b, c, partial, chunk, nchunks, st);
+  else if (p.DK == 64) launch_state<T, 64, 128>(p, a, b, c, partial, chunk, nchunks, st);
+  else if (p.DV == 64) launch_state<T, 128, 64>(p, a, b, c, partial, chunk, nchunks, st);
+  else launch_state<T, 128, 128>(p, a, b, c, partial, chunk, nchunks, st);
+}
+
+// Reserves the kernel's dynamic LDS once per instantiation and thread.
+template <typename K> static int reserve_lds(K kernel, int bytes, bool& done) {
+  if (done) return kOk;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) {
+    set_error("cannot reserve %d bytes of LDS: %s", bytes, hipGetErrorString(e));
+    return kErrLaunch;
+  }
+  done = true;
+  return kOk;
+}
+
+template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES>
+static int launch_rows_k(const Prob& p, const RowsJob& job, int chunk, int nchunks, hipStream_t st) {
+  using LY = RowsLayout<DR, DC, DEN, WAVES>;
+  auto kernel = rows_kernel<T, DR, DC, NORM, DEN, WAVES>;
+  static thread_local bool configured = false;
+  int rc = reserve_lds(kernel, LY::kTotal, configured);
+  if (rc != kOk) return rc;
+  const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(WAVES * 64);
+  kernel<<<grid, block, LY::kTotal, st>>>(p, job, chunk, nchunks);
+  return kOk;
 }
 
 template <typename T, int DR, int DC>
-static void launch_rows(const Prob& p, const RowsJob& job, hipStream_t st) {
-  const int chunk = rows_chunk(p);
+static int launch_rows(const Prob& p, const RowsJob& job, hipStream_t st) {
+  // 128 x 128 operands fill 64 KiB of LDS: one 8-wave workgroup per CU instead of
+  // several 4-wave ones
+  constexpr int WAVES = (DR == 128 && DC == 128) ? 8 : 4;
+  const int chunk = rows_chunk(p, DR, DC);
   const int nchunks = (int)cdiv64(p.L, chunk);
-  const unsigned grid = (unsigned)((int64_t)p.N * p.H * nchunks);
   const bool norm = job.xden != nullptr;
   const bool den = norm && job.xden != job.x;
-  if (!norm)
-    rows_kernel<T, DR, DC, false, false><<<dim3(grid), dim3(kThreads), 0, st>>>(p, job, chunk, nchunks);
-  else if (!den)
-    rows_kernel<T, DR, DC, true, false><<<dim3(grid), dim3(kThreads), 0, st>>>(p, job, chunk, nchunks);
-  else
-    rows_kernel<T, DR, DC, true, true><<<dim3(grid), dim3(kThreads), 0, st>>>(p, job, chunk, nchunks);
+  if (!norm) return launch_rows_k<T, DR, DC, false, false, WAVES>(p, job, chunk, nchunks, st);
+  if (!den) return launch_rows_k<T, DR, DC, true, false, WAVES>(p, job, chunk, nchunks, st);
+  if constexpr (DR == 64 && DC == 64)
+    return launch_rows_k<T, DR, DC, true, true, WAVES>(p, job, chunk, nchunks, st);
+  set_error("decoupled rows kernel exists only for 64 x 64 heads");
+  return kErrUnsupported;
 }
 
 template <typename T>
-void run_rows(const Prob& p, const RowsJob& job, int DR, int DC, hipStream_t st) {
-  (void)DR;
-  (void)DC;
-  launch_rows<T, 64, 64>(p, job, st);
+static int run_rows(const Prob& p, const RowsJob& job, int DR, int DC, hipStream_t st) {
+  if (DR == 64 && DC == 64) return launch_rows<T, 64, 64>(p, job, st);
+  if (DR == 64) return launch_rows<T, 64, 128>(p, job, st);
+  if (DC == 64) return launch_rows<T, 128, 64>(p, job, st);
+  return launch_rows<T, 128, 128>(p, job, st);
 }
 
 void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
@@ -922,9 +987,9 @@ void state(const Prob& p, int dtype, const void* kn, const void* v, const void* 
   else run_state<__bf16>(p, kn, v, kd, partial, chunk, nchunks, st);
 }
 
-void rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {
-  if (dtype == kF16) run_rows<_Float16>(p, job, DR, DC, st);
-  else run_rows<__bf16>(p, job, DR, DC, st);
+int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {
+  if (dtype == kF16) return run_rows<_Float16>(p, job, DR, DC, st);
+  return run_rows<__bf16>(p, job, DR, DC, st);
 }
 
 template <typename T, int DK, int DV, bool NORM, bool DEN>
@@ -936,15 +1001,8 @@ static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, 
                 "reduction buffer must fit in the tile area");
   auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN>;
   static thread_local bool configured = false;  // per instantiation
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, LY::kTotal);
-    if (e != hipSuccess) {
-      set_error("bwd_a: cannot reserve %d bytes of LDS: %s", LY::kTotal, hipGetErrorString(e));
-      return kErrLaunch;
-    }
-    configured = true;
-  }
+  int rc = reserve_lds(kernel, LY::kTotal, configured);
+  if (rc != kOk) return rc;
   const unsigned grid = (unsigned)((int64_t)p.N * p.H * nchunks);
   kernel<<<dim3(grid), dim3(kThreads), LY::kTotal, st>>>(p, qn, qd, dout, S, km, dqn, dqd, partial,
                                                          chunk, nchunks);

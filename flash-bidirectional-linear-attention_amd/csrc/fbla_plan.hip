@@ -24,7 +24,7 @@ static int fwd_chunk(const Prob& p, int dtype) {
   return mfma::supported(p, dtype) ? mfma::state_chunk(p) : generic::state_chunk(p);
 }
 static int bwd_chunk(const Prob& p, int dtype) {
-  return mfma::supported(p, dtype) ? mfma::bwd_a_chunk(p) : generic::state_chunk(p);
+  return mfma::bwd_a_supported(p, dtype) ? mfma::bwd_a_chunk(p) : generic::state_chunk(p);
 }
 
 size_t fwd_workspace_bytes(const Prob& p, int dtype) { return partial_bytes(p, fwd_chunk(p, dtype)); }
@@ -53,7 +53,8 @@ int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
   if (phases & kPhaseFwdOutput) {
     if (fast) {
       mfma::RowsJob job{qn, normalize ? a.q : nullptr, a.s, p.DV, 1, a.km, nullptr, a.o};
-      mfma::rows(p, dtype, job, p.DK, p.DV, st);
+      int rc = mfma::rows(p, dtype, job, p.DK, p.DV, st);
+      if (rc != kOk) return rc;
     } else {
       generic::output(p, dtype, qn, a.q, a.s, a.km, a.o, st);
     }
@@ -85,7 +86,7 @@ int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
   float* dkm = (float*)ws;
   const unsigned phases = phase_mask();
   if (phases & kPhaseBwdA) {
-    if (fast) {
+    if (mfma::bwd_a_supported(p, dtype)) {
       int rc = mfma::bwd_a(p, dtype, qn, a.q, a.dout, a.s, a.km, dqn, dqd, partial, chunk, nchunks, st);
       if (rc != kOk) return rc;
     } else {
@@ -99,10 +100,12 @@ int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
     if (fast) {
       // dk~_t = v_t (s dS)^T (+ dkm/L): contraction over dv, M(r=dv, c=dk) = dS[c][r]
       mfma::RowsJob jk{a.v, nullptr, dS, 1, p.DV, nullptr, (!dec && normalize) ? dkm : nullptr, dkn};
-      mfma::rows(p, dtype, jk, p.DV, p.DK, st);
+      int rc = mfma::rows(p, dtype, jk, p.DV, p.DK, st);
+      if (rc != kOk) return rc;
       // dv_t = k~_t (s dS): contraction over dk
       mfma::RowsJob jv{kn, nullptr, dS, p.DV, 1, nullptr, nullptr, a.dv};
-      mfma::rows(p, dtype, jv, p.DK, p.DV, st);
+      rc = mfma::rows(p, dtype, jv, p.DK, p.DV, st);
+      if (rc != kOk) return rc;
       if (dec) generic::broadcast_rows(p, dtype, dkm, dkd, st);
     } else {
       generic::bwd_b(p, dtype, kn, a.v, dS, dSt, dkm, dkn, dkd, a.dv, st);

@@ -62,6 +62,9 @@ def _check_dense(variant, B, H, L, DK, DV, dtype, scale=None, eps=1e-6, seed=42)
     (1, 2, 300, 128, 128),    # largest head dims
     (1, 2, 200, 128, 32),     # PolaFormer-like DK = 4 DV
     (1, 2, 200, 32, 64),
+    (2, 3, 333, 64, 128),     # mixed 64 / 128 head dims (MFMA path)
+    (2, 3, 333, 128, 64),
+    (1, 4, 4100, 128, 128),   # several chunks per head at the largest head dims
     (4, 16, 256, 32, 32),     # MLLA / RALA self-test shape (layers/mlla.py:102-127)
 ])
 def test_dense_parity(variant, B, H, L, DK, DV, dtype):
