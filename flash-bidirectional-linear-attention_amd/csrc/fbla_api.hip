@@ -55,13 +55,14 @@ static int check_dims(const char* what, int64_t N, int64_t H, int64_t L, int DK,
   return kOk;
 }
 
-static Prob make_prob(const int32_t* cu, int64_t N, int64_t H, int64_t L, int DK, int DV, int flags,
-                      float scale, float eps) {
+static Prob make_prob(const int32_t* cu, int64_t N, int64_t H, int64_t L, int64_t T, int DK, int DV,
+                      int flags, float scale, float eps) {
   Prob p;
   p.cu = cu;
   p.N = (int)N;
   p.H = (int)H;
   p.L = (int)L;
+  p.T = T;
   p.DK = DK;
   p.DV = DV;
   p.scale = scale;
@@ -113,7 +114,7 @@ const char* fbla_last_error(void) { return g_err; }
 size_t fbla_la_workspace_bytes(int pass, int64_t B, int64_t H, int64_t L, int DK, int DV, int dtype,
                                int flags) {
   if (check_dims("fbla_la_workspace_bytes", B, H, L, DK, DV, dtype, flags) != kOk) return 0;
-  Prob p = make_prob(nullptr, B, H, L, DK, DV, flags, 1.f, 0.f);
+  Prob p = make_prob(nullptr, B, H, L, B * L, DK, DV, flags, 1.f, 0.f);
   return workspace_bytes(p, dtype, pass);
 }
 
@@ -135,7 +136,7 @@ int fbla_la_fwd(const void* q, const void* k, const void* v, const void* q_rope,
       return kErrBadArg;
     }
   }
-  Prob p = make_prob(nullptr, B, H, L, DK, DV, flags, scale, eps);
+  Prob p = make_prob(nullptr, B, H, L, B * L, DK, DV, flags, scale, eps);
   FwdArgs a{q, k, v, q_rope, k_rope, o, s, km, workspace, workspace_bytes_};
   return run_fwd(what, p, dtype, a, (hipStream_t)stream);
 }
@@ -159,7 +160,7 @@ int fbla_la_bwd(const void* q, const void* k, const void* v, const void* q_rope,
     set_error("%s: null tensor pointer", what);
     return kErrBadArg;
   }
-  Prob p = make_prob(nullptr, B, H, L, DK, DV, flags, scale, eps);
+  Prob p = make_prob(nullptr, B, H, L, B * L, DK, DV, flags, scale, eps);
   BwdArgs a{q, k, v, q_rope, k_rope, dout, s, km, dq, dk, dv, dq_rope, dk_rope, workspace,
             workspace_bytes_};
   return run_bwd(what, p, dtype, a, (hipStream_t)stream);
@@ -167,11 +168,10 @@ int fbla_la_bwd(const void* q, const void* k, const void* v, const void* q_rope,
 
 size_t fbla_varlen_workspace_bytes(int pass, int64_t total_tokens, int64_t N, int64_t H,
                                    int64_t max_seqlen, int DK, int DV, int dtype, int flags) {
-  (void)total_tokens;
   if (check_dims("fbla_varlen_workspace_bytes", N, H, max_seqlen, DK, DV, dtype, flags) != kOk)
     return 0;
   static const int32_t dummy = 0;
-  Prob p = make_prob(&dummy, N, H, max_seqlen, DK, DV, flags, 1.f, 0.f);
+  Prob p = make_prob(&dummy, N, H, max_seqlen, total_tokens, DK, DV, flags, 1.f, 0.f);
   return workspace_bytes(p, dtype, pass);
 }
 
@@ -191,7 +191,7 @@ int fbla_varlen_fwd(const void* q, const void* k, const void* v, const int32_t* 
     set_error("%s: null tensor pointer", what);
     return kErrBadArg;
   }
-  Prob p = make_prob(cu_seqlens, N, H, max_seqlen, DK, DV, flags, scale, eps);
+  Prob p = make_prob(cu_seqlens, N, H, max_seqlen, total_tokens, DK, DV, flags, scale, eps);
   FwdArgs a{q, k, v, nullptr, nullptr, o, s, km, workspace, workspace_bytes_};
   return run_fwd(what, p, dtype, a, (hipStream_t)stream);
 }
@@ -213,7 +213,7 @@ int fbla_varlen_bwd(const void* q, const void* k, const void* v, const int32_t* 
     set_error("%s: null tensor pointer", what);
     return kErrBadArg;
   }
-  Prob p = make_prob(cu_seqlens, N, H, max_seqlen, DK, DV, flags, scale, eps);
+  Prob p = make_prob(cu_seqlens, N, H, max_seqlen, total_tokens, DK, DV, flags, scale, eps);
   BwdArgs a{q, k, v, nullptr, nullptr, dout, s, km, dq, dk, dv, nullptr, nullptr, workspace,
             workspace_bytes_};
   return run_bwd(what, p, dtype, a, (hipStream_t)stream);

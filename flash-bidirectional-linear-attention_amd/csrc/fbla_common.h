@@ -24,6 +24,7 @@ enum Flags : int {
 struct Prob {
   const int32_t* cu;
   int N, H, L;  // L: dense length, or max_seqlen upper bound when packed
+  int64_t T;    // total tokens (dense: N*L)
   int DK, DV;
   float scale;
   float eps;

@@ -81,6 +81,13 @@ void state(const Prob& p, int dtype, const void* kn, const void* v, const void* 
            int chunk, int nchunks, hipStream_t st);
 // out_t = (x_t M) / (xden_t . km + eps) + addvec   with M of shape DR x DC
 int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st);
+// two-kernel form of backward pass A for head dims above 64 (not decoupled):
+// bwd_tokens writes dq and tokscal = [1/z_t | dz_t] per (token, head) row, scaled_state
+// accumulates the partials of dS = sum_t q_t^T (dO_t / z_t) and dkm = sum_t dz_t q_t
+int bwd_tokens(const Prob& p, int dtype, const void* q, const void* dout, const float* S,
+               const float* km, void* dq, float* tokscal, int64_t total_rows, hipStream_t st);
+void scaled_state(const Prob& p, int dtype, const void* qn, const void* dout, const float* tokscal,
+                  int64_t total_rows, float* partial, int chunk, int nchunks, hipStream_t st);
 // backward pass A: dq~ (and dq when decoupled) + per-chunk partials of dS and dkm
 int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout, const float* S,
           const float* km, void* dqn, void* dqd, float* partial, int chunk, int nchunks,

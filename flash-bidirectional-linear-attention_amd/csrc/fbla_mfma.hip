@@ -206,11 +206,17 @@ __device__ __forceinline__ void reduce_store_partial(f32x16 (&acc)[CK][CV], floa
   }
 }
 
-template <typename T, int DK, int DV, bool SPLIT_KD, int TILES>
+// SCALED = true is the feature view of the backward for head dims above 64:
+// kn = q~, v = dO, every dO row is multiplied by 1/z_t (tokscal[row]) and split
+// into hi + lo before the MFMA, and the vector part is dkm = sum_t dz_t q_t
+// (dz_t = tokscal[total_rows + row]).
+template <typename T, int DK, int DV, bool SPLIT_KD, int TILES, bool SCALED>
 __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __restrict__ kn,
                                                          const T* __restrict__ v,
                                                          const T* __restrict__ kd,
-                                                         float* __restrict__ partial, int chunk,
+                                                         float* __restrict__ partial,
+                                                         const float* __restrict__ tokscal,
+                                                         int64_t total_rows, int chunk,
                                                          int nchunks) {
   // 128 x 128 states are split by value columns over wave pairs (256 accumulator
   // registers would not fit one wave): wave w owns columns [(w%NS)*DVW, +DVW).
@@ -268,6 +274,44 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
     for (int u = 0; u < TILES; ++u) {
       u32x4 A[CK], B[CV];
       transpose_rows<CK>(kw[u], A);
+      if constexpr (SCALED) {
+        RowWords<CV> vh, vl;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int tok = t0 + 16 * u + 8 * kb + j;
+          float rz = 0.f, dz = 0.f;
+          if (tok < t_end) {
+            const int64_t row = row0 + (int64_t)tok * rstride;
+            rz = tokscal[row];
+            dz = tokscal[total_rows + row];
+          }
+#pragma unroll
+          for (int c2 = 0; c2 < CV / 2; ++c2) {
+            const uint32_t w = vw[u].w[j][c2];
+            const float x0 = Ops<T>::lo(w) * rz, x1 = Ops<T>::hi(w) * rz;
+            const T h0 = (T)x0, h1 = (T)x1;
+            vh.w[j][c2] = pack2<T>((float)h0, (float)h1);
+            vl.w[j][c2] = pack2<T>(x0 - (float)h0, x1 - (float)h1);
+          }
+#pragma unroll
+          for (int c2 = 0; c2 < CK / 2; ++c2) {
+            const uint32_t w = SPLIT_KD ? kdw[u].w[j][c2] : kw[u].w[j][c2];
+            ks[2 * c2] = fmaf(dz, Ops<T>::lo(w), ks[2 * c2]);
+            ks[2 * c2 + 1] = fmaf(dz, Ops<T>::hi(w), ks[2 * c2 + 1]);
+          }
+        }
+        u32x4 Bl[CV];
+        transpose_rows<CV>(vh, B);
+        transpose_rows<CV>(vl, Bl);
+#pragma unroll
+        for (int a = 0; a < CK; ++a)
+#pragma unroll
+          for (int b = 0; b < CV; ++b) {
+            acc[a][b] = Ops<T>::mma(A[a], B[b], acc[a][b]);
+            acc[a][b] = Ops<T>::mma(A[a], Bl[b], acc[a][b]);
+          }
+        continue;
+      }
       transpose_rows<CV>(vw[u], B);
 #pragma unroll
       for (int a = 0; a < CK; ++a)
@@ -565,23 +609,27 @@ __device__ __forceinline__ void lds_rows(RowWords<C>& dst, const unsigned char* 
   }
 }
 
-template <int DK, int DV, bool NORM, bool DEN> struct BwdALayout {
+template <int DK, int DV, bool NORM, bool DEN, bool FUSED> struct BwdALayout {
   static constexpr int KS = DV / 16, NB = DK / 32;
   static constexpr int kOpnd = NB * KS * 2 * 1024;
   static constexpr int kQ = 32 * DK * 2, kG = 32 * DV * 2;
-  static constexpr int kWave = kQ + kG + (NORM ? kG : 0) + (DEN ? kQ : 0) + 128;  // + dz[32]
+  static constexpr int kWave = kQ + kG + (NORM && FUSED ? kG : 0) + (DEN ? kQ : 0) + 128;  // + dz[32]
   static constexpr int kKmPairs = kOpnd + kWaves * kWave;
   static constexpr int kKmF = kKmPairs + DK * 4;
   static constexpr int kMax = kKmF + DK * 4;
   static constexpr int kTotal = kMax + 64;
 };
 
-template <typename T, int DK, int DV, bool NORM, bool DEN>
+// FUSED = false runs the token view only (head dims whose dS accumulators do not
+// fit one wave): it writes 1/z_t and dz_t per (token, head) row to `tokscal`
+// ([2][total rows]) for scaled_state_kernel, and no partials.
+template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED>
 __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
     Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const T* __restrict__ dout,
     const float* __restrict__ S, const float* __restrict__ km, T* __restrict__ dqn,
-    T* __restrict__ dqd, float* __restrict__ partial, int chunk, int nchunks) {
-  using LY = BwdALayout<DK, DV, NORM, DEN>;
+    T* __restrict__ dqd, float* __restrict__ partial, float* __restrict__ tokscal,
+    int64_t total_rows, int chunk, int nchunks) {
+  using LY = BwdALayout<DK, DV, NORM, DEN, FUSED>;
   constexpr int KS = LY::KS, NB = LY::NB;
   constexpr int CK = DK / 32, CV = DV / 32;
   constexpr int QROWB = DK * 2, GROWB = DV * 2;
@@ -605,18 +653,18 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
   unsigned char* lds_opnd = smem;
   unsigned char* qt = smem + LY::kOpnd + wave * LY::kWave;
   unsigned char* gt = qt + LY::kQ;             // dO, later dO/z (hi part)
-  unsigned char* gl = gt + LY::kG;             // dO/z (lo part), NORM only
-  unsigned char* qdt = gl + (NORM ? LY::kG : 0);  // plain q, DEN only
+  unsigned char* gl = gt + LY::kG;             // dO/z (lo part), NORM && FUSED only
+  unsigned char* qdt = gl + (NORM && FUSED ? LY::kG : 0);  // plain q, DEN only
   float* dzs = reinterpret_cast<float*>(qdt + (DEN ? LY::kQ : 0));
   uint32_t* km_pairs = reinterpret_cast<uint32_t*>(smem + LY::kKmPairs);
   float* kmf = reinterpret_cast<float*>(smem + LY::kKmF);
   float* lds_max = reinterpret_cast<float*>(smem + LY::kMax);
 
-  f32x16 acc[CK][CV];
+  f32x16 acc[FUSED ? CK : 1][FUSED ? CV : 1];
 #pragma unroll
-  for (int a = 0; a < CK; ++a)
+  for (int a = 0; a < (FUSED ? CK : 1); ++a)
 #pragma unroll
-    for (int b = 0; b < CV; ++b)
+    for (int b = 0; b < (FUSED ? CV : 1); ++b)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
   float dkm[CK];
@@ -742,7 +790,15 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
       } else {
         rz = 0.f;  // padding rows contribute nothing
       }
-      if (kb == 0) dzs[ntok] = dz;
+      if constexpr (FUSED) {
+        if (kb == 0) dzs[ntok] = dz;
+      } else {
+        if (kb == 0 && t0 + ntok < t_end) {
+          const int64_t row = row0 + (int64_t)(t0 + ntok) * rstride;
+          tokscal[row] = rz;
+          tokscal[total_rows + row] = dz;
+        }
+      }
     }
     // dq~ (and dq when decoupled), packed; staged after the feature view is done with qt
     uint32_t dqp[DK / 4], dqdp[DEN ? DK / 4 : 1];
@@ -765,7 +821,7 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
       }
     }
     // dO / z as hi + lo, in place over this lane's own chunks of the dO tile
-    if constexpr (NORM) {
+    if constexpr (NORM && FUSED) {
 #pragma unroll
       for (int ch = 0; ch < GCH / 2; ++ch) {
         const int off = swz<GROWB>(ntok, (GCH / 2) * kb + ch);
@@ -785,6 +841,7 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
     wave_sync();
 
     // ---- feature view: two k-steps of 16 tokens ----
+    if constexpr (FUSED) {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       const int tok0 = 16 * ks + 8 * kb;
@@ -820,6 +877,7 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
         }
       }
     }
+    }
     wave_sync();  // qt (and qdt) are free: stage dq through them
 #pragma unroll
     for (int ch = 0; ch < QCH / 2; ++ch) {
@@ -835,9 +893,11 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
     t0 = tn;
   }
 
-  __syncthreads();  // every wave is done with its tiles: reuse them for the reduction
-  float* dst = partial + (int64_t)blockIdx.x * (DK * DV + DK);
-  reduce_store_partial<CK, CV, 1>(acc, dkm, reinterpret_cast<float*>(smem + LY::kOpnd), dst, wave, lane);
+  if constexpr (FUSED) {
+    __syncthreads();  // every wave is done with its tiles: reuse them for the reduction
+    float* dst = partial + (int64_t)blockIdx.x * (DK * DV + DK);
+    reduce_store_partial<CK, CV, 1>(acc, dkm, reinterpret_cast<float*>(smem + LY::kOpnd), dst, wave, lane);
+  }
 }
 
 // ===========================================================================
@@ -913,22 +973,25 @@ static int rows_chunk(const Prob& p, int DR, int DC) {
 
 template <typename T, int DK, int DV>
 static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, float* partial,
-                         int chunk, int nchunks, hipStream_t st) {
+                         const float* tokscal, int64_t total_rows, int chunk, int nchunks,
+                         hipStream_t st) {
   const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(kThreads);
-  if (p.flags & kDecoupled)
-    state_kernel<T, DK, DV, true, 1><<<grid, block, 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
+  if (tokscal)
+    state_kernel<T, DK, DV, false, 1, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, chunk, nchunks);
+  else if (p.flags & kDecoupled)
+    state_kernel<T, DK, DV, true, 1, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, chunk, nchunks);
   else
-    state_kernel<T, DK, DV, false, 1><<<grid, block, 0, st>>>(p, kn, v, kd, partial, chunk, nchunks);
+    state_kernel<T, DK, DV, false, 1, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, chunk, nchunks);
 }
 
 template <typename T>
 static void run_state(const Prob& p, const void* kn, const void* v, const void* kd, float* partial,
-                      int chunk, int nchunks, hipStream_t st) {
+                      const float* ts, int64_t rows, int chunk, int nchunks, hipStream_t st) {
   const T *a = (const T*)kn, *b = (const T*)v, *c = (const T*)kd;
-  if (p.DK == 64 && p.DV == 64) launch_state<T, 64, 64>(p, a, b, c, partial, chunk, nchunks, st);
-  else if (p.DK == 64) launch_state<T, 64, 128>(p, a, b, c, partial, chunk, nchunks, st);
-  else if (p.DV == 64) launch_state<T, 128, 64>(p, a, b, c, partial, chunk, nchunks, st);
-  else launch_state<T, 128, 128>(p, a, b, c, partial, chunk, nchunks, st);
+  if (p.DK == 64 && p.DV == 64) launch_state<T, 64, 64>(p, a, b, c, partial, ts, rows, chunk, nchunks, st);
+  else if (p.DK == 64) launch_state<T, 64, 128>(p, a, b, c, partial, ts, rows, chunk, nchunks, st);
+  else if (p.DV == 64) launch_state<T, 128, 64>(p, a, b, c, partial, ts, rows, chunk, nchunks, st);
+  else launch_state<T, 128, 128>(p, a, b, c, partial, ts, rows, chunk, nchunks, st);
 }
 
 // Reserves the kernel's dynamic LDS once per instantiation and thread.
@@ -983,8 +1046,14 @@ static int run_rows(const Prob& p, const RowsJob& job, int DR, int DC, hipStream
 
 void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
            int chunk, int nchunks, hipStream_t st) {
-  if (dtype == kF16) run_state<_Float16>(p, kn, v, kd, partial, chunk, nchunks, st);
-  else run_state<__bf16>(p, kn, v, kd, partial, chunk, nchunks, st);
+  if (dtype == kF16) run_state<_Float16>(p, kn, v, kd, partial, nullptr, 0, chunk, nchunks, st);
+  else run_state<__bf16>(p, kn, v, kd, partial, nullptr, 0, chunk, nchunks, st);
+}
+
+void scaled_state(const Prob& p, int dtype, const void* qn, const void* dout, const float* tokscal,
+                  int64_t total_rows, float* partial, int chunk, int nchunks, hipStream_t st) {
+  if (dtype == kF16) run_state<_Float16>(p, qn, dout, qn, partial, tokscal, total_rows, chunk, nchunks, st);
+  else run_state<__bf16>(p, qn, dout, qn, partial, tokscal, total_rows, chunk, nchunks, st);
 }
 
 int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {
@@ -992,20 +1061,22 @@ int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream
   return run_rows<__bf16>(p, job, DR, DC, st);
 }
 
-template <typename T, int DK, int DV, bool NORM, bool DEN>
+template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED>
 static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, const float* S,
-                        const float* km, T* dqn, T* dqd, float* partial, int chunk, int nchunks,
-                        hipStream_t st) {
-  using LY = BwdALayout<DK, DV, NORM, DEN>;
-  static_assert(LY::kTotal - LY::kOpnd >= (int)sizeof(float) * 64 * ((DK / 32) * (DV / 32) * 16 + DK / 32),
+                        const float* km, T* dqn, T* dqd, float* partial, float* tokscal,
+                        int64_t total_rows, int chunk, int nchunks, hipStream_t st) {
+  using LY = BwdALayout<DK, DV, NORM, DEN, FUSED>;
+  static_assert(!FUSED || LY::kTotal - LY::kOpnd >=
+                              (int)sizeof(float) * 64 * ((DK / 32) * (DV / 32) * 16 + DK / 32),
                 "reduction buffer must fit in the tile area");
-  auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN>;
+  static_assert(LY::kTotal <= 160 * 1024, "LDS budget of one workgroup");
+  auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN, FUSED>;
   static thread_local bool configured = false;  // per instantiation
   int rc = reserve_lds(kernel, LY::kTotal, configured);
   if (rc != kOk) return rc;
   const unsigned grid = (unsigned)((int64_t)p.N * p.H * nchunks);
   kernel<<<dim3(grid), dim3(kThreads), LY::kTotal, st>>>(p, qn, qd, dout, S, km, dqn, dqd, partial,
-                                                         chunk, nchunks);
+                                                         tokscal, total_rows, chunk, nchunks);
   return kOk;
 }
 
@@ -1016,10 +1087,10 @@ static int run_bwd_a(const Prob& p, const void* qn, const void* qd, const void* 
   const T *a = (const T*)qn, *b = (const T*)qd, *c = (const T*)dout;
   T *x = (T*)dqn, *y = (T*)dqd;
   if (!(p.flags & kNormalize))
-    return launch_bwd_a<T, 64, 64, false, false>(p, a, b, c, S, km, x, y, partial, chunk, nchunks, st);
+    return launch_bwd_a<T, 64, 64, false, false, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, chunk, nchunks, st);
   if (p.flags & kDecoupled)
-    return launch_bwd_a<T, 64, 64, true, true>(p, a, b, c, S, km, x, y, partial, chunk, nchunks, st);
-  return launch_bwd_a<T, 64, 64, true, false>(p, a, b, c, S, km, x, y, partial, chunk, nchunks, st);
+    return launch_bwd_a<T, 64, 64, true, true, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, chunk, nchunks, st);
+  return launch_bwd_a<T, 64, 64, true, false, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, chunk, nchunks, st);
 }
 
 int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout, const float* S,
@@ -1028,6 +1099,39 @@ int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* 
   if (dtype == kF16)
     return run_bwd_a<_Float16>(p, qn, qd, dout, S, km, dqn, dqd, partial, chunk, nchunks, st);
   return run_bwd_a<__bf16>(p, qn, qd, dout, S, km, dqn, dqd, partial, chunk, nchunks, st);
+}
+
+template <typename T, int DK, int DV>
+static int launch_bwd_tokens(const Prob& p, const void* q, const void* dout, const float* S,
+                             const float* km, void* dq, float* tokscal, int64_t total_rows,
+                             int chunk, int nchunks, hipStream_t st) {
+  const T *a = (const T*)q, *c = (const T*)dout;
+  if (p.flags & kNormalize)
+    return launch_bwd_a<T, DK, DV, true, false, false>(p, a, a, c, S, km, (T*)dq, nullptr, nullptr,
+                                                       tokscal, total_rows, chunk, nchunks, st);
+  return launch_bwd_a<T, DK, DV, false, false, false>(p, a, a, c, S, km, (T*)dq, nullptr, nullptr,
+                                                      tokscal, total_rows, chunk, nchunks, st);
+}
+
+template <typename T>
+static int run_bwd_tokens(const Prob& p, const void* q, const void* dout, const float* S,
+                          const float* km, void* dq, float* tokscal, int64_t total_rows,
+                          hipStream_t st) {
+  const int big = (p.DK == 128) + (p.DV == 128);
+  const int chunk = chunk_for(p, big == 2 ? 1 : 2, 1, 512, 128);
+  const int nchunks = (int)cdiv64(p.L, chunk);
+  if (p.DK == 64 && p.DV == 128)
+    return launch_bwd_tokens<T, 64, 128>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
+  if (p.DK == 128 && p.DV == 64)
+    return launch_bwd_tokens<T, 128, 64>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
+  return launch_bwd_tokens<T, 128, 128>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
+}
+
+// token view of the backward alone: dq and the per-row scalars 1/z_t, dz_t
+int bwd_tokens(const Prob& p, int dtype, const void* q, const void* dout, const float* S,
+               const float* km, void* dq, float* tokscal, int64_t total_rows, hipStream_t st) {
+  if (dtype == kF16) return run_bwd_tokens<_Float16>(p, q, dout, S, km, dq, tokscal, total_rows, st);
+  return run_bwd_tokens<__bf16>(p, q, dout, S, km, dq, tokscal, total_rows, st);
 }
 
 }  // namespace mfma

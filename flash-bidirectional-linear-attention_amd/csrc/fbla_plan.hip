@@ -24,14 +24,21 @@ static int fwd_chunk(const Prob& p, int dtype) {
   return mfma::supported(p, dtype) ? mfma::state_chunk(p) : generic::state_chunk(p);
 }
 static int bwd_chunk(const Prob& p, int dtype) {
-  return mfma::bwd_a_supported(p, dtype) ? mfma::bwd_a_chunk(p) : generic::state_chunk(p);
+  if (mfma::bwd_a_supported(p, dtype)) return mfma::bwd_a_chunk(p);
+  return mfma::supported(p, dtype) ? mfma::state_chunk(p) : generic::state_chunk(p);
+}
+// per-row scalars 1/z_t and dz_t of the two-kernel backward pass A
+static size_t tokscal_bytes(const Prob& p, int dtype) {
+  if (!mfma::supported(p, dtype) || mfma::bwd_a_supported(p, dtype)) return 0;
+  return align_up((size_t)2 * p.T * p.H * sizeof(float), 256);
 }
 
 size_t fwd_workspace_bytes(const Prob& p, int dtype) { return partial_bytes(p, fwd_chunk(p, dtype)); }
 
-// partials | S^T | s*dS | (s*dS)^T | dkm/L
+// partials | S^T | s*dS | (s*dS)^T | dkm/L | per-row scalars
 size_t bwd_workspace_bytes(const Prob& p, int dtype) {
-  return partial_bytes(p, bwd_chunk(p, dtype)) + 3 * state_bytes(p) + vec_bytes(p);
+  return partial_bytes(p, bwd_chunk(p, dtype)) + 3 * state_bytes(p) + vec_bytes(p) +
+         tokscal_bytes(p, dtype);
 }
 
 int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
@@ -84,11 +91,20 @@ int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
   float* dSt = (float*)ws;
   ws += state_bytes(p);
   float* dkm = (float*)ws;
+  ws += vec_bytes(p);
+  float* tokscal = (float*)ws;
   const unsigned phases = phase_mask();
   if (phases & kPhaseBwdA) {
     if (mfma::bwd_a_supported(p, dtype)) {
       int rc = mfma::bwd_a(p, dtype, qn, a.q, a.dout, a.s, a.km, dqn, dqd, partial, chunk, nchunks, st);
       if (rc != kOk) return rc;
+    } else if (fast) {
+      // head dims above 64: token view and feature view as two kernels
+      const int64_t rows = p.T * p.H;
+      int rc = mfma::bwd_tokens(p, dtype, a.q, a.dout, a.s, a.km, a.dq, tokscal, rows, st);
+      if (rc != kOk) return rc;
+      if (normalize) mfma::scaled_state(p, dtype, a.q, a.dout, tokscal, rows, partial, chunk, nchunks, st);
+      else mfma::state(p, dtype, a.q, a.dout, a.q, partial, chunk, nchunks, st);
     } else {
       generic::transpose_state(p, a.s, St, st);
       generic::bwd_a(p, dtype, qn, a.q, a.dout, a.s, St, a.km, dqn, dqd, partial, chunk, nchunks, st);
