@@ -162,6 +162,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sweep", action="store_true",
                     help="also print a table over T in {1024,4096,16384,32768} to stderr")
+    ap.add_argument("--configs", action="store_true",
+                    help="also time the other operator families / BASELINE configs (table on stderr)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path needs no collective: heads "
@@ -233,6 +235,8 @@ def main():
     }
     if args.sweep:
         sweep(dtype, dev, flush)
+    if args.configs:
+        other_configs(dev, flush)
     print(json.dumps(line), flush=True)
 
 
@@ -257,6 +261,93 @@ def sweep(dtype, dev, flush):
         print(json.dumps({"T": T, "fwd_ms": round(f[0], 5), "fwd_gbps": round(4 * nbytes / f[0] / 1e6, 1),
                           "fwd_bwd_ms": round(s[0], 5), "fwd_bwd_gbps": round(11 * nbytes / s[0] / 1e6, 1)}),
               file=sys.stderr, flush=True)
+
+
+def _report(name, nbytes_fwd, nbytes_step, fwd_fn, step_fn, flush, extra=None):
+    f = do_bench(fwd_fn, flush)
+    s = do_bench(step_fn, flush) if step_fn else None
+    row = {"config": name, "fwd_ms": round(f[0], 5), "fwd_gbps": round(nbytes_fwd / f[0] / 1e6, 1),
+           "fwd_frac": round(nbytes_fwd / f[0] / 1e6 / HBM_PEAK_GBPS, 4)}
+    if s:
+        row.update({"fwd_bwd_ms": round(s[0], 5), "fwd_bwd_gbps": round(nbytes_step / s[0] / 1e6, 1),
+                    "fwd_bwd_frac": round(nbytes_step / s[0] / 1e6 / HBM_PEAK_GBPS, 4)})
+    if extra:
+        row.update(extra)
+    print(json.dumps(row), file=sys.stderr, flush=True)
+
+
+def other_configs(dev, flush):
+    """Flushed-median timings of the remaining BASELINE configs and operator families."""
+    from flash_bla.ops.linear_attn.decoupled import decoupled_la
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    from flash_bla.ops.simple_la.fused import simple_la
+
+    def leaves(*ts):
+        return [t.requires_grad_() for t in ts]
+
+    # config 1 shape on the GPU (the CPU-runnable reference case): fp32, tiny
+    q, k, v, do = make_inputs(2, 4, 1024, 64, torch.float32, dev)
+    leaves(q, k, v)
+    nb = q.numel() * 4
+
+    def run(op, args, do_):
+        def step():
+            for t in args:
+                t.grad = None
+            op(*args).backward(do_)
+
+        def fwd():
+            with torch.no_grad():
+                return op(*args)
+        return fwd, step
+
+    f, s = run(linear_attention, (q, k, v), do)
+    _report("C1 linear_attn B2-H4-T1024-D64 fp32", 4 * nb, 11 * nb, f, s, flush)
+    f, s = run(simple_la, (q, k, v), do)
+    _report("C1 simple_la B2-H4-T1024-D64 fp32", 4 * nb, 11 * nb, f, s, flush)
+
+    # simple_la / decoupled at the headline shape, and bf16 linear_attn
+    for dtype, tag in ((torch.float16, "fp16"), (torch.bfloat16, "bf16")):
+        q, k, v, do = make_inputs(8, 16, 16384, 64, dtype, dev)
+        leaves(q, k, v)
+        nb = q.numel() * 2
+        if dtype == torch.bfloat16:
+            f, s = run(linear_attention, (q, k, v), do)
+            _report(f"linear_attn B8-H16-T16384-D64 {tag}", 4 * nb, 11 * nb, f, s, flush)
+        else:
+            f, s = run(simple_la, (q, k, v), do)
+            _report(f"simple_la B8-H16-T16384-D64 {tag}", 4 * nb, 11 * nb, f, s, flush)
+    q, k, v, do = make_inputs(2, 16, 16384, 64, torch.bfloat16, dev)
+    qr, kr, _, _ = make_inputs(2, 16, 16384, 64, torch.bfloat16, dev, seed=7)
+    leaves(q, k, qr, kr, v)
+    nb = q.numel() * 2
+    f, s = run(decoupled_la, (q, k, qr, kr, v), do)
+    _report("decoupled_la B2-H16-T16384-D64 bf16 (benchmark_decoupled_la.py shape)", 6 * nb, 16 * nb, f, s, flush)
+    del q, k, v, do, qr, kr
+
+    # config 3: packed variable-length, 64 sequences U[256, 2048], H=16, bf16
+    g = torch.Generator().manual_seed(42)
+    lengths = torch.randint(256, 2049, (64,), generator=g)
+    cu = torch.cat([torch.zeros(1, dtype=torch.int32), torch.cumsum(lengths, 0).to(torch.int32)]).to(dev)
+    total, max_len = int(lengths.sum()), int(lengths.max())
+    for D in (64, 128):
+        gg = torch.Generator(device=dev).manual_seed(42)
+        q = (F.elu(torch.randn(total, 16, D, generator=gg, device=dev)) + 1).bfloat16().requires_grad_()
+        k = (F.elu(torch.randn(total, 16, D, generator=gg, device=dev)) + 1).bfloat16().requires_grad_()
+        v = torch.randn(total, 16, D, generator=gg, device=dev).bfloat16().requires_grad_()
+        do = torch.randn(total, 16, D, generator=gg, device=dev).bfloat16()
+        nb = q.numel() * 2
+
+        def step():
+            q.grad = k.grad = v.grad = None
+            varlen_linear_attention(q, k, v, cu, max_len).backward(do)
+
+        def fwd():
+            with torch.no_grad():
+                return varlen_linear_attention(q, k, v, cu, max_len)
+        _report(f"C3 varlen 64 seqs U[256,2048] H16 D{D} bf16", 4 * nb, 11 * nb, fwd, step, flush,
+                {"total_tokens": total, "max_seqlen": max_len})
 
 
 if __name__ == "__main__":

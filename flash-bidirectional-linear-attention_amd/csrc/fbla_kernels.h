@@ -72,15 +72,27 @@ struct RowsJob {
   const float* km;      // per (sequence, head) [DR]; used when xden != null
   const float* addvec;  // per (sequence, head) [DC] added to every row, or null
   void* out;            // [rows][DC]
+  // pnchunks > 0: `mat` is instead the partial buffer written by the state kernel /
+  // backward pass A with chunking (pchunk, pnchunks); the kernel sums the partials
+  // itself (matrix times the state scale, vector times 1/len).  The vector is km
+  // (when xden is set) or the row added to the output (vec_is_add).  mat_out /
+  // vec_out (nullable) receive the reduced matrix [DK*DV] and vector [DK].
+  int pchunk = 0, pnchunks = 0;
+  bool vec_is_add = false;
+  float* mat_out = nullptr;
+  float* vec_out = nullptr;
 };
 bool supported(const Prob& p, int dtype);
 bool bwd_a_supported(const Prob& p, int dtype);
 int state_chunk(const Prob& p);
 int bwd_a_chunk(const Prob& p);
+int rows_chunk(const Prob& p, int DR, int DC);
 void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
            int chunk, int nchunks, hipStream_t st);
 // out_t = (x_t M) / (xden_t . km + eps) + addvec   with M of shape DR x DC
 int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st);
+int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, int DR, int DC,
+          hipStream_t st);
 // two-kernel form of backward pass A for head dims above 64 (not decoupled):
 // bwd_tokens writes dq and tokscal = [1/z_t | dz_t] per (token, head) row, scaled_state
 // accumulates the partials of dS = sum_t q_t^T (dO_t / z_t) and dkm = sum_t dz_t q_t

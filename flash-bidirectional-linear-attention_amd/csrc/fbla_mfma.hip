@@ -360,9 +360,15 @@ template <int ROWB> __device__ __forceinline__ int swz(int row, int chunk) {
 // 16-bit hi part and a 16-bit lo remainder (two MFMAs recover ~fp32 accuracy).
 // Returns the factor that undoes the normalisation.  Contains workgroup barriers;
 // the caller must __syncthreads() before reading the fragments.
+// `mat` may be the first of `nsum` partial matrices lying `sum_stride` floats apart
+// (the per-chunk partials of a reduction): they are added in index order and the
+// sum is multiplied by `mscale`; when `mat_out` is given the reduced matrix is
+// also written there in memory order.
 template <typename T, int DR, int DC, int NT = kThreads>
 __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* lds_max,
-                                               const float* __restrict__ mat, int ld_r, int ld_c) {
+                                               const float* __restrict__ mat, int ld_r, int ld_c,
+                                               int nsum = 1, int64_t sum_stride = 0,
+                                               float mscale = 1.f, float* mat_out = nullptr) {
   constexpr int KS = DR / 16;
   constexpr int kPer = DR * DC / (4 * NT);  // float4 loads per thread
   typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -371,8 +377,16 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
   f32x4 vals[kPer];
   float mx = 0.f;
 #pragma unroll
+  for (int i = 0; i < kPer; ++i) vals[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int c = 0; c < nsum; ++c) {
+#pragma unroll
+    for (int i = 0; i < kPer; ++i)
+      vals[i] += *reinterpret_cast<const f32x4*>(mat + (int64_t)c * sum_stride + 4 * (tid + NT * i));
+  }
+#pragma unroll
   for (int i = 0; i < kPer; ++i) {
-    vals[i] = *reinterpret_cast<const f32x4*>(mat + 4 * (tid + NT * i));
+    vals[i] *= mscale;
+    if (mat_out) *reinterpret_cast<f32x4*>(mat_out + 4 * (tid + NT * i)) = vals[i];
 #pragma unroll
     for (int j = 0; j < 4; ++j) mx = fmaxf(mx, fabsf(vals[i][j]));
   }
@@ -412,13 +426,34 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
 }
 
 // km as 16-bit hi/lo pairs (for v_dot2) : pairs[0][e] = hi(km[2e], km[2e+1]), pairs[1][e] = lo
+// `src` may be the vector part of the first of `nsum` partials (see build_operand);
+// the sum times `vscale` is the vector.  It is stored as pairs (when `pairs`), as
+// fp32 in LDS (when `f32`) and to memory (when `vec_out`).
 template <typename T, int NT = kThreads>
-__device__ __forceinline__ void build_km_pairs(uint32_t* pairs, const float* __restrict__ kmh, int D) {
+__device__ __forceinline__ void build_vec(uint32_t* pairs, float* f32, const float* __restrict__ src,
+                                          int D, int nsum = 1, int64_t sum_stride = 0,
+                                          float vscale = 1.f, float* vec_out = nullptr) {
   for (int e = threadIdx.x; e < D / 2; e += NT) {
-    const float a = kmh[2 * e], b = kmh[2 * e + 1];
-    const T ah = (T)a, bh = (T)b;
-    pairs[e] = pack2<T>((float)ah, (float)bh);
-    pairs[D / 2 + e] = pack2<T>(a - (float)ah, b - (float)bh);
+    float a = 0.f, b = 0.f;
+    for (int c = 0; c < nsum; ++c) {
+      a += src[(int64_t)c * sum_stride + 2 * e];
+      b += src[(int64_t)c * sum_stride + 2 * e + 1];
+    }
+    a *= vscale;
+    b *= vscale;
+    if (pairs) {
+      const T ah = (T)a, bh = (T)b;
+      pairs[e] = pack2<T>((float)ah, (float)bh);
+      pairs[D / 2 + e] = pack2<T>(a - (float)ah, b - (float)bh);
+    }
+    if (f32) {
+      f32[2 * e] = a;
+      f32[2 * e + 1] = b;
+    }
+    if (vec_out) {
+      vec_out[2 * e] = a;
+      vec_out[2 * e + 1] = b;
+    }
   }
 }
 
@@ -433,10 +468,15 @@ template <int DR, int DC, bool DEN, int WAVES> struct RowsLayout {
   static constexpr int kTotal = kMax + 64;
 };
 
+// One launch can carry two independent jobs of the same shape (the dk and dv
+// products of backward pass B): workgroups [0, wgs_per_job) run job0, the rest job1.
 template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job, int chunk,
-                                                          int nchunks) {
+__global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, RowsJob job1,
+                                                          int wgs_per_job, int chunk, int nchunks) {
   using LY = RowsLayout<DR, DC, DEN, WAVES>;
+  const bool second = (int)blockIdx.x >= wgs_per_job;
+  const RowsJob& job = second ? job1 : job0;
+  const int wg = second ? blockIdx.x - wgs_per_job : blockIdx.x;
   constexpr int NT = WAVES * 64;
   constexpr int KS = DR / 16;  // k-steps
   constexpr int NB = DC / 32;  // output blocks
@@ -449,13 +489,21 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job, i
   float* lds_add = reinterpret_cast<float*>(smem + LY::kAdd);
   float* lds_max = reinterpret_cast<float*>(smem + LY::kMax);
 
-  const int nh = blockIdx.x / nchunks, c = blockIdx.x - nh * nchunks;
+  const int nh = wg / nchunks, c = wg - nh * nchunks;
   const int n = nh / p.H, h = nh - n * p.H;
   int64_t bos, row0, rstride;
   int len;
   seq_range(p, n, bos, len);
   const int t_begin = c * chunk;
-  if (t_begin >= len) return;
+  if (t_begin >= len) {
+    if (c == 0 && job.pnchunks > 0) {  // empty sequence: its state is zero
+      if (job.mat_out)
+        for (int e = threadIdx.x; e < DR * DC; e += NT) job.mat_out[(int64_t)nh * DR * DC + e] = 0.f;
+      if (job.vec_out)
+        for (int e = threadIdx.x; e < p.DK; e += NT) job.vec_out[(int64_t)nh * p.DK + e] = 0.f;
+    }
+    return;
+  }
   const int t_end = min(len, t_begin + chunk);
   row_base(p, n, h, bos, row0, rstride);
 
@@ -463,7 +511,6 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job, i
   const T* x = (const T*)job.x;
   const T* xden = (const T*)job.xden;
   T* out = (T*)job.out;
-  const float* mat = job.mat + (int64_t)nh * DR * DC;
 
   // 32-token sub-tiles, interleaved over the waves; the first one is requested
   // before the prologue so that its latency overlaps the operand build.
@@ -501,9 +548,30 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job, i
   }
 
   // ---- prologue: matrix operand fragments, km pairs, addvec ----
-  const float denorm = build_operand<T, DR, DC, NT>(lds_opnd, lds_max, mat, job.ld_r, job.ld_c);
-  {
-    if constexpr (NORM) build_km_pairs<T, NT>(lds_km, job.km + (int64_t)nh * DR, DR);
+  // Either the finished matrix / vectors are given, or the per-chunk partials of
+  // the preceding reduction kernel, which are summed here in chunk order (every
+  // workgroup of a head computes the same sums; chunk 0 also stores them).
+  float denorm;
+  if (job.pnchunks > 0) {
+    constexpr int E = DR * DC;
+    const int64_t pstride = E + p.DK;
+    const int nsum = (len + job.pchunk - 1) / job.pchunk;
+    const float* part = job.mat + (int64_t)nh * job.pnchunks * pstride;
+    const bool writer = c == 0;
+    denorm = build_operand<T, DR, DC, NT>(lds_opnd, lds_max, part, job.ld_r, job.ld_c, nsum, pstride,
+                                          seq_scale(p, len),
+                                          writer && job.mat_out ? job.mat_out + (int64_t)nh * E : nullptr);
+    const float inv_len = 1.0f / (float)len;
+    float* vout = writer && job.vec_out ? job.vec_out + (int64_t)nh * p.DK : nullptr;
+    if (NORM || job.vec_is_add || vout)
+      build_vec<T, NT>(NORM ? lds_km : nullptr, job.vec_is_add ? lds_add : nullptr, part + E, p.DK,
+                       nsum, pstride, inv_len, vout);
+    if (!job.vec_is_add)
+      for (int e = tid; e < DC; e += NT) lds_add[e] = 0.f;
+  } else {
+    denorm = build_operand<T, DR, DC, NT>(lds_opnd, lds_max, job.mat + (int64_t)nh * DR * DC, job.ld_r,
+                                          job.ld_c);
+    if constexpr (NORM) build_vec<T, NT>(lds_km, nullptr, job.km + (int64_t)nh * DR, DR);
     for (int e = tid; e < DC; e += NT)
       lds_add[e] = job.addvec ? job.addvec[(int64_t)nh * DC + e] : 0.f;
   }
@@ -727,8 +795,7 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
   // g_t = dO_t S^T: contraction over dv, M(r = dv, c = dk) = S[c][r]
   const float denorm = build_operand<T, DV, DK>(lds_opnd, lds_max, S + (int64_t)nh * DK * DV, 1, DV);
   if constexpr (NORM) {
-    build_km_pairs<T>(km_pairs, km + (int64_t)nh * DK, DK);
-    for (int e = tid; e < DK; e += kThreads) kmf[e] = km[(int64_t)nh * DK + e];
+    build_vec<T>(km_pairs, kmf, km + (int64_t)nh * DK, DK);
   }
   __syncthreads();
 
@@ -963,7 +1030,7 @@ int bwd_a_chunk(const Prob& p) {
 }
 
 // Row-parallel kernels: long enough chunks to amortise the operand prologue.
-static int rows_chunk(const Prob& p, int DR, int DC) {
+int rows_chunk(const Prob& p, int DR, int DC) {
   static const int per_cu_knob = knob("FBLA_ROWS_WGS_PER_CU", 4);
   static const int rounds = knob("FBLA_ROWS_ROUNDS", 1);
   const int big = (DR == 128) + (DC == 128);
@@ -1008,19 +1075,21 @@ template <typename K> static int reserve_lds(K kernel, int bytes, bool& done) {
 }
 
 template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES>
-static int launch_rows_k(const Prob& p, const RowsJob& job, int chunk, int nchunks, hipStream_t st) {
+static int launch_rows_k(const Prob& p, const RowsJob& job, const RowsJob* job2, int chunk,
+                         int nchunks, hipStream_t st) {
   using LY = RowsLayout<DR, DC, DEN, WAVES>;
   auto kernel = rows_kernel<T, DR, DC, NORM, DEN, WAVES>;
   static thread_local bool configured = false;
   int rc = reserve_lds(kernel, LY::kTotal, configured);
   if (rc != kOk) return rc;
-  const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(WAVES * 64);
-  kernel<<<grid, block, LY::kTotal, st>>>(p, job, chunk, nchunks);
+  const int wgs = (int)((int64_t)p.N * p.H * nchunks);
+  const dim3 grid((unsigned)(job2 ? 2 * wgs : wgs)), block(WAVES * 64);
+  kernel<<<grid, block, LY::kTotal, st>>>(p, job, job2 ? *job2 : job, wgs, chunk, nchunks);
   return kOk;
 }
 
 template <typename T, int DR, int DC>
-static int launch_rows(const Prob& p, const RowsJob& job, hipStream_t st) {
+static int launch_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, hipStream_t st) {
   // 128 x 128 operands fill 64 KiB of LDS: one 8-wave workgroup per CU instead of
   // several 4-wave ones
   constexpr int WAVES = (DR == 128 && DC == 128) ? 8 : 4;
@@ -1028,20 +1097,21 @@ static int launch_rows(const Prob& p, const RowsJob& job, hipStream_t st) {
   const int nchunks = (int)cdiv64(p.L, chunk);
   const bool norm = job.xden != nullptr;
   const bool den = norm && job.xden != job.x;
-  if (!norm) return launch_rows_k<T, DR, DC, false, false, WAVES>(p, job, chunk, nchunks, st);
-  if (!den) return launch_rows_k<T, DR, DC, true, false, WAVES>(p, job, chunk, nchunks, st);
+  if (!norm) return launch_rows_k<T, DR, DC, false, false, WAVES>(p, job, job2, chunk, nchunks, st);
+  if (!den) return launch_rows_k<T, DR, DC, true, false, WAVES>(p, job, job2, chunk, nchunks, st);
   if constexpr (DR == 64 && DC == 64)
-    return launch_rows_k<T, DR, DC, true, true, WAVES>(p, job, chunk, nchunks, st);
+    return launch_rows_k<T, DR, DC, true, true, WAVES>(p, job, job2, chunk, nchunks, st);
   set_error("decoupled rows kernel exists only for 64 x 64 heads");
   return kErrUnsupported;
 }
 
 template <typename T>
-static int run_rows(const Prob& p, const RowsJob& job, int DR, int DC, hipStream_t st) {
-  if (DR == 64 && DC == 64) return launch_rows<T, 64, 64>(p, job, st);
-  if (DR == 64) return launch_rows<T, 64, 128>(p, job, st);
-  if (DC == 64) return launch_rows<T, 128, 64>(p, job, st);
-  return launch_rows<T, 128, 128>(p, job, st);
+static int run_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, int DR, int DC,
+                    hipStream_t st) {
+  if (DR == 64 && DC == 64) return launch_rows<T, 64, 64>(p, job, job2, st);
+  if (DR == 64) return launch_rows<T, 64, 128>(p, job, job2, st);
+  if (DC == 64) return launch_rows<T, 128, 64>(p, job, job2, st);
+  return launch_rows<T, 128, 128>(p, job, job2, st);
 }
 
 void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
@@ -1057,8 +1127,15 @@ void scaled_state(const Prob& p, int dtype, const void* qn, const void* dout, co
 }
 
 int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {
-  if (dtype == kF16) return run_rows<_Float16>(p, job, DR, DC, st);
-  return run_rows<__bf16>(p, job, DR, DC, st);
+  if (dtype == kF16) return run_rows<_Float16>(p, job, nullptr, DR, DC, st);
+  return run_rows<__bf16>(p, job, nullptr, DR, DC, st);
+}
+
+// two jobs of the same shape and normalisation mode in one launch
+int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, int DR, int DC,
+          hipStream_t st) {
+  if (dtype == kF16) return run_rows<_Float16>(p, job0, &job1, DR, DC, st);
+  return run_rows<__bf16>(p, job0, &job1, DR, DC, st);
 }
 
 template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED>

@@ -33,6 +33,17 @@ static size_t tokscal_bytes(const Prob& p, int dtype) {
   return align_up((size_t)2 * p.T * p.H * sizeof(float), 256);
 }
 
+// The rows kernels can sum the reduction partials in their prologue (saving the
+// reduce launch) or read a matrix reduced by a separate kernel.  Every workgroup
+// of a head repeats the sum, so folding pays only while that extra traffic is
+// small next to the cost of one more dependent launch.
+static bool fold_reduce(const Prob& p, int reduce_nchunks, int DR, int DC) {
+  const int64_t rows_nchunks = cdiv64(p.L, mfma::rows_chunk(p, DR, DC));
+  const double extra = (double)p.N * p.H * (double)(rows_nchunks - 1) * reduce_nchunks *
+                       ((double)p.DK * p.DV + p.DK) * sizeof(float);
+  return extra <= 16.0e6;
+}
+
 size_t fwd_workspace_bytes(const Prob& p, int dtype) { return partial_bytes(p, fwd_chunk(p, dtype)); }
 
 // partials | S^T | s*dS | (s*dS)^T | dkm/L | per-row scalars
@@ -55,11 +66,19 @@ int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
     if (fast) mfma::state(p, dtype, kn, a.v, a.k, partial, chunk, nchunks, st);
     else generic::state_partial(p, dtype, kn, a.v, a.k, partial, chunk, nchunks, st);
   }
-  if (phases & kPhaseFwdReduce)
+  const bool fold = fast && fold_reduce(p, nchunks, p.DK, p.DV);
+  if (!fold && (phases & kPhaseFwdReduce))
     generic::state_reduce(p, partial, chunk, nchunks, a.s, nullptr, a.km, st);
   if (phases & kPhaseFwdOutput) {
     if (fast) {
       mfma::RowsJob job{qn, normalize ? a.q : nullptr, a.s, p.DV, 1, a.km, nullptr, a.o};
+      if (fold) {  // the output kernel sums the partials itself and stores S and km on the way
+        job.mat = partial;
+        job.pchunk = chunk;
+        job.pnchunks = nchunks;
+        job.mat_out = a.s;
+        job.vec_out = a.km;
+      }
       int rc = mfma::rows(p, dtype, job, p.DK, p.DV, st);
       if (rc != kOk) return rc;
     } else {
@@ -110,17 +129,30 @@ int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
       generic::bwd_a(p, dtype, qn, a.q, a.dout, a.s, St, a.km, dqn, dqd, partial, chunk, nchunks, st);
     }
   }
-  if (phases & kPhaseBwdReduce)
+  const bool fold = fast && fold_reduce(p, nchunks, p.DV, p.DK);
+  if (!fold && (phases & kPhaseBwdReduce))
     generic::state_reduce(p, partial, chunk, nchunks, dS, fast ? nullptr : dSt, dkm, st);
   if (phases & kPhaseBwdB) {
     if (fast) {
       // dk~_t = v_t (s dS)^T (+ dkm/L): contraction over dv, M(r=dv, c=dk) = dS[c][r]
       mfma::RowsJob jk{a.v, nullptr, dS, 1, p.DV, nullptr, (!dec && normalize) ? dkm : nullptr, dkn};
-      int rc = mfma::rows(p, dtype, jk, p.DV, p.DK, st);
-      if (rc != kOk) return rc;
       // dv_t = k~_t (s dS): contraction over dk
       mfma::RowsJob jv{kn, nullptr, dS, p.DV, 1, nullptr, nullptr, a.dv};
-      rc = mfma::rows(p, dtype, jv, p.DK, p.DV, st);
+      if (fold) {  // both kernels sum the pass-A partials themselves (s dS, dkm/L)
+        jk.mat = jv.mat = partial;
+        jk.pchunk = jv.pchunk = chunk;
+        jk.pnchunks = jv.pnchunks = nchunks;
+        jk.addvec = nullptr;
+        jk.vec_is_add = !dec && normalize;
+        jk.vec_out = dec ? dkm : nullptr;
+      }
+      int rc;
+      if (p.DK == p.DV) {  // same shape: one launch
+        rc = mfma::rows2(p, dtype, jk, jv, p.DV, p.DK, st);
+      } else {
+        rc = mfma::rows(p, dtype, jk, p.DV, p.DK, st);
+        if (rc == kOk) rc = mfma::rows(p, dtype, jv, p.DK, p.DV, st);
+      }
       if (rc != kOk) return rc;
       if (dec) generic::broadcast_rows(p, dtype, dkm, dkd, st);
     } else {
