@@ -29,6 +29,18 @@ import torch.nn.functional as F  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
+# HBM bytes per launch of each large kernel at the default workload (B8-H16-D64,
+# T=16384, fp16), from two `rocprofv3 --pmc` runs of `bench.py --probe 3`
+# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch).  FETCH_SIZE is scaled by 2.0:
+# the 256 MiB device copy of the same run reads 256 MiB and the counter shows
+# 128.0 MiB; WRITE_SIZE shows 256.0 MiB for it (factor 1.0).
+MEASURED_TRAFFIC = {
+    "fwd_state": int((2 * 256.1 + 8.1) * 2 ** 20),
+    "fwd_output": int((2 * 136.2 + 256.0) * 2 ** 20),
+    "bwd_pass_a": int((2 * 260.2 + 264.1) * 2 ** 20),
+    "bwd_pass_b": int((2 * 272.2 + 512.0) * 2 ** 20),
+}
+
 PHASES = {  # name -> (phase bit, tensors read+written once, entry point)
     "fwd_state": (1, 2, "fwd"),     # reads k, v
     "fwd_output": (4, 2, "fwd"),    # reads q, writes o
@@ -162,6 +174,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sweep", action="store_true",
                     help="also print a table over T in {1024,4096,16384,32768} to stderr")
+    ap.add_argument("--probe", type=int, default=0, metavar="N",
+                    help="counter-collection mode for rocprofv3 --pmc: run N steps of the workload, each "
+                         "followed by a 256 MiB device copy of known traffic, then exit")
     ap.add_argument("--configs", action="store_true",
                     help="also time the other operator families / BASELINE configs (table on stderr)")
     args = ap.parse_args()
@@ -190,6 +205,16 @@ def main():
         with torch.no_grad():
             return linear_attention(q, k, v)
 
+    if args.probe:
+        a = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        b = torch.empty_like(a)
+        for _ in range(args.probe):
+            step()
+            b.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"probe_steps": args.probe, "copy_bytes_each_way": a.numel()}))
+        return
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -209,10 +234,18 @@ def main():
     dom = max(kern, key=lambda n: kern[n]["ms"])
     roofline = {
         "bound": "hbm", "kernel": dom, "achieved": kern[dom]["gbps"], "peak": HBM_PEAK_GBPS,
-        "unit": "GB/s", "frac": kern[dom]["frac"], "traffic": None,
+        "unit": "GB/s", "frac": kern[dom]["frac"],
+        "traffic": MEASURED_TRAFFIC.get(dom) if (T == 16384 and args.dtype == "fp16") else None,
         "alg_bytes_per_launch": kern[dom]["alg_bytes"], "avg_launch_ms": kern[dom]["ms"],
     }
     cpu = None if args.no_cpu else cpu_baseline(T, D, H, sample_batches=2)
+    # context: what a plain device-to-device copy reaches on this box (read + write bytes)
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    copy_ms = timed_loop(lambda: dst.copy_(src), 10)
+    copy_gbps = round(2 * src.numel() / copy_ms / 1e6, 1)
+    del src, dst
 
     line = {
         "metric": "linear_attn fwd+bwd ms and achieved HBM GB/s, B8-H16-D64 T=16384 fp16",
@@ -231,6 +264,7 @@ def main():
                 "gbps_p50": round(fwd_bytes / fwd_q[0] / 1e6, 1),
                 "frac_of_peak": round(fwd_bytes / fwd_q[0] / 1e6 / HBM_PEAK_GBPS, 4)},
         "kernels": kern,
+        "device_copy_gbps": copy_gbps,
         "parity": parity,
     }
     if args.sweep:
