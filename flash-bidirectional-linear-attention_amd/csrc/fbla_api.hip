@@ -219,4 +219,76 @@ int fbla_varlen_bwd(const void* q, const void* k, const void* v, const int32_t* 
   return run_bwd(what, p, dtype, a, (hipStream_t)stream);
 }
 
+size_t fbla_chunk_reduce_workspace_bytes(int64_t BH, int64_t T, int K, int V, int chunk, int dtype,
+                                         int with_norm) {
+  if (check_dims("fbla_chunk_reduce_workspace_bytes", BH, 1, T, K, V, dtype, 0) != kOk || chunk < 1)
+    return 0;
+  return piecewise::chunk_reduce_workspace_bytes(BH, T, K, V, chunk, dtype, with_norm != 0);
+}
+
+int fbla_chunk_reduce(const void* q, const void* k, const void* v, float* qc, float* kc, float* vc,
+                      float* h, float* h_norm, void* workspace, size_t workspace_bytes_, int64_t BH,
+                      int64_t T, int K, int V, int chunk, float p_norm, int dtype, void* stream) {
+  const char* what = "fbla_chunk_reduce";
+  int rc = check_dims(what, BH, 1, T, K, V, dtype, 0);
+  if (rc != kOk) return rc;
+  if (chunk < 1 || (h_norm && !(p_norm > 0.f))) {
+    set_error("%s: chunk must be positive and the norm order > 0", what);
+    return kErrBadArg;
+  }
+  if (BH == 0 || T == 0) return kOk;
+  if (!q || !k || !v || !qc || !kc || !vc || !h) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  const size_t need = piecewise::chunk_reduce_workspace_bytes(BH, T, K, V, chunk, dtype, h_norm != nullptr);
+  if (workspace_bytes_ < need || !workspace) {
+    set_error("%s: workspace too small (%zu < %zu bytes)", what, workspace_bytes_, need);
+    return kErrWorkspace;
+  }
+  rc = piecewise::chunk_reduce(q, k, v, qc, kc, vc, h, h_norm, workspace, BH, T, K, V, chunk, p_norm,
+                               dtype, (hipStream_t)stream);
+  if (rc != kOk) return rc;
+  return check_launch(what);
+}
+
+size_t fbla_piecewise_workspace_bytes(int64_t BH, int64_t T, int K, int V, int block, int dtype) {
+  if (check_dims("fbla_piecewise_workspace_bytes", BH, 1, T, K, V, dtype, 0) != kOk) return 0;
+  if (!piecewise::attention_supported(K, V, block, dtype)) return 0;
+  return piecewise::attention_workspace_bytes(BH, T, K, V);
+}
+
+int fbla_piecewise_fwd(const void* q, const void* k, const void* v, const float* kc, const float* vc,
+                       const float* h, const int32_t* indices, void* o, void* workspace,
+                       size_t workspace_bytes_, int64_t BH, int64_t T, int K, int V, int block, int NS,
+                       float scale, int dtype, void* stream) {
+  const char* what = "fbla_piecewise_fwd";
+  int rc = check_dims(what, BH, 1, T, K, V, dtype, 0);
+  if (rc != kOk) return rc;
+  if (!piecewise::attention_supported(K, V, block, dtype)) {
+    set_error("%s: needs fp16/bf16, head dims in {64,128} and 64-token blocks (got K=%d V=%d block=%d dtype=%d)",
+              what, K, V, block, dtype);
+    return kErrUnsupported;
+  }
+  const int64_t NT = (T + 63) / 64;
+  if (NS < 1 || NS > NT) {
+    set_error("%s: the number of selected blocks must be in [1, %lld], got %d", what, (long long)NT, NS);
+    return kErrBadArg;
+  }
+  if (BH == 0 || T == 0) return kOk;
+  if (!q || !k || !v || !kc || !vc || !h || !indices || !o) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  const size_t need = piecewise::attention_workspace_bytes(BH, T, K, V);
+  if (workspace_bytes_ < need || !workspace) {
+    set_error("%s: workspace too small (%zu < %zu bytes)", what, workspace_bytes_, need);
+    return kErrWorkspace;
+  }
+  rc = piecewise::attention(q, k, v, kc, vc, h, indices, o, workspace, BH, T, K, V, NS, scale, dtype,
+                            (hipStream_t)stream);
+  if (rc != kOk) return rc;
+  return check_launch(what);
+}
+
 }  // extern "C"

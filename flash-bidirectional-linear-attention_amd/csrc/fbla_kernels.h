@@ -106,4 +106,18 @@ int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* 
           hipStream_t st);
 }  // namespace mfma
 
+// Piecewise (PISA) attention, forward only (fbla_piecewise.hip).
+namespace piecewise {
+size_t chunk_reduce_workspace_bytes(int64_t BH, int64_t T, int K, int V, int chunk, int dtype,
+                                    bool per_chunk);
+int chunk_reduce(const void* q, const void* k, const void* v, float* qc, float* kc, float* vc,
+                 float* h, float* h_norm, void* workspace, int64_t BH, int64_t T, int K, int V,
+                 int chunk, float pnorm, int dtype, hipStream_t st);
+bool attention_supported(int K, int V, int block, int dtype);
+size_t attention_workspace_bytes(int64_t BH, int64_t T, int K, int V);
+int attention(const void* q, const void* k, const void* v, const float* kc, const float* vc,
+              const float* h, const int32_t* indices, void* o, void* workspace, int64_t BH, int64_t T,
+              int K, int V, int NS, float scale, int dtype, hipStream_t st);
+}  // namespace piecewise
+
 }  // namespace fbla

@@ -30,6 +30,10 @@ _SIGNATURES = {
     "fbla_varlen_workspace_bytes": (_sz, [_i32, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32]),
     "fbla_varlen_fwd": (_i32, [_vp] * 8 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_varlen_bwd": (_i32, [_vp] * 11 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
+    "fbla_chunk_reduce_workspace_bytes": (_sz, [_i64, _i64, _i32, _i32, _i32, _i32, _i32]),
+    "fbla_chunk_reduce": (_i32, [_vp] * 9 + [_sz, _i64, _i64, _i32, _i32, _i32, _f32, _i32, _vp]),
+    "fbla_piecewise_workspace_bytes": (_sz, [_i64, _i64, _i32, _i32, _i32, _i32]),
+    "fbla_piecewise_fwd": (_i32, [_vp] * 9 + [_sz, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
 }
 
 
@@ -175,3 +179,51 @@ def varlen_bwd(q, k, v, cu_seqlens, max_seqlen, do, s, km, scale, eps):
                                0.0 if scale is None else float(scale), float(eps), _stream(dev))
     _check(rc, "fbla_varlen_bwd")
     return dq, dk, dv
+
+
+def chunk_reduce(q, k, v, chunk, with_norm=False, p_norm=2.0):
+    """Block statistics of piecewise attention.  q,k:[B,H,T,K] v:[B,H,T,V] contiguous.
+    Returns fp32 (qc, kc, vc, h, h_norm or None)."""
+    _require_gpu(q, k, v)
+    L = lib()
+    B, H, T, K = k.shape
+    V = v.shape[-1]
+    NT = -(-T // chunk)
+    code = dtype_code(q)
+    dev = q.device
+    f32 = dict(dtype=torch.float32, device=dev)
+    qc, kc = torch.empty(B, H, NT, K, **f32), torch.empty(B, H, NT, K, **f32)
+    vc, h = torch.empty(B, H, NT, V, **f32), torch.empty(B, H, K, V, **f32)
+    h_norm = torch.empty(B, H, NT, **f32) if with_norm else None
+    with torch.cuda.device(dev):
+        ws = _workspace(L.fbla_chunk_reduce_workspace_bytes(B * H, T, K, V, chunk, code, int(with_norm)), dev)
+        rc = L.fbla_chunk_reduce(_ptr(q), _ptr(k), _ptr(v), _ptr(qc), _ptr(kc), _ptr(vc), _ptr(h),
+                                 _ptr(h_norm), _ptr(ws), ws.numel(), B * H, T, K, V, chunk,
+                                 float(p_norm), code, _stream(dev))
+    _check(rc, "fbla_chunk_reduce")
+    return qc, kc, vc, h, h_norm
+
+
+def piecewise_supported(q, v, block):
+    B, H, T, K = q.shape
+    return bool(q.dtype in (torch.float16, torch.bfloat16) and
+                lib().fbla_piecewise_workspace_bytes(B * H, T, K, v.shape[-1], block, dtype_code(q)))
+
+
+def piecewise_fwd(q, k, v, kc, vc, h, indices, block, scale):
+    """Piecewise attention forward; indices int32 [B,H,NT,NS]; kc, vc, h fp32 from chunk_reduce."""
+    _require_gpu(q, k, v, kc, vc, h, indices)
+    L = lib()
+    B, H, T, K = q.shape
+    V = v.shape[-1]
+    NS = indices.shape[-1]
+    code = dtype_code(q)
+    dev = q.device
+    o = torch.empty_like(v)
+    with torch.cuda.device(dev):
+        ws = _workspace(L.fbla_piecewise_workspace_bytes(B * H, T, K, V, block, code), dev)
+        rc = L.fbla_piecewise_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(kc), _ptr(vc), _ptr(h), _ptr(indices),
+                                  _ptr(o), _ptr(ws), ws.numel(), B * H, T, K, V, block, NS,
+                                  float(scale), code, _stream(dev))
+    _check(rc, "fbla_piecewise_fwd")
+    return o

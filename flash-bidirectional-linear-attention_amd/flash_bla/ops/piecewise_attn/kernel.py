@@ -1,0 +1,79 @@
+"""Piecewise (PISA) sparse attention, forward only (drop-in for
+flash_bla/ops/piecewise_attn/kernel.py:152-176,295-333).
+
+Key blocks of 64 tokens are ranked per query block by the product of block-mean
+queries and keys; the top `density` fraction is attended exactly (softmax), every
+other block contributes through its mean key and value sum (zeroth order) plus a
+first-order correction with H = sum_c (K_c - kc_c)^T V_c.  All block statistics
+are kept in fp32 (the reference stores them in the input dtype) and the running
+linear-branch normaliser is rescaled consistently with the running maximum.
+"""
+import torch
+
+from flash_bla import _hip
+
+
+def _check(q, k, v):
+    for t in (q, k, v):
+        if not isinstance(t, torch.Tensor) or t.ndim != 4:
+            raise ValueError("q, k, and v must have shape (B, H, T, D)")
+    if q.shape != k.shape or q.shape[:3] != v.shape[:3]:
+        raise ValueError(f"mismatching shapes: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
+    if not (q.dtype == k.dtype == v.dtype) or not (q.device == k.device == v.device):
+        raise ValueError("q, k, and v must have the same dtype and device")
+    if not q.is_cuda:
+        raise ValueError("piecewise attention needs GPU tensors")
+
+
+def fused_chunk_reduce(q, k, v, chunk_size, use_bias=False, p=2):
+    """Block statistics (kernel.py:152-176): qc, kc = chunk means `(B,H,N,K)`, vc = chunk
+    sums `(B,H,N,V)`, h = sum over chunks of `(K_c - kc_c)^T V_c` `(B,H,K,V)` and, with
+    `use_bias`, the p-norm of every chunk's matrix as `(B,H,1,N)` (else None).
+    Returned in the input dtype like the reference; `chunk_reduce_fp32` keeps fp32."""
+    qc, kc, vc, h, bias = chunk_reduce_fp32(q, k, v, chunk_size, use_bias, p)
+    return qc.to(k.dtype), kc.to(k.dtype), vc.to(v.dtype), h.to(v.dtype), bias
+
+
+def chunk_reduce_fp32(q, k, v, chunk_size, use_bias=False, p=2):
+    _check(q, k, v)
+    qc, kc, vc, h, h_norm = _hip.chunk_reduce(q.contiguous(), k.contiguous(), v.contiguous(),
+                                              int(chunk_size), use_bias, p)
+    return qc, kc, vc, h, (h_norm[..., None, :] if use_bias else None)
+
+
+def select_blocks(qc, kc, scale, density, bias=None):
+    """Top-k key blocks per query block (kernel.py:313-318): int64 indices `(B,H,N,top_k)`."""
+    NT = qc.shape[-2]
+    score = torch.einsum('bhid,bhjd->bhij', qc, kc * scale)
+    if bias is not None:
+        score = torch.softmax(score + torch.log(bias + 1e-5), dim=-1)
+    top_k = max(1, int(density * NT))
+    return torch.topk(score, k=top_k, dim=-1).indices
+
+
+def piecewise_sparse_attention(q, k, v, density=0.1, block_size=64, scale=None, use_bias=False,
+                               indices=None):
+    """
+    Args:
+        q, k: `(B, H, T, K)`; v: `(B, H, T, V)`; fp16 or bf16, K and V in {64, 128}.
+        density: fraction of key blocks attended exactly per query block (at least one).
+        block_size: tokens per block; the HIP kernel is built for 64.
+        scale: score scale, default `K ** -0.5`.
+        use_bias: rank blocks by softmax(score + log(norm of the block's first-order matrix)).
+        indices: optional precomputed selection `(B, H, N, top_k)` (not in the reference;
+            used to share a selection between implementations).
+    Returns `(B, H, T, V)` in the input dtype.  Forward only, as in the reference.
+    """
+    _check(q, k, v)
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    K = k.shape[-1]
+    scale = K ** -0.5 if scale is None else scale
+    if not _hip.piecewise_supported(q, v, block_size):
+        raise NotImplementedError(
+            "piecewise_sparse_attention on gfx950 needs fp16/bf16 inputs, head dims in {64, 128} and "
+            f"block_size 64 (got dtype {q.dtype}, K={K}, V={v.shape[-1]}, block_size={block_size})")
+    qc, kc, vc, h, bias = chunk_reduce_fp32(q, k, v, block_size, use_bias)
+    if indices is None:
+        indices = select_blocks(qc, kc, scale, density, bias)
+    indices = indices.to(torch.int32).contiguous()
+    return _hip.piecewise_fwd(q, k, v, kc, vc, h, indices, block_size, scale)

@@ -116,6 +116,37 @@ int fbla_varlen_bwd(const void* q, const void* k, const void* v, const int32_t* 
                     int64_t H, int64_t max_seqlen, int DK, int DV, int dtype, int flags,
                     float scale, float eps, void* stream);
 
+/* ---- piecewise (PISA) attention, forward only --------------------------------
+ * Tensors are contiguous [BH, T, K] / [BH, T, V] (batch and heads flattened). */
+
+/* Workspace of fbla_chunk_reduce (with_norm != 0 when h_norm is requested). */
+size_t fbla_chunk_reduce_workspace_bytes(int64_t BH, int64_t T, int K, int V, int chunk, int dtype,
+                                         int with_norm);
+
+/* Block statistics of the linear branch.  Replaces fused_chunk_reduce /
+ * fused_chunk_reduce_kernel (flash_bla/ops/piecewise_attn/kernel.py:89-128,152-176).
+ * With NT = ceil(T/chunk): qc, kc [BH,NT,K] = chunk means of q, k; vc [BH,NT,V] = chunk
+ * sums of v; h [BH,K,V] = sum_c (K_c - kc_c)^T V_c; h_norm [BH,NT] (optional, may be
+ * NULL) = p-norm of each chunk's (K_c - kc_c)^T V_c (kernel.py:172-174).  All outputs
+ * are fp32 (the reference stores them in the input dtype). */
+int fbla_chunk_reduce(const void* q, const void* k, const void* v, float* qc, float* kc, float* vc,
+                      float* h, float* h_norm, void* workspace, size_t workspace_bytes, int64_t BH,
+                      int64_t T, int K, int V, int chunk, float p_norm, int dtype, void* stream);
+
+/* Workspace of fbla_piecewise_fwd; 0 when the shape is not supported. */
+size_t fbla_piecewise_workspace_bytes(int64_t BH, int64_t T, int K, int V, int block, int dtype);
+
+/* Piecewise attention forward.  Replaces piecewise_sparse_attention_fwd_kernel
+ * (kernel.py:189-292): exact softmax attention over the NS selected 64-key blocks of
+ * every 64-query block (indices: int32 [BH, NT, NS]), the remaining blocks through
+ * their mean key / value sum (zeroth order) and h (first order).  kc, vc, h are the
+ * fp32 outputs of fbla_chunk_reduce with chunk = block.  fp16/bf16, K,V in {64,128},
+ * block = 64; anything else returns FBLA_ERR_UNSUPPORTED. */
+int fbla_piecewise_fwd(const void* q, const void* k, const void* v, const float* kc, const float* vc,
+                       const float* h, const int32_t* indices, void* o, void* workspace,
+                       size_t workspace_bytes, int64_t BH, int64_t T, int K, int V, int block, int NS,
+                       float scale, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

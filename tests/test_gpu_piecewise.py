@@ -1,0 +1,108 @@
+"""GPU parity of the piecewise (PISA) operators against the float64 oracle
+(oracle/piecewise.py).  The reference has neither a naive implementation nor a
+test for this operator: agreement with its Triton kernel is "parity unpinned";
+what is checked here is the mathematics the kernel text defines."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import TOL, assert_parity, max_rel_err, np64
+from oracle import piecewise as pw
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(B, H, T, K, V, dtype, seed=0, qk_scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    q = (qk_scale * torch.randn(B, H, T, K, generator=g)).to(dtype)
+    k = (qk_scale * torch.randn(B, H, T, K, generator=g)).to(dtype)
+    v = torch.randn(B, H, T, V, generator=g).to(dtype)
+    return q, k, v
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32], ids=str)
+@pytest.mark.parametrize("T,K,V,chunk", [(200, 64, 64, 64), (1000, 128, 128, 64), (130, 32, 16, 32),
+                                         (257, 64, 128, 64)])
+def test_fused_chunk_reduce(dtype, T, K, V, chunk):
+    from flash_bla.ops.piecewise_attn.kernel import chunk_reduce_fp32, fused_chunk_reduce
+    q, k, v = _inputs(1, 3, T, K, V, dtype, seed=1)
+    qc, kc, vc, h, bias = chunk_reduce_fp32(q.cuda(), k.cuda(), v.cuda(), chunk, use_bias=True)
+    for hd in range(3):
+        rq, rk, rv, rhc, rH, lens = pw.chunk_reduce(np64(q)[0, hd], np64(k)[0, hd], np64(v)[0, hd], chunk)
+        assert max_rel_err(qc[0, hd], rq) < 1e-5
+        assert max_rel_err(kc[0, hd], rk) < 1e-5
+        assert max_rel_err(vc[0, hd], rv) < 1e-5
+        assert max_rel_err(h[0, hd], rH) < 2e-5
+        ref_norm = np.sqrt((rhc.reshape(rhc.shape[0], -1) ** 2).sum(-1))
+        assert max_rel_err(bias[0, hd, 0], ref_norm) < 2e-5
+    # the reference-typed variant returns the input dtype and no bias by default
+    out = fused_chunk_reduce(q.cuda(), k.cuda(), v.cuda(), chunk)
+    assert out[0].dtype == dtype and out[3].dtype == dtype and out[4] is None
+    assert out[3].shape == (1, 3, K, V)
+
+
+def _oracle(q, k, v, indices, scale=None):
+    B, H = q.shape[:2]
+    out = np.zeros(v.shape, dtype=np.float64)
+    for b in range(B):
+        for h in range(H):
+            out[b, h] = pw.piecewise_forward(np64(q)[b, h], np64(k)[b, h], np64(v)[b, h],
+                                             indices[b, h].cpu().numpy(), 64, scale)
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("T,K,V,density", [
+    (256, 64, 64, 0.5),
+    (200, 64, 64, 0.3),        # ragged last block
+    (1000, 128, 128, 0.25),    # BASELINE config 5 head dims
+    (640, 128, 64, 0.1),
+    (520, 64, 128, 0.4),
+])
+def test_piecewise_attention_matches_oracle(dtype, T, K, V, density):
+    from flash_bla.ops.piecewise_attn.kernel import (chunk_reduce_fp32, piecewise_sparse_attention,
+                                                     select_blocks)
+    q, k, v = _inputs(1, 2, T, K, V, dtype, seed=2)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    qc, kc, vc, h, _ = chunk_reduce_fp32(qd, kd, vd, 64)
+    indices = select_blocks(qc, kc, K ** -0.5, density)
+    o = piecewise_sparse_attention(qd, kd, vd, density=density, indices=indices)
+    assert o.dtype == dtype and o.shape == v.shape
+    ref = _oracle(q, k, v, indices)
+    assert_parity(o, ref, dtype, f"T{T} K{K} V{V}")
+    # and with its own selection (same code path as select_blocks)
+    o2 = piecewise_sparse_attention(qd, kd, vd, density=density)
+    assert torch.equal(o, o2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_all_blocks_selected_is_softmax_attention(dtype):
+    from flash_bla.ops.piecewise_attn.kernel import piecewise_sparse_attention
+    q, k, v = _inputs(2, 2, 300, 64, 64, dtype, seed=3)
+    o = piecewise_sparse_attention(q.cuda(), k.cuda(), v.cuda(), density=1.0)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.double(), k.double(), v.double())
+    assert_parity(o, ref, dtype, "density 1")
+
+
+def test_small_scores_first_order_branch():
+    """Small logits: the linear branch carries real weight and the first-order term matters."""
+    from flash_bla.ops.piecewise_attn.kernel import chunk_reduce_fp32, piecewise_sparse_attention
+    q, k, v = _inputs(1, 2, 768, 64, 64, torch.float16, seed=4, qk_scale=0.3)
+    NT = 12
+    indices = torch.arange(NT).view(1, 1, NT, 1).expand(1, 2, NT, 1).contiguous().cuda()
+    o = piecewise_sparse_attention(q.cuda(), k.cuda(), v.cuda(), indices=indices, scale=0.5)
+    ref = _oracle(q, k, v, indices, scale=0.5)
+    assert_parity(o, ref, torch.float16, "first order")
+
+
+def test_use_bias_selection_and_errors():
+    from flash_bla.ops.piecewise_attn.kernel import piecewise_sparse_attention
+    q, k, v = _inputs(1, 2, 512, 64, 64, torch.bfloat16, seed=5)
+    o = piecewise_sparse_attention(q.cuda(), k.cuda(), v.cuda(), density=0.25, use_bias=True)
+    assert torch.isfinite(o).all()
+    with pytest.raises(NotImplementedError):
+        piecewise_sparse_attention(q.cuda().float(), k.cuda().float(), v.cuda().float())
+    with pytest.raises(NotImplementedError):
+        piecewise_sparse_attention(q.cuda(), k.cuda(), v.cuda(), block_size=32)
+    with pytest.raises(ValueError):
+        piecewise_sparse_attention(q, k, v)
