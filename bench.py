@@ -271,6 +271,7 @@ def main():
         sweep(dtype, dev, flush)
     if args.configs:
         other_configs(dev, flush)
+        piecewise_config(dev, flush)
     print(json.dumps(line), flush=True)
 
 
@@ -382,6 +383,32 @@ def other_configs(dev, flush):
                 return varlen_linear_attention(q, k, v, cu, max_len)
         _report(f"C3 varlen 64 seqs U[256,2048] H16 D{D} bf16", 4 * nb, 11 * nb, fwd, step, flush,
                 {"total_tokens": total, "max_seqlen": max_len})
+
+
+def piecewise_config(dev, flush):
+    """BASELINE config 5: PISA forward, B1-H24-T16384-D128 bf16, 64-token blocks, density 0.25."""
+    from flash_bla.ops.piecewise_attn.kernel import (chunk_reduce_fp32, piecewise_sparse_attention,
+                                                     select_blocks)
+    g = torch.Generator(device=dev).manual_seed(42)
+    shape = (1, 24, 16384, 128)
+    q = torch.randn(shape, generator=g, device=dev).bfloat16()
+    k = torch.randn(shape, generator=g, device=dev).bfloat16()
+    v = torch.randn(shape, generator=g, device=dev).bfloat16()
+    nb = q.numel() * 2
+    scale = 128 ** -0.5
+    qc, kc, vc, h, _ = chunk_reduce_fp32(q, k, v, 64)
+    indices = select_blocks(qc, kc, scale, 0.25)
+    flops_exact = 4.0 * 24 * 16384 * (indices.shape[-1] * 64) * 128
+    t_all = do_bench(lambda: piecewise_sparse_attention(q, k, v, density=0.25), flush)
+    t_red = do_bench(lambda: chunk_reduce_fp32(q, k, v, 64), flush)
+    t_att = do_bench(lambda: piecewise_sparse_attention(q, k, v, indices=indices), flush)
+    print(json.dumps({
+        "config": "C5 piecewise fwd B1-H24-T16384-D128 bf16 block64 density0.25",
+        "total_ms": round(t_all[0], 4), "chunk_reduce_ms": round(t_red[0], 4),
+        "chunk_reduce_gbps": round(3 * nb / t_red[0] / 1e6, 1),
+        "chunk_reduce_plus_attention_ms": round(t_att[0], 4),
+        "exact_branch_tflops": round(flops_exact / ((t_att[0] - t_red[0]) * 1e-3) / 1e12, 1),
+        "min_traffic_gbps": round(4 * nb / t_all[0] / 1e6, 1)}), file=sys.stderr, flush=True)
 
 
 if __name__ == "__main__":

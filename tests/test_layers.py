@@ -1,0 +1,85 @@
+"""Layer counterparts: `mode='torch'` runs anywhere (CPU shapes check), on the GPU
+`mode='triton'` (the HIP operators) must agree with it for the output and the
+input gradient, with the acceptance rule of the reference layers' self-tests
+(flash_bla/utils.py:55-67 with ratio 0.06; layers/linfusion.py:116-141 etc.)."""
+import pytest
+import torch
+
+from flash_bla.layers import (FocusedLinearAttention, GeneralizedLinearAttention, MambaLikeLinearAttention,
+                              PolaLinearAttention, RALALinearAttention)
+from flash_bla.utils import assert_close
+
+CASES = {
+    "linfusion": (lambda: GeneralizedLinearAttention(256, heads=4, dim_head=64), (2, 144, 256), ()),
+    "mlla": (lambda: MambaLikeLinearAttention(128, (12, 12), 4), (2, 144, 128), ()),
+    "rala": (lambda: RALALinearAttention(128, (12, 12), 4), (2, 144, 128), ()),
+    "focused": (lambda: FocusedLinearAttention(256, 144, num_heads=4), (2, 144, 256), (12, 12)),
+    "pola": (lambda: PolaLinearAttention(128, 144, num_heads=4), (2, 144, 128), (12, 12)),
+}
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_torch_mode_on_cpu(name):
+    torch.manual_seed(0)
+    make, shape, extra = CASES[name]
+    layer = make()
+    x = torch.randn(shape, requires_grad=True)
+    y = layer(x, *extra, mode='torch')
+    assert y.shape == x.shape and torch.isfinite(y).all()
+    y.sum().backward()
+    assert torch.isfinite(x.grad).all()
+    with pytest.raises(NotImplementedError):
+        layer(x, *extra, mode='flash')
+
+
+def test_linfusion_state_dict_names():
+    names = set(GeneralizedLinearAttention(64, heads=1, dim_head=64).state_dict())
+    assert {"to_q.weight", "to_k.weight", "to_v.weight", "to_out.0.weight", "to_out.0.bias",
+            "to_q_.0.weight", "to_q_.1.weight", "to_q_.3.bias", "to_k_.3.weight"} <= names
+    assert "to_q.bias" not in names
+
+
+GPU_CASES = {
+    # the shapes of the reference self-tests
+    "linfusion": (lambda: GeneralizedLinearAttention(1024, heads=16, dim_head=64), (2, 4096, 1024), ()),
+    "mlla": (lambda: MambaLikeLinearAttention(512, (16, 16), 16), (4, 256, 512), ()),
+    "rala": (lambda: RALALinearAttention(512, (16, 16), 16), (4, 256, 512), ()),
+    "focused": (lambda: FocusedLinearAttention(1024, 256, num_heads=16), (4, 256, 1024), (16, 16)),
+    "pola": (lambda: PolaLinearAttention(256, 256, num_heads=8), (4, 256, 256), (16, 16)),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16], ids=str)
+@pytest.mark.parametrize("name", sorted(GPU_CASES))
+def test_fast_mode_matches_torch_mode(name, dtype):
+    torch.manual_seed(1)
+    make, shape, extra = GPU_CASES[name]
+    if dtype == torch.float16 and name in ("mlla", "rala"):
+        pytest.skip("the rotary features of these blocks are fp32 (mlla.py:32-36)")
+    layer = make().to("cuda", dtype)
+    x = torch.randn(shape, device="cuda", dtype=dtype, requires_grad=True)
+    do = torch.randn(shape, device="cuda", dtype=dtype)
+    ref = layer(x, *extra, mode='torch')
+    ref.backward(do)
+    ref_dx, x.grad = x.grad.clone(), None
+    out = layer(x, *extra, mode='triton')
+    out.backward(do)
+    assert_close("o", ref, out, 0.06)
+    assert_close("dx", ref_dx, x.grad, 0.06)
+    if dtype == torch.float32:
+        assert (out - ref).abs().max() <= 1e-3 * ref.abs().max() + 1e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tokens,channels,heads", [(4096, 640, 10), (1024, 1280, 20)])
+def test_linfusion_sdxl_shapes_fp16(tokens, channels, heads):
+    """BASELINE config 4: SDXL self-attention shapes, B=2, fp16, forward only."""
+    torch.manual_seed(42)
+    layer = GeneralizedLinearAttention(channels, heads=heads, dim_head=64).to("cuda", torch.float16)
+    x = torch.randn(2, tokens, channels, device="cuda", dtype=torch.float16)
+    with torch.no_grad():
+        out = layer(x, mode='triton')
+        ref = layer.float()(x.float(), mode='torch')
+    assert_close("o", ref, out.float(), 0.06)
+    assert (out.float() - ref).abs().max() <= 5e-3 * ref.abs().max()
