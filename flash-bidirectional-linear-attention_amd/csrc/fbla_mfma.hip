@@ -1032,7 +1032,7 @@ int bwd_a_chunk(const Prob& p) {
 // Row-parallel kernels: long enough chunks to amortise the operand prologue.
 int rows_chunk(const Prob& p, int DR, int DC) {
   static const int per_cu_knob = knob("FBLA_ROWS_WGS_PER_CU", 4);
-  static const int rounds = knob("FBLA_ROWS_ROUNDS", 1);
+  static const int rounds = knob("FBLA_ROWS_ROUNDS", 4);
   const int big = (DR == 128) + (DC == 128);
   const int per_cu = big == 0 ? per_cu_knob : (big == 1 ? 2 : 1);
   return chunk_for(p, per_cu, rounds, 512, big == 2 ? 256 : 128);
