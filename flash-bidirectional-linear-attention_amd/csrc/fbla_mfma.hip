@@ -677,11 +677,11 @@ __device__ __forceinline__ void lds_rows(RowWords<C>& dst, const unsigned char* 
   }
 }
 
-template <int DK, int DV, bool NORM, bool DEN, bool FUSED> struct BwdALayout {
+template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struct BwdALayout {
   static constexpr int KS = DV / 16, NB = DK / 32;
   static constexpr int kOpnd = NB * KS * 2 * 1024;
   static constexpr int kQ = 32 * DK * 2, kG = 32 * DV * 2;
-  static constexpr int kWave = kQ + kG + (NORM && FUSED ? kG : 0) + (DEN ? kQ : 0) + 128;  // + dz[32]
+  static constexpr int kWave = kQ + kG + (NORM && FUSED && LO ? kG : 0) + (DEN ? kQ : 0) + 128;  // + dz[32]
   static constexpr int kKmPairs = kOpnd + kWaves * kWave;
   static constexpr int kKmF = kKmPairs + DK * 4;
   static constexpr int kMax = kKmF + DK * 4;
@@ -691,13 +691,13 @@ template <int DK, int DV, bool NORM, bool DEN, bool FUSED> struct BwdALayout {
 // FUSED = false runs the token view only (head dims whose dS accumulators do not
 // fit one wave): it writes 1/z_t and dz_t per (token, head) row to `tokscal`
 // ([2][total rows]) for scaled_state_kernel, and no partials.
-template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED>
+template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true>
 __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
     Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const T* __restrict__ dout,
     const float* __restrict__ S, const float* __restrict__ km, T* __restrict__ dqn,
     T* __restrict__ dqd, float* __restrict__ partial, float* __restrict__ tokscal,
     int64_t total_rows, int chunk, int nchunks) {
-  using LY = BwdALayout<DK, DV, NORM, DEN, FUSED>;
+  using LY = BwdALayout<DK, DV, NORM, DEN, FUSED, LO>;
   constexpr int KS = LY::KS, NB = LY::NB;
   constexpr int CK = DK / 32, CV = DV / 32;
   constexpr int QROWB = DK * 2, GROWB = DV * 2;
@@ -722,7 +722,7 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
   unsigned char* qt = smem + LY::kOpnd + wave * LY::kWave;
   unsigned char* gt = qt + LY::kQ;             // dO, later dO/z (hi part)
   unsigned char* gl = gt + LY::kG;             // dO/z (lo part), NORM && FUSED only
-  unsigned char* qdt = gl + (NORM && FUSED ? LY::kG : 0);  // plain q, DEN only
+  unsigned char* qdt = gl + (NORM && FUSED && LO ? LY::kG : 0);  // plain q, DEN only
   float* dzs = reinterpret_cast<float*>(qdt + (DEN ? LY::kQ : 0));
   uint32_t* km_pairs = reinterpret_cast<uint32_t*>(smem + LY::kKmPairs);
   float* kmf = reinterpret_cast<float*>(smem + LY::kKmF);
@@ -902,7 +902,7 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
           wl[i] = pack2<T>(a - (float)ah, b - (float)bh);
         }
         *reinterpret_cast<u32x4*>(gt + off) = wh;
-        *reinterpret_cast<u32x4*>(gl + off) = wl;
+        if constexpr (LO) *reinterpret_cast<u32x4*>(gl + off) = wl;
       }
     }
     wave_sync();
@@ -924,14 +924,16 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
 #pragma unroll
         for (int b = 0; b < CV; ++b) acc[a][b] = Ops<T>::mma(A[a], Bh[b], acc[a][b]);
       if constexpr (NORM) {
-        RowWords<CV> glw;
-        lds_rows<CV>(glw, gl, tok0, ntok);
-        u32x4 Bl[CV];
-        transpose_rows<CV>(glw, Bl);
+        if constexpr (LO) {
+          RowWords<CV> glw;
+          lds_rows<CV>(glw, gl, tok0, ntok);
+          u32x4 Bl[CV];
+          transpose_rows<CV>(glw, Bl);
 #pragma unroll
-        for (int a = 0; a < CK; ++a)
+          for (int a = 0; a < CK; ++a)
 #pragma unroll
-          for (int b = 0; b < CV; ++b) acc[a][b] = Ops<T>::mma(A[a], Bl[b], acc[a][b]);
+            for (int b = 0; b < CV; ++b) acc[a][b] = Ops<T>::mma(A[a], Bl[b], acc[a][b]);
+        }
         if constexpr (DEN) lds_rows<CK>(qw, qdt, tok0, ntok);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -1138,16 +1140,16 @@ int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, in
   return run_rows<__bf16>(p, job0, &job1, DR, DC, st);
 }
 
-template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED>
+template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true>
 static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, const float* S,
                         const float* km, T* dqn, T* dqd, float* partial, float* tokscal,
                         int64_t total_rows, int chunk, int nchunks, hipStream_t st) {
-  using LY = BwdALayout<DK, DV, NORM, DEN, FUSED>;
+  using LY = BwdALayout<DK, DV, NORM, DEN, FUSED, LO>;
   static_assert(!FUSED || LY::kTotal - LY::kOpnd >=
                               (int)sizeof(float) * 64 * ((DK / 32) * (DV / 32) * 16 + DK / 32),
                 "reduction buffer must fit in the tile area");
   static_assert(LY::kTotal <= 160 * 1024, "LDS budget of one workgroup");
-  auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN, FUSED>;
+  auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN, FUSED, LO>;
   static thread_local bool configured = false;  // per instantiation
   int rc = reserve_lds(kernel, LY::kTotal, configured);
   if (rc != kOk) return rc;
