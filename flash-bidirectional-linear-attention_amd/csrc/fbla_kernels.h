@@ -87,8 +87,10 @@ bool bwd_a_supported(const Prob& p, int dtype);
 int state_chunk(const Prob& p);
 int bwd_a_chunk(const Prob& p);
 int rows_chunk(const Prob& p, int DR, int DC);
+// fin_mat / fin_vec (only with nchunks == 1): store the finished, scaled matrix [N*H,DK,DV] and
+// vector [N*H,DK] directly instead of a partial (no reduce step needed)
 void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
-           int chunk, int nchunks, hipStream_t st);
+           int chunk, int nchunks, hipStream_t st, float* fin_mat = nullptr, float* fin_vec = nullptr);
 // out_t = (x_t M) / (xden_t . km + eps) + addvec   with M of shape DR x DC
 int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st);
 int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, int DR, int DC,
@@ -99,11 +101,12 @@ int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, in
 int bwd_tokens(const Prob& p, int dtype, const void* q, const void* dout, const float* S,
                const float* km, void* dq, float* tokscal, int64_t total_rows, hipStream_t st);
 void scaled_state(const Prob& p, int dtype, const void* qn, const void* dout, const float* tokscal,
-                  int64_t total_rows, float* partial, int chunk, int nchunks, hipStream_t st);
+                  int64_t total_rows, float* partial, int chunk, int nchunks, hipStream_t st,
+                  float* fin_mat = nullptr, float* fin_vec = nullptr);
 // backward pass A: dq~ (and dq when decoupled) + per-chunk partials of dS and dkm
 int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout, const float* S,
           const float* km, void* dqn, void* dqd, float* partial, int chunk, int nchunks,
-          hipStream_t st);
+          hipStream_t st, float* fin_mat = nullptr, float* fin_vec = nullptr);
 }  // namespace mfma
 
 // Piecewise (PISA) attention, forward only (fbla_piecewise.hip).

@@ -143,11 +143,13 @@ __device__ __forceinline__ void transpose_rows(const RowWords<C>& src, u32x4 (&o
 // the canonical [dk][dv] partial followed by the [dk] vector is written.
 // NS = 1: every wave holds the full DK x DV block (2 -> 0, 3 -> 1, 1 -> 0; wave 0 writes).
 // NS = 2: wave w holds value columns [(w%2)*32*CV, +32*CV) (2 -> 0, 3 -> 1; waves 0 and 1
-// write their halves, wave 0 the vector).  Register r of block (a,b) is dk = CK*m + a,
+// write their halves, wave 0 the vector).  The matrix goes to dst times mscale, the vector
+// to dst_vec (if given) times vscale.  Register r of block (a,b) is dk = CK*m + a,
 // dv = CV*pp + b with m = 8*(r/4) + 4*kb + r%4.  Must be reached by all waves.
 template <int CK, int CV, int NS>
 __device__ __forceinline__ void reduce_store_partial(f32x16 (&acc)[CK][CV], float (&ks)[CK],
-                                                     float* red, float* dst, int wave, int lane) {
+                                                     float* red, float* dst, float* dst_vec,
+                                                     float mscale, float vscale, int wave, int lane) {
   constexpr int kAcc = CK * CV * 16;
   constexpr int DK = 32 * CK, DVW = 32 * CV, DV = DVW * NS;
   const int pp = lane & 31, kb = lane >> 5;
@@ -195,13 +197,13 @@ __device__ __forceinline__ void reduce_store_partial(f32x16 (&acc)[CK][CV], floa
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = 8 * (r >> 2) + 4 * kb + (r & 3);
-        dst[(CK * m + a) * DV + dv_off + CV * pp + b] = acc[a][b][r];
+        dst[(CK * m + a) * DV + dv_off + CV * pp + b] = acc[a][b][r] * mscale;
       }
-  if (wave == 0) {
+  if (wave == 0 && dst_vec) {
 #pragma unroll
     for (int a = 0; a < CK; ++a) {
       const float tot = ks[a] + __shfl_xor(ks[a], 32);
-      if (kb == 0) dst[DK * DV + CK * pp + a] = tot;
+      if (kb == 0) dst_vec[CK * pp + a] = tot * vscale;
     }
   }
 }
@@ -216,8 +218,8 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
                                                          const T* __restrict__ kd,
                                                          float* __restrict__ partial,
                                                          const float* __restrict__ tokscal,
-                                                         int64_t total_rows, int chunk,
-                                                         int nchunks) {
+                                                         int64_t total_rows, float* fin_mat,
+                                                         float* fin_vec, int chunk, int nchunks) {
   // 128 x 128 states are split by value columns over wave pairs (256 accumulator
   // registers would not fit one wave): wave w owns columns [(w%NS)*DVW, +DVW).
   constexpr int NS = (DK == 128 && DV == 128) ? 2 : 1;
@@ -232,7 +234,14 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
   int len;
   seq_range(p, n, bos, len);
   const int t_begin = c * chunk;
-  if (t_begin >= len) return;
+  if (t_begin >= len) {
+    if (fin_mat && c == 0) {  // empty sequence: its state is zero
+      for (int e = threadIdx.x; e < DK * DV; e += kThreads) fin_mat[(int64_t)nh * DK * DV + e] = 0.f;
+      if (fin_vec)
+        for (int e = threadIdx.x; e < DK; e += kThreads) fin_vec[(int64_t)nh * DK + e] = 0.f;
+    }
+    return;
+  }
   const int t_end = min(len, t_begin + chunk);
   row_base(p, n, h, bos, row0, rstride);
 
@@ -340,8 +349,13 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
     t0 = tn;
   }
 
-  float* dst = partial + (int64_t)blockIdx.x * (DK * DV + DK);
-  reduce_store_partial<CK, CV, NS>(acc, ks, red, dst, wave, lane);
+  // one chunk per (sequence, head): the sum is final, store it scaled where the reduce
+  // kernel would have put it; otherwise store this chunk's partial
+  float* dst = fin_mat ? fin_mat + (int64_t)nh * DK * DV : partial + (int64_t)blockIdx.x * (DK * DV + DK);
+  float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * DK : nullptr) : dst + DK * DV;
+  const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
+  const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
+  reduce_store_partial<CK, CV, NS>(acc, ks, red, dst, dst_vec, mscale, vscale, wave, lane);
 }
 
 // ===========================================================================
@@ -696,7 +710,7 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
     Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const T* __restrict__ dout,
     const float* __restrict__ S, const float* __restrict__ km, T* __restrict__ dqn,
     T* __restrict__ dqd, float* __restrict__ partial, float* __restrict__ tokscal,
-    int64_t total_rows, int chunk, int nchunks) {
+    int64_t total_rows, float* fin_mat, float* fin_vec, int chunk, int nchunks) {
   using LY = BwdALayout<DK, DV, NORM, DEN, FUSED, LO>;
   constexpr int KS = LY::KS, NB = LY::NB;
   constexpr int CK = DK / 32, CV = DV / 32;
@@ -711,7 +725,14 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
   int len;
   seq_range(p, n, bos, len);
   const int t_begin = c * chunk;
-  if (t_begin >= len) return;
+  if (t_begin >= len) {
+    if (fin_mat && c == 0) {  // empty sequence: no gradient flows through its state
+      for (int e = threadIdx.x; e < DK * DV; e += kThreads) fin_mat[(int64_t)nh * DK * DV + e] = 0.f;
+      if (fin_vec)
+        for (int e = threadIdx.x; e < DK; e += kThreads) fin_vec[(int64_t)nh * DK + e] = 0.f;
+    }
+    return;
+  }
   const int t_end = min(len, t_begin + chunk);
   row_base(p, n, h, bos, row0, rstride);
 
@@ -964,8 +985,12 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
 
   if constexpr (FUSED) {
     __syncthreads();  // every wave is done with its tiles: reuse them for the reduction
-    float* dst = partial + (int64_t)blockIdx.x * (DK * DV + DK);
-    reduce_store_partial<CK, CV, 1>(acc, dkm, reinterpret_cast<float*>(smem + LY::kOpnd), dst, wave, lane);
+    float* red = reinterpret_cast<float*>(smem + LY::kOpnd);
+    float* dst = fin_mat ? fin_mat + (int64_t)nh * DK * DV : partial + (int64_t)blockIdx.x * (DK * DV + DK);
+    float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * DK : nullptr) : dst + DK * DV;
+    const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
+    const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
+    reduce_store_partial<CK, CV, 1>(acc, dkm, red, dst, dst_vec, mscale, vscale, wave, lane);
   }
 }
 
@@ -1042,25 +1067,26 @@ int rows_chunk(const Prob& p, int DR, int DC) {
 
 template <typename T, int DK, int DV>
 static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, float* partial,
-                         const float* tokscal, int64_t total_rows, int chunk, int nchunks,
-                         hipStream_t st) {
+                         const float* tokscal, int64_t total_rows, float* fm, float* fv, int chunk,
+                         int nchunks, hipStream_t st) {
   const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(kThreads);
   if (tokscal)
-    state_kernel<T, DK, DV, false, 1, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, chunk, nchunks);
+    state_kernel<T, DK, DV, false, 1, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fm, fv, chunk, nchunks);
   else if (p.flags & kDecoupled)
-    state_kernel<T, DK, DV, true, 1, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, chunk, nchunks);
+    state_kernel<T, DK, DV, true, 1, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks);
   else
-    state_kernel<T, DK, DV, false, 1, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, chunk, nchunks);
+    state_kernel<T, DK, DV, false, 1, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks);
 }
 
 template <typename T>
 static void run_state(const Prob& p, const void* kn, const void* v, const void* kd, float* partial,
-                      const float* ts, int64_t rows, int chunk, int nchunks, hipStream_t st) {
+                      const float* ts, int64_t rows, float* fm, float* fv, int chunk, int nchunks,
+                      hipStream_t st) {
   const T *a = (const T*)kn, *b = (const T*)v, *c = (const T*)kd;
-  if (p.DK == 64 && p.DV == 64) launch_state<T, 64, 64>(p, a, b, c, partial, ts, rows, chunk, nchunks, st);
-  else if (p.DK == 64) launch_state<T, 64, 128>(p, a, b, c, partial, ts, rows, chunk, nchunks, st);
-  else if (p.DV == 64) launch_state<T, 128, 64>(p, a, b, c, partial, ts, rows, chunk, nchunks, st);
-  else launch_state<T, 128, 128>(p, a, b, c, partial, ts, rows, chunk, nchunks, st);
+  if (p.DK == 64 && p.DV == 64) launch_state<T, 64, 64>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, st);
+  else if (p.DK == 64) launch_state<T, 64, 128>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, st);
+  else if (p.DV == 64) launch_state<T, 128, 64>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, st);
+  else launch_state<T, 128, 128>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, st);
 }
 
 // Reserves the kernel's dynamic LDS once per instantiation and thread.
@@ -1117,15 +1143,18 @@ static int run_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, int 
 }
 
 void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
-           int chunk, int nchunks, hipStream_t st) {
-  if (dtype == kF16) run_state<_Float16>(p, kn, v, kd, partial, nullptr, 0, chunk, nchunks, st);
-  else run_state<__bf16>(p, kn, v, kd, partial, nullptr, 0, chunk, nchunks, st);
+           int chunk, int nchunks, hipStream_t st, float* fin_mat, float* fin_vec) {
+  if (dtype == kF16) run_state<_Float16>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks, st);
+  else run_state<__bf16>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks, st);
 }
 
 void scaled_state(const Prob& p, int dtype, const void* qn, const void* dout, const float* tokscal,
-                  int64_t total_rows, float* partial, int chunk, int nchunks, hipStream_t st) {
-  if (dtype == kF16) run_state<_Float16>(p, qn, dout, qn, partial, tokscal, total_rows, chunk, nchunks, st);
-  else run_state<__bf16>(p, qn, dout, qn, partial, tokscal, total_rows, chunk, nchunks, st);
+                  int64_t total_rows, float* partial, int chunk, int nchunks, hipStream_t st,
+                  float* fin_mat, float* fin_vec) {
+  if (dtype == kF16)
+    run_state<_Float16>(p, qn, dout, qn, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, st);
+  else
+    run_state<__bf16>(p, qn, dout, qn, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, st);
 }
 
 int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {
@@ -1143,7 +1172,8 @@ int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, in
 template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true>
 static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, const float* S,
                         const float* km, T* dqn, T* dqd, float* partial, float* tokscal,
-                        int64_t total_rows, int chunk, int nchunks, hipStream_t st) {
+                        int64_t total_rows, float* fm, float* fv, int chunk, int nchunks,
+                        hipStream_t st) {
   using LY = BwdALayout<DK, DV, NORM, DEN, FUSED, LO>;
   static_assert(!FUSED || LY::kTotal - LY::kOpnd >=
                               (int)sizeof(float) * 64 * ((DK / 32) * (DV / 32) * 16 + DK / 32),
@@ -1155,29 +1185,29 @@ static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, 
   if (rc != kOk) return rc;
   const unsigned grid = (unsigned)((int64_t)p.N * p.H * nchunks);
   kernel<<<dim3(grid), dim3(kThreads), LY::kTotal, st>>>(p, qn, qd, dout, S, km, dqn, dqd, partial,
-                                                         tokscal, total_rows, chunk, nchunks);
+                                                         tokscal, total_rows, fm, fv, chunk, nchunks);
   return kOk;
 }
 
 template <typename T>
 static int run_bwd_a(const Prob& p, const void* qn, const void* qd, const void* dout, const float* S,
-                     const float* km, void* dqn, void* dqd, float* partial, int chunk, int nchunks,
-                     hipStream_t st) {
+                     const float* km, void* dqn, void* dqd, float* partial, float* fm, float* fv,
+                     int chunk, int nchunks, hipStream_t st) {
   const T *a = (const T*)qn, *b = (const T*)qd, *c = (const T*)dout;
   T *x = (T*)dqn, *y = (T*)dqd;
   if (!(p.flags & kNormalize))
-    return launch_bwd_a<T, 64, 64, false, false, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, chunk, nchunks, st);
+    return launch_bwd_a<T, 64, 64, false, false, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
   if (p.flags & kDecoupled)
-    return launch_bwd_a<T, 64, 64, true, true, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, chunk, nchunks, st);
-  return launch_bwd_a<T, 64, 64, true, false, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, chunk, nchunks, st);
+    return launch_bwd_a<T, 64, 64, true, true, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+  return launch_bwd_a<T, 64, 64, true, false, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
 }
 
 int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout, const float* S,
           const float* km, void* dqn, void* dqd, float* partial, int chunk, int nchunks,
-          hipStream_t st) {
+          hipStream_t st, float* fin_mat, float* fin_vec) {
   if (dtype == kF16)
-    return run_bwd_a<_Float16>(p, qn, qd, dout, S, km, dqn, dqd, partial, chunk, nchunks, st);
-  return run_bwd_a<__bf16>(p, qn, qd, dout, S, km, dqn, dqd, partial, chunk, nchunks, st);
+    return run_bwd_a<_Float16>(p, qn, qd, dout, S, km, dqn, dqd, partial, fin_mat, fin_vec, chunk, nchunks, st);
+  return run_bwd_a<__bf16>(p, qn, qd, dout, S, km, dqn, dqd, partial, fin_mat, fin_vec, chunk, nchunks, st);
 }
 
 template <typename T, int DK, int DV>
@@ -1187,9 +1217,11 @@ static int launch_bwd_tokens(const Prob& p, const void* q, const void* dout, con
   const T *a = (const T*)q, *c = (const T*)dout;
   if (p.flags & kNormalize)
     return launch_bwd_a<T, DK, DV, true, false, false>(p, a, a, c, S, km, (T*)dq, nullptr, nullptr,
-                                                       tokscal, total_rows, chunk, nchunks, st);
+                                                       tokscal, total_rows, nullptr, nullptr, chunk,
+                                                       nchunks, st);
   return launch_bwd_a<T, DK, DV, false, false, false>(p, a, a, c, S, km, (T*)dq, nullptr, nullptr,
-                                                      tokscal, total_rows, chunk, nchunks, st);
+                                                      tokscal, total_rows, nullptr, nullptr, chunk,
+                                                      nchunks, st);
 }
 
 template <typename T>

@@ -50,6 +50,56 @@ __global__ __launch_bounds__(kThreads) void chunk_sums_kernel(
   }
 }
 
+// The same for 16-bit inputs with D in {64, 128}: 16-byte loads, a lane owns one
+// 8-feature column group and every (64 / chunks-per-row)-th row, lanes are combined by
+// shuffles at the end.
+typedef uint32_t u32x4s __attribute__((ext_vector_type(4)));
+template <typename T, int D>
+__global__ __launch_bounds__(kThreads) void chunk_sums16_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, float* __restrict__ qc,
+    float* __restrict__ kc, float* __restrict__ vc, int64_t BH, int Tn, int NT, int chunk) {
+  constexpr int CH = D / 8, RPI = 64 / CH;  // chunks per row, rows per wave instruction
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t item = (int64_t)blockIdx.x * 4 + wave;
+  if (item >= BH * NT * 3) return;
+  const int which = (int)(item % 3);
+  const int64_t bc = item / 3;
+  const int c = (int)(bc % NT);
+  const int64_t bh = bc / NT;
+  const T* src = (which == 0 ? q : which == 1 ? k : v) + (bh * Tn + (int64_t)c * chunk) * D;
+  float* dst = (which == 0 ? qc : which == 1 ? kc : vc) + bc * D;
+  const int n = min(chunk, Tn - c * chunk);
+  const int ch = lane % CH, r0 = lane / CH;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  for (int base = 0; base < n; base += 4 * RPI) {
+    u32x4s w[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int row = base + u * RPI + r0;
+      w[u] = row < n ? *reinterpret_cast<const u32x4s*>(src + (int64_t)row * D + ch * 8)
+                     : u32x4s{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[2 * i] += (float)__builtin_bit_cast(T, (uint16_t)(w[u][i] & 0xffffu));
+        acc[2 * i + 1] += (float)__builtin_bit_cast(T, (uint16_t)(w[u][i] >> 16));
+      }
+  }
+#pragma unroll
+  for (int off = CH; off < 64; off <<= 1)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] += __shfl_xor(acc[i], off);
+  if (lane < CH) {
+    const float f = which == 2 ? 1.f : 1.f / (float)n;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dst[ch * 8 + i] = acc[i] * f;
+  }
+}
+
 // H[bh][dk][dv] = sum_p partial_p[dk][dv] - sum_c n_c kc_c[dk] vc_c[dv] / n_c ... with
 // kc the MEAN and vc the SUM of a chunk the correction is simply kc_c[dk] * vc_c[dv].
 __global__ __launch_bounds__(kThreads) void finish_h_kernel(
@@ -65,9 +115,18 @@ __global__ __launch_bounds__(kThreads) void finish_h_kernel(
   for (int pidx = 0; pidx < nparts; ++pidx) a += partial[(bh * nparts + pidx) * stride + e];
   const float* kch = kc + bh * NT * K;
   const float* vch = vc + bh * NT * V;
-  float corr = 0.f;
-  for (int c = 0; c < NT; ++c) corr = fmaf(kch[(int64_t)c * K + dk], vch[(int64_t)c * V + dv], corr);
-  h[bh * E + e] = a - corr;
+  // four independent chains so that the loads of many chunks are in flight at once
+  float c0 = 0.f, c1 = 0.f, c2 = 0.f, c3 = 0.f;
+  int c = 0;
+#pragma unroll 2
+  for (; c + 4 <= NT; c += 4) {
+    c0 = fmaf(kch[(int64_t)c * K + dk], vch[(int64_t)c * V + dv], c0);
+    c1 = fmaf(kch[(int64_t)(c + 1) * K + dk], vch[(int64_t)(c + 1) * V + dv], c1);
+    c2 = fmaf(kch[(int64_t)(c + 2) * K + dk], vch[(int64_t)(c + 2) * V + dv], c2);
+    c3 = fmaf(kch[(int64_t)(c + 3) * K + dk], vch[(int64_t)(c + 3) * V + dv], c3);
+  }
+  for (; c < NT; ++c) c0 = fmaf(kch[(int64_t)c * K + dk], vch[(int64_t)c * V + dv], c0);
+  h[bh * E + e] = a - ((c0 + c1) + (c2 + c3));
 }
 
 // Per-chunk norm of hc_c = K_c^T V_c - kc_c vc_c^T (kernel.py:172-174); partial holds one
@@ -234,6 +293,13 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
     }
   };
 
+  // per-lane LDS offsets of the operand reads (everything else is a compile-time constant)
+  int koff[KST], voff[DG];
+#pragma unroll
+  for (int s = 0; s < KST; ++s) koff[s] = kswz(nq, 4 * s + kb);
+#pragma unroll
+  for (int dg = 0; dg < DG; ++dg) voff[dg] = vswz_dword(4 * kb, 16 * dg + nq);
+
   float m_i = kNegInf, l_p = 0.f, g_p = 0.f;  // running max; per-lane partial sums
   f32x4 acc[DG][2];
 #pragma unroll
@@ -244,17 +310,18 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
   // One 64-key block: scores against NKT key tiles (summed), masked, online softmax,
   // then acc += P (V tile 0 [+ V tile 1]).  valid(key) / weight(key) describe the block.
   auto attend = [&](const unsigned char* kt0, const unsigned char* kt1, const unsigned char* vt0,
-                    const unsigned char* vt1, auto valid, auto weight, bool weighted) {
+                    const unsigned char* vt1, auto valid, auto weight, bool weighted, bool all_valid) {
     f32x4 st[4];
 #pragma unroll
     for (int jb = 0; jb < 4; ++jb) {
       st[jb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < KST; ++s) {
-        const u32x4 ak = *reinterpret_cast<const u32x4*>(kt0 + kswz(16 * jb + nq, 4 * s + kb));
+        // row 16jb + nq: same swizzle as row nq (16jb is a multiple of 8)
+        const u32x4 ak = *reinterpret_cast<const u32x4*>(kt0 + koff[s] + jb * (16 * K * 2));
         st[jb] = Mma16<T>::run(ak, qop[s], st[jb]);
         if (kt1) {
-          const u32x4 al = *reinterpret_cast<const u32x4*>(kt1 + kswz(16 * jb + nq, 4 * s + kb));
+          const u32x4 al = *reinterpret_cast<const u32x4*>(kt1 + koff[s] + jb * (16 * K * 2));
           st[jb] = Mma16<T>::run(al, qop[s], st[jb]);
         }
       }
@@ -265,7 +332,7 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
     for (int jb = 0; jb < 4; ++jb)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float x = valid(16 * jb + 4 * kb + r) ? st[jb][r] * sm_scale : kNegInf;
+        const float x = (all_valid || valid(16 * jb + 4 * kb + r)) ? st[jb][r] * sm_scale : kNegInf;
         st[jb][r] = x;
         mx = fmaxf(mx, x);
       }
@@ -273,7 +340,7 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const float m_new = fmaxf(m_i, mx);
     const float m_safe = m_new == kNegInf ? 0.f : m_new;
-    const float alpha = exp2f(m_i - m_safe);
+    const float alpha = __builtin_amdgcn_exp2f(m_i - m_safe);
     m_i = m_new;
     float psum = 0.f, wsum = 0.f;
     uint32_t pw[8];
@@ -282,7 +349,7 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
       float pv[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        pv[r] = exp2f(st[jb][r] - m_safe);
+        pv[r] = __builtin_amdgcn_exp2f(st[jb][r] - m_safe);
         psum += pv[r];
         if (weighted) wsum = fmaf(pv[r], weight(16 * jb + 4 * kb + r), wsum);
       }
@@ -296,10 +363,12 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
       l_p = l_p * alpha + psum;
       g_p = g_p * alpha;
     }
+    if (__any(alpha != 1.f)) {  // the running maximum rarely moves after the first blocks
 #pragma unroll
-    for (int dg = 0; dg < DG; ++dg)
+      for (int dg = 0; dg < DG; ++dg)
 #pragma unroll
-      for (int par = 0; par < 2; ++par) acc[dg][par] *= alpha;
+        for (int par = 0; par < 2; ++par) acc[dg][par] *= alpha;
+    }
     // O^T += V^T P^T: k-step sp covers key sub-blocks 2sp, 2sp+1; slot i of lane kb is
     // key 32sp + 4kb + i (i < 4) or 32sp + 16 + 4kb + (i - 4)
 #pragma unroll
@@ -314,8 +383,9 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
           uint32_t w[8];
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
-            const int row = 32 * sp + 16 * (i >> 2) + 4 * kb + (i & 3);
-            w[i] = *reinterpret_cast<const uint32_t*>(vt + vswz_dword(row, 16 * dg + nq));
+            // row 32sp + 16(i/4) + 4kb + i%4: the swizzle bit (row/4)%2 equals kb%2 as in row 4kb
+            w[i] = *reinterpret_cast<const uint32_t*>(vt + voff[dg] +
+                                                      (32 * sp + 16 * (i >> 2) + (i & 3)) * (V * 2));
           }
           u32x4 ae, ao;
 #pragma unroll
@@ -332,10 +402,12 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
 
   // ---- phase 1: selected blocks, K/V tiles double-buffered ----
   u32x4 rk[KLD], rv[VLD];
+  // rows of block b that exist (0 for an index outside [0, NT): the block is skipped)
+  auto block_rows = [&](int b) { return b >= 0 && b < a.NT ? min(64, a.T - b * 64) : 0; };
   {
-    const int b0 = idx[0];
-    load_tile_k(rk, kbase, b0 * 64, a.T - b0 * 64);
-    load_tile_v(rv, vbase, b0 * 64, a.T - b0 * 64);
+    const int b0 = idx[0], n0 = block_rows(b0);
+    load_tile_k(rk, kbase, n0 ? b0 * 64 : 0, n0);
+    load_tile_v(rv, vbase, n0 ? b0 * 64 : 0, n0);
     store_tile_k(rk, smem);
     store_tile_v(rv, smem + LY::kKT);
   }
@@ -346,13 +418,13 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
     unsigned char* nxt = smem + ((i + 1) & 1) * LY::kSet;
     const bool more = i + 1 < a.NS;
     if (more) {
-      const int bn = idx[i + 1];
-      load_tile_k(rk, kbase, bn * 64, a.T - bn * 64);
-      load_tile_v(rv, vbase, bn * 64, a.T - bn * 64);
+      const int bn = idx[i + 1], nn = block_rows(bn);
+      load_tile_k(rk, kbase, nn ? bn * 64 : 0, nn);
+      load_tile_v(rv, vbase, nn ? bn * 64 : 0, nn);
     }
-    const int key0 = blk * 64;
-    attend(cur, nullptr, cur + LY::kKT, nullptr, [&](int key) { return key0 + key < a.T; },
-           [](int) { return 0.f; }, false);
+    const int nrows = block_rows(blk);
+    attend(cur, nullptr, cur + LY::kKT, nullptr, [&](int key) { return key < nrows; },
+           [](int) { return 0.f; }, false, nrows == 64);
     if (more) {
       store_tile_k(rk, nxt);
       store_tile_v(rv, nxt + LY::kKT);
@@ -383,7 +455,7 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
     const int c0 = grp * 64;
     attend(smem, smem + LY::kSet, smem + LY::kKT, smem + LY::kSet + LY::kKT,
            [&](int key) { return c0 + key < a.NT && !sel[c0 + key]; },
-           [&](int key) { return c0 + key == a.NT - 1 ? (float)last_len : 64.f; }, true);
+           [&](int key) { return c0 + key == a.NT - 1 ? (float)last_len : 64.f; }, true, false);
     __syncthreads();
   }
 
@@ -480,6 +552,17 @@ template <typename T>
 static void launch_sums(const void* q, const void* k, const void* v, float* qc, float* kc, float* vc,
                         int64_t BH, int Tn, int NT, int chunk, int K, int V, hipStream_t st) {
   const int64_t items = BH * NT * 3;
+  if constexpr (sizeof(T) == 2) {
+    const dim3 grid((unsigned)cdiv64(items, 4)), block(kThreads);
+    if (K == 64 && V == 64) {
+      chunk_sums16_kernel<T, 64><<<grid, block, 0, st>>>((const T*)q, (const T*)k, (const T*)v, qc, kc, vc, BH, Tn, NT, chunk);
+      return;
+    }
+    if (K == 128 && V == 128) {
+      chunk_sums16_kernel<T, 128><<<grid, block, 0, st>>>((const T*)q, (const T*)k, (const T*)v, qc, kc, vc, BH, Tn, NT, chunk);
+      return;
+    }
+  }
   chunk_sums_kernel<T><<<dim3((unsigned)cdiv64(items, 4)), dim3(kThreads), 0, st>>>(
       (const T*)q, (const T*)k, (const T*)v, qc, kc, vc, BH, Tn, NT, chunk, K, V);
 }

@@ -62,12 +62,17 @@ int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
   const int nchunks = (int)cdiv64(p.L, chunk);
   float* partial = (float*)a.workspace;
   const unsigned phases = phase_mask();
+  // one chunk per (sequence, head): the state kernel stores the finished S and km itself
+  const bool direct = fast && nchunks == 1;
   if (phases & kPhaseFwdState) {
-    if (fast) mfma::state(p, dtype, kn, a.v, a.k, partial, chunk, nchunks, st);
-    else generic::state_partial(p, dtype, kn, a.v, a.k, partial, chunk, nchunks, st);
+    if (fast)
+      mfma::state(p, dtype, kn, a.v, a.k, partial, chunk, nchunks, st, direct ? a.s : nullptr,
+                  direct ? a.km : nullptr);
+    else
+      generic::state_partial(p, dtype, kn, a.v, a.k, partial, chunk, nchunks, st);
   }
-  const bool fold = fast && fold_reduce(p, nchunks, p.DK, p.DV);
-  if (!fold && (phases & kPhaseFwdReduce))
+  const bool fold = fast && !direct && fold_reduce(p, nchunks, p.DK, p.DV);
+  if (!fold && !direct && (phases & kPhaseFwdReduce))
     generic::state_reduce(p, partial, chunk, nchunks, a.s, nullptr, a.km, st);
   if (phases & kPhaseFwdOutput) {
     if (fast) {
@@ -113,24 +118,30 @@ int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
   ws += vec_bytes(p);
   float* tokscal = (float*)ws;
   const unsigned phases = phase_mask();
+  const bool direct = fast && nchunks == 1;  // pass A stores the finished s*dS and dkm/L itself
+  float* fm = direct ? dS : nullptr;
+  float* fv = direct ? dkm : nullptr;
   if (phases & kPhaseBwdA) {
     if (mfma::bwd_a_supported(p, dtype)) {
-      int rc = mfma::bwd_a(p, dtype, qn, a.q, a.dout, a.s, a.km, dqn, dqd, partial, chunk, nchunks, st);
+      int rc = mfma::bwd_a(p, dtype, qn, a.q, a.dout, a.s, a.km, dqn, dqd, partial, chunk, nchunks, st,
+                           fm, fv);
       if (rc != kOk) return rc;
     } else if (fast) {
       // head dims above 64: token view and feature view as two kernels
       const int64_t rows = p.T * p.H;
       int rc = mfma::bwd_tokens(p, dtype, a.q, a.dout, a.s, a.km, a.dq, tokscal, rows, st);
       if (rc != kOk) return rc;
-      if (normalize) mfma::scaled_state(p, dtype, a.q, a.dout, tokscal, rows, partial, chunk, nchunks, st);
-      else mfma::state(p, dtype, a.q, a.dout, a.q, partial, chunk, nchunks, st);
+      if (normalize)
+        mfma::scaled_state(p, dtype, a.q, a.dout, tokscal, rows, partial, chunk, nchunks, st, fm, fv);
+      else
+        mfma::state(p, dtype, a.q, a.dout, a.q, partial, chunk, nchunks, st, fm, fv);
     } else {
       generic::transpose_state(p, a.s, St, st);
       generic::bwd_a(p, dtype, qn, a.q, a.dout, a.s, St, a.km, dqn, dqd, partial, chunk, nchunks, st);
     }
   }
-  const bool fold = fast && fold_reduce(p, nchunks, p.DV, p.DK);
-  if (!fold && (phases & kPhaseBwdReduce))
+  const bool fold = fast && !direct && fold_reduce(p, nchunks, p.DV, p.DK);
+  if (!fold && !direct && (phases & kPhaseBwdReduce))
     generic::state_reduce(p, partial, chunk, nchunks, dS, fast ? nullptr : dSt, dkm, st);
   if (phases & kPhaseBwdB) {
     if (fast) {

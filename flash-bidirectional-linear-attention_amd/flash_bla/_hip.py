@@ -9,7 +9,9 @@ import os
 
 import torch
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "libfbla_hip.so")
+# FBLA_LIB_PATH selects another build of the library (A/B comparisons of kernel changes).
+_LIB_PATH = os.environ.get("FBLA_LIB_PATH") or os.path.join(
+    os.path.dirname(os.path.abspath(__file__)), "_lib", "libfbla_hip.so")
 _lib = None
 
 F16, BF16, F32 = 0, 1, 2
