@@ -93,6 +93,27 @@ __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Packed sequences have different lengths, and workgroups are dispatched in index
+// order: handing out the longest sequences first (LPT) keeps the last round of
+// workgroups short.  Returns the index of the sequence with the `rank`-th largest
+// length (ties by index); the identity for dense problems, a single sequence, or
+// more sequences than the LDS table holds.  Called by all threads of the workgroup.
+constexpr int kLptMax = 1024;
+__device__ __forceinline__ int lpt_sequence(const Prob& p, int rank, int* lens /* [kLptMax + 1] */) {
+  if (!p.cu || p.N < 2 || p.N > kLptMax) return rank;
+  const int nthreads = blockDim.x;
+  for (int i = threadIdx.x; i < p.N; i += nthreads) lens[i] = p.cu[i + 1] - p.cu[i];
+  __syncthreads();
+  for (int j = threadIdx.x; j < p.N; j += nthreads) {
+    const int lj = lens[j];
+    int r = 0;
+    for (int i = 0; i < p.N; ++i) r += (lens[i] > lj) || (lens[i] == lj && i < j);
+    if (r == rank) lens[kLptMax] = j;
+  }
+  __syncthreads();
+  return lens[kLptMax];
+}
+
 // ===========================================================================
 // state kernel
 // ===========================================================================
@@ -228,8 +249,11 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
   constexpr int kAcc = CK * CV * 16;          // accumulator floats per lane
   __shared__ float red[64 * (kAcc + CK)];      // cross-wave reduction buffer, [value][lane]
 
-  const int nh = blockIdx.x / nchunks, c = blockIdx.x - nh * nchunks;
-  const int n = nh / p.H, h = nh - n * p.H;
+  __shared__ int lpt_lens[kLptMax + 1];
+  const int wg_nh = blockIdx.x / nchunks, c = blockIdx.x - wg_nh * nchunks;
+  const int h = wg_nh % p.H;
+  const int n = lpt_sequence(p, wg_nh / p.H, lpt_lens);
+  const int nh = n * p.H + h;
   int64_t bos, row0, rstride;
   int len;
   seq_range(p, n, bos, len);
@@ -351,7 +375,8 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
 
   // one chunk per (sequence, head): the sum is final, store it scaled where the reduce
   // kernel would have put it; otherwise store this chunk's partial
-  float* dst = fin_mat ? fin_mat + (int64_t)nh * DK * DV : partial + (int64_t)blockIdx.x * (DK * DV + DK);
+  float* dst = fin_mat ? fin_mat + (int64_t)nh * DK * DV
+                       : partial + ((int64_t)nh * nchunks + c) * (DK * DV + DK);
   float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * DK : nullptr) : dst + DK * DV;
   const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
   const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
@@ -479,7 +504,8 @@ template <int DR, int DC, bool DEN, int WAVES> struct RowsLayout {
   static constexpr int kKm = kStages + WAVES * (DEN ? 2 : 1) * kStage;
   static constexpr int kAdd = kKm + DR * 4;
   static constexpr int kMax = kAdd + DC * 4;
-  static constexpr int kTotal = kMax + 64;
+  static constexpr int kLpt = kMax + 64;
+  static constexpr int kTotal = kLpt + (kLptMax + 1) * 4;
 };
 
 // One launch can carry two independent jobs of the same shape (the dk and dv
@@ -503,8 +529,10 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
   float* lds_add = reinterpret_cast<float*>(smem + LY::kAdd);
   float* lds_max = reinterpret_cast<float*>(smem + LY::kMax);
 
-  const int nh = wg / nchunks, c = wg - nh * nchunks;
-  const int n = nh / p.H, h = nh - n * p.H;
+  const int wg_nh = wg / nchunks, c = wg - wg_nh * nchunks;
+  const int h = wg_nh % p.H;
+  const int n = lpt_sequence(p, wg_nh / p.H, reinterpret_cast<int*>(smem + LY::kLpt));
+  const int nh = n * p.H + h;
   int64_t bos, row0, rstride;
   int len;
   seq_range(p, n, bos, len);
@@ -699,7 +727,8 @@ template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struc
   static constexpr int kKmPairs = kOpnd + kWaves * kWave;
   static constexpr int kKmF = kKmPairs + DK * 4;
   static constexpr int kMax = kKmF + DK * 4;
-  static constexpr int kTotal = kMax + 64;
+  static constexpr int kLpt = kMax + 64;
+  static constexpr int kTotal = kLpt + (kLptMax + 1) * 4;
 };
 
 // FUSED = false runs the token view only (head dims whose dS accumulators do not
@@ -719,8 +748,10 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
   constexpr int QI = 32 * QCH / 64, GI = 32 * GCH / 64;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
-  const int nh = blockIdx.x / nchunks, c = blockIdx.x - nh * nchunks;
-  const int n = nh / p.H, h = nh - n * p.H;
+  const int wg_nh = blockIdx.x / nchunks, c = blockIdx.x - wg_nh * nchunks;
+  const int h = wg_nh % p.H;
+  const int n = lpt_sequence(p, wg_nh / p.H, reinterpret_cast<int*>(smem + LY::kLpt));
+  const int nh = n * p.H + h;
   int64_t bos, row0, rstride;
   int len;
   seq_range(p, n, bos, len);
@@ -986,7 +1017,8 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
   if constexpr (FUSED) {
     __syncthreads();  // every wave is done with its tiles: reuse them for the reduction
     float* red = reinterpret_cast<float*>(smem + LY::kOpnd);
-    float* dst = fin_mat ? fin_mat + (int64_t)nh * DK * DV : partial + (int64_t)blockIdx.x * (DK * DV + DK);
+    float* dst = fin_mat ? fin_mat + (int64_t)nh * DK * DV
+                         : partial + ((int64_t)nh * nchunks + c) * (DK * DV + DK);
     float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * DK : nullptr) : dst + DK * DV;
     const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
     const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
@@ -1059,7 +1091,11 @@ int bwd_a_chunk(const Prob& p) {
 // Row-parallel kernels: long enough chunks to amortise the operand prologue.
 int rows_chunk(const Prob& p, int DR, int DC) {
   static const int per_cu_knob = knob("FBLA_ROWS_WGS_PER_CU", 4);
-  static const int rounds = knob("FBLA_ROWS_ROUNDS", 4);
+  // dense: several rounds of short workgroups (page locality); packed: one workgroup per
+  // (sequence, head) where possible, handed out longest first, so fewer operand prologues
+  static const int dense_rounds = knob("FBLA_ROWS_ROUNDS", 4);
+  static const int packed_rounds = knob("FBLA_ROWS_ROUNDS_PACKED", 1);
+  const int rounds = p.cu ? packed_rounds : dense_rounds;
   const int big = (DR == 128) + (DC == 128);
   const int per_cu = big == 0 ? per_cu_knob : (big == 1 ? 2 : 1);
   return chunk_for(p, per_cu, rounds, 512, big == 2 ? 256 : 128);
