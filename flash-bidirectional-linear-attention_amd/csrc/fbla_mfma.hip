@@ -122,29 +122,42 @@ __device__ __forceinline__ int lpt_sequence(const Prob& p, int rank, int* lens /
 // column c: 8 tokens of one feature = 4 dwords.
 template <int C> struct RowWords { uint32_t w[8][C / 2]; };
 
+// Loads eight consecutive token rows of a 16-token tile: rows rel0 .. rel0+7 (rel0 = 0 for
+// the lower, 8 for the upper half-wave) relative to `tile`, the wave-uniform address of the
+// tile's first row; `step` = elements between consecutive token rows.  `full` (uniform) says
+// that all 16 rows of the tile exist; otherwise rows above `lim` (uniform, >= 0: the last
+// valid row relative to the tile) re-read row `lim` and the caller zeroes them.  Both forms
+// issue the same eight loads and no load sits behind a divergent branch, so the loads of the
+// next step stay in flight while the current one is multiplied.
 template <typename T, int C>
-__device__ __forceinline__ void load_rows(RowWords<C>& dst, const T* __restrict__ base,
-                                          int64_t row0, int64_t rstride, int D, int tok0, int t_end,
-                                          int p) {
-  const T* ptr0 = base + (row0 + (int64_t)tok0 * rstride) * D + C * p;
-  const int64_t step = rstride * D;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int tok = tok0 + j;
-    if (tok < t_end) {
-      const T* ptr = ptr0 + j * step;
-      if constexpr (C == 2) {
-        dst.w[j][0] = *reinterpret_cast<const uint32_t*>(ptr);
-      } else {
-        u32x2 x = *reinterpret_cast<const u32x2*>(ptr);
-        dst.w[j][0] = x[0];
-        dst.w[j][1] = x[1];
-      }
+__device__ __forceinline__ void load_rows(RowWords<C>& dst, const T* __restrict__ tile, uint32_t step,
+                                          int rel0, int lim, int p, bool full) {
+  auto get = [&](const T* base, uint32_t off, int j) {
+    if constexpr (C == 2) {
+      dst.w[j][0] = *reinterpret_cast<const uint32_t*>(base + off);
     } else {
-#pragma unroll
-      for (int c = 0; c < C / 2; ++c) dst.w[j][c] = 0u;
+      u32x2 x = *reinterpret_cast<const u32x2*>(base + off);
+      dst.w[j][0] = x[0];
+      dst.w[j][1] = x[1];
     }
+  };
+  if (full) {
+    const uint32_t off0 = (uint32_t)rel0 * step + (uint32_t)(C * p);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) get(tile + (size_t)j * step, off0, j);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) get(tile, (uint32_t)min(rel0 + j, lim) * step + (uint32_t)(C * p), j);
   }
+}
+
+// zeroes the rows at or past t_end
+template <int C>
+__device__ __forceinline__ void mask_rows(RowWords<C>& r, int tok0, int t_end) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int c = 0; c < C / 2; ++c) r.w[j][c] = tok0 + j < t_end ? r.w[j][c] : 0u;
 }
 
 // token-pair packing: operand c gets feature c of tokens (2i, 2i+1) in dword i
@@ -229,25 +242,98 @@ __device__ __forceinline__ void reduce_store_partial(f32x16 (&acc)[CK][CV], floa
   }
 }
 
+// The state kernel's form of the same reduction.  The DK x DV state is tiled into 64 x 64
+// blocks; a block is owned by G = 4 / (number of blocks) waves that take interleaved token
+// tiles (g = the wave's index inside its group).  The group's accumulators are summed in a
+// fixed order through the group's LDS buffer `red` (64 * 66 floats; unused for G = 1) and
+// wave g = 0 stores the block: dst points at the block's first element inside the [DK][DV]
+// matrix (leading dimension ld), dst_vec (optional) at the block's 64 entries of the vector.
+// Register r of accumulator (a,b) is row 2*m + a, column 2*pp + b with
+// m = 8*(r/4) + 4*kb + r%4.  Must be reached by all waves of the workgroup.
+template <int G>
+__device__ __forceinline__ void reduce_store_block(f32x16 (&acc)[2][2], float (&ks)[2], float* red,
+                                                   float* dst, int ld, float* dst_vec, float mscale,
+                                                   float vscale, int g, int lane) {
+  const int pp = lane & 31, kb = lane >> 5;
+  auto spill = [&]() {
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) red[((a * 2 + b) * 16 + r) * 64 + lane] = acc[a][b][r];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) red[(64 + a) * 64 + lane] = ks[a];
+  };
+  auto absorb = [&]() {
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] += red[((a * 2 + b) * 16 + r) * 64 + lane];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) ks[a] += red[(64 + a) * 64 + lane];
+  };
+  if constexpr (G == 4) {  // 2 -> 0, 3 -> 1, 1 -> 0
+    if (g == 2) spill();
+    __syncthreads();
+    if (g == 0) absorb();
+    __syncthreads();
+    if (g == 3) spill();
+    __syncthreads();
+    if (g == 1) absorb();
+    __syncthreads();
+    if (g == 1) spill();
+    __syncthreads();
+    if (g == 0) absorb();
+  } else if constexpr (G == 2) {
+    if (g == 1) spill();
+    __syncthreads();
+    if (g == 0) absorb();
+  }
+  if (g != 0) return;
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = 8 * (r >> 2) + 4 * kb + (r & 3);
+        dst[(2 * m + a) * ld + 2 * pp + b] = acc[a][b][r] * mscale;
+      }
+  if (dst_vec) {
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      const float tot = ks[a] + __shfl_xor(ks[a], 32);
+      if (kb == 0) dst_vec[2 * pp + a] = tot * vscale;
+    }
+  }
+}
+
 // SCALED = true is the feature view of the backward for head dims above 64:
 // kn = q~, v = dO, every dO row is multiplied by 1/z_t (tokscal[row]) and split
 // into hi + lo before the MFMA, and the vector part is dkm = sum_t dz_t q_t
 // (dz_t = tokscal[total_rows + row]).
+#ifndef FBLA_STATE128_TILES
+#define FBLA_STATE128_TILES 1
+#endif
 template <typename T, int DK, int DV, bool SPLIT_KD, int TILES, bool SCALED>
-__global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __restrict__ kn,
+__global__ __launch_bounds__(kThreads, 2) void state_kernel(Prob p, const T* __restrict__ kn,
                                                          const T* __restrict__ v,
                                                          const T* __restrict__ kd,
                                                          float* __restrict__ partial,
                                                          const float* __restrict__ tokscal,
                                                          int64_t total_rows, float* fin_mat,
                                                          float* fin_vec, int chunk, int nchunks) {
-  // 128 x 128 states are split by value columns over wave pairs (256 accumulator
-  // registers would not fit one wave): wave w owns columns [(w%NS)*DVW, +DVW).
-  constexpr int NS = (DK == 128 && DV == 128) ? 2 : 1;
-  constexpr int DVW = DV / NS, G = kWaves / NS;
-  constexpr int CK = DK / 32, CV = DVW / 32;
-  constexpr int kAcc = CK * CV * 16;          // accumulator floats per lane
-  __shared__ float red[64 * (kAcc + CK)];      // cross-wave reduction buffer, [value][lane]
+  // The state is tiled into 64 x 64 blocks (64 accumulator registers per lane); a block is
+  // owned by G waves that take interleaved token tiles.  For a 128 x 128 state the four
+  // waves of the workgroup therefore read the same tokens, each the 64 key and 64 value
+  // columns of its block: every row is fetched from HBM once and served to two waves by
+  // the cache.
+  constexpr int KB = DK / 64, VB = DV / 64, NB = KB * VB, G = kWaves / NB;
+  constexpr int CK = 2, CV = 2;
+  __shared__ float red[G > 1 ? NB * 64 * 66 : 1];  // per-group reduction buffers, [value][lane]
 
   __shared__ int lpt_lens[kLptMax + 1];
   const int wg_nh = blockIdx.x / nchunks, c = blockIdx.x - wg_nh * nchunks;
@@ -269,8 +355,12 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
   const int t_end = min(len, t_begin + chunk);
   row_base(p, n, h, bos, row0, rstride);
 
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int pp = lane & 31, kb = lane >> 5;
+  const int blk = wave / G, g = wave % G, bk = blk / VB, bv = blk % VB;
+  const T* kcol = kn + 64 * bk;
+  const T* vcol = v + 64 * bv;
+  const T* kdcol = kd + 64 * bk;
 
   f32x16 acc[CK][CV];
 #pragma unroll
@@ -283,44 +373,67 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
 #pragma unroll
   for (int a = 0; a < CK; ++a) ks[a] = 0.f;
 
-  // Each wave walks TILES consecutive 16-token tiles per step, the steps of the 4
-  // waves interleaved; the next step's rows are in flight while the current ones
-  // are multiplied.
+  // Each wave walks TILES consecutive 16-token tiles per step, the steps of the G waves
+  // interleaved.  Two register buffers alternate (the loop is unrolled by two so that no
+  // copy is needed): the loads of the next step are issued, unconditionally, before the
+  // current step is multiplied.
   constexpr int kStep = 16 * TILES;
-  const T* vcol = v + (wave % NS) * DVW;
-  int t0 = t_begin + kStep * (wave / NS);
-  RowWords<CK> kw[TILES], kw_n[TILES], kdw[TILES], kdw_n[TILES];
-  RowWords<CV> vw[TILES], vw_n[TILES];
-  auto fetch = [&](RowWords<CK>(&dk_)[TILES], RowWords<CV>(&dv_)[TILES], RowWords<CK>(&dd_)[TILES], int tok) {
+  struct Buf {
+    RowWords<CK> k[TILES];
+    RowWords<CV> v[TILES];
+    RowWords<CK> d[SPLIT_KD ? TILES : 1];
+    float rz[SCALED ? TILES : 1][8], dz[SCALED ? TILES : 1][8];
+  };
+  const uint32_t kstep = (uint32_t)(rstride * DK), vstep = (uint32_t)(rstride * DV);
+  auto fetch = [&](Buf& b, int tok) {
+    const bool full = tok + kStep <= t_end;
 #pragma unroll
     for (int u = 0; u < TILES; ++u) {
-      load_rows<T, CK>(dk_[u], kn, row0, rstride, DK, tok + 16 * u + 8 * kb, t_end, pp);
-      load_rows<T, CV>(dv_[u], vcol, row0, rstride, DV, tok + 16 * u + 8 * kb, t_end, pp);
-      if constexpr (SPLIT_KD) load_rows<T, CK>(dd_[u], kd, row0, rstride, DK, tok + 16 * u + 8 * kb, t_end, pp);
+      const int tc = min(tok + 16 * u, t_end - 1);  // first row of the tile, kept inside the chunk
+      const int lim = t_end - 1 - tc;
+      const int64_t row = row0 + (int64_t)tc * rstride;
+      load_rows<T, CK>(b.k[u], kcol + row * DK, kstep, 8 * kb, lim, pp, full);
+      load_rows<T, CV>(b.v[u], vcol + row * DV, vstep, 8 * kb, lim, pp, full);
+      if constexpr (SPLIT_KD) load_rows<T, CK>(b.d[u], kdcol + row * DK, kstep, 8 * kb, lim, pp, full);
+      if constexpr (SCALED) {
+        const float* ts = tokscal + row;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const uint32_t off = (uint32_t)min(8 * kb + j, lim) * (uint32_t)rstride;
+          b.rz[u][j] = ts[off];
+          b.dz[u][j] = ts[total_rows + off];
+        }
+      }
     }
   };
-  if (t0 < t_end) fetch(kw, vw, kdw, t0);
-  while (t0 < t_end) {
-    const int tn = t0 + kStep * G;
-    if (tn < t_end) fetch(kw_n, vw_n, kdw_n, tn);
+  auto compute = [&](Buf& b, int tok) {
+    if (tok + kStep > t_end) {  // last, partial step of the chunk
+#pragma unroll
+      for (int u = 0; u < TILES; ++u) {
+        const int tk = tok + 16 * u + 8 * kb;
+        mask_rows<CK>(b.k[u], tk, t_end);
+        if constexpr (SPLIT_KD) mask_rows<CK>(b.d[u], tk, t_end);
+        if constexpr (SCALED) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            b.rz[u][j] = tk + j < t_end ? b.rz[u][j] : 0.f;
+            b.dz[u][j] = tk + j < t_end ? b.dz[u][j] : 0.f;
+          }
+        }
+      }
+    }
 #pragma unroll
     for (int u = 0; u < TILES; ++u) {
       u32x4 A[CK], B[CV];
-      transpose_rows<CK>(kw[u], A);
+      transpose_rows<CK>(b.k[u], A);
       if constexpr (SCALED) {
         RowWords<CV> vh, vl;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const int tok = t0 + 16 * u + 8 * kb + j;
-          float rz = 0.f, dz = 0.f;
-          if (tok < t_end) {
-            const int64_t row = row0 + (int64_t)tok * rstride;
-            rz = tokscal[row];
-            dz = tokscal[total_rows + row];
-          }
+          const float rz = b.rz[u][j], dz = b.dz[u][j];
 #pragma unroll
           for (int c2 = 0; c2 < CV / 2; ++c2) {
-            const uint32_t w = vw[u].w[j][c2];
+            const uint32_t w = b.v[u].w[j][c2];
             const float x0 = Ops<T>::lo(w) * rz, x1 = Ops<T>::hi(w) * rz;
             const T h0 = (T)x0, h1 = (T)x1;
             vh.w[j][c2] = pack2<T>((float)h0, (float)h1);
@@ -328,7 +441,7 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
           }
 #pragma unroll
           for (int c2 = 0; c2 < CK / 2; ++c2) {
-            const uint32_t w = SPLIT_KD ? kdw[u].w[j][c2] : kw[u].w[j][c2];
+            const uint32_t w = SPLIT_KD ? b.d[u].w[j][c2] : b.k[u].w[j][c2];
             ks[2 * c2] = fmaf(dz, Ops<T>::lo(w), ks[2 * c2]);
             ks[2 * c2 + 1] = fmaf(dz, Ops<T>::hi(w), ks[2 * c2 + 1]);
           }
@@ -339,48 +452,57 @@ __global__ __launch_bounds__(kThreads) void state_kernel(Prob p, const T* __rest
 #pragma unroll
         for (int a = 0; a < CK; ++a)
 #pragma unroll
-          for (int b = 0; b < CV; ++b) {
-            acc[a][b] = Ops<T>::mma(A[a], B[b], acc[a][b]);
-            acc[a][b] = Ops<T>::mma(A[a], Bl[b], acc[a][b]);
+          for (int bb = 0; bb < CV; ++bb) {
+            acc[a][bb] = Ops<T>::mma(A[a], B[bb], acc[a][bb]);
+            acc[a][bb] = Ops<T>::mma(A[a], Bl[bb], acc[a][bb]);
           }
-        continue;
-      }
-      transpose_rows<CV>(vw[u], B);
-#pragma unroll
-      for (int a = 0; a < CK; ++a)
-#pragma unroll
-        for (int b = 0; b < CV; ++b) acc[a][b] = Ops<T>::mma(A[a], B[b], acc[a][b]);
-      if constexpr (SPLIT_KD) {
-        u32x4 D[CK];
-        transpose_rows<CK>(kdw[u], D);
-#pragma unroll
-        for (int a = 0; a < CK; ++a)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) ks[a] = Ops<T>::dot2(D[a][i], Ops<T>::kOnes, ks[a]);
       } else {
+        transpose_rows<CV>(b.v[u], B);
 #pragma unroll
         for (int a = 0; a < CK; ++a)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) ks[a] = Ops<T>::dot2(A[a][i], Ops<T>::kOnes, ks[a]);
+          for (int bb = 0; bb < CV; ++bb) acc[a][bb] = Ops<T>::mma(A[a], B[bb], acc[a][bb]);
+        if constexpr (SPLIT_KD) {
+          u32x4 Dd[CK];
+          transpose_rows<CK>(b.d[u], Dd);
+#pragma unroll
+          for (int a = 0; a < CK; ++a)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ks[a] = Ops<T>::dot2(Dd[a][i], Ops<T>::kOnes, ks[a]);
+        } else {
+#pragma unroll
+          for (int a = 0; a < CK; ++a)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ks[a] = Ops<T>::dot2(A[a][i], Ops<T>::kOnes, ks[a]);
+        }
       }
     }
-#pragma unroll
-    for (int u = 0; u < TILES; ++u) {
-      kw[u] = kw_n[u];
-      vw[u] = vw_n[u];
-      if constexpr (SPLIT_KD) kdw[u] = kdw_n[u];
+  };
+  int t0 = t_begin + kStep * g;
+  if (t0 < t_end) {
+    Buf b0, b1;
+    fetch(b0, t0);
+    while (true) {
+      fetch(b1, t0 + kStep * G);
+      compute(b0, t0);
+      t0 += kStep * G;
+      if (t0 >= t_end) break;
+      fetch(b0, t0 + kStep * G);
+      compute(b1, t0);
+      t0 += kStep * G;
+      if (t0 >= t_end) break;
     }
-    t0 = tn;
   }
 
   // one chunk per (sequence, head): the sum is final, store it scaled where the reduce
   // kernel would have put it; otherwise store this chunk's partial
-  float* dst = fin_mat ? fin_mat + (int64_t)nh * DK * DV
+  float* mat = fin_mat ? fin_mat + (int64_t)nh * DK * DV
                        : partial + ((int64_t)nh * nchunks + c) * (DK * DV + DK);
-  float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * DK : nullptr) : dst + DK * DV;
+  float* vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * DK : nullptr) : mat + DK * DV;
   const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
   const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
-  reduce_store_partial<CK, CV, NS>(acc, ks, red, dst, dst_vec, mscale, vscale, wave, lane);
+  reduce_store_block<G>(acc, ks, red + (G > 1 ? blk * 64 * 66 : 0), mat + (64 * bk) * DV + 64 * bv, DV,
+                        (vec && bv == 0) ? vec + 64 * bk : nullptr, mscale, vscale, g, lane);
 }
 
 // ===========================================================================
@@ -1106,12 +1228,13 @@ static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, fl
                          const float* tokscal, int64_t total_rows, float* fm, float* fv, int chunk,
                          int nchunks, hipStream_t st) {
   const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(kThreads);
+  constexpr int TL = (DK == 128 && DV == 128) ? FBLA_STATE128_TILES : 1;
   if (tokscal)
-    state_kernel<T, DK, DV, false, 1, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fm, fv, chunk, nchunks);
+    state_kernel<T, DK, DV, false, TL, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fm, fv, chunk, nchunks);
   else if (p.flags & kDecoupled)
-    state_kernel<T, DK, DV, true, 1, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks);
+    state_kernel<T, DK, DV, true, TL, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks);
   else
-    state_kernel<T, DK, DV, false, 1, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks);
+    state_kernel<T, DK, DV, false, TL, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks);
 }
 
 template <typename T>

@@ -100,33 +100,57 @@ __global__ __launch_bounds__(kThreads) void chunk_sums16_kernel(
   }
 }
 
-// H[bh][dk][dv] = sum_p partial_p[dk][dv] - sum_c n_c kc_c[dk] vc_c[dv] / n_c ... with
-// kc the MEAN and vc the SUM of a chunk the correction is simply kc_c[dk] * vc_c[dv].
+// H[bh][dk][dv] = sum_p partial_p[dk][dv] - sum_c kc_c[dk] * vc_c[dv]   (kc the MEAN and vc
+// the SUM of chunk c, so their product is the whole correction of that chunk).
+// One workgroup per (head, 32x32 tile of H); a thread owns a 2x2 patch.  The chunk
+// statistics go through LDS in slabs of 64 chunks (coalesced loads, every value is
+// then used 16 times from LDS); the chunk order of the sum is fixed.
+constexpr int kHTile = 32, kHSlab = 64;
 __global__ __launch_bounds__(kThreads) void finish_h_kernel(
     const float* __restrict__ partial, int nparts, const float* __restrict__ kc,
     const float* __restrict__ vc, float* __restrict__ h, int NT, int K, int V) {
-  const int E = K * V, stride = E + K;
-  const int blocks_per_head = (E + kThreads - 1) / kThreads;
-  const int64_t bh = blockIdx.x / blocks_per_head;
-  const int e = (blockIdx.x % blocks_per_head) * kThreads + threadIdx.x;
-  if (e >= E) return;
-  const int dk = e / V, dv = e - dk * V;
-  float a = 0.f;
-  for (int pidx = 0; pidx < nparts; ++pidx) a += partial[(bh * nparts + pidx) * stride + e];
+  __shared__ float ks[kHSlab][kHTile + 1];
+  __shared__ float vs[kHSlab][kHTile + 1];
+  const int tk = (K + kHTile - 1) / kHTile, tv = (V + kHTile - 1) / kHTile;
+  const int tile = blockIdx.x % (tk * tv);
+  const int64_t bh = blockIdx.x / (tk * tv);
+  const int dk0 = (tile / tv) * kHTile, dv0 = (tile % tv) * kHTile;
+  const int ty = threadIdx.x / 16, tx = threadIdx.x % 16;  // patch rows 2ty.., cols tx, tx+16
   const float* kch = kc + bh * NT * K;
   const float* vch = vc + bh * NT * V;
-  // four independent chains so that the loads of many chunks are in flight at once
-  float c0 = 0.f, c1 = 0.f, c2 = 0.f, c3 = 0.f;
-  int c = 0;
-#pragma unroll 2
-  for (; c + 4 <= NT; c += 4) {
-    c0 = fmaf(kch[(int64_t)c * K + dk], vch[(int64_t)c * V + dv], c0);
-    c1 = fmaf(kch[(int64_t)(c + 1) * K + dk], vch[(int64_t)(c + 1) * V + dv], c1);
-    c2 = fmaf(kch[(int64_t)(c + 2) * K + dk], vch[(int64_t)(c + 2) * V + dv], c2);
-    c3 = fmaf(kch[(int64_t)(c + 3) * K + dk], vch[(int64_t)(c + 3) * V + dv], c3);
+  float c00 = 0.f, c01 = 0.f, c10 = 0.f, c11 = 0.f;
+  for (int cb = 0; cb < NT; cb += kHSlab) {
+    const int nc = min(kHSlab, NT - cb);
+    __syncthreads();
+    for (int i = threadIdx.x; i < kHSlab * kHTile; i += kThreads) {
+      const int c = i / kHTile, d = i % kHTile;
+      ks[c][d] = (c < nc && dk0 + d < K) ? kch[(int64_t)(cb + c) * K + dk0 + d] : 0.f;
+      vs[c][d] = (c < nc && dv0 + d < V) ? vch[(int64_t)(cb + c) * V + dv0 + d] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int c = 0; c < kHSlab; ++c) {
+      const float k0 = ks[c][2 * ty], k1 = ks[c][2 * ty + 1];
+      const float v0 = vs[c][tx], v1 = vs[c][tx + 16];
+      c00 = fmaf(k0, v0, c00);
+      c01 = fmaf(k0, v1, c01);
+      c10 = fmaf(k1, v0, c10);
+      c11 = fmaf(k1, v1, c11);
+    }
   }
-  for (; c < NT; ++c) c0 = fmaf(kch[(int64_t)c * K + dk], vch[(int64_t)c * V + dv], c0);
-  h[bh * E + e] = a - ((c0 + c1) + (c2 + c3));
+  const int E = K * V, stride = E + K;
+  const float corr[2][2] = {{c00, c01}, {c10, c11}};
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int dk = dk0 + 2 * ty + i, dv = dv0 + tx + 16 * j;
+      if (dk >= K || dv >= V) continue;
+      const int e = dk * V + dv;
+      float a = 0.f;
+      for (int pidx = 0; pidx < nparts; ++pidx) a += partial[(bh * nparts + pidx) * stride + e];
+      h[bh * E + e] = a - corr[i][j];
+    }
 }
 
 // Per-chunk norm of hc_c = K_c^T V_c - kc_c vc_c^T (kernel.py:172-174); partial holds one
@@ -584,8 +608,8 @@ int chunk_reduce(const void* q, const void* k, const void* v, float* qc, float* 
   if (per_chunk)
     chunk_norm_kernel<<<dim3((unsigned)(BH * NT)), dim3(kThreads), 0, st>>>(partial, kc, vc, h_norm, K,
                                                                           V, pnorm);
-  const int blocks_per_head = (K * V + kThreads - 1) / kThreads;
-  finish_h_kernel<<<dim3((unsigned)(BH * blocks_per_head)), dim3(kThreads), 0, st>>>(
+  const int tiles_per_head = (int)(cdiv64(K, kHTile) * cdiv64(V, kHTile));
+  finish_h_kernel<<<dim3((unsigned)(BH * tiles_per_head)), dim3(kThreads), 0, st>>>(
       partial, nparts, kc, vc, h, NT, K, V);
   return kOk;
 }
