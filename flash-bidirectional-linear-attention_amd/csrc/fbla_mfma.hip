@@ -111,7 +111,7 @@ __device__ __forceinline__ int lpt_sequence(const Prob& p, int rank, int* lens /
     if (r == rank) lens[kLptMax] = j;
   }
   __syncthreads();
-  return lens[kLptMax];
+  return __builtin_amdgcn_readfirstlane(lens[kLptMax]);  // the same for all lanes: keep it scalar
 }
 
 // ===========================================================================
@@ -122,42 +122,55 @@ __device__ __forceinline__ int lpt_sequence(const Prob& p, int rank, int* lens /
 // column c: 8 tokens of one feature = 4 dwords.
 template <int C> struct RowWords { uint32_t w[8][C / 2]; };
 
-// Loads eight consecutive token rows of a 16-token tile: rows rel0 .. rel0+7 (rel0 = 0 for
-// the lower, 8 for the upper half-wave) relative to `tile`, the wave-uniform address of the
-// tile's first row; `step` = elements between consecutive token rows.  `full` (uniform) says
-// that all 16 rows of the tile exist; otherwise rows above `lim` (uniform, >= 0: the last
-// valid row relative to the tile) re-read row `lim` and the caller zeroes them.  Both forms
-// issue the same eight loads and no load sits behind a divergent branch, so the loads of the
-// next step stay in flight while the current one is multiplied.
+// Loads eight consecutive token rows of a 16-token tile.  `tile` is the wave-uniform address
+// of the tile's first row, `step` the elements between consecutive token rows and `voff` the
+// lane's constant offset (its half-wave's first row, 0 or 8, times step, plus its feature
+// column).  No branch, no per-row address arithmetic in vector registers: the loads of the
+// next step can stay in flight while the current one is multiplied.
 template <typename T, int C>
 __device__ __forceinline__ void load_rows(RowWords<C>& dst, const T* __restrict__ tile, uint32_t step,
-                                          int rel0, int lim, int p, bool full) {
-  auto get = [&](const T* base, uint32_t off, int j) {
+                                          uint32_t voff) {
+  // byte arithmetic in 32 bits on top of a uniform 64-bit base: the scalar-base + vector-offset
+  // addressing form, one shared offset register for all eight rows
+  const char* base = reinterpret_cast<const char*>(tile);
+  const uint32_t step_b = step * (uint32_t)sizeof(T), voff_b = voff * (uint32_t)sizeof(T);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const char* row = base + (size_t)((uint32_t)j * step_b);
     if constexpr (C == 2) {
-      dst.w[j][0] = *reinterpret_cast<const uint32_t*>(base + off);
+      dst.w[j][0] = *reinterpret_cast<const uint32_t*>(row + voff_b);
     } else {
-      u32x2 x = *reinterpret_cast<const u32x2*>(base + off);
+      u32x2 x = *reinterpret_cast<const u32x2*>(row + voff_b);
       dst.w[j][0] = x[0];
       dst.w[j][1] = x[1];
     }
-  };
-  if (full) {
-    const uint32_t off0 = (uint32_t)rel0 * step + (uint32_t)(C * p);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) get(tile + (size_t)j * step, off0, j);
-  } else {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) get(tile, (uint32_t)min(rel0 + j, lim) * step + (uint32_t)(C * p), j);
   }
 }
 
-// zeroes the rows at or past t_end
+// The same with a bounds check per row, for chunks shorter than one tile: rows at or past
+// `rows` (relative to the tile) are not read and come back as zero.
+template <typename T, int C>
+__device__ __forceinline__ void load_rows_checked(RowWords<C>& dst, const T* __restrict__ tile,
+                                                  uint32_t step, int rel0, int p, int rows) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+#pragma unroll
+    for (int c = 0; c < C / 2; ++c) dst.w[j][c] = 0u;
+    if (rel0 + j < rows) {
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(tile + (size_t)(rel0 + j) * step + C * p);
+#pragma unroll
+      for (int c = 0; c < C / 2; ++c) dst.w[j][c] = src[c];
+    }
+  }
+}
+
+// zeroes the rows below `lo` (relative to the tile; rel0 = the lane's first row, 0 or 8)
 template <int C>
-__device__ __forceinline__ void mask_rows(RowWords<C>& r, int tok0, int t_end) {
+__device__ __forceinline__ void mask_rows(RowWords<C>& r, int rel0, int lo) {
 #pragma unroll
   for (int j = 0; j < 8; ++j)
 #pragma unroll
-    for (int c = 0; c < C / 2; ++c) r.w[j][c] = tok0 + j < t_end ? r.w[j][c] : 0u;
+    for (int c = 0; c < C / 2; ++c) r.w[j][c] = rel0 + j >= lo ? r.w[j][c] : 0u;
 }
 
 // token-pair packing: operand c gets feature c of tokens (2i, 2i+1) in dword i
@@ -319,7 +332,7 @@ __device__ __forceinline__ void reduce_store_block(f32x16 (&acc)[2][2], float (&
 #define FBLA_STATE128_TILES 1
 #endif
 template <typename T, int DK, int DV, bool SPLIT_KD, int TILES, bool SCALED>
-__global__ __launch_bounds__(kThreads, 2) void state_kernel(Prob p, const T* __restrict__ kn,
+__global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2) void state_kernel(Prob p, const T* __restrict__ kn,
                                                          const T* __restrict__ v,
                                                          const T* __restrict__ kd,
                                                          float* __restrict__ partial,
@@ -384,40 +397,62 @@ __global__ __launch_bounds__(kThreads, 2) void state_kernel(Prob p, const T* __r
     RowWords<CK> d[SPLIT_KD ? TILES : 1];
     float rz[SCALED ? TILES : 1][8], dz[SCALED ? TILES : 1][8];
   };
+  // A tile that would cross the end of the chunk is moved back so that it ends there; its
+  // first `lo` rows were already part of the previous tile and are zeroed before use.  Every
+  // tile therefore reads 16 valid rows with the same address pattern (chunks shorter than
+  // one tile take the checked path below).
   const uint32_t kstep = (uint32_t)(rstride * DK), vstep = (uint32_t)(rstride * DV);
+  const uint32_t kvoff = (uint32_t)(8 * kb) * kstep + (uint32_t)(CK * pp);
+  const uint32_t vvoff = (uint32_t)(8 * kb) * vstep + (uint32_t)(CV * pp);
+  const uint32_t tvoff = (uint32_t)(8 * kb) * (uint32_t)rstride;
   auto fetch = [&](Buf& b, int tok) {
-    const bool full = tok + kStep <= t_end;
 #pragma unroll
     for (int u = 0; u < TILES; ++u) {
-      const int tc = min(tok + 16 * u, t_end - 1);  // first row of the tile, kept inside the chunk
-      const int lim = t_end - 1 - tc;
-      const int64_t row = row0 + (int64_t)tc * rstride;
-      load_rows<T, CK>(b.k[u], kcol + row * DK, kstep, 8 * kb, lim, pp, full);
-      load_rows<T, CV>(b.v[u], vcol + row * DV, vstep, 8 * kb, lim, pp, full);
-      if constexpr (SPLIT_KD) load_rows<T, CK>(b.d[u], kdcol + row * DK, kstep, 8 * kb, lim, pp, full);
+      const int tb = min(tok + 16 * u, t_end - 16);
+      const int64_t row = row0 + (int64_t)tb * rstride;
+      load_rows<T, CK>(b.k[u], kcol + row * DK, kstep, kvoff);
+      load_rows<T, CV>(b.v[u], vcol + row * DV, vstep, vvoff);
+      if constexpr (SPLIT_KD) load_rows<T, CK>(b.d[u], kdcol + row * DK, kstep, kvoff);
       if constexpr (SCALED) {
         const float* ts = tokscal + row;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const uint32_t off = (uint32_t)min(8 * kb + j, lim) * (uint32_t)rstride;
-          b.rz[u][j] = ts[off];
-          b.dz[u][j] = ts[total_rows + off];
+          b.rz[u][j] = ts[tvoff + (uint32_t)j * (uint32_t)rstride];
+          b.dz[u][j] = ts[total_rows + tvoff + (uint32_t)j * (uint32_t)rstride];
         }
       }
     }
   };
-  auto compute = [&](Buf& b, int tok) {
-    if (tok + kStep > t_end) {  // last, partial step of the chunk
+  auto fetch_checked = [&](Buf& b, int tok) {  // chunk shorter than a tile
+#pragma unroll
+    for (int u = 0; u < TILES; ++u) {
+      const int rows = t_end - (tok + 16 * u);
+      const int64_t row = row0 + (int64_t)(tok + 16 * u) * rstride;
+      load_rows_checked<T, CK>(b.k[u], kcol + row * DK, kstep, 8 * kb, pp, rows);
+      load_rows_checked<T, CV>(b.v[u], vcol + row * DV, vstep, 8 * kb, pp, rows);
+      if constexpr (SPLIT_KD) load_rows_checked<T, CK>(b.d[u], kdcol + row * DK, kstep, 8 * kb, pp, rows);
+      if constexpr (SCALED) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const bool ok = 8 * kb + j < rows;
+          b.rz[u][j] = ok ? tokscal[row + (8 * kb + j) * rstride] : 0.f;
+          b.dz[u][j] = ok ? tokscal[total_rows + row + (8 * kb + j) * rstride] : 0.f;
+        }
+      }
+    }
+  };
+  auto compute = [&](Buf& b, int tok, bool checked) {
+    if (!checked && tok + kStep > t_end) {  // last step of the chunk: some tiles were moved back
 #pragma unroll
       for (int u = 0; u < TILES; ++u) {
-        const int tk = tok + 16 * u + 8 * kb;
-        mask_rows<CK>(b.k[u], tk, t_end);
-        if constexpr (SPLIT_KD) mask_rows<CK>(b.d[u], tk, t_end);
+        const int lo = min(16, tok + 16 * u - min(tok + 16 * u, t_end - 16));
+        mask_rows<CK>(b.k[u], 8 * kb, lo);
+        if constexpr (SPLIT_KD) mask_rows<CK>(b.d[u], 8 * kb, lo);
         if constexpr (SCALED) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
-            b.rz[u][j] = tk + j < t_end ? b.rz[u][j] : 0.f;
-            b.dz[u][j] = tk + j < t_end ? b.dz[u][j] : 0.f;
+            b.rz[u][j] = 8 * kb + j >= lo ? b.rz[u][j] : 0.f;
+            b.dz[u][j] = 8 * kb + j >= lo ? b.dz[u][j] : 0.f;
           }
         }
       }
@@ -479,16 +514,22 @@ __global__ __launch_bounds__(kThreads, 2) void state_kernel(Prob p, const T* __r
     }
   };
   int t0 = t_begin + kStep * g;
-  if (t0 < t_end) {
+  if (t_end - t_begin < 16) {
+    if (t0 < t_end) {
+      Buf b0;
+      fetch_checked(b0, t0);
+      compute(b0, t0, true);
+    }
+  } else if (t0 < t_end) {
     Buf b0, b1;
     fetch(b0, t0);
     while (true) {
       fetch(b1, t0 + kStep * G);
-      compute(b0, t0);
+      compute(b0, t0, false);
       t0 += kStep * G;
       if (t0 >= t_end) break;
       fetch(b0, t0 + kStep * G);
-      compute(b1, t0);
+      compute(b1, t0, false);
       t0 += kStep * G;
       if (t0 >= t_end) break;
     }
@@ -1217,8 +1258,9 @@ int rows_chunk(const Prob& p, int DR, int DC) {
   // (sequence, head) where possible, handed out longest first, so fewer operand prologues
   static const int dense_rounds = knob("FBLA_ROWS_ROUNDS", 4);
   static const int packed_rounds = knob("FBLA_ROWS_ROUNDS_PACKED", 1);
-  const int rounds = p.cu ? packed_rounds : dense_rounds;
+  // a 128 x 128 operand costs as much to build as 512 tokens cost to stream: one round there
   const int big = (DR == 128) + (DC == 128);
+  const int rounds = p.cu ? packed_rounds : (big == 2 ? 1 : big == 1 ? (dense_rounds + 1) / 2 : dense_rounds);
   const int per_cu = big == 0 ? per_cu_knob : (big == 1 ? 2 : 1);
   return chunk_for(p, per_cu, rounds, 512, big == 2 ? 256 : 128);
 }
