@@ -177,6 +177,8 @@ def main():
     ap.add_argument("--probe", type=int, default=0, metavar="N",
                     help="counter-collection mode for rocprofv3 --pmc: run N steps of the workload, each "
                          "followed by a 256 MiB device copy of known traffic, then exit")
+    ap.add_argument("--tables", action="store_true",
+                    help="also print the reference's benchmark tables (torch formula, this library, SDPA) on stderr")
     ap.add_argument("--configs", action="store_true",
                     help="also time the other operator families / BASELINE configs (table on stderr)")
     args = ap.parse_args()
@@ -277,7 +279,10 @@ def main():
         sweep(dtype, dev, flush)
     if args.configs:
         other_configs(dev, flush)
+        layer_config(dev, flush)
         piecewise_config(dev, flush)
+    if args.tables:
+        reference_tables(dev, flush)
     print(json.dumps(line), flush=True)
 
 
@@ -389,6 +394,79 @@ def other_configs(dev, flush):
                 return varlen_linear_attention(q, k, v, cu, max_len)
         _report(f"C3 varlen 64 seqs U[256,2048] H16 D{D} bf16", 4 * nb, 11 * nb, fwd, step, flush,
                 {"total_tokens": total, "max_seqlen": max_len})
+
+
+def layer_config(dev, flush):
+    """BASELINE config 4: the LinFusion attention block, forward only, fp16, random-init weights:
+    B2 with (L4096, C640, 10 heads x 64) and (L1024, C1280, 20 heads x 64).  Reports the whole
+    layer with the HIP operator ('triton' mode name kept from the reference), the whole layer
+    with the torch formula, and the operator alone."""
+    from flash_bla.layers.linfusion import GeneralizedLinearAttention
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    for L, C, heads in ((4096, 640, 10), (1024, 1280, 20)):
+        torch.manual_seed(42)
+        layer = GeneralizedLinearAttention(query_dim=C, heads=heads, dim_head=64).to(dev).half().eval()
+        x = torch.randn(2, L, C, generator=torch.Generator().manual_seed(42)).half().to(dev)
+        q = (F.elu(torch.randn(2, heads, L, 64, device=dev)) + 1).half()
+        k = (F.elu(torch.randn(2, heads, L, 64, device=dev)) + 1).half()
+        v = torch.randn(2, heads, L, 64, device=dev).half()
+        with torch.no_grad():
+            t_fast = do_bench(lambda: layer(x, mode="triton"), flush)
+            t_torch = do_bench(lambda: layer(x, mode="torch"), flush)
+            t_op = do_bench(lambda: linear_attention(q, k, v, eps=1e-4), flush)
+            err = (layer(x, mode="triton").float() - layer(x, mode="torch").float()).abs().max().item()
+            ref = layer(x, mode="torch").float().abs().max().item()
+        nb = 4 * q.numel() * 2
+        print(json.dumps({"config": f"C4 LinFusion layer fwd B2-L{L}-C{C}-{heads}x64 fp16",
+                          "layer_ms": round(t_fast[0], 5), "layer_torch_mode_ms": round(t_torch[0], 5),
+                          "op_ms": round(t_op[0], 5), "op_gbps": round(nb / t_op[0] / 1e6, 1),
+                          "modes_max_abs_diff_over_max": round(err / ref, 6)}), file=sys.stderr, flush=True)
+
+
+def reference_tables(dev, flush):
+    """The tables of the reference's benchmark scripts, with the torch formula and torch's
+    scaled_dot_product_attention beside the HIP operators (benchmarks/ops/benchmark_linear_attn.py:
+    B8-H16-D64 fp16 over T; benchmark_varlen_linear_attn.py:20-52: 8 sequences, padded batch
+    against the packed operator at max_seqlen 256/1024/4096)."""
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    from flash_bla.ops.linear_attn.naive import naive_linear_attn
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    for T in (1024, 4096, 16384):
+        q, k, v, do = make_inputs(8, 16, T, 64, torch.float16, dev)
+        for t in (q, k, v):
+            t.requires_grad_()
+
+        def bwd_of(fn):
+            def step():
+                q.grad = k.grad = v.grad = None
+                fn().backward(do)
+            return step
+        row = {"table": "linear_attn B8-H16-D64 fp16", "T": T}
+        for name, fn in (("torch_la", lambda: naive_linear_attn(q, k, v)),
+                         ("flash_bla", lambda: linear_attention(q, k, v)),
+                         ("torch_sdpa", lambda: F.scaled_dot_product_attention(q, k, v))):
+            with torch.no_grad():
+                row[name + "_fwd_ms"] = round(do_bench(fn, flush)[0], 4)
+            row[name + "_fwd_bwd_ms"] = round(do_bench(bwd_of(fn), flush)[0], 4)
+        print(json.dumps(row), file=sys.stderr, flush=True)
+    g = torch.Generator().manual_seed(42)
+    for max_len in (256, 1024, 4096):
+        lengths = torch.randint(max_len // 4, max_len + 1, (8,), generator=g)
+        lengths[0] = max_len
+        cu = torch.cat([torch.zeros(1, dtype=torch.int32), torch.cumsum(lengths, 0).to(torch.int32)]).to(dev)
+        total = int(lengths.sum())
+        qp = (F.elu(torch.randn(total, 16, 64, device=dev)) + 1).half()
+        kp = (F.elu(torch.randn(total, 16, 64, device=dev)) + 1).half()
+        vp = torch.randn(total, 16, 64, device=dev).half()
+        qd = (F.elu(torch.randn(8, 16, max_len, 64, device=dev)) + 1).half()
+        kd = (F.elu(torch.randn(8, 16, max_len, 64, device=dev)) + 1).half()
+        vd = torch.randn(8, 16, max_len, 64, device=dev).half()
+        with torch.no_grad():
+            t_pad = do_bench(lambda: linear_attention(qd, kd, vd), flush)[0]
+            t_var = do_bench(lambda: varlen_linear_attention(qp, kp, vp, cu, max_len), flush)[0]
+        print(json.dumps({"table": "varlen 8 seqs H16 D64 fp16 fwd", "max_seqlen": max_len, "total_tokens": total,
+                          "padded_dense_ms": round(t_pad, 4), "varlen_ms": round(t_var, 4)}),
+              file=sys.stderr, flush=True)
 
 
 def piecewise_config(dev, flush):

@@ -1,0 +1,119 @@
+"""Properties of the C-ABI boundary itself: work goes to the caller's stream and nowhere
+else, nothing synchronises or allocates behind the caller's back (so the entry points can be
+captured into a HIP graph), and the entry points are re-entrant across host threads."""
+import threading
+
+import pytest
+import torch
+
+from helpers import make_qkv
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    from flash_bla import _hip
+    return _hip
+
+
+def _step(hip, q, k, v, do, scale):
+    o, s, km = hip.la_fwd(q, k, v, None, None, scale, 1e-6, hip.NORMALIZE)
+    dq, dk, dv, _, _ = hip.la_bwd(q, k, v, None, None, do, s, km, scale, 1e-6, hip.NORMALIZE)
+    return o, dq, dk, dv
+
+
+@pytest.mark.parametrize("shape", [(2, 4, 1024, 64), (1, 2, 700, 128)])
+def test_graph_capture_replays_match_eager(shape):
+    """Forward + backward captured once, replayed four times on fresh inputs with eager work
+    and synchronisations in between; every replay must equal the eager result bit for bit
+    (the reductions are fixed-order)."""
+    hip = _ops()
+    dev = torch.device("cuda")
+    B, H, L, D = shape
+    scale = 1.0 / L
+    static = [t.to(dev) for t in make_qkv(shape, shape, torch.float16, seed=1)[:4]]
+    _step(hip, *static, scale)  # warm-up outside the capture (module load, LDS attributes)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = _step(hip, *static, scale)
+    for seed in (2, 3, 4, 5):
+        fresh = [t.to(dev) for t in make_qkv(shape, shape, torch.float16, seed=seed)[:4]]
+        eager = [t.clone() for t in _step(hip, *fresh, scale)]
+        torch.cuda.synchronize()
+        for dst, src in zip(static, fresh):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("o", "dq", "dk", "dv"), outs, eager):
+            assert torch.equal(a, b), f"replay with seed {seed}: {name} differs from the eager result"
+
+
+def test_side_stream_only():
+    """Launched on a side stream while the default stream is busy: the result is complete once
+    that side stream is synchronised, and equals the default-stream result."""
+    hip = _ops()
+    dev = torch.device("cuda")
+    shape = (2, 4, 2048, 64)
+    q, k, v, do = (t.to(dev) for t in make_qkv(shape, shape, torch.bfloat16, seed=9)[:4])
+    ref = [t.clone() for t in _step(hip, q, k, v, do, 1.0 / 2048)]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    busy = torch.empty(64 << 20, dtype=torch.float32, device=dev)
+    for _ in range(8):
+        busy.normal_()  # keeps the default stream occupied
+    with torch.cuda.stream(side):
+        got = _step(hip, q, k, v, do, 1.0 / 2048)
+    side.synchronize()
+    for a, b in zip(got, ref):
+        assert torch.equal(a, b)
+    torch.cuda.synchronize()
+
+
+def test_two_host_threads():
+    """Two host threads, each with its own stream and problem, call the entry points at the
+    same time (error text and profiling mask are per thread; there is no other mutable state)."""
+    hip = _ops()
+    dev = torch.device("cuda")
+    shapes = [(2, 4, 1536, 64), (1, 8, 1000, 64)]
+    inputs = [[t.to(dev) for t in make_qkv(s, s, torch.float16, seed=20 + i)[:4]] for i, s in enumerate(shapes)]
+    refs = [[t.clone() for t in _step(hip, *inp, 1.0 / s[2])] for inp, s in zip(inputs, shapes)]
+    torch.cuda.synchronize()
+    results, errors = [None, None], []
+
+    def work(i):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    out = _step(hip, *inputs[i], 1.0 / shapes[i][2])
+            stream.synchronize()
+            results[i] = out
+        except Exception as exc:  # surfaced below: an exception in a thread would otherwise be lost
+            errors.append(exc)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for got, ref in zip(results, refs):
+        for a, b in zip(got, ref):
+            assert torch.equal(a, b)
+
+
+def test_error_is_per_thread_and_does_not_poison():
+    """A rejected call reports through the return code / last-error text and leaves the library
+    usable: the next valid call succeeds."""
+    hip = _ops()
+    dev = torch.device("cuda")
+    L = hip.lib()
+    rc = L.fbla_la_fwd(None, None, None, None, None, None, None, None, None, 0, 1, 1, 16, 64, 64, 0, 1,
+                       1.0, 1e-6, None)
+    assert rc < 0
+    assert L.fbla_last_error().decode() != ""
+    shape = (1, 2, 256, 64)
+    q, k, v, do = (t.to(dev) for t in make_qkv(shape, shape, torch.float16, seed=3)[:4])
+    o, *_ = _step(hip, q, k, v, do, 1.0 / 256)
+    assert torch.isfinite(o).all()
