@@ -10,6 +10,7 @@
 // materialised unless the optional bias (per-chunk norm of (K_c - kc_c)^T V_c)
 // is requested.
 #include <algorithm>
+#include <type_traits>
 
 #include "fbla_kernels.h"
 
@@ -139,18 +140,43 @@ __global__ __launch_bounds__(kThreads) void finish_h_kernel(
     }
   }
   const int E = K * V, stride = E + K;
+  // the four partial sums advance together, four partials per trip: sixteen independent
+  // loads in flight instead of one (the order of each sum stays p = 0, 1, 2, ...)
+  const int dk_a = dk0 + 2 * ty, dv_a = dv0 + tx;
+  const bool ok[2][2] = {{dk_a < K && dv_a < V, dk_a < K && dv_a + 16 < V},
+                         {dk_a + 1 < K && dv_a < V, dk_a + 1 < K && dv_a + 16 < V}};
+  const int e00 = dk_a * V + dv_a;
+  const int eo[2][2] = {{ok[0][0] ? e00 : 0, ok[0][1] ? e00 + 16 : 0},
+                        {ok[1][0] ? e00 + V : 0, ok[1][1] ? e00 + V + 16 : 0}};
+  const float* pb = partial + bh * nparts * stride;
+  float a[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+  int pidx = 0;
+  for (; pidx + 4 <= nparts; pidx += 4) {
+    float x[4][2][2];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) x[u][i][j] = pb[(int64_t)(pidx + u) * stride + eo[i][j]];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) a[i][j] += x[u][i][j];
+  }
+  for (; pidx < nparts; ++pidx)
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) a[i][j] += pb[(int64_t)pidx * stride + eo[i][j]];
   const float corr[2][2] = {{c00, c01}, {c10, c11}};
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int dk = dk0 + 2 * ty + i, dv = dv0 + tx + 16 * j;
-      if (dk >= K || dv >= V) continue;
-      const int e = dk * V + dv;
-      float a = 0.f;
-      for (int pidx = 0; pidx < nparts; ++pidx) a += partial[(bh * nparts + pidx) * stride + e];
-      h[bh * E + e] = a - corr[i][j];
-    }
+    for (int j = 0; j < 2; ++j)
+      if (ok[i][j]) h[bh * E + eo[i][j]] = a[i][j] - corr[i][j];
 }
 
 // Per-chunk norm of hc_c = K_c^T V_c - kc_c vc_c^T (kernel.py:172-174); partial holds one
@@ -177,42 +203,12 @@ __global__ __launch_bounds__(kThreads) void chunk_norm_kernel(
   }
 }
 
-// ===========================================================================
-// attention kernel
-// ===========================================================================
-// One workgroup (4 waves) per (head, 64-query block); each wave owns 16 queries.
-// MFMA: v_mfma_f32_16x16x32_{f16,bf16} (A lane l: m=l%16, k=8*(l/16)+i; B lane l:
-// n=l%16, k=8*(l/16)+i; C lane l: n=l%16, rows 4*(l/16)+r).  Scores are computed
-// transposed, S^T = K Q^T, so that a lane holds 16 keys of ONE query: the row
-// maximum needs two shuffles, and exp(S^T) packed to 16 bits is directly the B
-// operand of O^T += V^T P^T (the key order of that contraction is chosen to match).
-// V^T operands come from LDS with the dword + v_perm transposition.
-//
-//   phase 1  exact softmax attention over the NS selected 64-key blocks
-//   phase 2  the unselected blocks, each represented by its mean key (weight n_c in
-//            the denominator) and its value sum; means/sums are hi+lo 16-bit pairs
-//   phase 3  first-order term: acc += (q H) * (G/T) * scale, q H precomputed per token
-//   o = acc / (l + G)
-// Unlike the Triton kernel (kernel.py:263-276) the running G is rescaled together
-// with acc and l whenever the running maximum grows.
+// 16-bit pack / unpack helpers of the attention kernel
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-template <typename T> struct Mma16;
-template <> struct Mma16<_Float16> {
-  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
-                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-  }
-};
-template <> struct Mma16<__bf16> {
-  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
-                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-  }
-};
 template <typename T> __device__ __forceinline__ uint32_t pack_pair(float a, float b) {
   return (uint32_t)__builtin_bit_cast(uint16_t, (T)a) |
          ((uint32_t)__builtin_bit_cast(uint16_t, (T)b) << 16);
@@ -224,47 +220,101 @@ template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t w) {
   return (float)__builtin_bit_cast(T, (uint16_t)(w >> 16));
 }
 
-struct AttnArgs {
-  const void *q, *k, *v;         // [BH, T, K], [BH, T, K], [BH, T, V]
-  const void *kc_hi, *kc_lo;     // [BH, NTp, K] 16-bit: chunk mean keys, hi + lo
-  const void *vc_hi, *vc_lo;     // [BH, NTp, V] 16-bit: chunk value sums, hi + lo
-  const void* r;                 // [BH, T, V] 16-bit: q H per token
-  const int32_t* indices;        // [BH, NT, NS] selected key blocks per query block
+// ===========================================================================
+// attention kernel
+// ===========================================================================
+// One workgroup (4 waves) per (head, 64-query block).  Wave w owns queries
+// 32*(w%2) .. +31 and, of every 64-key block, keys 32*(w/2) .. +31: the two waves that
+// share a query half keep separate running maxima / sums / accumulators for their key
+// halves and are merged once at the end.  MFMA: v_mfma_f32_32x32x16 (A lane l: m = l%32,
+// k = 8*(l/32)+i; B lane l: n = l%32, same k; C lane l: column l%32, register r is row
+// 8*(r/4) + 4*(l/32) + r%4).
+//   S^T[key][query] = K Q^T      A = K tile row (16 B of one key), B = Q^T in registers
+//   O^T[vcol][query] += V^T P^T  A = V^T tile row (16 B = 8 keys of one value column),
+//                                B = exp2(S^T) packed to 16 bits, straight from the
+//                                accumulator registers: k-slot i of k-step t is register
+//                                8t+i, i.e. key 16t + 8*(i/4) + 4*(l/32) + i%4
+//   phase 1  exact softmax attention over the NS selected 64-key blocks
+//   phase 2  the unselected blocks, each represented by its mean key (weight n_c in the
+//            denominator) and its value sum; means / sums are hi + lo 16-bit pairs
+//   phase 3  first-order term: acc += (q H) * (G/T) * scale, q H precomputed per token
+//   o = acc / (l + G)
+// Unlike the Triton kernel (kernel.py:263-276) the running G is rescaled together with
+// acc and l whenever the running maximum grows.
+// Values arrive transposed ([BH, V, Tp], Tp = 64*NT, zero padded) so that a V^T tile row
+// is 128 contiguous bytes; inside every group of 16 keys the LDS copy is stored in the
+// order (4b+j, 8+4b+j) so that the eight keys of a k-slot group are one 16-byte read.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <typename T> struct Mma32;
+template <> struct Mma32<_Float16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma32<__bf16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+
+struct Attn32Args {
+  const void *q, *k;             // [BH, T, K]
+  const void* vt;                // [BH, V, Tp] transposed values, zero padded
+  const void *kc_hi, *kc_lo;     // [BH, NTp, K] chunk mean keys, hi + lo
+  const void *vct_hi, *vct_lo;   // [BH, V, NTp] transposed chunk value sums, hi + lo
+  const void* r;                 // [BH, T, V] q H per token
+  const int32_t* indices;        // [BH, NT, NS]
   void* o;                       // [BH, T, V]
   int T, NT, NTp, NS;
   float scale;
 };
 
-template <int K, int V> struct AttnLayout {
-  static constexpr int kKT = 64 * K * 2, kVT = 64 * V * 2;  // one 64-row tile
+template <int K, int V> struct Attn32Layout {
+  static constexpr int kKT = 64 * K * 2;   // K tile: 64 keys x K features
+  static constexpr int kVT = V * 128;      // V^T tile: V value columns x 64 keys
   static constexpr int kSet = kKT + kVT;
-  static constexpr int kSel = 2 * kSet;
-  static constexpr int kTotalNoSel = 2 * kSet;
+  static constexpr int kTiles = 2 * kSet;  // double buffer; the selected-block bitmap follows
 };
 
+typedef uint32_t u32x2p __attribute__((ext_vector_type(2)));
+
 template <typename T, int K, int V>
-__global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
-  using LY = AttnLayout<K, V>;
-  constexpr int KCH = K / 8, VCH = V / 8;        // 16-byte chunks per row
-  constexpr int KST = K / 32;                    // k-steps of the score product
-  constexpr int DG = V / 32;                     // 32-wide value column groups
-  constexpr int KLD = 64 * KCH / kThreads, VLD = 64 * VCH / kThreads;  // chunks per thread per tile
+__global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) {
+  using LY = Attn32Layout<K, V>;
+  constexpr int KCH = K / 8;                 // 16-byte chunks per K tile row
+  constexpr int KS = K / 16;                 // k-steps of the score product
+  constexpr int MB = V / 32;                 // 32-row blocks of O^T
+  constexpr int KLD = 64 * KCH / kThreads;   // 16-byte chunks per thread per K tile
+  constexpr int VLD = V * 8 / kThreads;      // ... per V^T tile
+  constexpr int OLD = 64 * (V / 8) / kThreads;
   constexpr float kNegInf = -__builtin_huge_valf();
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  unsigned char* sel = smem + LY::kSel;
+  unsigned char* sel = smem + LY::kTiles;
 
   const int tq = blockIdx.x % a.NT;
   const int64_t bh = blockIdx.x / a.NT;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int nq = lane & 15, kb = lane >> 4;
-  const int qtok = tq * 64 + wave * 16 + nq;  // this lane's query token
-  const float sm_scale = a.scale * 1.44269504f;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int qh = wave & 1, kh = wave >> 1;
+  const int n = lane & 31, kg = lane >> 5;
+  const int qtok = tq * 64 + 32 * qh + n;  // this lane's query
+  const float c2 = a.scale * 1.44269504f;  // scores are kept unscaled; p = exp2(s*c2 - m*c2)
+  const int Tp = a.NT * 64;
 
   const T* qb = (const T*)a.q + bh * a.T * K;
-  const T* kbase = (const T*)a.k + bh * a.T * K;
-  const T* vbase = (const T*)a.v + bh * a.T * V;
+  auto descriptor = [](const void* base, int64_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+  };
+  const auto k_rs = descriptor((const T*)a.k + bh * a.T * K, (int64_t)a.T * K * 2);
+  const auto vt_rs = descriptor((const T*)a.vt + bh * V * (int64_t)Tp, (int64_t)V * Tp * 2);
+  const auto kch_rs = descriptor((const T*)a.kc_hi + bh * a.NTp * K, (int64_t)a.NTp * K * 2);
+  const auto kcl_rs = descriptor((const T*)a.kc_lo + bh * a.NTp * K, (int64_t)a.NTp * K * 2);
+  const auto vch_rs = descriptor((const T*)a.vct_hi + bh * V * (int64_t)a.NTp, (int64_t)V * a.NTp * 2);
+  const auto vcl_rs = descriptor((const T*)a.vct_lo + bh * V * (int64_t)a.NTp, (int64_t)V * a.NTp * 2);
 
-  // selected-block bitmap
   for (int i = tid; i < a.NTp; i += kThreads) sel[i] = 0;
   __syncthreads();
   const int32_t* idx = a.indices + (bh * a.NT + tq) * a.NS;
@@ -273,34 +323,33 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
     if (b >= 0 && b < a.NT) sel[b] = 1;
   }
 
-  // Q^T operand: k-step s covers d = 32s + 8kb + i
-  u32x4 qop[KST];
+  // Q^T operand: k-step s covers features 16s + 8kg + i
+  u32x4 qop[KS];
 #pragma unroll
-  for (int s = 0; s < KST; ++s)
-    qop[s] = qtok < a.T ? *reinterpret_cast<const u32x4*>(qb + (int64_t)qtok * K + 32 * s + 8 * kb)
+  for (int s = 0; s < KS; ++s)
+    qop[s] = qtok < a.T ? *reinterpret_cast<const u32x4*>(qb + (int64_t)qtok * K + 16 * s + 8 * kg)
                         : u32x4{0u, 0u, 0u, 0u};
 
-  // tile swizzles: K rows are read 16 B per lane down a column of 16 rows; V rows are
-  // read one dword per lane, four rows (one per kb) at a time
-  auto kswz = [](int row, int ch) { return row * (K * 2) + ((ch ^ (row & 7)) << 4); };
-  auto vswz_chunk = [](int row, int ch) { return row * (V * 2) + ((ch ^ (((row >> 2) & 1) << 2)) << 4); };
-  auto vswz_dword = [](int row, int dw) { return row * (V * 2) + ((dw ^ (((row >> 2) & 1) << 4)) << 2); };
+  // 16-byte chunk ch of row `row`, XOR-swizzled (rows are 128 or 256 bytes: a column of
+  // rows would otherwise sit in one bank group)
+  // (the LDS serves 16 lanes x 16 bytes per cycle from 64 banks: 16 consecutive rows of a
+  // column must land in 16 different 16-byte bank groups; 256-byte rows need all four low
+  // row bits, 128-byte rows come in pairs that already differ in the upper half of the banks)
+  auto swz256 = [](int row, int ch) { return row * 256 + ((ch ^ (row & 15)) << 4); };
+  auto swz128 = [](int row, int ch) { return row * 128 + ((ch ^ ((row >> 1) & 7)) << 4); };
+  auto kswz = [&](int row, int ch) { return K == 128 ? swz256(row, ch) : swz128(row, ch); };
+  auto vswz = [&](int row, int ch) { return swz128(row, ch); };
+  auto oswz = [&](int row, int ch) { return V == 128 ? swz256(row, ch) : swz128(row, ch); };
 
-  auto load_tile_k = [&](u32x4(&dst)[KLD], const T* src, int row0, int nrows) {
+  // Tiles are fetched with buffer loads: one lane offset register, the tile / row-group
+  // offsets are scalars, and rows past the end of the tensor come back as zero (the
+  // descriptor's byte count is the bounds check).
+  const uint32_t k_lane_off = (uint32_t)(((tid / KCH) * K + (tid % KCH) * 8) * 2);
+  auto load_tile_k = [&](u32x4(&dst)[KLD], __amdgpu_buffer_rsrc_t rs, int row0) {
 #pragma unroll
-    for (int j = 0; j < KLD; ++j) {
-      const int qq = tid + kThreads * j, row = qq / KCH, ch = qq % KCH;
-      dst[j] = row < nrows ? *reinterpret_cast<const u32x4*>(src + (int64_t)(row0 + row) * K + ch * 8)
-                           : u32x4{0u, 0u, 0u, 0u};
-    }
-  };
-  auto load_tile_v = [&](u32x4(&dst)[VLD], const T* src, int row0, int nrows) {
-#pragma unroll
-    for (int j = 0; j < VLD; ++j) {
-      const int qq = tid + kThreads * j, row = qq / VCH, ch = qq % VCH;
-      dst[j] = row < nrows ? *reinterpret_cast<const u32x4*>(src + (int64_t)(row0 + row) * V + ch * 8)
-                           : u32x4{0u, 0u, 0u, 0u};
-    }
+    for (int j = 0; j < KLD; ++j)  // chunk tid + 256j: row tid/KCH + j*(256/KCH)
+      dst[j] = __builtin_amdgcn_raw_buffer_load_b128(
+          rs, k_lane_off, (row0 + j * (kThreads / KCH)) * (K * 2), 0);
   };
   auto store_tile_k = [&](const u32x4(&src)[KLD], unsigned char* tile) {
 #pragma unroll
@@ -309,78 +358,97 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
       *reinterpret_cast<u32x4*>(tile + kswz(qq / KCH, qq % KCH)) = src[j];
     }
   };
+  // V^T tile: row = value column, 8 chunks of 8 keys; source row stride `ld` elements
+  auto load_tile_v = [&](u32x4(&dst)[VLD], __amdgpu_buffer_rsrc_t rs, int ld, int col0) {
+    const uint32_t lane_off = (uint32_t)(((tid >> 3) * ld + (tid & 7) * 8) * 2);
+#pragma unroll
+    for (int j = 0; j < VLD; ++j)  // chunk tid + 256j: row tid/8 + 32j
+      dst[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, (col0 + j * 32 * ld) * 2, 0);
+  };
+  // keys 8ch .. 8ch+7 of a row: (ch odd ? a = 1 : a = 0) half-groups b = 0, 1 go to positions
+  // 8b + 4a of 16-key group ch/2, i.e. chunk 2*(ch/2) + b, byte 8a
   auto store_tile_v = [&](const u32x4(&src)[VLD], unsigned char* tile) {
 #pragma unroll
     for (int j = 0; j < VLD; ++j) {
-      const int qq = tid + kThreads * j;
-      *reinterpret_cast<u32x4*>(tile + vswz_chunk(qq / VCH, qq % VCH)) = src[j];
+      const int qq = tid + kThreads * j, row = qq >> 3, ch = qq & 7;
+      const int g2 = ch & ~1, aa = ch & 1;
+      *reinterpret_cast<u32x2p*>(tile + vswz(row, g2) + 8 * aa) = u32x2p{src[j][0], src[j][1]};
+      *reinterpret_cast<u32x2p*>(tile + vswz(row, g2 + 1) + 8 * aa) = u32x2p{src[j][2], src[j][3]};
     }
   };
 
-  // per-lane LDS offsets of the operand reads (everything else is a compile-time constant)
-  int koff[KST], voff[DG];
+  // per-lane LDS offsets of the operand reads
+  int koff[KS], voff[2];
 #pragma unroll
-  for (int s = 0; s < KST; ++s) koff[s] = kswz(nq, 4 * s + kb);
+  for (int s = 0; s < KS; ++s) koff[s] = kswz(32 * kh + n, 2 * s + kg);
 #pragma unroll
-  for (int dg = 0; dg < DG; ++dg) voff[dg] = vswz_dword(4 * kb, 16 * dg + nq);
+  for (int t = 0; t < 2; ++t) voff[t] = vswz(n, 2 * (2 * kh + t) + kg);
 
-  float m_i = kNegInf, l_p = 0.f, g_p = 0.f;  // running max; per-lane partial sums
-  f32x4 acc[DG][2];
+  float m_i = kNegInf, l_p = 0.f, g_p = 0.f;  // running max (unscaled); per-lane partial sums
+  f32x16 acc[MB];
 #pragma unroll
-  for (int dg = 0; dg < DG; ++dg)
+  for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-    for (int par = 0; par < 2; ++par) acc[dg][par] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int r = 0; r < 16; ++r) acc[mb][r] = 0.f;
 
-  // One 64-key block: scores against NKT key tiles (summed), masked, online softmax,
-  // then acc += P (V tile 0 [+ V tile 1]).  valid(key) / weight(key) describe the block.
-  auto attend = [&](const unsigned char* kt0, const unsigned char* kt1, const unsigned char* vt0,
-                    const unsigned char* vt1, auto valid, auto weight, bool weighted, bool all_valid) {
-    f32x4 st[4];
+  // One 64-key block in three stages; this wave's keys are key(r) = 32kh + 8(r/4) + 4kg + r%4.
+  // The tags are compile-time (std::true_type / false_type): masked = some keys are invalid,
+  // weighted = the block statistics branch (hi + lo tiles, sums weighted by chunk length).
+  //   scores:   S^T = K Q^T, two accumulators (two independent MFMA chains)
+  //   softmax:  running maximum, p = exp2(...), partial sums, accumulator rescale; p packed
+  //   values:   O^T += V^T P^T
+  auto scores = [&](const unsigned char* kt0, const unsigned char* kt1, auto weighted_tag) {
+    constexpr bool weighted = decltype(weighted_tag)::value;
+    f32x16 st, st2;
 #pragma unroll
-    for (int jb = 0; jb < 4; ++jb) {
-      st[jb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int r = 0; r < 16; ++r) st[r] = st2[r] = 0.f;
 #pragma unroll
-      for (int s = 0; s < KST; ++s) {
-        // row 16jb + nq: same swizzle as row nq (16jb is a multiple of 8)
-        const u32x4 ak = *reinterpret_cast<const u32x4*>(kt0 + koff[s] + jb * (16 * K * 2));
-        st[jb] = Mma16<T>::run(ak, qop[s], st[jb]);
-        if (kt1) {
-          const u32x4 al = *reinterpret_cast<const u32x4*>(kt1 + koff[s] + jb * (16 * K * 2));
-          st[jb] = Mma16<T>::run(al, qop[s], st[jb]);
-        }
+    for (int s = 0; s < KS; s += 2) {
+      const u32x4 ak = *reinterpret_cast<const u32x4*>(kt0 + koff[s]);
+      const u32x4 ak2 = *reinterpret_cast<const u32x4*>(kt0 + koff[s + 1]);
+      st = Mma32<T>::run(ak, qop[s], st);
+      st2 = Mma32<T>::run(ak2, qop[s + 1], st2);
+      if constexpr (weighted) {
+        const u32x4 al = *reinterpret_cast<const u32x4*>(kt1 + koff[s]);
+        const u32x4 al2 = *reinterpret_cast<const u32x4*>(kt1 + koff[s + 1]);
+        st = Mma32<T>::run(al, qop[s], st);
+        st2 = Mma32<T>::run(al2, qop[s + 1], st2);
       }
     }
-    // this lane: keys 16jb + 4kb + r of query nq
+#pragma unroll
+    for (int r = 0; r < 16; ++r) st[r] += st2[r];
+    return st;
+  };
+  auto softmax = [&](f32x16 st, u32x4(&pw)[2], auto valid, auto weight, auto masked_tag, auto weighted_tag) {
+    constexpr bool masked = decltype(masked_tag)::value, weighted = decltype(weighted_tag)::value;
     float mx = kNegInf;
 #pragma unroll
-    for (int jb = 0; jb < 4; ++jb)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float x = (all_valid || valid(16 * jb + 4 * kb + r)) ? st[jb][r] * sm_scale : kNegInf;
-        st[jb][r] = x;
-        mx = fmaxf(mx, x);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    for (int r = 0; r < 16; ++r) {
+      if constexpr (masked) st[r] = valid(32 * kh + 8 * (r >> 2) + 4 * kg + (r & 3)) ? st[r] : kNegInf;
+      mx = fmaxf(mx, st[r]);
+    }
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const float m_new = fmaxf(m_i, mx);
     const float m_safe = m_new == kNegInf ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_i - m_safe);
+    const float alpha = __builtin_amdgcn_exp2f((m_i - m_safe) * c2);
+    const float mc = m_safe * c2;
     m_i = m_new;
     float psum = 0.f, wsum = 0.f;
-    uint32_t pw[8];
 #pragma unroll
-    for (int jb = 0; jb < 4; ++jb) {
-      float pv[4];
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        pv[r] = __builtin_amdgcn_exp2f(st[jb][r] - m_safe);
-        psum += pv[r];
-        if (weighted) wsum = fmaf(pv[r], weight(16 * jb + 4 * kb + r), wsum);
+      for (int i = 0; i < 4; ++i) {
+        const int r = 8 * t + 2 * i;
+        const float p0 = __builtin_amdgcn_exp2f(fmaf(st[r], c2, -mc));
+        const float p1 = __builtin_amdgcn_exp2f(fmaf(st[r + 1], c2, -mc));
+        psum += p0 + p1;
+        if constexpr (weighted) {
+          wsum = fmaf(p0, weight(32 * kh + 8 * (r >> 2) + 4 * kg + (r & 3)), wsum);
+          wsum = fmaf(p1, weight(32 * kh + 8 * ((r + 1) >> 2) + 4 * kg + ((r + 1) & 3)), wsum);
+        }
+        pw[t][i] = pack_pair<T>(p0, p1);
       }
-      pw[2 * jb] = pack_pair<T>(pv[0], pv[1]);
-      pw[2 * jb + 1] = pack_pair<T>(pv[2], pv[3]);
-    }
-    if (weighted) {
+    if constexpr (weighted) {
       g_p = g_p * alpha + wsum;
       l_p = l_p * alpha;
     } else {
@@ -389,136 +457,202 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(AttnArgs a) {
     }
     if (__any(alpha != 1.f)) {  // the running maximum rarely moves after the first blocks
 #pragma unroll
-      for (int dg = 0; dg < DG; ++dg)
+      for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int par = 0; par < 2; ++par) acc[dg][par] *= alpha;
-    }
-    // O^T += V^T P^T: k-step sp covers key sub-blocks 2sp, 2sp+1; slot i of lane kb is
-    // key 32sp + 4kb + i (i < 4) or 32sp + 16 + 4kb + (i - 4)
-#pragma unroll
-    for (int sp = 0; sp < 2; ++sp) {
-      const u32x4 bp = u32x4{pw[4 * sp], pw[4 * sp + 1], pw[4 * sp + 2], pw[4 * sp + 3]};
-#pragma unroll
-      for (int dg = 0; dg < DG; ++dg) {
-#pragma unroll
-        for (int tile = 0; tile < 2; ++tile) {
-          const unsigned char* vt = tile == 0 ? vt0 : vt1;
-          if (!vt) continue;
-          uint32_t w[8];
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            // row 32sp + 16(i/4) + 4kb + i%4: the swizzle bit (row/4)%2 equals kb%2 as in row 4kb
-            w[i] = *reinterpret_cast<const uint32_t*>(vt + voff[dg] +
-                                                      (32 * sp + 16 * (i >> 2) + (i & 3)) * (V * 2));
-          }
-          u32x4 ae, ao;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            ae[i] = __builtin_amdgcn_perm(w[2 * i + 1], w[2 * i], 0x05040100u);
-            ao[i] = __builtin_amdgcn_perm(w[2 * i + 1], w[2 * i], 0x07060302u);
-          }
-          acc[dg][0] = Mma16<T>::run(ae, bp, acc[dg][0]);
-          acc[dg][1] = Mma16<T>::run(ao, bp, acc[dg][1]);
-        }
-      }
+        for (int r = 0; r < 16; ++r) acc[mb][r] *= alpha;
     }
   };
+  auto values = [&](const unsigned char* vt0, const unsigned char* vt1, const u32x4(&pw)[2],
+                    auto weighted_tag) {
+    constexpr bool weighted = decltype(weighted_tag)::value;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const u32x4 av = *reinterpret_cast<const u32x4*>(vt0 + voff[t] + mb * (32 * 128));
+        acc[mb] = Mma32<T>::run(av, pw[t], acc[mb]);
+        if constexpr (weighted) {
+          const u32x4 al = *reinterpret_cast<const u32x4*>(vt1 + voff[t] + mb * (32 * 128));
+          acc[mb] = Mma32<T>::run(al, pw[t], acc[mb]);
+        }
+      }
+  };
+  const std::true_type yes{};
+  const std::false_type no{};
 
-  // ---- phase 1: selected blocks, K/V tiles double-buffered ----
+  // ---- phase 1: selected blocks.  Software pipeline: the value product of block i-1 is
+  // issued between the score product and the softmax of block i, so that the matrix unit
+  // works on it while the vector unit does the exponentials.  K and V^T tiles alternate
+  // between two LDS sets (the loop is unrolled by two: constant addresses); the tile of
+  // block i+1 travels through registers during block i and is stored between two barriers
+  // (its V^T slot held block i-1, which every wave has consumed by then).
   u32x4 rk[KLD], rv[VLD];
-  // rows of block b that exist (0 for an index outside [0, NT): the block is skipped)
   auto block_rows = [&](int b) { return b >= 0 && b < a.NT ? min(64, a.T - b * 64) : 0; };
   {
     const int b0 = idx[0], n0 = block_rows(b0);
-    load_tile_k(rk, kbase, n0 ? b0 * 64 : 0, n0);
-    load_tile_v(rv, vbase, n0 ? b0 * 64 : 0, n0);
+    load_tile_k(rk, k_rs, n0 ? b0 * 64 : 0);
+    load_tile_v(rv, vt_rs, Tp, n0 ? b0 * 64 : 0);
     store_tile_k(rk, smem);
     store_tile_v(rv, smem + LY::kKT);
   }
   __syncthreads();
-  for (int i = 0; i < a.NS; ++i) {
-    const int blk = idx[i];
-    unsigned char* cur = smem + (i & 1) * LY::kSet;
-    unsigned char* nxt = smem + ((i + 1) & 1) * LY::kSet;
-    const bool more = i + 1 < a.NS;
-    if (more) {
-      const int bn = idx[i + 1], nn = block_rows(bn);
-      load_tile_k(rk, kbase, nn ? bn * 64 : 0, nn);
-      load_tile_v(rv, vbase, nn ? bn * 64 : 0, nn);
+  u32x4 pw[2];
+  bool pending = false;  // pw holds the probabilities of the previous block, not yet multiplied
+  auto prefetch = [&](int i) {  // tile of selected block i -> registers
+    if (i < a.NS) {
+      const int bn = idx[i], nn = block_rows(bn);
+      load_tile_k(rk, k_rs, nn ? bn * 64 : 0);
+      load_tile_v(rv, vt_rs, Tp, nn ? bn * 64 : 0);
     }
-    const int nrows = block_rows(blk);
-    attend(cur, nullptr, cur + LY::kKT, nullptr, [&](int key) { return key < nrows; },
-           [](int) { return 0.f; }, false, nrows == 64);
-    if (more) {
+  };
+  prefetch(1);
+  auto step = [&](int i, unsigned char* cur, unsigned char* nxt) {
+    const int nrows = block_rows(idx[i]);
+    const auto none = [](int) { return 0.f; };
+    f32x16 st;
+    if (nrows > 0) st = scores(cur, cur, no);
+    if (pending) values(nxt + LY::kKT, nxt, pw, no);  // block i-1 lives in the other set
+    pending = nrows > 0;
+    if (nrows == 64)
+      softmax(st, pw, [](int) { return true; }, none, no, no);
+    else if (nrows > 0)
+      softmax(st, pw, [&](int key) { return key < nrows; }, none, yes, no);
+    __syncthreads();
+    if (i + 1 < a.NS) {
       store_tile_k(rk, nxt);
       store_tile_v(rv, nxt + LY::kKT);
     }
+    prefetch(i + 2);  // in flight during the barrier and all of the next block
     __syncthreads();
+  };
+  for (int i = 0; i < a.NS; i += 2) {
+    step(i, smem, smem + LY::kSet);
+    if (i + 1 < a.NS) step(i + 1, smem + LY::kSet, smem);
   }
+  if (pending) values(smem + ((a.NS - 1) & 1) * LY::kSet + LY::kKT, smem, pw, no);
+  __syncthreads();
 
   // ---- phase 2: unselected blocks through their means / sums ----
   const int last_len = a.T - (a.NT - 1) * 64;
   for (int grp = 0; grp * 64 < a.NT; ++grp) {
-    const int64_t row0 = bh * a.NTp + grp * 64;
-    // four tiles: kc hi | vc hi | kc lo | vc lo
     {
-      const T* src = (const T*)a.kc_hi + row0 * K;
-      load_tile_k(rk, src, 0, 64);
+      load_tile_k(rk, kch_rs, grp * 64);
       store_tile_k(rk, smem);
-      src = (const T*)a.kc_lo + row0 * K;
-      load_tile_k(rk, src, 0, 64);
+      load_tile_k(rk, kcl_rs, grp * 64);
       store_tile_k(rk, smem + LY::kSet);
-      const T* vsrc = (const T*)a.vc_hi + row0 * V;
-      load_tile_v(rv, vsrc, 0, 64);
+      load_tile_v(rv, vch_rs, a.NTp, grp * 64);
       store_tile_v(rv, smem + LY::kKT);
-      vsrc = (const T*)a.vc_lo + row0 * V;
-      load_tile_v(rv, vsrc, 0, 64);
+      load_tile_v(rv, vcl_rs, a.NTp, grp * 64);
       store_tile_v(rv, smem + LY::kSet + LY::kKT);
     }
     __syncthreads();
     const int c0 = grp * 64;
-    attend(smem, smem + LY::kSet, smem + LY::kKT, smem + LY::kSet + LY::kKT,
-           [&](int key) { return c0 + key < a.NT && !sel[c0 + key]; },
-           [&](int key) { return c0 + key == a.NT - 1 ? (float)last_len : 64.f; }, true, false);
+    const f32x16 st = scores(smem, smem + LY::kSet, yes);
+    softmax(st, pw, [&](int key) { return c0 + key < a.NT && !sel[c0 + key]; },
+            [&](int key) { return c0 + key == a.NT - 1 ? (float)last_len : 64.f; }, yes, yes);
+    values(smem + LY::kKT, smem + LY::kSet + LY::kKT, pw, yes);
     __syncthreads();
   }
 
-  // ---- phase 3 and output ----
-  float L = l_p, G = g_p;
-  L += __shfl_xor(L, 16);
-  L += __shfl_xor(L, 32);
-  G += __shfl_xor(G, 16);
-  G += __shfl_xor(G, 32);
-  {
-    const T* rsrc = (const T*)a.r + (bh * a.T + (int64_t)tq * 64) * V;
-    load_tile_v(rv, rsrc, 0, a.T - tq * 64);
-    store_tile_v(rv, smem + LY::kKT);
+  // ---- merge the two key halves: waves kh = 1 hand their state to waves kh = 0 ----
+  float L = l_p + __shfl_xor(l_p, 32), G = g_p + __shfl_xor(g_p, 32);
+  float* mrg = reinterpret_cast<float*>(smem) + qh * (64 * (MB * 16 + 3));  // [value][lane]
+  if (kh == 1) {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mrg[(mb * 16 + r) * 64 + lane] = acc[mb][r];
+    mrg[(MB * 16 + 0) * 64 + lane] = m_i;
+    mrg[(MB * 16 + 1) * 64 + lane] = L;
+    mrg[(MB * 16 + 2) * 64 + lane] = G;
   }
   __syncthreads();
-  const float corr = G / (float)a.T * a.scale;
-  const float inv = 1.f / (L + G);
-  unsigned char* rt = smem + LY::kKT;    // q H tile
-  unsigned char* ot = smem + LY::kSet + LY::kKT;  // output tile
-  const int qrow = wave * 16 + nq;
+  if (kh == 0) {
+    const float m1 = mrg[(MB * 16 + 0) * 64 + lane];
+    const float m = fmaxf(m_i, m1);
+    const float ms = m == kNegInf ? 0.f : m;
+    const float a0 = __builtin_amdgcn_exp2f((m_i - ms) * c2), a1 = __builtin_amdgcn_exp2f((m1 - ms) * c2);
+    L = L * a0 + mrg[(MB * 16 + 1) * 64 + lane] * a1;
+    G = G * a0 + mrg[(MB * 16 + 2) * 64 + lane] * a1;
 #pragma unroll
-  for (int dg = 0; dg < DG; ++dg)
+    for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      // acc[dg][par][r] is value column 32dg + 2(4kb + r) + par: one dword per (dg, r)
-      const int dw = 16 * dg + 4 * kb + r;
-      const uint32_t rw = *reinterpret_cast<const uint32_t*>(rt + vswz_dword(qrow, dw));
-      const float o0 = (acc[dg][0][r] + unpack_lo<T>(rw) * corr) * inv;
-      const float o1 = (acc[dg][1][r] + unpack_hi<T>(rw) * corr) * inv;
-      *reinterpret_cast<uint32_t*>(ot + vswz_dword(qrow, dw)) = pack_pair<T>(o0, o1);
+      for (int r = 0; r < 16; ++r) acc[mb][r] = acc[mb][r] * a0 + mrg[(mb * 16 + r) * 64 + lane] * a1;
+  }
+  __syncthreads();
+
+  // ---- phase 3 and output (waves kh = 0): acc += (q H) * (G/T) * scale, o = acc / (L + G) ----
+  unsigned char* rt = smem;                 // q H tile [64][V]
+  unsigned char* ot = smem + 64 * V * 2;    // output tile [64][V]
+  {
+    const T* rsrc = (const T*)a.r + (bh * a.T + (int64_t)tq * 64) * V;
+    const int nrows = a.T - tq * 64;
+#pragma unroll
+    for (int j = 0; j < OLD; ++j) {
+      const int qq = tid + kThreads * j, row = qq / (V / 8), ch = qq % (V / 8);
+      const u32x4 x = row < nrows ? *reinterpret_cast<const u32x4*>(rsrc + (int64_t)row * V + ch * 8)
+                                  : u32x4{0u, 0u, 0u, 0u};
+      *reinterpret_cast<u32x4*>(rt + oswz(row, ch)) = x;
     }
+  }
+  __syncthreads();
+  if (kh == 0) {
+    const float corr = G / (float)a.T * a.scale;
+    const float inv = 1.f / (L + G);
+    const int qrow = 32 * qh + n;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        // registers 4*r4 .. +3: value columns 32mb + 8*r4 + 4kg + 0..3 = 8 bytes of chunk 4mb + r4
+        const int off = oswz(qrow, 4 * mb + r4) + 8 * kg;
+        const u32x2p rw = *reinterpret_cast<const u32x2p*>(rt + off);
+        const float o0 = (acc[mb][4 * r4 + 0] + unpack_lo<T>(rw[0]) * corr) * inv;
+        const float o1 = (acc[mb][4 * r4 + 1] + unpack_hi<T>(rw[0]) * corr) * inv;
+        const float o2 = (acc[mb][4 * r4 + 2] + unpack_lo<T>(rw[1]) * corr) * inv;
+        const float o3 = (acc[mb][4 * r4 + 3] + unpack_hi<T>(rw[1]) * corr) * inv;
+        *reinterpret_cast<u32x2p*>(ot + off) = u32x2p{pack_pair<T>(o0, o1), pack_pair<T>(o2, o3)};
+      }
+  }
   __syncthreads();
   T* ob = (T*)a.o + (bh * a.T + (int64_t)tq * 64) * V;
 #pragma unroll
-  for (int j = 0; j < VLD; ++j) {
-    const int qq = tid + kThreads * j, row = qq / VCH, ch = qq % VCH;
+  for (int j = 0; j < OLD; ++j) {
+    const int qq = tid + kThreads * j, row = qq / (V / 8), ch = qq % (V / 8);
     if (tq * 64 + row < a.T)
       *reinterpret_cast<u32x4*>(ob + (int64_t)row * V + ch * 8) =
-          *reinterpret_cast<const u32x4*>(ot + vswz_chunk(row, ch));
+          *reinterpret_cast<const u32x4*>(ot + oswz(row, ch));
+  }
+}
+
+// values [BH, T, V] -> [BH, V, Tp] (Tp = 64 * NT, zero padded): one workgroup per (head,
+// 64-token block), through a padded LDS tile
+template <typename T, int V>
+__global__ __launch_bounds__(kThreads) void transpose_values_kernel(const T* __restrict__ v,
+                                                                   T* __restrict__ vt, int Tn, int NT) {
+  constexpr int LDW = V + 2;  // row stride in elements: odd number of dwords
+  __shared__ T tile[64 * LDW];
+  const int tb = blockIdx.x % NT;
+  const int64_t bh = blockIdx.x / NT;
+  const int nrows = min(64, Tn - tb * 64);
+  const T* src = v + (bh * Tn + (int64_t)tb * 64) * V;
+  for (int qq = threadIdx.x; qq < 64 * (V / 2); qq += kThreads) {
+    const int row = qq / (V / 2), dw = qq % (V / 2);
+    const uint32_t x = row < nrows ? *reinterpret_cast<const uint32_t*>(src + (int64_t)row * V + 2 * dw) : 0u;
+    *reinterpret_cast<uint32_t*>(&tile[row * LDW + 2 * dw]) = x;
+  }
+  __syncthreads();
+  T* dst = vt + bh * V * (int64_t)NT * 64 + (int64_t)tb * 64;
+  for (int qq = threadIdx.x; qq < V * 8; qq += kThreads) {
+    const int col = qq >> 3, ch = qq & 7;
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint16_t lo = __builtin_bit_cast(uint16_t, tile[(8 * ch + 2 * i) * LDW + col]);
+      const uint16_t hi = __builtin_bit_cast(uint16_t, tile[(8 * ch + 2 * i + 1) * LDW + col]);
+      w[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+    }
+    *reinterpret_cast<u32x4*>(dst + (int64_t)col * NT * 64 + ch * 8) = u32x4{w[0], w[1], w[2], w[3]};
   }
 }
 
@@ -534,6 +668,26 @@ __global__ __launch_bounds__(kThreads) void split_hi_lo_kernel(const float* __re
     const int64_t bc = e / D;
     const int c = (int)(bc % NTp);
     const int64_t bh = bc / NTp;
+    float x = 0.f;
+    if (c < NT) x = src[(bh * NT + c) * D + d];
+    const T h = (T)x;
+    hi[e] = h;
+    lo[e] = (T)(x - (float)h);
+  }
+}
+
+// The same, transposed: [BH, NT, D] -> [BH, D, NTp]
+template <typename T>
+__global__ __launch_bounds__(kThreads) void split_hi_lo_t_kernel(const float* __restrict__ src,
+                                                                 T* __restrict__ hi, T* __restrict__ lo,
+                                                                 int64_t BH, int NT, int NTp, int D) {
+  const int64_t total = BH * D * NTp;
+  for (int64_t e = (int64_t)blockIdx.x * kThreads + threadIdx.x; e < total;
+       e += (int64_t)gridDim.x * kThreads) {
+    const int c = (int)(e % NTp);
+    const int64_t bd = e / NTp;
+    const int d = (int)(bd % D);
+    const int64_t bh = bd / D;
     float x = 0.f;
     if (c < NT) x = src[(bh * NT + c) * D + d];
     const T h = (T)x;
@@ -621,22 +775,22 @@ bool attention_supported(int K, int V, int block, int dtype) {
 
 static int64_t padded_chunks(int64_t T) { return cdiv64(cdiv64(T, 64), 64) * 64; }
 
-// kc_hi | kc_lo | vc_hi | vc_lo | r
+// kc_hi | kc_lo | vc_hi | vc_lo (transposed) | r | v transposed
 size_t attention_workspace_bytes(int64_t BH, int64_t T, int K, int V) {
-  const int64_t NTp = padded_chunks(T);
+  const int64_t NTp = padded_chunks(T), Tp = cdiv64(T, 64) * 64;
   return 2 * align_up((size_t)BH * NTp * K * 2, 256) + 2 * align_up((size_t)BH * NTp * V * 2, 256) +
-         align_up((size_t)BH * T * V * 2, 256);
+         align_up((size_t)BH * T * V * 2, 256) + align_up((size_t)BH * V * Tp * 2, 256);
 }
 
 template <typename T, int K, int V>
-static int launch_attention(const AttnArgs& a, int64_t BH, hipStream_t st) {
-  using LY = AttnLayout<K, V>;
-  const int lds = LY::kSel + a.NTp;
-  if (lds > 160 * 1024) {
+static int launch_attention(const Attn32Args& a, const void* v, int64_t BH, hipStream_t st) {
+  using LY = Attn32Layout<K, V>;
+  const int lds = LY::kTiles + a.NTp;
+  if (lds > 80 * 1024) {
     set_error("piecewise attention: %d key blocks need more LDS than a workgroup has", a.NT);
     return kErrUnsupported;
   }
-  auto kernel = attention_kernel<T, K, V>;
+  auto kernel = attention32_kernel<T, K, V>;
   static thread_local int reserved = 0;
   if (lds > reserved) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -647,6 +801,8 @@ static int launch_attention(const AttnArgs& a, int64_t BH, hipStream_t st) {
     }
     reserved = lds;
   }
+  transpose_values_kernel<T, V><<<dim3((unsigned)(BH * a.NT)), dim3(kThreads), 0, st>>>(
+      (const T*)v, (T*)const_cast<void*>(a.vt), a.T, a.NT);
   kernel<<<dim3((unsigned)(BH * a.NT)), dim3(kThreads), lds, st>>>(a);
   return kOk;
 }
@@ -656,31 +812,34 @@ static int attention_t(const void* q, const void* k, const void* v, const float*
                        const float* h, const int32_t* indices, void* o, void* workspace, int64_t BH,
                        int64_t Tn, int K, int V, int NS, float scale, int dtype, hipStream_t st) {
   const int NT = (int)cdiv64(Tn, 64);
-  const int64_t NTp = padded_chunks(Tn);
+  const int64_t NTp = padded_chunks(Tn), Tp = (int64_t)NT * 64;
   char* ws = (char*)workspace;
   T* kc_hi = (T*)ws;
   ws += align_up((size_t)BH * NTp * K * 2, 256);
   T* kc_lo = (T*)ws;
   ws += align_up((size_t)BH * NTp * K * 2, 256);
-  T* vc_hi = (T*)ws;
+  T* vct_hi = (T*)ws;
   ws += align_up((size_t)BH * NTp * V * 2, 256);
-  T* vc_lo = (T*)ws;
+  T* vct_lo = (T*)ws;
   ws += align_up((size_t)BH * NTp * V * 2, 256);
   T* r = (T*)ws;
+  ws += align_up((size_t)BH * Tn * V * 2, 256);
+  T* vt = (T*)ws;
+  (void)Tp;
   const unsigned gk = (unsigned)std::min<int64_t>(cdiv64(BH * NTp * K, kThreads), 4096);
   const unsigned gv = (unsigned)std::min<int64_t>(cdiv64(BH * NTp * V, kThreads), 4096);
   split_hi_lo_kernel<T><<<dim3(gk), dim3(kThreads), 0, st>>>(kc, kc_hi, kc_lo, BH, NT, (int)NTp, K);
-  split_hi_lo_kernel<T><<<dim3(gv), dim3(kThreads), 0, st>>>(vc, vc_hi, vc_lo, BH, NT, (int)NTp, V);
+  split_hi_lo_t_kernel<T><<<dim3(gv), dim3(kThreads), 0, st>>>(vc, vct_hi, vct_lo, BH, NT, (int)NTp, V);
   // r_t = q_t H: the row-parallel kernel with M = H
   const Prob p = dense_prob(BH, Tn, K, V);
   mfma::RowsJob job{q, nullptr, h, V, 1, nullptr, nullptr, r};
   int rc = mfma::rows(p, dtype, job, K, V, st);
   if (rc != kOk) return rc;
-  AttnArgs a{q, k, v, kc_hi, kc_lo, vc_hi, vc_lo, r, indices, o, (int)Tn, NT, (int)NTp, NS, scale};
-  if (K == 64 && V == 64) return launch_attention<T, 64, 64>(a, BH, st);
-  if (K == 64) return launch_attention<T, 64, 128>(a, BH, st);
-  if (V == 64) return launch_attention<T, 128, 64>(a, BH, st);
-  return launch_attention<T, 128, 128>(a, BH, st);
+  Attn32Args a{q, k, vt, kc_hi, kc_lo, vct_hi, vct_lo, r, indices, o, (int)Tn, NT, (int)NTp, NS, scale};
+  if (K == 64 && V == 64) return launch_attention<T, 64, 64>(a, v, BH, st);
+  if (K == 64) return launch_attention<T, 64, 128>(a, v, BH, st);
+  if (V == 64) return launch_attention<T, 128, 64>(a, v, BH, st);
+  return launch_attention<T, 128, 128>(a, v, BH, st);
 }
 
 int attention(const void* q, const void* k, const void* v, const float* kc, const float* vc,
