@@ -549,9 +549,15 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
 // ===========================================================================
 // rows kernel: out_t = (x_t M) * rowscale_t + addvec
 // ===========================================================================
-// byte offset of 16-byte chunk `chunk` of row `row` inside a swizzled tile
+// Byte offset of 16-byte chunk `chunk` of row `row` inside a swizzled tile.  The LDS serves
+// 16 lanes x 16 bytes per cycle out of 64 banks, so the reads of one chunk column over 16
+// consecutive rows must fall into 16 different 16-byte bank groups: 256-byte rows use all
+// four low row bits; 128-byte rows come in pairs that already sit in different halves of
+// the banks, so the pair index is used.
 template <int ROWB> __device__ __forceinline__ int swz(int row, int chunk) {
-  return row * ROWB + ((chunk ^ (row & 7)) << 4);
+  if constexpr (ROWB == 256) return row * ROWB + ((chunk ^ (row & 15)) << 4);
+  else if constexpr (ROWB == 128) return row * ROWB + ((chunk ^ ((row >> 1) & 7)) << 4);
+  else return row * ROWB + ((chunk ^ (row & 7)) << 4);
 }
 
 // LDS layout of a DR x DC matrix operand M: fragment f = (b*KS + s)*2 + hl holds,
