@@ -91,6 +91,11 @@ int rows_chunk(const Prob& p, int DR, int DC);
 // vector [N*H,DK] directly instead of a partial (no reduce step needed)
 void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
            int chunk, int nchunks, hipStream_t st, float* fin_mat = nullptr, float* fin_vec = nullptr);
+// The state partials (as `state` with kd = kn, no final store) plus the block statistics of
+// piecewise attention: per 64-token block the mean key kc [N*H, NT, DK] and the value sum
+// vc [N*H, NT, DV] (fp32).  chunk must be a multiple of 64.
+void state_with_block_stats(const Prob& p, int dtype, const void* k, const void* v, float* partial,
+                            int chunk, int nchunks, float* kc, float* vc, int NT, hipStream_t st);
 // out_t = (x_t M) / (xden_t . km + eps) + addvec   with M of shape DR x DC
 int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st);
 int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, int DR, int DC,

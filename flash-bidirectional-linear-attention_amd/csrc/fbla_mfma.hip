@@ -331,14 +331,26 @@ __device__ __forceinline__ void reduce_store_block(f32x16 (&acc)[2][2], float (&
 #ifndef FBLA_STATE128_TILES
 #define FBLA_STATE128_TILES 1
 #endif
-template <typename T, int DK, int DV, bool SPLIT_KD, int TILES, bool SCALED>
+// STATS = true additionally writes, for every 64-token block of the sequence, the mean key
+// (kc [N*H, NT, DK]) and the value sum (vc [N*H, NT, DV]): the block statistics of piecewise
+// attention.  The waves then walk whole 64-token blocks (four tiles in a row) instead of
+// interleaving single tiles, so that a block's sums stay inside one wave.
+struct BlockStats {
+  float* kc;
+  float* vc;
+  int NT;
+};
+
+template <typename T, int DK, int DV, bool SPLIT_KD, int TILES, bool SCALED, bool STATS = false>
 __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2) void state_kernel(Prob p, const T* __restrict__ kn,
                                                          const T* __restrict__ v,
                                                          const T* __restrict__ kd,
                                                          float* __restrict__ partial,
                                                          const float* __restrict__ tokscal,
                                                          int64_t total_rows, float* fin_mat,
-                                                         float* fin_vec, int chunk, int nchunks) {
+                                                         float* fin_vec, int chunk, int nchunks,
+                                                         BlockStats stats) {
+  static_assert(!STATS || (TILES == 1 && !SCALED && !SPLIT_KD), "block statistics: plain variant only");
   // The state is tiled into 64 x 64 blocks (64 accumulator registers per lane); a block is
   // owned by G waves that take interleaved token tiles.  For a 128 x 128 state the four
   // waves of the workgroup therefore read the same tokens, each the 64 key and 64 value
@@ -385,6 +397,7 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
   float ks[CK];
 #pragma unroll
   for (int a = 0; a < CK; ++a) ks[a] = 0.f;
+  float kcs[CK] = {0.f, 0.f}, vcs[CV] = {0.f, 0.f};  // STATS: sums over the current 64-token block
 
   // Each wave walks TILES consecutive 16-token tiles per step, the steps of the G waves
   // interleaved.  Two register buffers alternate (the loop is unrolled by two so that no
@@ -447,6 +460,7 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
       for (int u = 0; u < TILES; ++u) {
         const int lo = min(16, tok + 16 * u - min(tok + 16 * u, t_end - 16));
         mask_rows<CK>(b.k[u], 8 * kb, lo);
+        if constexpr (STATS) mask_rows<CV>(b.v[u], 8 * kb, lo);
         if constexpr (SPLIT_KD) mask_rows<CK>(b.d[u], 8 * kb, lo);
         if constexpr (SCALED) {
 #pragma unroll
@@ -504,6 +518,19 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
           for (int a = 0; a < CK; ++a)
 #pragma unroll
             for (int i = 0; i < 4; ++i) ks[a] = Ops<T>::dot2(Dd[a][i], Ops<T>::kOnes, ks[a]);
+        } else if constexpr (STATS) {
+#pragma unroll
+          for (int a = 0; a < CK; ++a) {
+            float tk = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) tk = Ops<T>::dot2(A[a][i], Ops<T>::kOnes, tk);
+            ks[a] += tk;
+            kcs[a] += tk;
+          }
+#pragma unroll
+          for (int bb = 0; bb < CV; ++bb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) vcs[bb] = Ops<T>::dot2(B[bb][i], Ops<T>::kOnes, vcs[bb]);
         } else {
 #pragma unroll
           for (int a = 0; a < CK; ++a)
@@ -512,8 +539,33 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
         }
       }
     }
+    if constexpr (STATS) {
+      // last tile of its 64-token block (or of the sequence): write the block's statistics
+      if (((tok + 16) & 63) == 0 || tok + 16 >= t_end) {
+        const int cb = tok >> 6;
+        const float inv_n = 1.0f / (float)min(64, len - 64 * cb);
+        const int64_t slot = (int64_t)nh * stats.NT + cb;
+#pragma unroll
+        for (int a = 0; a < CK; ++a) {
+          const float tot = kcs[a] + __shfl_xor(kcs[a], 32);
+          if (kb == 0 && bv == 0) stats.kc[slot * DK + 64 * bk + CK * pp + a] = tot * inv_n;
+          kcs[a] = 0.f;
+        }
+#pragma unroll
+        for (int bb = 0; bb < CV; ++bb) {
+          const float tot = vcs[bb] + __shfl_xor(vcs[bb], 32);
+          if (kb == 0 && bk == 0) stats.vc[slot * DV + 64 * bv + CV * pp + bb] = tot;
+          vcs[bb] = 0.f;
+        }
+      }
+    }
   };
-  int t0 = t_begin + kStep * g;
+  // token walk: single tiles interleaved over the G waves, or (STATS) whole 64-token blocks
+  auto next = [&](int t) {
+    if constexpr (STATS) return ((t + 16) & 63) ? t + 16 : t + 16 + 64 * (G - 1);
+    else return t + kStep * G;
+  };
+  int t0 = t_begin + (STATS ? 64 : kStep) * g;
   if (t_end - t_begin < 16) {
     if (t0 < t_end) {
       Buf b0;
@@ -524,13 +576,15 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
     Buf b0, b1;
     fetch(b0, t0);
     while (true) {
-      fetch(b1, t0 + kStep * G);
+      int tn = next(t0);
+      fetch(b1, tn);
       compute(b0, t0, false);
-      t0 += kStep * G;
+      t0 = tn;
       if (t0 >= t_end) break;
-      fetch(b0, t0 + kStep * G);
+      tn = next(t0);
+      fetch(b0, tn);
       compute(b1, t0, false);
-      t0 += kStep * G;
+      t0 = tn;
       if (t0 >= t_end) break;
     }
   }
@@ -1274,26 +1328,28 @@ int rows_chunk(const Prob& p, int DR, int DC) {
 template <typename T, int DK, int DV>
 static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, float* partial,
                          const float* tokscal, int64_t total_rows, float* fm, float* fv, int chunk,
-                         int nchunks, hipStream_t st) {
+                         int nchunks, BlockStats bs, hipStream_t st) {
   const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(kThreads);
   constexpr int TL = (DK == 128 && DV == 128) ? FBLA_STATE128_TILES : 1;
-  if (tokscal)
-    state_kernel<T, DK, DV, false, TL, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fm, fv, chunk, nchunks);
+  if (bs.kc)
+    state_kernel<T, DK, DV, false, 1, false, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
+  else if (tokscal)
+    state_kernel<T, DK, DV, false, TL, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fm, fv, chunk, nchunks, bs);
   else if (p.flags & kDecoupled)
-    state_kernel<T, DK, DV, true, TL, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks);
+    state_kernel<T, DK, DV, true, TL, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
   else
-    state_kernel<T, DK, DV, false, TL, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks);
+    state_kernel<T, DK, DV, false, TL, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
 }
 
 template <typename T>
 static void run_state(const Prob& p, const void* kn, const void* v, const void* kd, float* partial,
                       const float* ts, int64_t rows, float* fm, float* fv, int chunk, int nchunks,
-                      hipStream_t st) {
+                      BlockStats bs, hipStream_t st) {
   const T *a = (const T*)kn, *b = (const T*)v, *c = (const T*)kd;
-  if (p.DK == 64 && p.DV == 64) launch_state<T, 64, 64>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, st);
-  else if (p.DK == 64) launch_state<T, 64, 128>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, st);
-  else if (p.DV == 64) launch_state<T, 128, 64>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, st);
-  else launch_state<T, 128, 128>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, st);
+  if (p.DK == 64 && p.DV == 64) launch_state<T, 64, 64>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
+  else if (p.DK == 64) launch_state<T, 64, 128>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
+  else if (p.DV == 64) launch_state<T, 128, 64>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
+  else launch_state<T, 128, 128>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
 }
 
 // Reserves the kernel's dynamic LDS once per instantiation and thread.
@@ -1351,17 +1407,26 @@ static int run_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, int 
 
 void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
            int chunk, int nchunks, hipStream_t st, float* fin_mat, float* fin_vec) {
-  if (dtype == kF16) run_state<_Float16>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks, st);
-  else run_state<__bf16>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks, st);
+  const BlockStats none{nullptr, nullptr, 0};
+  if (dtype == kF16) run_state<_Float16>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks, none, st);
+  else run_state<__bf16>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks, none, st);
+}
+
+void state_with_block_stats(const Prob& p, int dtype, const void* k, const void* v, float* partial,
+                            int chunk, int nchunks, float* kc, float* vc, int NT, hipStream_t st) {
+  const BlockStats bs{kc, vc, NT};
+  if (dtype == kF16) run_state<_Float16>(p, k, v, k, partial, nullptr, 0, nullptr, nullptr, chunk, nchunks, bs, st);
+  else run_state<__bf16>(p, k, v, k, partial, nullptr, 0, nullptr, nullptr, chunk, nchunks, bs, st);
 }
 
 void scaled_state(const Prob& p, int dtype, const void* qn, const void* dout, const float* tokscal,
                   int64_t total_rows, float* partial, int chunk, int nchunks, hipStream_t st,
                   float* fin_mat, float* fin_vec) {
+  const BlockStats none{nullptr, nullptr, 0};
   if (dtype == kF16)
-    run_state<_Float16>(p, qn, dout, qn, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, st);
+    run_state<_Float16>(p, qn, dout, qn, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, none, st);
   else
-    run_state<__bf16>(p, qn, dout, qn, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, st);
+    run_state<__bf16>(p, qn, dout, qn, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, none, st);
 }
 
 int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {

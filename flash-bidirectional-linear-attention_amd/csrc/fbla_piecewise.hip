@@ -58,13 +58,14 @@ typedef uint32_t u32x4s __attribute__((ext_vector_type(4)));
 template <typename T, int D>
 __global__ __launch_bounds__(kThreads) void chunk_sums16_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, float* __restrict__ qc,
-    float* __restrict__ kc, float* __restrict__ vc, int64_t BH, int Tn, int NT, int chunk) {
+    float* __restrict__ kc, float* __restrict__ vc, int64_t BH, int Tn, int NT, int chunk, int nten) {
+  // nten = 3: q, k and v; nten = 1: q only (k and v statistics come from the state kernel)
   constexpr int CH = D / 8, RPI = 64 / CH;  // chunks per row, rows per wave instruction
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t item = (int64_t)blockIdx.x * 4 + wave;
-  if (item >= BH * NT * 3) return;
-  const int which = (int)(item % 3);
-  const int64_t bc = item / 3;
+  if (item >= BH * NT * nten) return;
+  const int which = (int)(item % nten);
+  const int64_t bc = item / nten;
   const int c = (int)(bc % NT);
   const int64_t bh = bc / NT;
   const T* src = (which == 0 ? q : which == 1 ? k : v) + (bh * Tn + (int64_t)c * chunk) * D;
@@ -728,20 +729,19 @@ size_t chunk_reduce_workspace_bytes(int64_t BH, int64_t T, int K, int V, int chu
 
 template <typename T>
 static void launch_sums(const void* q, const void* k, const void* v, float* qc, float* kc, float* vc,
-                        int64_t BH, int Tn, int NT, int chunk, int K, int V, hipStream_t st) {
-  const int64_t items = BH * NT * 3;
+                        int64_t BH, int Tn, int NT, int chunk, int K, int V, bool q_only, hipStream_t st) {
   if constexpr (sizeof(T) == 2) {
-    const dim3 grid((unsigned)cdiv64(items, 4)), block(kThreads);
-    if (K == 64 && V == 64) {
-      chunk_sums16_kernel<T, 64><<<grid, block, 0, st>>>((const T*)q, (const T*)k, (const T*)v, qc, kc, vc, BH, Tn, NT, chunk);
-      return;
-    }
-    if (K == 128 && V == 128) {
-      chunk_sums16_kernel<T, 128><<<grid, block, 0, st>>>((const T*)q, (const T*)k, (const T*)v, qc, kc, vc, BH, Tn, NT, chunk);
+    if ((K == 64 || K == 128) && (q_only || V == K)) {
+      const int nten = q_only ? 1 : 3;
+      const dim3 grid((unsigned)cdiv64(BH * NT * nten, 4)), block(kThreads);
+      if (K == 64)
+        chunk_sums16_kernel<T, 64><<<grid, block, 0, st>>>((const T*)q, (const T*)k, (const T*)v, qc, kc, vc, BH, Tn, NT, chunk, nten);
+      else
+        chunk_sums16_kernel<T, 128><<<grid, block, 0, st>>>((const T*)q, (const T*)k, (const T*)v, qc, kc, vc, BH, Tn, NT, chunk, nten);
       return;
     }
   }
-  chunk_sums_kernel<T><<<dim3((unsigned)cdiv64(items, 4)), dim3(kThreads), 0, st>>>(
+  chunk_sums_kernel<T><<<dim3((unsigned)cdiv64(BH * NT * 3, 4)), dim3(kThreads), 0, st>>>(
       (const T*)q, (const T*)k, (const T*)v, qc, kc, vc, BH, Tn, NT, chunk, K, V);
 }
 
@@ -754,10 +754,14 @@ int chunk_reduce(const void* q, const void* k, const void* v, float* qc, float* 
   const int sc = state_chunk_for(p, dtype, chunk, per_chunk);
   const int nparts = (int)cdiv64(T, sc);
   float* partial = (float*)workspace;
-  if (dtype == kF16) launch_sums<_Float16>(q, k, v, qc, kc, vc, BH, (int)T, NT, chunk, K, V, st);
-  else if (dtype == kBF16) launch_sums<__bf16>(q, k, v, qc, kc, vc, BH, (int)T, NT, chunk, K, V, st);
-  else launch_sums<float>(q, k, v, qc, kc, vc, BH, (int)T, NT, chunk, K, V, st);
-  if (mfma::supported(p, dtype)) mfma::state(p, dtype, k, v, k, partial, sc, nparts, st);
+  // 16-bit, MFMA-sized heads, 64-token blocks: k and v are read once, by the state kernel,
+  // which also writes their block statistics; q has its own streaming pass
+  const bool fused = mfma::supported(p, dtype) && chunk == 64 && !per_chunk;
+  if (dtype == kF16) launch_sums<_Float16>(q, k, v, qc, kc, vc, BH, (int)T, NT, chunk, K, V, fused, st);
+  else if (dtype == kBF16) launch_sums<__bf16>(q, k, v, qc, kc, vc, BH, (int)T, NT, chunk, K, V, fused, st);
+  else launch_sums<float>(q, k, v, qc, kc, vc, BH, (int)T, NT, chunk, K, V, false, st);
+  if (fused) mfma::state_with_block_stats(p, dtype, k, v, partial, sc, nparts, kc, vc, NT, st);
+  else if (mfma::supported(p, dtype)) mfma::state(p, dtype, k, v, k, partial, sc, nparts, st);
   else generic::state_partial(p, dtype, k, v, k, partial, sc, nparts, st);
   if (per_chunk)
     chunk_norm_kernel<<<dim3((unsigned)(BH * NT)), dim3(kThreads), 0, st>>>(partial, kc, vc, h_norm, K,
