@@ -291,4 +291,30 @@ int fbla_piecewise_fwd(const void* q, const void* k, const void* v, const float*
   return check_launch(what);
 }
 
+int fbla_select_blocks(const float* qc, const float* kc, const float* bias, int32_t* indices,
+                       int64_t BH, int64_t NT, int K, int NS, float scale, void* stream) {
+  const char* what = "fbla_select_blocks";
+  if (BH < 0 || NT < 0 || NT > 0x7fffffffLL / 64) {
+    set_error("%s: bad sizes BH=%lld NT=%lld", what, (long long)BH, (long long)NT);
+    return kErrBadArg;
+  }
+  if (BH == 0 || NT == 0) return kOk;
+  if (NS < 1 || NS > NT) {
+    set_error("%s: the number of selected blocks must be in [1, %lld], got %d", what, (long long)NT, NS);
+    return kErrBadArg;
+  }
+  if (!piecewise::select_blocks_supported((int)NT, K)) {
+    set_error("%s: needs K in {64,128} and a score row that fits LDS (got K=%d NT=%lld)", what, K,
+              (long long)NT);
+    return kErrUnsupported;
+  }
+  if (!qc || !kc || !indices) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  int rc = piecewise::select_blocks(qc, kc, bias, indices, BH, (int)NT, K, NS, scale, (hipStream_t)stream);
+  if (rc != kOk) return rc;
+  return check_launch(what);
+}
+
 }  // extern "C"

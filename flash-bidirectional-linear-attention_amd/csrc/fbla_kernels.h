@@ -121,6 +121,10 @@ size_t chunk_reduce_workspace_bytes(int64_t BH, int64_t T, int K, int V, int chu
 int chunk_reduce(const void* q, const void* k, const void* v, float* qc, float* kc, float* vc,
                  float* h, float* h_norm, void* workspace, int64_t BH, int64_t T, int K, int V,
                  int chunk, float pnorm, int dtype, hipStream_t st);
+// top-NS key blocks per query block from the block means (ascending block order)
+bool select_blocks_supported(int NT, int K);
+int select_blocks(const float* qc, const float* kc, const float* bias, int32_t* indices, int64_t BH,
+                  int NT, int K, int NS, float scale, hipStream_t st);
 bool attention_supported(int K, int V, int block, int dtype);
 size_t attention_workspace_bytes(int64_t BH, int64_t T, int K, int V);
 int attention(const void* q, const void* k, const void* v, const float* kc, const float* vc,

@@ -697,6 +697,143 @@ __global__ __launch_bounds__(kThreads) void split_hi_lo_t_kernel(const float* __
   }
 }
 
+// ===========================================================================
+// block selection (replaces score = qc (kc*scale)^T; torch.topk, kernel.py:304-318)
+// ===========================================================================
+// One workgroup per (head, 16 query blocks).  Scores of its 16 rows against all NT key
+// blocks are computed with fp32 FMAs out of LDS tiles (64 key blocks at a time) and kept in
+// LDS; then every wave selects, for four of the rows, the NS largest scores: the threshold
+// (the NS-th largest value) comes from a bitwise descent over the order-preserving integer
+// image of the floats with wave-wide counts, and the selected block indices are written in
+// ascending index order (ties at the threshold: lower index first).  With a bias (the
+// per-block norms), log(bias + 1e-5) is added to the score: the softmax of the reference
+// (kernel.py:314-315) is monotonic per row and does not change the selection.
+constexpr int kSelRows = 16, kSelKeys = 64;
+
+__device__ __forceinline__ uint32_t order_bits(float x) {
+  const uint32_t b = __builtin_bit_cast(uint32_t, x);
+  return b ^ ((b >> 31) ? 0xffffffffu : 0x80000000u);
+}
+
+template <int K>
+__global__ __launch_bounds__(kThreads) void select_blocks_kernel(
+    const float* __restrict__ qc, const float* __restrict__ kc, const float* __restrict__ bias,
+    int32_t* __restrict__ indices, int NT, int NS, float scale) {
+  constexpr int KLD = K + 4;  // padded key rows: 16-byte reads of 16 lanes hit 16 bank groups
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float* qs = reinterpret_cast<float*>(smem);          // [16][K]
+  float* kt = qs + kSelRows * K;                       // [64][K + 4]
+  float* sc = kt + kSelKeys * KLD;                     // [16][NTs]
+  const int NTs = (NT + 63) & ~63;
+  const int nrt = (NT + kSelRows - 1) / kSelRows;
+  const int r0 = (blockIdx.x % nrt) * kSelRows;
+  const int64_t bh = blockIdx.x / nrt;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const float* qh = qc + bh * NT * K;
+  const float* kh = kc + bh * NT * K;
+  typedef float f4 __attribute__((ext_vector_type(4)));
+
+  for (int e = tid; e < kSelRows * (K / 4); e += kThreads) {
+    const int row = e / (K / 4), c4 = e % (K / 4);
+    f4 x = f4{0.f, 0.f, 0.f, 0.f};
+    if (r0 + row < NT) x = *reinterpret_cast<const f4*>(qh + (int64_t)(r0 + row) * K + 4 * c4);
+    *reinterpret_cast<f4*>(qs + row * K + 4 * c4) = x;
+  }
+  for (int j0 = 0; j0 < NT; j0 += kSelKeys) {
+    __syncthreads();  // previous tile consumed (first trip: nothing to wait for but cheap)
+    for (int e = tid; e < kSelKeys * (K / 4); e += kThreads) {
+      const int row = e / (K / 4), c4 = e % (K / 4);
+      f4 x = f4{0.f, 0.f, 0.f, 0.f};
+      if (j0 + row < NT) x = *reinterpret_cast<const f4*>(kh + (int64_t)(j0 + row) * K + 4 * c4);
+      *reinterpret_cast<f4*>(kt + row * KLD + 4 * c4) = x;
+    }
+    __syncthreads();
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;  // rows 4*wave .. +3 against key j0 + lane
+    const float* kr = kt + lane * KLD;
+    const float* q0 = qs + (4 * wave) * K;
+#pragma unroll 4
+    for (int d = 0; d < K; d += 4) {
+      const f4 kv = *reinterpret_cast<const f4*>(kr + d);
+      const f4 x0 = *reinterpret_cast<const f4*>(q0 + d);
+      const f4 x1 = *reinterpret_cast<const f4*>(q0 + K + d);
+      const f4 x2 = *reinterpret_cast<const f4*>(q0 + 2 * K + d);
+      const f4 x3 = *reinterpret_cast<const f4*>(q0 + 3 * K + d);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a0 = fmaf(x0[i], kv[i], a0);
+        a1 = fmaf(x1[i], kv[i], a1);
+        a2 = fmaf(x2[i], kv[i], a2);
+        a3 = fmaf(x3[i], kv[i], a3);
+      }
+    }
+    const int key = j0 + lane;
+    const float off = key < NT ? (bias ? logf(bias[bh * NT + key] + 1e-5f) : 0.f) : -__builtin_huge_valf();
+    sc[(4 * wave + 0) * NTs + key] = key < NT ? a0 * scale + off : off;
+    sc[(4 * wave + 1) * NTs + key] = key < NT ? a1 * scale + off : off;
+    sc[(4 * wave + 2) * NTs + key] = key < NT ? a2 * scale + off : off;
+    sc[(4 * wave + 3) * NTs + key] = key < NT ? a3 * scale + off : off;
+  }
+  __syncthreads();
+
+  for (int rr = 0; rr < 4; ++rr) {
+    const int row = 4 * wave + rr;
+    if (r0 + row >= NT) break;  // uniform over the wave
+    const float* srow = sc + row * NTs;
+    // threshold: greatest t with count(u >= t) >= NS
+    uint32_t thr = 0;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t t = thr | (1u << bit);
+      int cnt = 0;
+      for (int j = lane; j < NTs; j += 64) cnt += __popcll(__ballot(order_bits(srow[j]) >= t));
+      if (cnt >= NS) thr = t;
+    }
+    int above = 0;
+    for (int j = lane; j < NTs; j += 64) above += __popcll(__ballot(order_bits(srow[j]) > thr));
+    int ties_left = NS - above, written = 0;
+    int32_t* dst = indices + (bh * NT + (r0 + row)) * (int64_t)NS;
+    for (int j = lane; j < NTs; j += 64) {
+      const uint32_t u = order_bits(srow[j]);
+      const uint64_t tie_mask = __ballot(u == thr);
+      const int tie_rank = __popcll(tie_mask & ((1ull << lane) - 1ull));
+      const bool take = u > thr || (u == thr && tie_rank < ties_left);
+      const uint64_t take_mask = __ballot(take);
+      if (take) dst[written + __popcll(take_mask & ((1ull << lane) - 1ull))] = j;
+      written += __popcll(take_mask);
+      ties_left -= min(ties_left, (int)__popcll(tie_mask));
+    }
+  }
+}
+
+size_t select_blocks_lds_bytes(int NT, int K) {
+  const int NTs = (NT + 63) & ~63;
+  return (size_t)(kSelRows * K + kSelKeys * (K + 4) + kSelRows * NTs) * sizeof(float);
+}
+
+bool select_blocks_supported(int NT, int K) {
+  return (K == 64 || K == 128) && select_blocks_lds_bytes(NT, K) <= 160 * 1024;
+}
+
+int select_blocks(const float* qc, const float* kc, const float* bias, int32_t* indices, int64_t BH,
+                  int NT, int K, int NS, float scale, hipStream_t st) {
+  const int lds = (int)select_blocks_lds_bytes(NT, K);
+  const int nrt = (NT + kSelRows - 1) / kSelRows;
+  const dim3 grid((unsigned)(BH * nrt)), block(kThreads);
+  auto run = [&](auto kernel) {
+    if (lds > 64 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      if (e != hipSuccess) {
+        set_error("block selection: cannot reserve %d bytes of LDS: %s", lds, hipGetErrorString(e));
+        return (int)kErrLaunch;
+      }
+    }
+    kernel<<<grid, block, lds, st>>>(qc, kc, bias, indices, NT, NS, scale);
+    return (int)kOk;
+  };
+  if (K == 64) return run(select_blocks_kernel<64>);
+  return run(select_blocks_kernel<128>);
+}
+
 static Prob dense_prob(int64_t BH, int64_t T, int K, int V) {
   Prob p;
   p.cu = nullptr;

@@ -34,6 +34,7 @@ _SIGNATURES = {
     "fbla_varlen_bwd": (_i32, [_vp] * 11 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_chunk_reduce_workspace_bytes": (_sz, [_i64, _i64, _i32, _i32, _i32, _i32, _i32]),
     "fbla_chunk_reduce": (_i32, [_vp] * 9 + [_sz, _i64, _i64, _i32, _i32, _i32, _f32, _i32, _vp]),
+    "fbla_select_blocks": (_i32, [_vp] * 4 + [_i64, _i64, _i32, _i32, _f32, _vp]),
     "fbla_piecewise_workspace_bytes": (_sz, [_i64, _i64, _i32, _i32, _i32, _i32]),
     "fbla_piecewise_fwd": (_i32, [_vp] * 9 + [_sz, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
 }
@@ -204,6 +205,20 @@ def chunk_reduce(q, k, v, chunk, with_norm=False, p_norm=2.0):
                                  float(p_norm), code, _stream(dev))
     _check(rc, "fbla_chunk_reduce")
     return qc, kc, vc, h, h_norm
+
+
+def select_blocks(qc, kc, bias, top_k, scale):
+    """Indices (int32, ascending) of the top_k key blocks per query block; qc, kc fp32 [B,H,NT,K]."""
+    _require_gpu(qc, kc, bias)
+    L = lib()
+    B, H, NT, K = qc.shape
+    dev = qc.device
+    idx = torch.empty(B, H, NT, top_k, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = L.fbla_select_blocks(_ptr(qc), _ptr(kc), _ptr(bias), _ptr(idx), B * H, NT, K, top_k,
+                                  float(scale), _stream(dev))
+    _check(rc, "fbla_select_blocks")
+    return idx
 
 
 def piecewise_supported(q, v, block):

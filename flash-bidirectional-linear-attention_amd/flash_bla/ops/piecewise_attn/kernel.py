@@ -42,13 +42,16 @@ def chunk_reduce_fp32(q, k, v, chunk_size, use_bias=False, p=2):
 
 
 def select_blocks(qc, kc, scale, density, bias=None):
-    """Top-k key blocks per query block (kernel.py:313-318): int64 indices `(B,H,N,top_k)`."""
+    """Top-k key blocks per query block (kernel.py:304-318): int32 indices `(B,H,N,top_k)` in
+    ascending block order (the reference's torch.topk orders them by score; the attention
+    result does not depend on the order).  `bias`: optional per-block norms `(B,H,N)`."""
     NT = qc.shape[-2]
-    score = torch.einsum('bhid,bhjd->bhij', qc, kc * scale)
-    if bias is not None:
-        score = torch.softmax(score + torch.log(bias + 1e-5), dim=-1)
     top_k = max(1, int(density * NT))
-    return torch.topk(score, k=top_k, dim=-1).indices
+    qc = qc.float().contiguous()
+    kc = kc.float().contiguous()
+    if bias is not None:
+        bias = bias.float().contiguous()
+    return _hip.select_blocks(qc, kc, bias, top_k, scale)
 
 
 def piecewise_sparse_attention(q, k, v, density=0.1, block_size=64, scale=None, use_bias=False,

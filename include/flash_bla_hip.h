@@ -133,6 +133,17 @@ int fbla_chunk_reduce(const void* q, const void* k, const void* v, float* qc, fl
                       float* h, float* h_norm, void* workspace, size_t workspace_bytes, int64_t BH,
                       int64_t T, int K, int V, int chunk, float p_norm, int dtype, void* stream);
 
+/* Block selection.  Replaces the score matrix and torch.topk of the wrapper
+ * (flash_bla/ops/piecewise_attn/kernel.py:304-318): for every query block the NS key blocks
+ * with the largest qc . kc * scale (+ log(bias + 1e-5) when bias [BH,NT], the h_norm output
+ * of fbla_chunk_reduce, is given; kernel.py:314-315 applies a softmax on top, which does not
+ * change the order).  qc, kc: fp32 [BH,NT,K] from fbla_chunk_reduce; indices: int32
+ * [BH,NT,NS], written in ascending block order (torch.topk orders by score; the attention
+ * result does not depend on the order); ties at the threshold go to the lower block index.
+ * K in {64,128}. */
+int fbla_select_blocks(const float* qc, const float* kc, const float* bias, int32_t* indices,
+                       int64_t BH, int64_t NT, int K, int NS, float scale, void* stream);
+
 /* Workspace of fbla_piecewise_fwd; 0 when the shape is not supported. */
 size_t fbla_piecewise_workspace_bytes(int64_t BH, int64_t T, int K, int V, int block, int dtype);
 

@@ -106,3 +106,42 @@ def test_use_bias_selection_and_errors():
         piecewise_sparse_attention(q.cuda(), k.cuda(), v.cuda(), block_size=32)
     with pytest.raises(ValueError):
         piecewise_sparse_attention(q, k, v)
+
+
+@pytest.mark.parametrize("NT,K,top_density", [(256, 128, 0.25), (37, 64, 0.3), (1, 64, 1.0), (130, 128, 0.01),
+                                              (64, 64, 1.0)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_block_selection_matches_topk(NT, K, top_density, with_bias):
+    """The selection kernel against torch.topk on the same fp32 scores, as sets (torch orders
+    by score, the kernel by block index); random scores have no ties."""
+    from flash_bla.ops.piecewise_attn.kernel import select_blocks
+    g = torch.Generator().manual_seed(NT * 7 + K)
+    qc = torch.randn(2, 3, NT, K, generator=g).cuda()
+    kc = torch.randn(2, 3, NT, K, generator=g).cuda()
+    bias = (torch.rand(2, 3, NT, generator=g) * 4 + 0.1).cuda() if with_bias else None
+    scale = K ** -0.5
+    idx = select_blocks(qc, kc, scale, top_density, bias)
+    top_k = max(1, int(top_density * NT))
+    assert idx.dtype == torch.int32 and idx.shape == (2, 3, NT, top_k)
+    score = torch.einsum('bhid,bhjd->bhij', qc.double(), kc.double() * scale)
+    if with_bias:
+        score = score + torch.log(bias.double() + 1e-5).unsqueeze(-2)
+    want = torch.topk(score, k=top_k, dim=-1).indices.sort(dim=-1).values
+    got = idx.long()
+    assert (got[..., 1:] > got[..., :-1]).all(), "indices must be strictly ascending"
+    mismatch = (got != want).any(dim=-1)
+    if mismatch.any():  # fp32 vs fp64 scores may swap two blocks whose scores agree to ~1e-6
+        kth = torch.topk(score, k=min(top_k + 1, NT), dim=-1).values
+        gap = (kth[..., top_k - 1] - kth[..., -1]).abs() if top_k < NT else torch.ones_like(kth[..., 0])
+        assert (gap[mismatch] < 1e-4).all()
+
+
+def test_block_selection_ties_go_to_lower_index():
+    from flash_bla.ops.piecewise_attn.kernel import select_blocks
+    NT, K = 96, 64
+    qc = torch.ones(1, 1, NT, K).cuda()
+    kc = torch.zeros(1, 1, NT, K)
+    kc[0, 0, 10] = 1.0   # one clear winner, everything else ties at 0
+    idx = select_blocks(qc, kc.cuda(), 1.0, 5 / NT)
+    assert idx.shape[-1] == 5
+    assert (idx.cpu() == torch.tensor([0, 1, 2, 3, 10], dtype=torch.int32)).all()
