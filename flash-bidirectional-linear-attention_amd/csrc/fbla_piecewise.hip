@@ -288,12 +288,14 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
   constexpr int KCH = K / 8;                 // 16-byte chunks per K tile row
   constexpr int KS = K / 16;                 // k-steps of the score product
   constexpr int MB = V / 32;                 // 32-row blocks of O^T
-  constexpr int KLD = 64 * KCH / kThreads;   // 16-byte chunks per thread per K tile
-  constexpr int VLD = V * 8 / kThreads;      // ... per V^T tile
   constexpr int OLD = 64 * (V / 8) / kThreads;
   constexpr float kNegInf = -__builtin_huge_valf();
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  unsigned char* sel = smem + LY::kTiles;
+  // Two tile sets as two separate LDS objects: the compiler can then tell that a tile load
+  // in flight towards one set does not touch the set being read, and does not make the reads
+  // wait for it.  The selected-block bitmap is the dynamic part.
+  __shared__ __attribute__((aligned(1024))) unsigned char set_a[LY::kSet];
+  __shared__ __attribute__((aligned(1024))) unsigned char set_b[LY::kSet];
+  extern __shared__ __attribute__((aligned(16))) unsigned char sel[];
 
   const int tq = blockIdx.x % a.NT;
   const int64_t bh = blockIdx.x / a.NT;
@@ -342,40 +344,33 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
   auto vswz = [&](int row, int ch) { return swz128(row, ch); };
   auto oswz = [&](int row, int ch) { return V == 128 ? swz256(row, ch) : swz128(row, ch); };
 
-  // Tiles are fetched with buffer loads: one lane offset register, the tile / row-group
-  // offsets are scalars, and rows past the end of the tensor come back as zero (the
-  // descriptor's byte count is the bounds check).
-  const uint32_t k_lane_off = (uint32_t)(((tid / KCH) * K + (tid % KCH) * 8) * 2);
-  auto load_tile_k = [&](u32x4(&dst)[KLD], __amdgpu_buffer_rsrc_t rs, int row0) {
+  // Tiles go from global memory straight into LDS (buffer load with the LDS destination:
+  // lane l of a wave instruction delivers 16 bytes to destination + 16*l, so one instruction
+  // fills 1 KiB = 4 or 8 whole tile rows).  The swizzle is applied on the global side: the
+  // lane that owns LDS slot s of row r fetches chunk s ^ swizzle(r).  Rows past the end of
+  // the tensor arrive as zeros (the descriptor's byte count is the bounds check).
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  constexpr int KROWB = K * 2, KRW = 1024 / KROWB, KJ = 64 / (4 * KRW);
+  const int krow_l = KRW * wave + lane / (KROWB / 16), kslot = lane % (KROWB / 16);
+  const uint32_t k_lane_off =
+      (uint32_t)(krow_l * KROWB + ((kslot ^ (K == 128 ? (krow_l & 15) : ((krow_l >> 1) & 7))) << 4));
+  auto dma_tile_k = [&](__amdgpu_buffer_rsrc_t rs, unsigned char* tile, int row0) {
 #pragma unroll
-    for (int j = 0; j < KLD; ++j)  // chunk tid + 256j: row tid/KCH + j*(256/KCH)
-      dst[j] = __builtin_amdgcn_raw_buffer_load_b128(
-          rs, k_lane_off, (row0 + j * (kThreads / KCH)) * (K * 2), 0);
+    for (int j = 0; j < KJ; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(tile + (4 * KRW * j + KRW * wave) * KROWB), 16,
+                                               k_lane_off, (row0 + 4 * KRW * j) * KROWB, 0, 0);
   };
-  auto store_tile_k = [&](const u32x4(&src)[KLD], unsigned char* tile) {
+  // V^T tile: V rows of 128 bytes (64 keys, permuted inside groups of 16 in global memory
+  // already); source row stride `ld` elements
+  constexpr int VJ = V / 32;
+  const int vrow_l = 8 * wave + (lane >> 3), vslot = lane & 7;
+  const uint32_t v_lane_chunk = (uint32_t)((vslot ^ ((vrow_l >> 1) & 7)) << 4);
+  auto dma_tile_v = [&](__amdgpu_buffer_rsrc_t rs, unsigned char* tile, int ld, int col0) {
+    const uint32_t lane_off = (uint32_t)(vrow_l * ld * 2) + v_lane_chunk;
 #pragma unroll
-    for (int j = 0; j < KLD; ++j) {
-      const int qq = tid + kThreads * j;
-      *reinterpret_cast<u32x4*>(tile + kswz(qq / KCH, qq % KCH)) = src[j];
-    }
-  };
-  // V^T tile: row = value column, 8 chunks of 8 keys; source row stride `ld` elements
-  auto load_tile_v = [&](u32x4(&dst)[VLD], __amdgpu_buffer_rsrc_t rs, int ld, int col0) {
-    const uint32_t lane_off = (uint32_t)(((tid >> 3) * ld + (tid & 7) * 8) * 2);
-#pragma unroll
-    for (int j = 0; j < VLD; ++j)  // chunk tid + 256j: row tid/8 + 32j
-      dst[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_off, (col0 + j * 32 * ld) * 2, 0);
-  };
-  // keys 8ch .. 8ch+7 of a row: (ch odd ? a = 1 : a = 0) half-groups b = 0, 1 go to positions
-  // 8b + 4a of 16-key group ch/2, i.e. chunk 2*(ch/2) + b, byte 8a
-  auto store_tile_v = [&](const u32x4(&src)[VLD], unsigned char* tile) {
-#pragma unroll
-    for (int j = 0; j < VLD; ++j) {
-      const int qq = tid + kThreads * j, row = qq >> 3, ch = qq & 7;
-      const int g2 = ch & ~1, aa = ch & 1;
-      *reinterpret_cast<u32x2p*>(tile + vswz(row, g2) + 8 * aa) = u32x2p{src[j][0], src[j][1]};
-      *reinterpret_cast<u32x2p*>(tile + vswz(row, g2 + 1) + 8 * aa) = u32x2p{src[j][2], src[j][3]};
-    }
+    for (int j = 0; j < VJ; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(tile + (32 * j + 8 * wave) * 128), 16, lane_off,
+                                               (col0 + 32 * j * ld) * 2, 0, 0);
   };
 
   // per-lane LDS offsets of the operand reads
@@ -403,17 +398,22 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
     f32x16 st, st2;
 #pragma unroll
     for (int r = 0; r < 16; ++r) st[r] = st2[r] = 0.f;
+    // all operand reads are issued before the first MFMA: their latencies overlap
+    u32x4 ak[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) ak[s] = *reinterpret_cast<const u32x4*>(kt0 + koff[s]);
 #pragma unroll
     for (int s = 0; s < KS; s += 2) {
-      const u32x4 ak = *reinterpret_cast<const u32x4*>(kt0 + koff[s]);
-      const u32x4 ak2 = *reinterpret_cast<const u32x4*>(kt0 + koff[s + 1]);
-      st = Mma32<T>::run(ak, qop[s], st);
-      st2 = Mma32<T>::run(ak2, qop[s + 1], st2);
-      if constexpr (weighted) {
-        const u32x4 al = *reinterpret_cast<const u32x4*>(kt1 + koff[s]);
-        const u32x4 al2 = *reinterpret_cast<const u32x4*>(kt1 + koff[s + 1]);
-        st = Mma32<T>::run(al, qop[s], st);
-        st2 = Mma32<T>::run(al2, qop[s + 1], st2);
+      st = Mma32<T>::run(ak[s], qop[s], st);
+      st2 = Mma32<T>::run(ak[s + 1], qop[s + 1], st2);
+    }
+    if constexpr (weighted) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) ak[s] = *reinterpret_cast<const u32x4*>(kt1 + koff[s]);
+#pragma unroll
+      for (int s = 0; s < KS; s += 2) {
+        st = Mma32<T>::run(ak[s], qop[s], st);
+        st2 = Mma32<T>::run(ak[s + 1], qop[s + 1], st2);
       }
     }
 #pragma unroll
@@ -466,98 +466,83 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
   auto values = [&](const unsigned char* vt0, const unsigned char* vt1, const u32x4(&pw)[2],
                     auto weighted_tag) {
     constexpr bool weighted = decltype(weighted_tag)::value;
+    u32x4 av[2][MB];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        const u32x4 av = *reinterpret_cast<const u32x4*>(vt0 + voff[t] + mb * (32 * 128));
-        acc[mb] = Mma32<T>::run(av, pw[t], acc[mb]);
-        if constexpr (weighted) {
-          const u32x4 al = *reinterpret_cast<const u32x4*>(vt1 + voff[t] + mb * (32 * 128));
-          acc[mb] = Mma32<T>::run(al, pw[t], acc[mb]);
-        }
-      }
+      for (int mb = 0; mb < MB; ++mb)
+        av[t][mb] = *reinterpret_cast<const u32x4*>(vt0 + voff[t] + mb * (32 * 128));
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) acc[mb] = Mma32<T>::run(av[t][mb], pw[t], acc[mb]);
+    if constexpr (weighted) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          av[t][mb] = *reinterpret_cast<const u32x4*>(vt1 + voff[t] + mb * (32 * 128));
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[mb] = Mma32<T>::run(av[t][mb], pw[t], acc[mb]);
+    }
   };
   const std::true_type yes{};
   const std::false_type no{};
 
-  // ---- phase 1: selected blocks.  Software pipeline: the value product of block i-1 is
-  // issued between the score product and the softmax of block i, so that the matrix unit
-  // works on it while the vector unit does the exponentials.  K and V^T tiles alternate
-  // between two LDS sets (the loop is unrolled by two: constant addresses); the tile of
-  // block i+1 travels through registers during block i and is stored between two barriers
-  // (its V^T slot held block i-1, which every wave has consumed by then).
-  u32x4 rk[KLD], rv[VLD];
+  // ---- phase 1: selected blocks.  The tile of block i+1 is in flight towards the other LDS
+  // set while block i is computed (the loop is unrolled by two: constant addresses).
   auto block_rows = [&](int b) { return b >= 0 && b < a.NT ? min(64, a.T - b * 64) : 0; };
-  {
-    const int b0 = idx[0], n0 = block_rows(b0);
-    load_tile_k(rk, k_rs, n0 ? b0 * 64 : 0);
-    load_tile_v(rv, vt_rs, Tp, n0 ? b0 * 64 : 0);
-    store_tile_k(rk, smem);
-    store_tile_v(rv, smem + LY::kKT);
-  }
-  __syncthreads();
-  u32x4 pw[2];
-  bool pending = false;  // pw holds the probabilities of the previous block, not yet multiplied
-  auto prefetch = [&](int i) {  // tile of selected block i -> registers
+  auto fetch_block = [&](int i, unsigned char* set) {
     if (i < a.NS) {
       const int bn = idx[i], nn = block_rows(bn);
-      load_tile_k(rk, k_rs, nn ? bn * 64 : 0);
-      load_tile_v(rv, vt_rs, Tp, nn ? bn * 64 : 0);
+      dma_tile_k(k_rs, set, nn ? bn * 64 : 0);
+      dma_tile_v(vt_rs, set + LY::kKT, Tp, nn ? bn * 64 : 0);
     }
   };
-  prefetch(1);
+  fetch_block(0, set_a);
+  __syncthreads();
+  u32x4 pw[2];
   auto step = [&](int i, unsigned char* cur, unsigned char* nxt) {
+    fetch_block(i + 1, nxt);
     const int nrows = block_rows(idx[i]);
     const auto none = [](int) { return 0.f; };
-    f32x16 st;
-    if (nrows > 0) st = scores(cur, cur, no);
-    if (pending) values(nxt + LY::kKT, nxt, pw, no);  // block i-1 lives in the other set
-    pending = nrows > 0;
-    if (nrows == 64)
+    if (nrows == 64) {
+      const f32x16 st = scores(cur, cur, no);
       softmax(st, pw, [](int) { return true; }, none, no, no);
-    else if (nrows > 0)
+      values(cur + LY::kKT, cur, pw, no);
+    } else if (nrows > 0) {
+      const f32x16 st = scores(cur, cur, no);
       softmax(st, pw, [&](int key) { return key < nrows; }, none, yes, no);
-    __syncthreads();
-    if (i + 1 < a.NS) {
-      store_tile_k(rk, nxt);
-      store_tile_v(rv, nxt + LY::kKT);
+      values(cur + LY::kKT, cur, pw, no);
     }
-    prefetch(i + 2);  // in flight during the barrier and all of the next block
     __syncthreads();
   };
   for (int i = 0; i < a.NS; i += 2) {
-    step(i, smem, smem + LY::kSet);
-    if (i + 1 < a.NS) step(i + 1, smem + LY::kSet, smem);
+    step(i, set_a, set_b);
+    if (i + 1 < a.NS) step(i + 1, set_b, set_a);
   }
-  if (pending) values(smem + ((a.NS - 1) & 1) * LY::kSet + LY::kKT, smem, pw, no);
-  __syncthreads();
 
   // ---- phase 2: unselected blocks through their means / sums ----
   const int last_len = a.T - (a.NT - 1) * 64;
   for (int grp = 0; grp * 64 < a.NT; ++grp) {
-    {
-      load_tile_k(rk, kch_rs, grp * 64);
-      store_tile_k(rk, smem);
-      load_tile_k(rk, kcl_rs, grp * 64);
-      store_tile_k(rk, smem + LY::kSet);
-      load_tile_v(rv, vch_rs, a.NTp, grp * 64);
-      store_tile_v(rv, smem + LY::kKT);
-      load_tile_v(rv, vcl_rs, a.NTp, grp * 64);
-      store_tile_v(rv, smem + LY::kSet + LY::kKT);
-    }
+    dma_tile_k(kch_rs, set_a, grp * 64);
+    dma_tile_k(kcl_rs, set_b, grp * 64);
+    dma_tile_v(vch_rs, set_a + LY::kKT, a.NTp, grp * 64);
+    dma_tile_v(vcl_rs, set_b + LY::kKT, a.NTp, grp * 64);
     __syncthreads();
     const int c0 = grp * 64;
-    const f32x16 st = scores(smem, smem + LY::kSet, yes);
+    const f32x16 st = scores(set_a, set_b, yes);
     softmax(st, pw, [&](int key) { return c0 + key < a.NT && !sel[c0 + key]; },
             [&](int key) { return c0 + key == a.NT - 1 ? (float)last_len : 64.f; }, yes, yes);
-    values(smem + LY::kKT, smem + LY::kSet + LY::kKT, pw, yes);
+    values(set_a + LY::kKT, set_b + LY::kKT, pw, yes);
     __syncthreads();
   }
 
   // ---- merge the two key halves: waves kh = 1 hand their state to waves kh = 0 ----
   float L = l_p + __shfl_xor(l_p, 32), G = g_p + __shfl_xor(g_p, 32);
-  float* mrg = reinterpret_cast<float*>(smem) + qh * (64 * (MB * 16 + 3));  // [value][lane]
+  float* mrg = reinterpret_cast<float*>(qh ? set_b : set_a);  // [value][lane], 64 * (16 MB + 3) floats
   if (kh == 1) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -583,8 +568,8 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
   __syncthreads();
 
   // ---- phase 3 and output (waves kh = 0): acc += (q H) * (G/T) * scale, o = acc / (L + G) ----
-  unsigned char* rt = smem;                 // q H tile [64][V]
-  unsigned char* ot = smem + 64 * V * 2;    // output tile [64][V]
+  unsigned char* rt = set_a;  // q H tile [64][V]
+  unsigned char* ot = set_b;  // output tile [64][V]
   {
     const T* rsrc = (const T*)a.r + (bh * a.T + (int64_t)tq * 64) * V;
     const int nrows = a.T - tq * 64;
@@ -646,11 +631,16 @@ __global__ __launch_bounds__(kThreads) void transpose_values_kernel(const T* __r
   T* dst = vt + bh * V * (int64_t)NT * 64 + (int64_t)tb * 64;
   for (int qq = threadIdx.x; qq < V * 8; qq += kThreads) {
     const int col = qq >> 3, ch = qq & 7;
+    // positions 8ch .. 8ch+7 of the row hold keys 16g + 4b + (0..3), 16g + 8 + 4b + (0..3)
+    // (g = ch/2, b = ch%2): the order in which the attention kernel's accumulator registers
+    // hold the keys of a group of 16
+    const int kb0 = 16 * (ch >> 1) + 4 * (ch & 1);
     uint32_t w[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const uint16_t lo = __builtin_bit_cast(uint16_t, tile[(8 * ch + 2 * i) * LDW + col]);
-      const uint16_t hi = __builtin_bit_cast(uint16_t, tile[(8 * ch + 2 * i + 1) * LDW + col]);
+      const int key = kb0 + 8 * (i >> 1) + 2 * (i & 1);
+      const uint16_t lo = __builtin_bit_cast(uint16_t, tile[key * LDW + col]);
+      const uint16_t hi = __builtin_bit_cast(uint16_t, tile[(key + 1) * LDW + col]);
       w[i] = (uint32_t)lo | ((uint32_t)hi << 16);
     }
     *reinterpret_cast<u32x4*>(dst + (int64_t)col * NT * 64 + ch * 8) = u32x4{w[0], w[1], w[2], w[3]};
@@ -677,7 +667,8 @@ __global__ __launch_bounds__(kThreads) void split_hi_lo_kernel(const float* __re
   }
 }
 
-// The same, transposed: [BH, NT, D] -> [BH, D, NTp]
+// The same, transposed: [BH, NT, D] -> [BH, D, NTp], with the order inside groups of 16 chunks
+// that the attention kernel expects of a V^T tile row
 template <typename T>
 __global__ __launch_bounds__(kThreads) void split_hi_lo_t_kernel(const float* __restrict__ src,
                                                                  T* __restrict__ hi, T* __restrict__ lo,
@@ -685,7 +676,9 @@ __global__ __launch_bounds__(kThreads) void split_hi_lo_t_kernel(const float* __
   const int64_t total = BH * D * NTp;
   for (int64_t e = (int64_t)blockIdx.x * kThreads + threadIdx.x; e < total;
        e += (int64_t)gridDim.x * kThreads) {
-    const int c = (int)(e % NTp);
+    const int cpos = (int)(e % NTp);  // position; chunks are permuted inside groups of 16 like keys
+    const int pos = cpos & 15;
+    const int c = (cpos & ~15) + 8 * ((pos >> 2) & 1) + 4 * (pos >> 3) + (pos & 3);
     const int64_t bd = e / NTp;
     const int d = (int)(bd % D);
     const int64_t bh = bd / D;
@@ -926,22 +919,12 @@ size_t attention_workspace_bytes(int64_t BH, int64_t T, int K, int V) {
 template <typename T, int K, int V>
 static int launch_attention(const Attn32Args& a, const void* v, int64_t BH, hipStream_t st) {
   using LY = Attn32Layout<K, V>;
-  const int lds = LY::kTiles + a.NTp;
-  if (lds > 80 * 1024) {
+  if (LY::kTiles + a.NTp > 80 * 1024) {
     set_error("piecewise attention: %d key blocks need more LDS than a workgroup has", a.NT);
     return kErrUnsupported;
   }
+  const int lds = a.NTp;  // the tile sets are static
   auto kernel = attention32_kernel<T, K, V>;
-  static thread_local int reserved = 0;
-  if (lds > reserved) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) {
-      set_error("piecewise attention: cannot reserve %d bytes of LDS: %s", lds, hipGetErrorString(e));
-      return kErrLaunch;
-    }
-    reserved = lds;
-  }
   transpose_values_kernel<T, V><<<dim3((unsigned)(BH * a.NT)), dim3(kThreads), 0, st>>>(
       (const T*)v, (T*)const_cast<void*>(a.vt), a.T, a.NT);
   kernel<<<dim3((unsigned)(BH * a.NT)), dim3(kThreads), lds, st>>>(a);
