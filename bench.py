@@ -179,6 +179,9 @@ def main():
                          "followed by a 256 MiB device copy of known traffic, then exit")
     ap.add_argument("--tables", action="store_true",
                     help="also print the reference's benchmark tables (torch formula, this library, SDPA) on stderr")
+    ap.add_argument("--only", choices=["c3", "c5"], default=None,
+                    help="profiling aid: time just BASELINE config 3 (packed variable-length, D=64 and "
+                         "D=128) or config 5 (piecewise attention), table on stderr, no headline line")
     ap.add_argument("--configs", action="store_true",
                     help="also time the other operator families / BASELINE configs (table on stderr)")
     args = ap.parse_args()
@@ -194,6 +197,13 @@ def main():
     dtype = {"fp16": torch.float16, "bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
     B, H, D, T = 8, 16, 64, args.T
     dev = torch.device("cuda:0")
+    if args.only:
+        flush = torch.empty(256 << 20, dtype=torch.int8, device=dev)
+        if args.only == "c3":
+            varlen_config(dev, flush)
+        else:
+            piecewise_config(dev, flush)
+        return
     q, k, v, do = make_inputs(B, H, T, D, dtype, dev)
     q.requires_grad_(), k.requires_grad_(), v.requires_grad_()
     tensor_bytes = q.numel() * q.element_size()
@@ -372,7 +382,12 @@ def other_configs(dev, flush):
     _report("decoupled_la B2-H16-T16384-D64 bf16 (benchmark_decoupled_la.py shape)", 6 * nb, 16 * nb, f, s, flush)
     del q, k, v, do, qr, kr
 
-    # config 3: packed variable-length, 64 sequences U[256, 2048], H=16, bf16
+    varlen_config(dev, flush)
+
+
+def varlen_config(dev, flush):
+    """BASELINE config 3: packed variable-length, 64 sequences U[256, 2048], H=16, bf16."""
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
     g = torch.Generator().manual_seed(42)
     lengths = torch.randint(256, 2049, (64,), generator=g)
     cu = torch.cat([torch.zeros(1, dtype=torch.int32), torch.cumsum(lengths, 0).to(torch.int32)]).to(dev)
