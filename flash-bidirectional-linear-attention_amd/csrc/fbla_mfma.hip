@@ -23,11 +23,11 @@
 #include <stdlib.h>
 
 #include "fbla_kernels.h"
+#include "fbla_mfma_shared.h"
 
 namespace fbla {
 namespace mfma {
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
@@ -82,36 +82,6 @@ template <> struct Ops<__bf16> {
 
 template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b) {
   return Ops<T>::bits(a) | (Ops<T>::bits(b) << 16);
-}
-
-// Orders this wave's LDS traffic: everything written before is visible to every
-// lane of the wave after (LDS executes a wave's instructions in order; this keeps
-// the compiler from moving accesses across the point).
-__device__ __forceinline__ void wave_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
-// Packed sequences have different lengths, and workgroups are dispatched in index
-// order: handing out the longest sequences first (LPT) keeps the last round of
-// workgroups short.  Returns the index of the sequence with the `rank`-th largest
-// length (ties by index); the identity for dense problems, a single sequence, or
-// more sequences than the LDS table holds.  Called by all threads of the workgroup.
-constexpr int kLptMax = 1024;
-__device__ __forceinline__ int lpt_sequence(const Prob& p, int rank, int* lens /* [kLptMax + 1] */) {
-  if (!p.cu || p.N < 2 || p.N > kLptMax) return rank;
-  const int nthreads = blockDim.x;
-  for (int i = threadIdx.x; i < p.N; i += nthreads) lens[i] = p.cu[i + 1] - p.cu[i];
-  __syncthreads();
-  for (int j = threadIdx.x; j < p.N; j += nthreads) {
-    const int lj = lens[j];
-    int r = 0;
-    for (int i = 0; i < p.N; ++i) r += (lens[i] > lj) || (lens[i] == lj && i < j);
-    if (r == rank) lens[kLptMax] = j;
-  }
-  __syncthreads();
-  return __builtin_amdgcn_readfirstlane(lens[kLptMax]);  // the same for all lanes: keep it scalar
 }
 
 // ===========================================================================
@@ -251,75 +221,6 @@ __device__ __forceinline__ void reduce_store_partial(f32x16 (&acc)[CK][CV], floa
     for (int a = 0; a < CK; ++a) {
       const float tot = ks[a] + __shfl_xor(ks[a], 32);
       if (kb == 0) dst_vec[CK * pp + a] = tot * vscale;
-    }
-  }
-}
-
-// The state kernel's form of the same reduction.  The DK x DV state is tiled into 64 x 64
-// blocks; a block is owned by G = 4 / (number of blocks) waves that take interleaved token
-// tiles (g = the wave's index inside its group).  The group's accumulators are summed in a
-// fixed order through the group's LDS buffer `red` (64 * 66 floats; unused for G = 1) and
-// wave g = 0 stores the block: dst points at the block's first element inside the [DK][DV]
-// matrix (leading dimension ld), dst_vec (optional) at the block's 64 entries of the vector.
-// Register r of accumulator (a,b) is row 2*m + a, column 2*pp + b with
-// m = 8*(r/4) + 4*kb + r%4.  Must be reached by all waves of the workgroup.
-template <int G>
-__device__ __forceinline__ void reduce_store_block(f32x16 (&acc)[2][2], float (&ks)[2], float* red,
-                                                   float* dst, int ld, float* dst_vec, float mscale,
-                                                   float vscale, int g, int lane) {
-  const int pp = lane & 31, kb = lane >> 5;
-  auto spill = [&]() {
-#pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-      for (int b = 0; b < 2; ++b)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) red[((a * 2 + b) * 16 + r) * 64 + lane] = acc[a][b][r];
-#pragma unroll
-    for (int a = 0; a < 2; ++a) red[(64 + a) * 64 + lane] = ks[a];
-  };
-  auto absorb = [&]() {
-#pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-      for (int b = 0; b < 2; ++b)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][b][r] += red[((a * 2 + b) * 16 + r) * 64 + lane];
-#pragma unroll
-    for (int a = 0; a < 2; ++a) ks[a] += red[(64 + a) * 64 + lane];
-  };
-  if constexpr (G == 4) {  // 2 -> 0, 3 -> 1, 1 -> 0
-    if (g == 2) spill();
-    __syncthreads();
-    if (g == 0) absorb();
-    __syncthreads();
-    if (g == 3) spill();
-    __syncthreads();
-    if (g == 1) absorb();
-    __syncthreads();
-    if (g == 1) spill();
-    __syncthreads();
-    if (g == 0) absorb();
-  } else if constexpr (G == 2) {
-    if (g == 1) spill();
-    __syncthreads();
-    if (g == 0) absorb();
-  }
-  if (g != 0) return;
-#pragma unroll
-  for (int a = 0; a < 2; ++a)
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = 8 * (r >> 2) + 4 * kb + (r & 3);
-        dst[(2 * m + a) * ld + 2 * pp + b] = acc[a][b][r] * mscale;
-      }
-  if (dst_vec) {
-#pragma unroll
-    for (int a = 0; a < 2; ++a) {
-      const float tot = ks[a] + __shfl_xor(ks[a], 32);
-      if (kb == 0) dst_vec[2 * pp + a] = tot * vscale;
     }
   }
 }
@@ -603,17 +504,6 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
 // ===========================================================================
 // rows kernel: out_t = (x_t M) * rowscale_t + addvec
 // ===========================================================================
-// Byte offset of 16-byte chunk `chunk` of row `row` inside a swizzled tile.  The LDS serves
-// 16 lanes x 16 bytes per cycle out of 64 banks, so the reads of one chunk column over 16
-// consecutive rows must fall into 16 different 16-byte bank groups: 256-byte rows use all
-// four low row bits; 128-byte rows come in pairs that already sit in different halves of
-// the banks, so the pair index is used.
-template <int ROWB> __device__ __forceinline__ int swz(int row, int chunk) {
-  if constexpr (ROWB == 256) return row * ROWB + ((chunk ^ (row & 15)) << 4);
-  else if constexpr (ROWB == 128) return row * ROWB + ((chunk ^ ((row >> 1) & 7)) << 4);
-  else return row * ROWB + ((chunk ^ (row & 7)) << 4);
-}
-
 // LDS layout of a DR x DC matrix operand M: fragment f = (b*KS + s)*2 + hl holds,
 // for lane l = (m = l%32, kb = l/32), the 8 values  M[(DR/2)*kb + 8s + i][sigma(b,m)]
 // where sigma(b, m = 8g + 4kb' + j) = (DC/2)*kb' + 16b + 4g + j, so that after the
@@ -1254,6 +1144,7 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
 // ===========================================================================
 // 16-bit inputs with head dims 64 or 128; the decoupled operator only at 64 x 64.
 bool supported(const Prob& p, int dtype) {
+  if (dtype == kF32) return mfma32::supported(p);
   if (dtype != kF16 && dtype != kBF16) return false;
   if (!((p.DK == 64 || p.DK == 128) && (p.DV == 64 || p.DV == 128))) return false;
   if ((p.flags & kDecoupled) && !(p.DK == 64 && p.DV == 64)) return false;
@@ -1262,7 +1153,7 @@ bool supported(const Prob& p, int dtype) {
 
 // The fused backward pass A exists for 64 x 64 heads.
 bool bwd_a_supported(const Prob& p, int dtype) {
-  return supported(p, dtype) && p.DK == 64 && p.DV == 64;
+  return dtype != kF32 && supported(p, dtype) && p.DK == 64 && p.DV == 64;
 }
 
 // Number of compute units of the current device (256 on MI355X; also the value
@@ -1408,6 +1299,9 @@ static int run_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, int 
 void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
            int chunk, int nchunks, hipStream_t st, float* fin_mat, float* fin_vec) {
   const BlockStats none{nullptr, nullptr, 0};
+  if (dtype == kF32)
+    return mfma32::state(p, (const float*)kn, (const float*)v, (const float*)kd, partial, nullptr, 0, chunk,
+                         nchunks, st, fin_mat, fin_vec);
   if (dtype == kF16) run_state<_Float16>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks, none, st);
   else run_state<__bf16>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks, none, st);
 }
@@ -1423,6 +1317,9 @@ void scaled_state(const Prob& p, int dtype, const void* qn, const void* dout, co
                   int64_t total_rows, float* partial, int chunk, int nchunks, hipStream_t st,
                   float* fin_mat, float* fin_vec) {
   const BlockStats none{nullptr, nullptr, 0};
+  if (dtype == kF32)
+    return mfma32::state(p, (const float*)qn, (const float*)dout, (const float*)qn, partial, tokscal,
+                         total_rows, chunk, nchunks, st, fin_mat, fin_vec);
   if (dtype == kF16)
     run_state<_Float16>(p, qn, dout, qn, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, none, st);
   else
@@ -1430,6 +1327,7 @@ void scaled_state(const Prob& p, int dtype, const void* qn, const void* dout, co
 }
 
 int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {
+  if (dtype == kF32) return mfma32::rows(p, job, nullptr, st);
   if (dtype == kF16) return run_rows<_Float16>(p, job, nullptr, DR, DC, st);
   return run_rows<__bf16>(p, job, nullptr, DR, DC, st);
 }
@@ -1437,6 +1335,7 @@ int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream
 // two jobs of the same shape and normalisation mode in one launch
 int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, int DR, int DC,
           hipStream_t st) {
+  if (dtype == kF32) return mfma32::rows(p, job0, &job1, st);
   if (dtype == kF16) return run_rows<_Float16>(p, job0, &job1, DR, DC, st);
   return run_rows<__bf16>(p, job0, &job1, DR, DC, st);
 }
@@ -1513,6 +1412,8 @@ static int run_bwd_tokens(const Prob& p, const void* q, const void* dout, const 
 // token view of the backward alone: dq and the per-row scalars 1/z_t, dz_t
 int bwd_tokens(const Prob& p, int dtype, const void* q, const void* dout, const float* S,
                const float* km, void* dq, float* tokscal, int64_t total_rows, hipStream_t st) {
+  if (dtype == kF32)
+    return mfma32::bwd_tokens(p, (const float*)q, (const float*)dout, S, km, (float*)dq, tokscal, total_rows, st);
   if (dtype == kF16) return run_bwd_tokens<_Float16>(p, q, dout, S, km, dq, tokscal, total_rows, st);
   return run_bwd_tokens<__bf16>(p, q, dout, S, km, dq, tokscal, total_rows, st);
 }

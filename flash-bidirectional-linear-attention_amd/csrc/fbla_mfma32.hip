@@ -1,0 +1,478 @@
+// MFMA kernels for fp32 inputs, 64 x 64 heads (dense and packed layouts, with or
+// without the denominator; the decoupled operator and other head sizes stay on the
+// shape-generic kernels).  v_mfma_f32_32x32x2_f32 computes in fp32 throughout, so
+// there is no operand splitting here: A lane l holds A[m = l%32][k = l/32], B lane l
+// holds B[k = l/32][n = l%32], C register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32].
+// One instruction covers two values of the contraction index and takes 64 cycles:
+// at 16 flop per byte these kernels keep the matrix unit about half busy at HBM speed.
+//
+//  state32_kernel   S_part = K^T V and sum_t k_t over a token chunk.  A lane owns one
+//                   feature of the token rows 2s + kb: row loads are 128 contiguous
+//                   bytes per half-wave and need no transposition at all.  SCALED: the
+//                   feature view of the backward, v = dO scaled by 1/z_t per row and the
+//                   vector part sum_t dz_t q_t.
+//  rows32_kernel    out_t = (x_t M) * rowscale_t + addvec: forward output and both
+//                   products of backward pass B.  TOKENS: the token view of backward
+//                   pass A (x = dO, M = S^T; then q.g, z, dz, dq and the per-row scalars).
+// The backward pass A is therefore two kernels (5 tensor passes), as for 16-bit heads
+// above 64.
+#include <stdlib.h>
+
+#include "fbla_kernels.h"
+#include "fbla_mfma_shared.h"
+
+namespace fbla {
+namespace mfma32 {
+
+using mfma::f32x16;
+using mfma::kLptMax;
+using mfma::lpt_sequence;
+using mfma::reduce_store_block;
+using mfma::swz;
+using mfma::wave_sync;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr int D = 64;  // head dim of both operands
+
+__device__ __forceinline__ f32x16 mma(float a, float b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+// ===========================================================================
+// state kernel
+// ===========================================================================
+// Lane l = (f = l%32, kb = l/32).  A 16-token tile is eight k-steps; in k-step s the lane
+// holds feature 32a + f of token 2s + kb for the key blocks a = 0, 1 and the value blocks
+// b = 0, 1.  Four waves take interleaved tiles; two register buffers alternate.
+template <bool SPLIT_KD, bool SCALED>
+__global__ __launch_bounds__(kThreads, 2) void state32_kernel(
+    Prob p, const float* __restrict__ kn, const float* __restrict__ v, const float* __restrict__ kd,
+    float* __restrict__ partial, const float* __restrict__ tokscal, int64_t total_rows, float* fin_mat,
+    float* fin_vec, int chunk, int nchunks) {
+  __shared__ float red[64 * 66];
+  __shared__ int lpt_lens[kLptMax + 1];
+  const int wg_nh = blockIdx.x / nchunks, c = blockIdx.x - wg_nh * nchunks;
+  const int h = wg_nh % p.H;
+  const int n = lpt_sequence(p, wg_nh / p.H, lpt_lens);
+  const int nh = n * p.H + h;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t_begin = c * chunk;
+  if (t_begin >= len) {
+    if (fin_mat && c == 0) {  // empty sequence: its state is zero
+      for (int e = threadIdx.x; e < D * D; e += kThreads) fin_mat[(int64_t)nh * D * D + e] = 0.f;
+      if (fin_vec)
+        for (int e = threadIdx.x; e < D; e += kThreads) fin_vec[(int64_t)nh * D + e] = 0.f;
+    }
+    return;
+  }
+  const int t_end = min(len, t_begin + chunk);
+  row_base(p, n, h, bos, row0, rstride);
+
+  const int g = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int f = lane & 31, kb = lane >> 5;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  float ks[2] = {0.f, 0.f};
+
+  struct Buf {
+    float k[8][2], v[8][2];
+    float d[SPLIT_KD ? 8 : 1][2];
+    float rz[SCALED ? 8 : 1], dz[SCALED ? 8 : 1];
+  };
+  const uint32_t step = (uint32_t)(rstride * D);
+  const uint32_t voff = (uint32_t)kb * step + (uint32_t)f;
+  // A tile that would cross the end of the chunk is moved back so that it ends there; the
+  // rows it shares with the previous tile are zeroed before use.
+  auto fetch = [&](Buf& b, int tok) {
+    const int tb = min(tok, t_end - 16);
+    const int64_t row = row0 + (int64_t)tb * rstride;
+    const float* kp = kn + row * D;
+    const float* vp = v + row * D;
+    const float* dp = kd + row * D;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const size_t ro = (size_t)(2 * s) * step;
+#pragma unroll
+      for (int a = 0; a < 2; ++a) {
+        b.k[s][a] = kp[ro + voff + 32 * a];
+        b.v[s][a] = vp[ro + voff + 32 * a];
+        if constexpr (SPLIT_KD) b.d[s][a] = dp[ro + voff + 32 * a];
+      }
+      if constexpr (SCALED) {
+        const int64_t r = row + (int64_t)(2 * s + kb) * rstride;
+        b.rz[s] = tokscal[r];
+        b.dz[s] = tokscal[total_rows + r];
+      }
+    }
+  };
+  auto fetch_checked = [&](Buf& b, int tok) {  // chunk shorter than a tile
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int t = tok + 2 * s + kb;
+      const bool ok = t < t_end;
+      const int64_t r = row0 + (int64_t)t * rstride;
+#pragma unroll
+      for (int a = 0; a < 2; ++a) {
+        b.k[s][a] = ok ? kn[r * D + 32 * a + f] : 0.f;
+        b.v[s][a] = ok ? v[r * D + 32 * a + f] : 0.f;
+        if constexpr (SPLIT_KD) b.d[s][a] = ok ? kd[r * D + 32 * a + f] : 0.f;
+      }
+      if constexpr (SCALED) {
+        b.rz[s] = ok ? tokscal[r] : 0.f;
+        b.dz[s] = ok ? tokscal[total_rows + r] : 0.f;
+      }
+    }
+  };
+  auto compute = [&](Buf& b, int tok, bool checked) {
+    if (!checked && tok + 16 > t_end) {
+      const int lo = tok - (t_end - 16);  // rows below lo belong to the previous tile
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        const bool keep = 2 * s + kb >= lo;
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+          b.k[s][a] = keep ? b.k[s][a] : 0.f;
+          if constexpr (SPLIT_KD) b.d[s][a] = keep ? b.d[s][a] : 0.f;
+        }
+        if constexpr (SCALED) b.dz[s] = keep ? b.dz[s] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      float vv[2] = {b.v[s][0], b.v[s][1]};
+      if constexpr (SCALED) {
+        vv[0] *= b.rz[s];
+        vv[1] *= b.rz[s];
+      }
+#pragma unroll
+      for (int a = 0; a < 2; ++a) {
+#pragma unroll
+        for (int bb = 0; bb < 2; ++bb) acc[a][bb] = mma(b.k[s][a], vv[bb], acc[a][bb]);
+        if constexpr (SCALED) ks[a] = fmaf(b.dz[s], b.k[s][a], ks[a]);
+        else ks[a] += SPLIT_KD ? b.d[s][a] : b.k[s][a];
+      }
+    }
+  };
+  int t0 = t_begin + 16 * g;
+  if (t_end - t_begin < 16) {
+    if (t0 < t_end) {
+      Buf b0;
+      fetch_checked(b0, t0);
+      compute(b0, t0, true);
+    }
+  } else if (t0 < t_end) {
+    Buf b0, b1;
+    fetch(b0, t0);
+    while (true) {
+      fetch(b1, t0 + 16 * kWaves);
+      compute(b0, t0, false);
+      t0 += 16 * kWaves;
+      if (t0 >= t_end) break;
+      fetch(b0, t0 + 16 * kWaves);
+      compute(b1, t0, false);
+      t0 += 16 * kWaves;
+      if (t0 >= t_end) break;
+    }
+  }
+
+  float* mat = fin_mat ? fin_mat + (int64_t)nh * D * D
+                       : partial + ((int64_t)nh * nchunks + c) * (D * D + D);
+  float* vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * D : nullptr) : mat + D * D;
+  const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
+  const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
+  reduce_store_block<4, false>(acc, ks, red, mat, D, vec, mscale, vscale, g, lane);
+}
+
+// ===========================================================================
+// rows kernel
+// ===========================================================================
+// C[m][n = token] = sum_k A[m][k] B[k][n] with A = the operand M (from LDS) and B = x.
+// The contraction index of k-step s and half-wave kb is feature r(s, kb) = 4*(s/2) + 2*kb
+// + s%2: a lane's B values of k-steps 2i, 2i+1 are then 8 contiguous bytes of the staged
+// x tile, and the A values of four k-steps one 16-byte read.  Row m = 8g + 4kb' + j of
+// block b is output feature sigma(b, m) = 32*kb' + 16*b + 4*g + j: after the MFMA a lane
+// (token, kb') owns 32 consecutive output features.
+//
+// Operand fragments in LDS: frag[((b*8 + s/4)*64 + lane)*4 + s%4] = M[r(s,kb)][sigma(b,m)],
+// lane = m + 32*kb.  M is read as mat[r*ld_r + c*ld_c] times mscale.
+__device__ __forceinline__ void build_operand32(float* frag, const float* __restrict__ mat, int ld_r,
+                                                int ld_c, float mscale) {
+  for (int e = threadIdx.x; e < D * D; e += blockDim.x) {
+    // walk the matrix along its contiguous direction
+    const int r = ld_c == 1 ? e / D : e % D, cc = ld_c == 1 ? e % D : e / D;
+    const int s = 2 * (r >> 2) + (r & 1), kb = (r >> 1) & 1;
+    const int kbp = cc >> 5, b = (cc >> 4) & 1, gq = (cc >> 2) & 3, j = cc & 3;
+    const int m = 8 * gq + 4 * kbp + j;
+    frag[((b * 8 + (s >> 2)) * 64 + m + 32 * kb) * 4 + (s & 3)] = mat[(int64_t)r * ld_r + (int64_t)cc * ld_c] * mscale;
+  }
+}
+
+struct Rows32Job {
+  const float* x;       // [rows, 64] B operand
+  const float* xden;    // NORM: rows for the denominator (== x here); TOKENS: q
+  const float* mat;     // operand M, element (r, c) at mat[nh*4096 + r*ld_r + c*ld_c]
+  int ld_r, ld_c;
+  const float* km;      // [NH, 64] mean key (NORM / TOKENS with the denominator)
+  const float* addvec;  // [NH, 64] added to every output row, or null
+  float* out;           // [rows, 64]
+  float* tokscal;       // TOKENS: [2][total rows]: 1/z_t, dz_t
+  int64_t total_rows;
+};
+
+struct Rows32Layout {
+  static constexpr int kFrag = D * D * 4;        // 16 KiB
+  static constexpr int kStage = 32 * D * 4;      // one 32-token tile, 8 KiB per wave
+  static constexpr int kKm = kFrag + kWaves * kStage;
+  static constexpr int kAdd = kKm + D * 4;
+  static constexpr int kLpt = kAdd + D * 4;
+  static constexpr int kTotal = kLpt + (kLptMax + 1) * 4;
+};
+
+// NORM: rowscale = 1 / (x_t . km + eps).  TOKENS (implies the job's q in xden): the token
+// view of backward pass A: g = x_t M (x = dO, M = S^T), P = q_t . g, z = q_t . km + eps,
+// dz = -P / z^2, out = dq_t = g / z + dz km (without the denominator: out = g), and the
+// per-row scalars 1/z_t, dz_t go to tokscal.
+template <bool NORM, bool TOKENS>
+__global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0, Rows32Job job1,
+                                                          int wgs_per_job, int chunk, int nchunks) {
+  using LY = Rows32Layout;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const bool second = (int)blockIdx.x >= wgs_per_job;
+  const Rows32Job& job = second ? job1 : job0;
+  const int wg = second ? blockIdx.x - wgs_per_job : blockIdx.x;
+  const int wg_nh = wg / nchunks, c = wg - wg_nh * nchunks;
+  const int h = wg_nh % p.H;
+  const int n = lpt_sequence(p, wg_nh / p.H, reinterpret_cast<int*>(smem + LY::kLpt));
+  const int nh = n * p.H + h;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t_begin = c * chunk;
+  if (t_begin >= len) return;
+  const int t_end = min(len, t_begin + chunk);
+  row_base(p, n, h, bos, row0, rstride);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ntok = lane & 31, kb = lane >> 5;
+  float* frag = reinterpret_cast<float*>(smem);
+  unsigned char* stage = smem + LY::kFrag + wave * LY::kStage;
+  float* kmv = reinterpret_cast<float*>(smem + LY::kKm);
+  float* addv = reinterpret_cast<float*>(smem + LY::kAdd);
+
+  // x tile: 32 rows of 256 bytes = 512 chunks, 8 per lane, flat and coalesced
+  auto load_tile = [&](f32x4(&dst)[8], const float* src, int tok0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q = lane + 64 * i, row = q >> 4, ch = q & 15;
+      const int tok = tok0 + row;
+      dst[i] = tok < t_end ? *reinterpret_cast<const f32x4*>(src + (row0 + (int64_t)tok * rstride) * D + ch * 4)
+                           : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  int t0 = t_begin + 32 * wave;
+  f32x4 xr[8];
+  if (t0 < t_end) load_tile(xr, job.x, t0);
+
+  build_operand32(frag, job.mat + (int64_t)nh * D * D, job.ld_r, job.ld_c, 1.f);
+  for (int e = tid; e < D; e += kThreads) {
+    kmv[e] = (NORM || TOKENS) && job.km ? job.km[(int64_t)nh * D + e] : 0.f;
+    addv[e] = job.addvec ? job.addvec[(int64_t)nh * D + e] : 0.f;
+  }
+  __syncthreads();
+  const bool with_den = (NORM || TOKENS) && job.km != nullptr;
+
+  while (t0 < t_end) {
+    wave_sync();  // the previous tile's staged output has been read out
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q = lane + 64 * i;
+      *reinterpret_cast<f32x4*>(stage + swz<256>(q >> 4, q & 15)) = xr[i];
+    }
+    const int tn = t0 + 32 * kWaves;
+    if (tn < t_end) load_tile(xr, job.x, tn);
+    wave_sync();
+
+    f32x16 acc[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[b][r] = 0.f;
+    float z = 0.f;
+#pragma unroll
+    for (int sg = 0; sg < 8; ++sg) {
+      // k-steps 4sg .. 4sg+3: x features 8sg + 2kb + {0,1} and 8sg + 4 + 2kb + {0,1}
+      const f32x2 x01 = *reinterpret_cast<const f32x2*>(stage + swz<256>(ntok, 2 * sg) + 8 * kb);
+      const f32x2 x23 = *reinterpret_cast<const f32x2*>(stage + swz<256>(ntok, 2 * sg + 1) + 8 * kb);
+      const float xv[4] = {x01[0], x01[1], x23[0], x23[1]};
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const f32x4 a4 = *reinterpret_cast<const f32x4*>(frag + ((b * 8 + sg) * 64 + lane) * 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[b] = mma(a4[e], xv[e], acc[b]);
+      }
+      if constexpr (NORM) {
+        const f32x2 k01 = *reinterpret_cast<const f32x2*>(kmv + 8 * sg + 2 * kb);
+        const f32x2 k23 = *reinterpret_cast<const f32x2*>(kmv + 8 * sg + 4 + 2 * kb);
+        z = fmaf(x01[0], k01[0], z);
+        z = fmaf(x01[1], k01[1], z);
+        z = fmaf(x23[0], k23[0], z);
+        z = fmaf(x23[1], k23[1], z);
+      }
+    }
+    // this lane: token ntok, output features 32*kb + 16*b + r
+    float rs = 1.f, dz = 0.f;
+    if constexpr (NORM) {
+      z += __shfl_xor(z, 32);
+      rs = 1.f / (z + p.eps);
+    }
+    if constexpr (TOKENS) {
+      if (with_den) {
+        // q row half of this lane straight from global memory (a full 128-byte line per lane)
+        const int tok = min(t0 + ntok, t_end - 1);
+        const float* qrow = job.xden + (row0 + (int64_t)tok * rstride) * D + 32 * kb;
+        float P = 0.f, zz = 0.f;
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const f32x4 qv = *reinterpret_cast<const f32x4*>(qrow + 16 * b + 4 * i);
+            const f32x4 kv = *reinterpret_cast<const f32x4*>(kmv + 32 * kb + 16 * b + 4 * i);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              P = fmaf(qv[j], acc[b][4 * i + j], P);
+              zz = fmaf(qv[j], kv[j], zz);
+            }
+          }
+        P += __shfl_xor(P, 32);
+        zz += __shfl_xor(zz, 32);
+        rs = 1.f / (zz + p.eps);
+        dz = -P * rs * rs;
+        if (kb == 0 && t0 + ntok < t_end) {
+          const int64_t row = row0 + (int64_t)(t0 + ntok) * rstride;
+          job.tokscal[row] = rs;
+          job.tokscal[job.total_rows + row] = dz;
+        }
+      }
+    }
+    wave_sync();  // all lanes have read their x values; the staging tile is reused for out
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c0 = 32 * kb + 16 * b + 4 * i;
+        f32x4 w;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float o = fmaf(acc[b][4 * i + j], rs, addv[c0 + j]);
+          if constexpr (TOKENS) o = fmaf(dz, kmv[c0 + j], o);
+          w[j] = o;
+        }
+        *reinterpret_cast<f32x4*>(stage + swz<256>(ntok, c0 >> 2)) = w;
+      }
+    wave_sync();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q = lane + 64 * i, row = q >> 4, ch = q & 15;
+      const int tok = t0 + row;
+      if (tok < t_end)
+        *reinterpret_cast<f32x4*>(job.out + (row0 + (int64_t)tok * rstride) * D + ch * 4) =
+            *reinterpret_cast<const f32x4*>(stage + swz<256>(row, ch));
+    }
+    t0 = tn;
+  }
+}
+
+// ===========================================================================
+// host side
+// ===========================================================================
+bool supported(const Prob& p) {
+  return p.DK == D && p.DV == D && !(p.flags & kDecoupled);
+}
+
+void state(const Prob& p, const float* kn, const float* v, const float* kd, float* partial,
+           const float* tokscal, int64_t total_rows, int chunk, int nchunks, hipStream_t st, float* fin_mat,
+           float* fin_vec) {
+  const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(kThreads);
+  if (tokscal)
+    state32_kernel<false, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks);
+  else
+    state32_kernel<false, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks);
+}
+
+template <bool NORM, bool TOKENS>
+static int launch_rows(const Prob& p, const Rows32Job& j0, const Rows32Job* j1, hipStream_t st) {
+  auto kernel = rows32_kernel<NORM, TOKENS>;
+  static thread_local bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, Rows32Layout::kTotal);
+    if (e != hipSuccess) {
+      set_error("cannot reserve %d bytes of LDS: %s", Rows32Layout::kTotal, hipGetErrorString(e));
+      return kErrLaunch;
+    }
+    configured = true;
+  }
+  const int chunk = mfma::rows_chunk(p, D, D);
+  const int nchunks = (int)cdiv64(p.L, chunk);
+  const int wgs = (int)((int64_t)p.N * p.H * nchunks);
+  const dim3 grid((unsigned)(j1 ? 2 * wgs : wgs)), block(kThreads);
+  kernel<<<grid, block, Rows32Layout::kTotal, st>>>(p, j0, j1 ? *j1 : j0, wgs, chunk, nchunks);
+  return kOk;
+}
+
+static Rows32Job convert(const mfma::RowsJob& j) {
+  Rows32Job r;
+  r.x = (const float*)j.x;
+  r.xden = (const float*)j.xden;
+  r.mat = j.mat;
+  r.ld_r = j.ld_r;
+  r.ld_c = j.ld_c;
+  r.km = j.km;
+  r.addvec = j.addvec;
+  r.out = (float*)j.out;
+  r.tokscal = nullptr;
+  r.total_rows = 0;
+  return r;
+}
+
+int rows(const Prob& p, const mfma::RowsJob& job, const mfma::RowsJob* job2, hipStream_t st) {
+  const Rows32Job a = convert(job);
+  if (job.xden) return launch_rows<true, false>(p, a, nullptr, st);
+  if (job2) {
+    const Rows32Job b = convert(*job2);
+    return launch_rows<false, false>(p, a, &b, st);
+  }
+  return launch_rows<false, false>(p, a, nullptr, st);
+}
+
+int bwd_tokens(const Prob& p, const float* q, const float* dout, const float* S, const float* km, float* dq,
+               float* tokscal, int64_t total_rows, hipStream_t st) {
+  Rows32Job j;
+  j.x = dout;
+  j.xden = q;
+  j.mat = S;  // M(r = dv, c = dk) = S[c][r]
+  j.ld_r = 1;
+  j.ld_c = D;
+  j.km = (p.flags & kNormalize) ? km : nullptr;
+  j.addvec = nullptr;
+  j.out = dq;
+  j.tokscal = tokscal;
+  j.total_rows = total_rows;
+  return launch_rows<false, true>(p, j, nullptr, st);
+}
+
+}  // namespace mfma32
+}  // namespace fbla

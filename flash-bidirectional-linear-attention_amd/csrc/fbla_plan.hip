@@ -1,6 +1,7 @@
 // The plan: which kernels run, in which order, for each entry point, and how the
 // caller's workspace is carved up.  MFMA kernels are used for the shapes they
-// cover (16-bit inputs, head dims 64); everything else runs on the generic kernels.
+// cover (16-bit inputs with head dims 64 / 128, fp32 inputs with 64 x 64 heads);
+// everything else runs on the generic kernels.
 //
 // forward :  state partials -> fixed-order reduce (S, km) -> output rows
 // backward:  S^T -> pass A (dq, partial dS/dkm) -> reduce (s dS, its transpose, dkm/L)
@@ -71,7 +72,7 @@ int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
     else
       generic::state_partial(p, dtype, kn, a.v, a.k, partial, chunk, nchunks, st);
   }
-  const bool fold = fast && !direct && fold_reduce(p, nchunks, p.DK, p.DV);
+  const bool fold = fast && !direct && dtype != kF32 && fold_reduce(p, nchunks, p.DK, p.DV);
   if (!fold && !direct && (phases & kPhaseFwdReduce))
     generic::state_reduce(p, partial, chunk, nchunks, a.s, nullptr, a.km, st);
   if (phases & kPhaseFwdOutput) {
@@ -140,7 +141,7 @@ int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
       generic::bwd_a(p, dtype, qn, a.q, a.dout, a.s, St, a.km, dqn, dqd, partial, chunk, nchunks, st);
     }
   }
-  const bool fold = fast && !direct && fold_reduce(p, nchunks, p.DV, p.DK);
+  const bool fold = fast && !direct && dtype != kF32 && fold_reduce(p, nchunks, p.DV, p.DK);
   if (!fold && !direct && (phases & kPhaseBwdReduce))
     generic::state_reduce(p, partial, chunk, nchunks, dS, fast ? nullptr : dSt, dkm, st);
   if (phases & kPhaseBwdB) {
