@@ -149,3 +149,12 @@ def test_matches_autograd_of_torch_formula_on_gpu():
     for name, x, y in zip("qkv", b, a):
         assert_close("d" + name, x.grad, y.grad, 0.06)
         assert max_rel_err(y.grad, x.grad) < 1e-4
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("variant", ["linear", "simple"])
+@pytest.mark.parametrize("L", [1, 5, 15, 16, 17, 31, 33, 47, 8200])
+def test_matrix_core_paths_at_awkward_lengths(variant, L, dtype):
+    """64 x 64 heads run on the MFMA kernels for all three dtypes; their token loops work in
+    tiles of 16 and 32 tokens with a moved-back last tile and a checked path below one tile."""
+    _check_dense(variant, 1, 3, L, 64, 64, dtype, seed=L)
