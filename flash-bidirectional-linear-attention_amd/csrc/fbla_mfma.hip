@@ -848,7 +848,7 @@ template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struc
 // fit one wave): it writes 1/z_t and dz_t per (token, head) row to `tokscal`
 // ([2][total rows]) for scaled_state_kernel, and no partials.
 template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true>
-__global__ __launch_bounds__(kThreads) void bwd_a_kernel(
+__global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const T* __restrict__ dout,
     const float* __restrict__ S, const float* __restrict__ km, T* __restrict__ dqn,
     T* __restrict__ dqd, float* __restrict__ partial, float* __restrict__ tokscal,
