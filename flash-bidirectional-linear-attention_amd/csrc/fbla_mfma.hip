@@ -156,82 +156,10 @@ __device__ __forceinline__ void transpose_rows(const RowWords<C>& src, u32x4 (&o
     }
 }
 
-// Fixed-order sum of the four waves' accumulators through one LDS buffer, then
-// the canonical [dk][dv] partial followed by the [dk] vector is written.
-// NS = 1: every wave holds the full DK x DV block (2 -> 0, 3 -> 1, 1 -> 0; wave 0 writes).
-// NS = 2: wave w holds value columns [(w%2)*32*CV, +32*CV) (2 -> 0, 3 -> 1; waves 0 and 1
-// write their halves, wave 0 the vector).  The matrix goes to dst times mscale, the vector
-// to dst_vec (if given) times vscale.  Register r of block (a,b) is dk = CK*m + a,
-// dv = CV*pp + b with m = 8*(r/4) + 4*kb + r%4.  Must be reached by all waves.
-template <int CK, int CV, int NS>
-__device__ __forceinline__ void reduce_store_partial(f32x16 (&acc)[CK][CV], float (&ks)[CK],
-                                                     float* red, float* dst, float* dst_vec,
-                                                     float mscale, float vscale, int wave, int lane) {
-  constexpr int kAcc = CK * CV * 16;
-  constexpr int DK = 32 * CK, DVW = 32 * CV, DV = DVW * NS;
-  const int pp = lane & 31, kb = lane >> 5;
-  auto spill = [&]() {
-#pragma unroll
-    for (int a = 0; a < CK; ++a)
-#pragma unroll
-      for (int b = 0; b < CV; ++b)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) red[((a * CV + b) * 16 + r) * 64 + lane] = acc[a][b][r];
-#pragma unroll
-    for (int a = 0; a < CK; ++a) red[(kAcc + a) * 64 + lane] = ks[a];
-  };
-  auto absorb = [&]() {
-#pragma unroll
-    for (int a = 0; a < CK; ++a)
-#pragma unroll
-      for (int b = 0; b < CV; ++b)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][b][r] += red[((a * CV + b) * 16 + r) * 64 + lane];
-#pragma unroll
-    for (int a = 0; a < CK; ++a) ks[a] += red[(kAcc + a) * 64 + lane];
-  };
-  if (wave == 2) spill();
-  __syncthreads();
-  if (wave == 0) absorb();
-  __syncthreads();
-  if (wave == 3) spill();
-  __syncthreads();
-  if (wave == 1) absorb();
-  if constexpr (NS == 1) {
-    __syncthreads();
-    if (wave == 1) spill();
-    __syncthreads();
-    if (wave != 0) return;
-    absorb();
-  } else {
-    if (wave > 1) return;
-  }
-  const int dv_off = NS == 1 ? 0 : wave * DVW;
-#pragma unroll
-  for (int a = 0; a < CK; ++a)
-#pragma unroll
-    for (int b = 0; b < CV; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = 8 * (r >> 2) + 4 * kb + (r & 3);
-        dst[(CK * m + a) * DV + dv_off + CV * pp + b] = acc[a][b][r] * mscale;
-      }
-  if (wave == 0 && dst_vec) {
-#pragma unroll
-    for (int a = 0; a < CK; ++a) {
-      const float tot = ks[a] + __shfl_xor(ks[a], 32);
-      if (kb == 0) dst_vec[CK * pp + a] = tot * vscale;
-    }
-  }
-}
-
 // SCALED = true is the feature view of the backward for head dims above 64:
 // kn = q~, v = dO, every dO row is multiplied by 1/z_t (tokscal[row]) and split
 // into hi + lo before the MFMA, and the vector part is dkm = sum_t dz_t q_t
 // (dz_t = tokscal[total_rows + row]).
-#ifndef FBLA_STATE128_TILES
-#define FBLA_STATE128_TILES 1
-#endif
 // STATS = true additionally writes, for every 64-token block of the sequence, the mean key
 // (kc [N*H, NT, DK]) and the value sum (vc [N*H, NT, DV]): the block statistics of piecewise
 // attention.  The waves then walk whole 64-token blocks (four tiles in a row) instead of
@@ -1135,7 +1063,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * DK : nullptr) : dst + DK * DV;
     const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
     const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
-    reduce_store_partial<CK, CV, 1>(acc, dkm, red, dst, dst_vec, mscale, vscale, wave, lane);
+    reduce_store_block<4>(acc, dkm, red, dst, DV, dst_vec, mscale, vscale, wave, lane);
   }
 }
 
@@ -1221,7 +1149,7 @@ static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, fl
                          const float* tokscal, int64_t total_rows, float* fm, float* fv, int chunk,
                          int nchunks, BlockStats bs, hipStream_t st) {
   const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(kThreads);
-  constexpr int TL = (DK == 128 && DV == 128) ? FBLA_STATE128_TILES : 1;
+  constexpr int TL = 1;  // 16-token tiles per step and wave
   if (bs.kc)
     state_kernel<T, DK, DV, false, 1, false, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
   else if (tokscal)

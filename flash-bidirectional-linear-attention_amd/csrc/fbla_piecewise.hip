@@ -768,27 +768,33 @@ __global__ __launch_bounds__(kThreads) void select_blocks_kernel(
   }
   __syncthreads();
 
+  // the wave's four rows advance through the bitwise descent together: four independent
+  // chains of LDS reads and wave-wide counts instead of one
+  uint32_t thr[4] = {0u, 0u, 0u, 0u};
+  for (int bit = 31; bit >= 0; --bit) {
+    int cnt[4] = {0, 0, 0, 0};
+    for (int j = lane; j < NTs; j += 64)
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr)
+        cnt[rr] += __popcll(__ballot(order_bits(sc[(4 * wave + rr) * NTs + j]) >= (thr[rr] | (1u << bit))));
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr)
+      if (cnt[rr] >= NS) thr[rr] |= 1u << bit;
+  }
   for (int rr = 0; rr < 4; ++rr) {
     const int row = 4 * wave + rr;
     if (r0 + row >= NT) break;  // uniform over the wave
     const float* srow = sc + row * NTs;
-    // threshold: greatest t with count(u >= t) >= NS
-    uint32_t thr = 0;
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t t = thr | (1u << bit);
-      int cnt = 0;
-      for (int j = lane; j < NTs; j += 64) cnt += __popcll(__ballot(order_bits(srow[j]) >= t));
-      if (cnt >= NS) thr = t;
-    }
+    const uint32_t t = thr[rr];
     int above = 0;
-    for (int j = lane; j < NTs; j += 64) above += __popcll(__ballot(order_bits(srow[j]) > thr));
+    for (int j = lane; j < NTs; j += 64) above += __popcll(__ballot(order_bits(srow[j]) > t));
     int ties_left = NS - above, written = 0;
     int32_t* dst = indices + (bh * NT + (r0 + row)) * (int64_t)NS;
     for (int j = lane; j < NTs; j += 64) {
       const uint32_t u = order_bits(srow[j]);
-      const uint64_t tie_mask = __ballot(u == thr);
+      const uint64_t tie_mask = __ballot(u == t);
       const int tie_rank = __popcll(tie_mask & ((1ull << lane) - 1ull));
-      const bool take = u > thr || (u == thr && tie_rank < ties_left);
+      const bool take = u > t || (u == t && tie_rank < ties_left);
       const uint64_t take_mask = __ballot(take);
       if (take) dst[written + __popcll(take_mask & ((1ull << lane) - 1ull))] = j;
       written += __popcll(take_mask);
