@@ -126,3 +126,33 @@ def test_piecewise_config_full_size():
     assert_parity(o[0, hd], ref, dtype, "piecewise head 11")
     rq, rk, rv, _, rH, _ = pw.chunk_reduce(np64(q)[0, hd], np64(k)[0, hd], np64(v)[0, hd], 64)
     assert max_rel_err(h[0, hd], rH) < 1e-4 and max_rel_err(kc[0, hd], rk) < 1e-5
+
+
+def test_more_than_2_31_elements_per_tensor():
+    """B=2, H=16, T=1048576, D=64 fp16: 2^31 elements (4 GiB) per tensor, so every element
+    offset of the second batch entry needs more than 31 bits.  Sampled heads from both ends
+    against the float64 oracle, forward and backward."""
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    dtype, B, H, T, D = torch.float16, 2, 16, 1 << 20, 64
+    g = torch.Generator(device="cuda").manual_seed(7)
+    q = torch.empty(B, H, T, D, dtype=dtype, device="cuda")
+    k = torch.empty_like(q)
+    v = torch.empty_like(q)
+    do = torch.empty_like(q)
+    for b in range(B):  # filled per batch entry: the fp32 temporaries stay small
+        q[b] = (F.elu(torch.randn(H, T, D, generator=g, device="cuda")) + 1).to(dtype)
+        k[b] = (F.elu(torch.randn(H, T, D, generator=g, device="cuda")) + 1).to(dtype)
+        v[b] = torch.randn(H, T, D, generator=g, device="cuda").to(dtype)
+        do[b] = torch.randn(H, T, D, generator=g, device="cuda").to(dtype)
+    assert q.numel() >= 2 ** 31
+    leaves = [t.requires_grad_() for t in (q, k, v)]
+    o = linear_attention(*leaves)
+    o.backward(do)
+    torch.cuda.synchronize()
+    for b, h in ((0, 0), (1, 0), (1, 15)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        ref = cf.dense_backward(np64(q[sl].detach()), np64(k[sl].detach()), np64(v[sl].detach()), np64(do[sl]),
+                                1.0 / T)
+        assert_parity(o[sl], ref["o"], dtype, f"o[{b},{h}]")
+        for name, t in zip(("dq", "dk", "dv"), leaves):
+            assert_parity(t.grad[sl], ref[name], dtype, f"{name}[{b},{h}]", ref.get(name + "_mag"))
