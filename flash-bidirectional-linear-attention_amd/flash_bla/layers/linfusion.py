@@ -12,6 +12,20 @@ import torch.nn.functional as F
 
 from flash_bla.layers._common import check_mode, torch_linear_attention
 from flash_bla.ops.linear_attn.fused import linear_attention
+from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+
+
+_CU_CACHE = {}
+
+
+def _equal_cu_seqlens(batch, tokens, device):
+    """int32 [0, n, 2n, ...] on `device`, cached per (batch, tokens, device)."""
+    key = (batch, tokens, str(device))
+    cu = _CU_CACHE.get(key)
+    if cu is None:
+        cu = torch.arange(0, (batch + 1) * tokens, tokens, dtype=torch.int32, device=device)
+        _CU_CACHE[key] = cu
+    return cu
 
 
 def get_none_linear_projection(query_dim, mid_dim=None):
@@ -55,6 +69,15 @@ class GeneralizedLinearAttention(nn.Module):
         q = self.to_q(hidden_states + self.to_q_(hidden_states))
         k = self.to_k(context + self.to_k_(context))
         v = self.to_v(context)
+        if fast and q.shape[1] == k.shape[1]:
+            # The projections come out token-major, (batch, tokens, heads * dim): that is the
+            # packed layout of the variable-length operator with equal lengths, so the head
+            # split / merge copies of the reference (linfusion.py:98,102) are not needed at all.
+            b, n, _ = q.shape
+            q, k = F.elu(q) + 1.0, F.elu(k) + 1.0
+            packed = [t.reshape(b * n, self.heads, -1) for t in (q, k, v)]
+            out = varlen_linear_attention(*packed, _equal_cu_seqlens(b, n, q.device), n, eps=1e-4)
+            return self.to_out[1](self.to_out[0](out.reshape(b, n, -1)))
         q, k, v = (self.head_to_batch_dim(t) for t in (q, k, v))
         q, k = F.elu(q) + 1.0, F.elu(k) + 1.0
         if fast:
