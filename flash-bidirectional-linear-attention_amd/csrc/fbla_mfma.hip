@@ -121,13 +121,13 @@ __device__ __forceinline__ void load_rows(RowWords<C>& dst, const T* __restrict_
 // `rows` (relative to the tile) are not read and come back as zero.
 template <typename T, int C>
 __device__ __forceinline__ void load_rows_checked(RowWords<C>& dst, const T* __restrict__ tile,
-                                                  uint32_t step, int rel0, int p, int rows) {
+                                                  uint32_t step, int rel0, int col, int rows) {
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
 #pragma unroll
     for (int c = 0; c < C / 2; ++c) dst.w[j][c] = 0u;
     if (rel0 + j < rows) {
-      const uint32_t* src = reinterpret_cast<const uint32_t*>(tile + (size_t)(rel0 + j) * step + C * p);
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(tile + (size_t)(rel0 + j) * step + col);
 #pragma unroll
       for (int c = 0; c < C / 2; ++c) dst.w[j][c] = src[c];
     }
@@ -141,6 +141,16 @@ __device__ __forceinline__ void mask_rows(RowWords<C>& r, int rel0, int lo) {
   for (int j = 0; j < 8; ++j)
 #pragma unroll
     for (int c = 0; c < C / 2; ++c) r.w[j][c] = rel0 + j >= lo ? r.w[j][c] : 0u;
+}
+
+// keeps (keep = all ones) or clears (keep = 0) every word: lanes whose feature columns lie
+// past the head dim (padding up to the 64-wide block) load a valid column and drop it here
+template <int C>
+__device__ __forceinline__ void keep_rows(RowWords<C>& r, uint32_t keep) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int c = 0; c < C / 2; ++c) r.w[j][c] &= keep;
 }
 
 // token-pair packing: operand c gets feature c of tokens (2i, 2i+1) in dword i
@@ -164,13 +174,17 @@ __device__ __forceinline__ void transpose_rows(const RowWords<C>& src, u32x4 (&o
 // (kc [N*H, NT, DK]) and the value sum (vc [N*H, NT, DV]): the block statistics of piecewise
 // attention.  The waves then walk whole 64-token blocks (four tiles in a row) instead of
 // interleaving single tiles, so that a block's sums stay inside one wave.
+// PAD = true: the head dims (p.DK, p.DV, multiples of 8) are smaller than the template's
+// DK, DV, which then only fix the tiling: rows are p.DK / p.DV elements long in memory, lanes
+// of feature columns past the head dim contribute zeros, and the stored state has the true
+// shape [p.DK][p.DV].
 struct BlockStats {
   float* kc;
   float* vc;
   int NT;
 };
 
-template <typename T, int DK, int DV, bool SPLIT_KD, int TILES, bool SCALED, bool STATS = false>
+template <typename T, int DK, int DV, bool SPLIT_KD, int TILES, bool SCALED, bool STATS = false, bool PAD = false>
 __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2) void state_kernel(Prob p, const T* __restrict__ kn,
                                                          const T* __restrict__ v,
                                                          const T* __restrict__ kd,
@@ -179,7 +193,8 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
                                                          int64_t total_rows, float* fin_mat,
                                                          float* fin_vec, int chunk, int nchunks,
                                                          BlockStats stats) {
-  static_assert(!STATS || (TILES == 1 && !SCALED && !SPLIT_KD), "block statistics: plain variant only");
+  static_assert(!STATS || (TILES == 1 && !SCALED && !SPLIT_KD && !PAD), "block statistics: plain variant only");
+  const int dk = PAD ? p.DK : DK, dv = PAD ? p.DV : DV;  // row lengths in memory
   // The state is tiled into 64 x 64 blocks (64 accumulator registers per lane); a block is
   // owned by G waves that take interleaved token tiles.  For a 128 x 128 state the four
   // waves of the workgroup therefore read the same tokens, each the 64 key and 64 value
@@ -200,9 +215,9 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
   const int t_begin = c * chunk;
   if (t_begin >= len) {
     if (fin_mat && c == 0) {  // empty sequence: its state is zero
-      for (int e = threadIdx.x; e < DK * DV; e += kThreads) fin_mat[(int64_t)nh * DK * DV + e] = 0.f;
+      for (int e = threadIdx.x; e < dk * dv; e += kThreads) fin_mat[(int64_t)nh * dk * dv + e] = 0.f;
       if (fin_vec)
-        for (int e = threadIdx.x; e < DK; e += kThreads) fin_vec[(int64_t)nh * DK + e] = 0.f;
+        for (int e = threadIdx.x; e < dk; e += kThreads) fin_vec[(int64_t)nh * dk + e] = 0.f;
     }
     return;
   }
@@ -212,6 +227,10 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int pp = lane & 31, kb = lane >> 5;
   const int blk = wave / G, g = wave % G, bk = blk / VB, bv = blk % VB;
+  // this lane's feature columns inside its block, and whether they exist
+  const bool k_ok = !PAD || 64 * bk + CK * pp < dk, v_ok = !PAD || 64 * bv + CV * pp < dv;
+  const int kcol0 = k_ok ? CK * pp : 0, vcol0 = v_ok ? CV * pp : 0;
+  const uint32_t k_keep = k_ok ? ~0u : 0u, v_keep = v_ok ? ~0u : 0u;
   const T* kcol = kn + 64 * bk;
   const T* vcol = v + 64 * bv;
   const T* kdcol = kd + 64 * bk;
@@ -243,18 +262,18 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
   // first `lo` rows were already part of the previous tile and are zeroed before use.  Every
   // tile therefore reads 16 valid rows with the same address pattern (chunks shorter than
   // one tile take the checked path below).
-  const uint32_t kstep = (uint32_t)(rstride * DK), vstep = (uint32_t)(rstride * DV);
-  const uint32_t kvoff = (uint32_t)(8 * kb) * kstep + (uint32_t)(CK * pp);
-  const uint32_t vvoff = (uint32_t)(8 * kb) * vstep + (uint32_t)(CV * pp);
+  const uint32_t kstep = (uint32_t)(rstride * dk), vstep = (uint32_t)(rstride * dv);
+  const uint32_t kvoff = (uint32_t)(8 * kb) * kstep + (uint32_t)kcol0;
+  const uint32_t vvoff = (uint32_t)(8 * kb) * vstep + (uint32_t)vcol0;
   const uint32_t tvoff = (uint32_t)(8 * kb) * (uint32_t)rstride;
   auto fetch = [&](Buf& b, int tok) {
 #pragma unroll
     for (int u = 0; u < TILES; ++u) {
       const int tb = min(tok + 16 * u, t_end - 16);
       const int64_t row = row0 + (int64_t)tb * rstride;
-      load_rows<T, CK>(b.k[u], kcol + row * DK, kstep, kvoff);
-      load_rows<T, CV>(b.v[u], vcol + row * DV, vstep, vvoff);
-      if constexpr (SPLIT_KD) load_rows<T, CK>(b.d[u], kdcol + row * DK, kstep, kvoff);
+      load_rows<T, CK>(b.k[u], kcol + row * dk, kstep, kvoff);
+      load_rows<T, CV>(b.v[u], vcol + row * dv, vstep, vvoff);
+      if constexpr (SPLIT_KD) load_rows<T, CK>(b.d[u], kdcol + row * dk, kstep, kvoff);
       if constexpr (SCALED) {
         const float* ts = tokscal + row;
 #pragma unroll
@@ -270,9 +289,9 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
     for (int u = 0; u < TILES; ++u) {
       const int rows = t_end - (tok + 16 * u);
       const int64_t row = row0 + (int64_t)(tok + 16 * u) * rstride;
-      load_rows_checked<T, CK>(b.k[u], kcol + row * DK, kstep, 8 * kb, pp, rows);
-      load_rows_checked<T, CV>(b.v[u], vcol + row * DV, vstep, 8 * kb, pp, rows);
-      if constexpr (SPLIT_KD) load_rows_checked<T, CK>(b.d[u], kdcol + row * DK, kstep, 8 * kb, pp, rows);
+      load_rows_checked<T, CK>(b.k[u], kcol + row * dk, kstep, 8 * kb, kcol0, rows);
+      load_rows_checked<T, CV>(b.v[u], vcol + row * dv, vstep, 8 * kb, vcol0, rows);
+      if constexpr (SPLIT_KD) load_rows_checked<T, CK>(b.d[u], kdcol + row * dk, kstep, 8 * kb, kcol0, rows);
       if constexpr (SCALED) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -284,6 +303,14 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
     }
   };
   auto compute = [&](Buf& b, int tok, bool checked) {
+    if constexpr (PAD) {
+#pragma unroll
+      for (int u = 0; u < TILES; ++u) {
+        keep_rows<CK>(b.k[u], k_keep);
+        keep_rows<CV>(b.v[u], v_keep);
+        if constexpr (SPLIT_KD) keep_rows<CK>(b.d[u], k_keep);
+      }
+    }
     if (!checked && tok + kStep > t_end) {  // last step of the chunk: some tiles were moved back
 #pragma unroll
       for (int u = 0; u < TILES; ++u) {
@@ -420,13 +447,14 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
 
   // one chunk per (sequence, head): the sum is final, store it scaled where the reduce
   // kernel would have put it; otherwise store this chunk's partial
-  float* mat = fin_mat ? fin_mat + (int64_t)nh * DK * DV
-                       : partial + ((int64_t)nh * nchunks + c) * (DK * DV + DK);
-  float* vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * DK : nullptr) : mat + DK * DV;
+  float* mat = fin_mat ? fin_mat + (int64_t)nh * dk * dv
+                       : partial + ((int64_t)nh * nchunks + c) * (dk * dv + dk);
+  float* vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : mat + dk * dv;
   const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
   const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
-  reduce_store_block<G>(acc, ks, red + (G > 1 ? blk * 64 * 66 : 0), mat + (64 * bk) * DV + 64 * bv, DV,
-                        (vec && bv == 0) ? vec + 64 * bk : nullptr, mscale, vscale, g, lane);
+  reduce_store_block<G>(acc, ks, red + (G > 1 ? blk * 64 * 66 : 0), mat + (64 * bk) * dv + 64 * bv, dv,
+                        (vec && bv == 0) ? vec + 64 * bk : nullptr, mscale, vscale, g, lane,
+                        PAD ? dk - 64 * bk : 64, PAD ? dv - 64 * bv : 64);
 }
 
 // ===========================================================================
@@ -444,11 +472,14 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
 // (the per-chunk partials of a reduction): they are added in index order and the
 // sum is multiplied by `mscale`; when `mat_out` is given the reduced matrix is
 // also written there in memory order.
-template <typename T, int DR, int DC, int NT = kThreads>
+// PAD = true: the matrix in memory is dr x dc (multiples of 8, at most DR x DC); the
+// operand's remaining rows and columns are zero.
+template <typename T, int DR, int DC, int NT = kThreads, bool PAD = false>
 __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* lds_max,
                                                const float* __restrict__ mat, int ld_r, int ld_c,
                                                int nsum = 1, int64_t sum_stride = 0,
-                                               float mscale = 1.f, float* mat_out = nullptr) {
+                                               float mscale = 1.f, float* mat_out = nullptr,
+                                               int dr = DR, int dc = DC) {
   constexpr int KS = DR / 16;
   constexpr int kPer = DR * DC / (4 * NT);  // float4 loads per thread
   typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -456,17 +487,29 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
   // one coalesced sweep over the matrix as it lies in memory; values stay in registers
   f32x4 vals[kPer];
   float mx = 0.f;
+  const bool c_fast = ld_c == 1;  // memory index = r*dc + c, else c*dr + r
+  // where this thread's i-th group of four operand elements lies in memory (-1: padding)
+  auto mem_index = [&](int i) {
+    const int e = 4 * (tid + NT * i);
+    if constexpr (!PAD) return e;
+    const int r = c_fast ? e / DC : e % DR, cc = c_fast ? e % DC : e / DR;
+    if (r >= dr || cc >= dc) return -1;
+    return c_fast ? r * dc + cc : cc * dr + r;
+  };
 #pragma unroll
   for (int i = 0; i < kPer; ++i) vals[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int c = 0; c < nsum; ++c) {
 #pragma unroll
-    for (int i = 0; i < kPer; ++i)
-      vals[i] += *reinterpret_cast<const f32x4*>(mat + (int64_t)c * sum_stride + 4 * (tid + NT * i));
+    for (int i = 0; i < kPer; ++i) {
+      const int idx = mem_index(i);
+      if (!PAD || idx >= 0) vals[i] += *reinterpret_cast<const f32x4*>(mat + (int64_t)c * sum_stride + idx);
+    }
   }
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
     vals[i] *= mscale;
-    if (mat_out) *reinterpret_cast<f32x4*>(mat_out + 4 * (tid + NT * i)) = vals[i];
+    const int idx = mem_index(i);
+    if (mat_out && (!PAD || idx >= 0)) *reinterpret_cast<f32x4*>(mat_out + idx) = vals[i];
 #pragma unroll
     for (int j = 0; j < 4; ++j) mx = fmaxf(mx, fabsf(vals[i][j]));
   }
@@ -484,7 +527,6 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
     norm = ldexpf(1.f, 4 - e);
   }
   uint16_t* op16 = reinterpret_cast<uint16_t*>(lds_opnd);
-  const bool c_fast = ld_c == 1;  // memory index = r*DC + c, else c*DR + r
 #pragma unroll
   for (int i = 0; i < kPer; ++i)
 #pragma unroll
@@ -509,13 +551,16 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
 // `src` may be the vector part of the first of `nsum` partials (see build_operand);
 // the sum times `vscale` is the vector.  It is stored as pairs (when `pairs`), as
 // fp32 in LDS (when `f32`) and to memory (when `vec_out`).
+// The LDS copies hold DP >= D entries (DP = 0 stands for D), zero past the first D.
 template <typename T, int NT = kThreads>
 __device__ __forceinline__ void build_vec(uint32_t* pairs, float* f32, const float* __restrict__ src,
                                           int D, int nsum = 1, int64_t sum_stride = 0,
-                                          float vscale = 1.f, float* vec_out = nullptr) {
-  for (int e = threadIdx.x; e < D / 2; e += NT) {
+                                          float vscale = 1.f, float* vec_out = nullptr, int DP = 0) {
+  if (DP == 0) DP = D;
+  for (int e = threadIdx.x; e < DP / 2; e += NT) {
     float a = 0.f, b = 0.f;
-    for (int c = 0; c < nsum; ++c) {
+    const bool real = 2 * e < D;
+    for (int c = 0; real && c < nsum; ++c) {
       a += src[(int64_t)c * sum_stride + 2 * e];
       b += src[(int64_t)c * sum_stride + 2 * e + 1];
     }
@@ -524,13 +569,13 @@ __device__ __forceinline__ void build_vec(uint32_t* pairs, float* f32, const flo
     if (pairs) {
       const T ah = (T)a, bh = (T)b;
       pairs[e] = pack2<T>((float)ah, (float)bh);
-      pairs[D / 2 + e] = pack2<T>(a - (float)ah, b - (float)bh);
+      pairs[DP / 2 + e] = pack2<T>(a - (float)ah, b - (float)bh);
     }
     if (f32) {
       f32[2 * e] = a;
       f32[2 * e + 1] = b;
     }
-    if (vec_out) {
+    if (vec_out && real) {
       vec_out[2 * e] = a;
       vec_out[2 * e + 1] = b;
     }
@@ -551,9 +596,14 @@ template <int DR, int DC, bool DEN, int WAVES> struct RowsLayout {
 
 // One launch can carry two independent jobs of the same shape (the dk and dv
 // products of backward pass B): workgroups [0, wgs_per_job) run job0, the rest job1.
-template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES>
+// PAD = true: rows are dr (x) and dc (out) elements long in memory, multiples of 8 below the
+// template's DR, DC; the staged tiles keep the padded width, with zeros in the padding.
+template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD = false>
 __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, RowsJob job1,
-                                                          int wgs_per_job, int chunk, int nchunks) {
+                                                          int wgs_per_job, int chunk, int nchunks,
+                                                          int dr_true, int dc_true) {
+  const int dr = PAD ? dr_true : DR, dc = PAD ? dc_true : DC;
+  const int dpk = PAD ? (p.DK <= 64 ? 64 : 128) : p.DK;  // padded length of the km / dkm vector
   using LY = RowsLayout<DR, DC, DEN, WAVES>;
   const bool second = (int)blockIdx.x >= wgs_per_job;
   const RowsJob& job = second ? job1 : job0;
@@ -581,7 +631,7 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
   if (t_begin >= len) {
     if (c == 0 && job.pnchunks > 0) {  // empty sequence: its state is zero
       if (job.mat_out)
-        for (int e = threadIdx.x; e < DR * DC; e += NT) job.mat_out[(int64_t)nh * DR * DC + e] = 0.f;
+        for (int e = threadIdx.x; e < dr * dc; e += NT) job.mat_out[(int64_t)nh * dr * dc + e] = 0.f;
       if (job.vec_out)
         for (int e = threadIdx.x; e < p.DK; e += NT) job.vec_out[(int64_t)nh * p.DK + e] = 0.f;
     }
@@ -608,8 +658,8 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
     for (int i = 0; i < XI; ++i) {
       const int q = lane + 64 * i, row = q / XCH, ch = q % XCH;
       const int tok = tok0 + row;
-      if (tok < t_end) {
-        dst[i] = *reinterpret_cast<const u32x4*>(src + (row0 + (int64_t)tok * rstride) * DR + ch * 8);
+      if (tok < t_end && (!PAD || ch * 8 < dr)) {
+        dst[i] = *reinterpret_cast<const u32x4*>(src + (row0 + (int64_t)tok * rstride) * dr + ch * 8);
       } else {
         dst[i] = u32x4{0u, 0u, 0u, 0u};
       }
@@ -636,27 +686,28 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
   // workgroup of a head computes the same sums; chunk 0 also stores them).
   float denorm;
   if (job.pnchunks > 0) {
-    constexpr int E = DR * DC;
+    const int E = dr * dc;
     const int64_t pstride = E + p.DK;
     const int nsum = (len + job.pchunk - 1) / job.pchunk;
     const float* part = job.mat + (int64_t)nh * job.pnchunks * pstride;
     const bool writer = c == 0;
-    denorm = build_operand<T, DR, DC, NT>(lds_opnd, lds_max, part, job.ld_r, job.ld_c, nsum, pstride,
-                                          seq_scale(p, len),
-                                          writer && job.mat_out ? job.mat_out + (int64_t)nh * E : nullptr);
+    denorm = build_operand<T, DR, DC, NT, PAD>(lds_opnd, lds_max, part, job.ld_r, job.ld_c, nsum, pstride,
+                                               seq_scale(p, len),
+                                               writer && job.mat_out ? job.mat_out + (int64_t)nh * E : nullptr,
+                                               dr, dc);
     const float inv_len = 1.0f / (float)len;
     float* vout = writer && job.vec_out ? job.vec_out + (int64_t)nh * p.DK : nullptr;
     if (NORM || job.vec_is_add || vout)
       build_vec<T, NT>(NORM ? lds_km : nullptr, job.vec_is_add ? lds_add : nullptr, part + E, p.DK,
-                       nsum, pstride, inv_len, vout);
+                       nsum, pstride, inv_len, vout, dpk);
     if (!job.vec_is_add)
       for (int e = tid; e < DC; e += NT) lds_add[e] = 0.f;
   } else {
-    denorm = build_operand<T, DR, DC, NT>(lds_opnd, lds_max, job.mat + (int64_t)nh * DR * DC, job.ld_r,
-                                          job.ld_c);
-    if constexpr (NORM) build_vec<T, NT>(lds_km, nullptr, job.km + (int64_t)nh * DR, DR);
+    denorm = build_operand<T, DR, DC, NT, PAD>(lds_opnd, lds_max, job.mat + (int64_t)nh * dr * dc, job.ld_r,
+                                               job.ld_c, 1, 0, 1.f, nullptr, dr, dc);
+    if constexpr (NORM) build_vec<T, NT>(lds_km, nullptr, job.km + (int64_t)nh * dr, dr, 1, 0, 1.f, nullptr, DR);
     for (int e = tid; e < DC; e += NT)
-      lds_add[e] = job.addvec ? job.addvec[(int64_t)nh * DC + e] : 0.f;
+      lds_add[e] = (job.addvec && e < dc) ? job.addvec[(int64_t)nh * dc + e] : 0.f;
   }
   __syncthreads();
 
@@ -724,9 +775,9 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
     for (int i = 0; i < OI; ++i) {
       const int q = lane + 64 * i, row = q / OCH, ch = q % OCH;
       const int tok = t0 + row;
-      if (tok < t_end) {
+      if (tok < t_end && (!PAD || ch * 8 < dc)) {
         const u32x4 w = *reinterpret_cast<const u32x4*>(stage + swz<OROWB>(row, ch));
-        *reinterpret_cast<u32x4*>(out + (row0 + (int64_t)tok * rstride) * DC + ch * 8) = w;
+        *reinterpret_cast<u32x4*>(out + (row0 + (int64_t)tok * rstride) * dc + ch * 8) = w;
       }
     }
     t0 = tn;
@@ -775,7 +826,9 @@ template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struc
 // FUSED = false runs the token view only (head dims whose dS accumulators do not
 // fit one wave): it writes 1/z_t and dz_t per (token, head) row to `tokscal`
 // ([2][total rows]) for scaled_state_kernel, and no partials.
-template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true>
+// PAD = true: head dims p.DK, p.DV (multiples of 8) below the template's DK, DV, as in the
+// other kernels: true row lengths in memory, zero padding in the staged tiles and operands.
+template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true, bool PAD = false>
 __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const T* __restrict__ dout,
     const float* __restrict__ S, const float* __restrict__ km, T* __restrict__ dqn,
@@ -784,6 +837,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
   using LY = BwdALayout<DK, DV, NORM, DEN, FUSED, LO>;
   constexpr int KS = LY::KS, NB = LY::NB;
   constexpr int CK = DK / 32, CV = DV / 32;
+  const int dk = PAD ? p.DK : DK, dv = PAD ? p.DV : DV;
   constexpr int QROWB = DK * 2, GROWB = DV * 2;
   constexpr int QCH = QROWB / 16, GCH = GROWB / 16;
   constexpr int QI = 32 * QCH / 64, GI = 32 * GCH / 64;
@@ -799,9 +853,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
   const int t_begin = c * chunk;
   if (t_begin >= len) {
     if (fin_mat && c == 0) {  // empty sequence: no gradient flows through its state
-      for (int e = threadIdx.x; e < DK * DV; e += kThreads) fin_mat[(int64_t)nh * DK * DV + e] = 0.f;
+      for (int e = threadIdx.x; e < dk * dv; e += kThreads) fin_mat[(int64_t)nh * dk * dv + e] = 0.f;
       if (fin_vec)
-        for (int e = threadIdx.x; e < DK; e += kThreads) fin_vec[(int64_t)nh * DK + e] = 0.f;
+        for (int e = threadIdx.x; e < dk; e += kThreads) fin_vec[(int64_t)nh * dk + e] = 0.f;
     }
     return;
   }
@@ -837,8 +891,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     for (int i = 0; i < QI; ++i) {
       const int q = lane + 64 * i, row = q / QCH, ch = q % QCH;
       const int tok = tok0 + row;
-      dst[i] = tok < t_end
-                   ? *reinterpret_cast<const u32x4*>(src + (row0 + (int64_t)tok * rstride) * DK + ch * 8)
+      dst[i] = (tok < t_end && (!PAD || ch * 8 < dk))
+                   ? *reinterpret_cast<const u32x4*>(src + (row0 + (int64_t)tok * rstride) * dk + ch * 8)
                    : u32x4{0u, 0u, 0u, 0u};
     }
   };
@@ -847,8 +901,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     for (int i = 0; i < GI; ++i) {
       const int q = lane + 64 * i, row = q / GCH, ch = q % GCH;
       const int tok = tok0 + row;
-      dst[i] = tok < t_end
-                   ? *reinterpret_cast<const u32x4*>(src + (row0 + (int64_t)tok * rstride) * DV + ch * 8)
+      dst[i] = (tok < t_end && (!PAD || ch * 8 < dv))
+                   ? *reinterpret_cast<const u32x4*>(src + (row0 + (int64_t)tok * rstride) * dv + ch * 8)
                    : u32x4{0u, 0u, 0u, 0u};
     }
   };
@@ -871,8 +925,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     for (int i = 0; i < QI; ++i) {
       const int q = lane + 64 * i, row = q / QCH, ch = q % QCH;
       const int tok = tok0 + row;
-      if (tok < t_end)
-        *reinterpret_cast<u32x4*>(dst + (row0 + (int64_t)tok * rstride) * DK + ch * 8) =
+      if (tok < t_end && (!PAD || ch * 8 < dk))
+        *reinterpret_cast<u32x4*>(dst + (row0 + (int64_t)tok * rstride) * dk + ch * 8) =
             *reinterpret_cast<const u32x4*>(srcb + swz<QROWB>(row, ch));
     }
   };
@@ -886,9 +940,10 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
   }
 
   // g_t = dO_t S^T: contraction over dv, M(r = dv, c = dk) = S[c][r]
-  const float denorm = build_operand<T, DV, DK>(lds_opnd, lds_max, S + (int64_t)nh * DK * DV, 1, DV);
+  const float denorm = build_operand<T, DV, DK, kThreads, PAD>(lds_opnd, lds_max, S + (int64_t)nh * dk * dv, 1,
+                                                               dv, 1, 0, 1.f, nullptr, dv, dk);
   if constexpr (NORM) {
-    build_vec<T>(km_pairs, kmf, km + (int64_t)nh * DK, DK);
+    build_vec<T>(km_pairs, kmf, km + (int64_t)nh * dk, dk, 1, 0, 1.f, nullptr, DK);
   }
   __syncthreads();
 
@@ -1058,30 +1113,36 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
   if constexpr (FUSED) {
     __syncthreads();  // every wave is done with its tiles: reuse them for the reduction
     float* red = reinterpret_cast<float*>(smem + LY::kOpnd);
-    float* dst = fin_mat ? fin_mat + (int64_t)nh * DK * DV
-                         : partial + ((int64_t)nh * nchunks + c) * (DK * DV + DK);
-    float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * DK : nullptr) : dst + DK * DV;
+    float* dst = fin_mat ? fin_mat + (int64_t)nh * dk * dv
+                         : partial + ((int64_t)nh * nchunks + c) * (dk * dv + dk);
+    float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : dst + dk * dv;
     const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
     const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
-    reduce_store_block<4>(acc, dkm, red, dst, DV, dst_vec, mscale, vscale, wave, lane);
+    reduce_store_block<4>(acc, dkm, red, dst, dv, dst_vec, mscale, vscale, wave, lane, dk, dv);
   }
 }
 
 // ===========================================================================
 // host side
 // ===========================================================================
-// 16-bit inputs with head dims 64 or 128; the decoupled operator only at 64 x 64.
+// The kernels tile a head into 64-wide blocks: a head dim runs as the next of 64 / 128 above
+// it, the padded variants (PAD) when it is not one of the two.
+static int tiled_dim(int d) { return d <= 64 ? 64 : 128; }
+static bool padded(const Prob& p) { return p.DK != tiled_dim(p.DK) || p.DV != tiled_dim(p.DV); }
+
+// 16-bit inputs with head dims that are multiples of 8 (16-byte row pieces) up to 128; the
+// decoupled operator up to 64 x 64.
 bool supported(const Prob& p, int dtype) {
   if (dtype == kF32) return mfma32::supported(p);
   if (dtype != kF16 && dtype != kBF16) return false;
-  if (!((p.DK == 64 || p.DK == 128) && (p.DV == 64 || p.DV == 128))) return false;
-  if ((p.flags & kDecoupled) && !(p.DK == 64 && p.DV == 64)) return false;
+  if (p.DK < 8 || p.DV < 8 || p.DK > 128 || p.DV > 128 || p.DK % 8 || p.DV % 8) return false;
+  if ((p.flags & kDecoupled) && !(p.DK <= 64 && p.DV <= 64)) return false;
   return true;
 }
 
-// The fused backward pass A exists for 64 x 64 heads.
+// The fused backward pass A exists for heads up to 64 x 64.
 bool bwd_a_supported(const Prob& p, int dtype) {
-  return dtype != kF32 && supported(p, dtype) && p.DK == 64 && p.DV == 64;
+  return dtype != kF32 && supported(p, dtype) && p.DK <= 64 && p.DV <= 64;
 }
 
 // Number of compute units of the current device (256 on MI355X; also the value
@@ -1138,26 +1199,38 @@ int rows_chunk(const Prob& p, int DR, int DC) {
   static const int dense_rounds = knob("FBLA_ROWS_ROUNDS", 4);
   static const int packed_rounds = knob("FBLA_ROWS_ROUNDS_PACKED", 1);
   // a 128 x 128 operand costs as much to build as 512 tokens cost to stream: one round there
-  const int big = (DR == 128) + (DC == 128);
+  const int big = (tiled_dim(DR) == 128) + (tiled_dim(DC) == 128);
   const int rounds = p.cu ? packed_rounds : (big == 2 ? 1 : big == 1 ? (dense_rounds + 1) / 2 : dense_rounds);
   const int per_cu = big == 0 ? per_cu_knob : (big == 1 ? 2 : 1);
   return chunk_for(p, per_cu, rounds, 512, big == 2 ? 256 : 128);
 }
 
-template <typename T, int DK, int DV>
+template <typename T, int DK, int DV, bool PAD>
 static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, float* partial,
                          const float* tokscal, int64_t total_rows, float* fm, float* fv, int chunk,
                          int nchunks, BlockStats bs, hipStream_t st) {
   const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(kThreads);
   constexpr int TL = 1;  // 16-token tiles per step and wave
-  if (bs.kc)
-    state_kernel<T, DK, DV, false, 1, false, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
-  else if (tokscal)
-    state_kernel<T, DK, DV, false, TL, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fm, fv, chunk, nchunks, bs);
+  if (bs.kc) {
+    if constexpr (!PAD)
+      state_kernel<T, DK, DV, false, 1, false, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
+  } else if (tokscal)
+    state_kernel<T, DK, DV, false, TL, true, false, PAD><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fm, fv, chunk, nchunks, bs);
   else if (p.flags & kDecoupled)
-    state_kernel<T, DK, DV, true, TL, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
+    state_kernel<T, DK, DV, true, TL, false, false, PAD><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
   else
-    state_kernel<T, DK, DV, false, TL, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
+    state_kernel<T, DK, DV, false, TL, false, false, PAD><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
+}
+
+template <typename T, bool PAD>
+static void run_state_dims(const Prob& p, const T* a, const T* b, const T* c, float* partial,
+                           const float* ts, int64_t rows, float* fm, float* fv, int chunk, int nchunks,
+                           BlockStats bs, hipStream_t st) {
+  const int DK = tiled_dim(p.DK), DV = tiled_dim(p.DV);
+  if (DK == 64 && DV == 64) launch_state<T, 64, 64, PAD>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
+  else if (DK == 64) launch_state<T, 64, 128, PAD>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
+  else if (DV == 64) launch_state<T, 128, 64, PAD>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
+  else launch_state<T, 128, 128, PAD>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
 }
 
 template <typename T>
@@ -1165,10 +1238,8 @@ static void run_state(const Prob& p, const void* kn, const void* v, const void* 
                       const float* ts, int64_t rows, float* fm, float* fv, int chunk, int nchunks,
                       BlockStats bs, hipStream_t st) {
   const T *a = (const T*)kn, *b = (const T*)v, *c = (const T*)kd;
-  if (p.DK == 64 && p.DV == 64) launch_state<T, 64, 64>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
-  else if (p.DK == 64) launch_state<T, 64, 128>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
-  else if (p.DV == 64) launch_state<T, 128, 64>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
-  else launch_state<T, 128, 128>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
+  if (padded(p)) run_state_dims<T, true>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
+  else run_state_dims<T, false>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
 }
 
 // Reserves the kernel's dynamic LDS once per instantiation and thread.
@@ -1184,22 +1255,23 @@ template <typename K> static int reserve_lds(K kernel, int bytes, bool& done) {
   return kOk;
 }
 
-template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES>
+template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD>
 static int launch_rows_k(const Prob& p, const RowsJob& job, const RowsJob* job2, int chunk,
-                         int nchunks, hipStream_t st) {
+                         int nchunks, int dr, int dc, hipStream_t st) {
   using LY = RowsLayout<DR, DC, DEN, WAVES>;
-  auto kernel = rows_kernel<T, DR, DC, NORM, DEN, WAVES>;
+  auto kernel = rows_kernel<T, DR, DC, NORM, DEN, WAVES, PAD>;
   static thread_local bool configured = false;
   int rc = reserve_lds(kernel, LY::kTotal, configured);
   if (rc != kOk) return rc;
   const int wgs = (int)((int64_t)p.N * p.H * nchunks);
   const dim3 grid((unsigned)(job2 ? 2 * wgs : wgs)), block(WAVES * 64);
-  kernel<<<grid, block, LY::kTotal, st>>>(p, job, job2 ? *job2 : job, wgs, chunk, nchunks);
+  kernel<<<grid, block, LY::kTotal, st>>>(p, job, job2 ? *job2 : job, wgs, chunk, nchunks, dr, dc);
   return kOk;
 }
 
-template <typename T, int DR, int DC>
-static int launch_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, hipStream_t st) {
+template <typename T, int DR, int DC, bool PAD>
+static int launch_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, int dr, int dc,
+                       hipStream_t st) {
   // 128 x 128 operands fill 64 KiB of LDS: one 8-wave workgroup per CU instead of
   // several 4-wave ones
   constexpr int WAVES = (DR == 128 && DC == 128) ? 8 : 4;
@@ -1207,21 +1279,29 @@ static int launch_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, h
   const int nchunks = (int)cdiv64(p.L, chunk);
   const bool norm = job.xden != nullptr;
   const bool den = norm && job.xden != job.x;
-  if (!norm) return launch_rows_k<T, DR, DC, false, false, WAVES>(p, job, job2, chunk, nchunks, st);
-  if (!den) return launch_rows_k<T, DR, DC, true, false, WAVES>(p, job, job2, chunk, nchunks, st);
+  if (!norm) return launch_rows_k<T, DR, DC, false, false, WAVES, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
+  if (!den) return launch_rows_k<T, DR, DC, true, false, WAVES, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
   if constexpr (DR == 64 && DC == 64)
-    return launch_rows_k<T, DR, DC, true, true, WAVES>(p, job, job2, chunk, nchunks, st);
-  set_error("decoupled rows kernel exists only for 64 x 64 heads");
+    return launch_rows_k<T, DR, DC, true, true, WAVES, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
+  set_error("decoupled rows kernel exists only for heads up to 64 x 64");
   return kErrUnsupported;
 }
 
+template <typename T, bool PAD>
+static int run_rows_dims(const Prob& p, const RowsJob& job, const RowsJob* job2, int dr, int dc,
+                         hipStream_t st) {
+  const int DR = tiled_dim(dr), DC = tiled_dim(dc);
+  if (DR == 64 && DC == 64) return launch_rows<T, 64, 64, PAD>(p, job, job2, dr, dc, st);
+  if (DR == 64) return launch_rows<T, 64, 128, PAD>(p, job, job2, dr, dc, st);
+  if (DC == 64) return launch_rows<T, 128, 64, PAD>(p, job, job2, dr, dc, st);
+  return launch_rows<T, 128, 128, PAD>(p, job, job2, dr, dc, st);
+}
+
 template <typename T>
-static int run_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, int DR, int DC,
+static int run_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, int dr, int dc,
                     hipStream_t st) {
-  if (DR == 64 && DC == 64) return launch_rows<T, 64, 64>(p, job, job2, st);
-  if (DR == 64) return launch_rows<T, 64, 128>(p, job, job2, st);
-  if (DC == 64) return launch_rows<T, 128, 64>(p, job, job2, st);
-  return launch_rows<T, 128, 128>(p, job, job2, st);
+  if (padded(p)) return run_rows_dims<T, true>(p, job, job2, dr, dc, st);
+  return run_rows_dims<T, false>(p, job, job2, dr, dc, st);
 }
 
 void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
@@ -1268,17 +1348,18 @@ int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, in
   return run_rows<__bf16>(p, job0, &job1, DR, DC, st);
 }
 
-template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true>
+template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool PAD>
 static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, const float* S,
                         const float* km, T* dqn, T* dqd, float* partial, float* tokscal,
                         int64_t total_rows, float* fm, float* fv, int chunk, int nchunks,
                         hipStream_t st) {
+  constexpr bool LO = true;
   using LY = BwdALayout<DK, DV, NORM, DEN, FUSED, LO>;
   static_assert(!FUSED || LY::kTotal - LY::kOpnd >=
                               (int)sizeof(float) * 64 * ((DK / 32) * (DV / 32) * 16 + DK / 32),
                 "reduction buffer must fit in the tile area");
   static_assert(LY::kTotal <= 160 * 1024, "LDS budget of one workgroup");
-  auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN, FUSED, LO>;
+  auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN, FUSED, LO, PAD>;
   static thread_local bool configured = false;  // per instantiation
   int rc = reserve_lds(kernel, LY::kTotal, configured);
   if (rc != kOk) return rc;
@@ -1288,17 +1369,25 @@ static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, 
   return kOk;
 }
 
+template <typename T, bool PAD>
+static int run_bwd_a_pad(const Prob& p, const void* qn, const void* qd, const void* dout, const float* S,
+                         const float* km, void* dqn, void* dqd, float* partial, float* fm, float* fv,
+                         int chunk, int nchunks, hipStream_t st) {
+  const T *a = (const T*)qn, *b = (const T*)qd, *c = (const T*)dout;
+  T *x = (T*)dqn, *y = (T*)dqd;
+  if (!(p.flags & kNormalize))
+    return launch_bwd_a<T, 64, 64, false, false, true, PAD>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+  if (p.flags & kDecoupled)
+    return launch_bwd_a<T, 64, 64, true, true, true, PAD>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+  return launch_bwd_a<T, 64, 64, true, false, true, PAD>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+}
+
 template <typename T>
 static int run_bwd_a(const Prob& p, const void* qn, const void* qd, const void* dout, const float* S,
                      const float* km, void* dqn, void* dqd, float* partial, float* fm, float* fv,
                      int chunk, int nchunks, hipStream_t st) {
-  const T *a = (const T*)qn, *b = (const T*)qd, *c = (const T*)dout;
-  T *x = (T*)dqn, *y = (T*)dqd;
-  if (!(p.flags & kNormalize))
-    return launch_bwd_a<T, 64, 64, false, false, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
-  if (p.flags & kDecoupled)
-    return launch_bwd_a<T, 64, 64, true, true, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
-  return launch_bwd_a<T, 64, 64, true, false, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+  if (padded(p)) return run_bwd_a_pad<T, true>(p, qn, qd, dout, S, km, dqn, dqd, partial, fm, fv, chunk, nchunks, st);
+  return run_bwd_a_pad<T, false>(p, qn, qd, dout, S, km, dqn, dqd, partial, fm, fv, chunk, nchunks, st);
 }
 
 int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout, const float* S,
@@ -1309,32 +1398,42 @@ int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* 
   return run_bwd_a<__bf16>(p, qn, qd, dout, S, km, dqn, dqd, partial, fin_mat, fin_vec, chunk, nchunks, st);
 }
 
-template <typename T, int DK, int DV>
+template <typename T, int DK, int DV, bool PAD>
 static int launch_bwd_tokens(const Prob& p, const void* q, const void* dout, const float* S,
                              const float* km, void* dq, float* tokscal, int64_t total_rows,
                              int chunk, int nchunks, hipStream_t st) {
   const T *a = (const T*)q, *c = (const T*)dout;
   if (p.flags & kNormalize)
-    return launch_bwd_a<T, DK, DV, true, false, false>(p, a, a, c, S, km, (T*)dq, nullptr, nullptr,
-                                                       tokscal, total_rows, nullptr, nullptr, chunk,
-                                                       nchunks, st);
-  return launch_bwd_a<T, DK, DV, false, false, false>(p, a, a, c, S, km, (T*)dq, nullptr, nullptr,
-                                                      tokscal, total_rows, nullptr, nullptr, chunk,
-                                                      nchunks, st);
+    return launch_bwd_a<T, DK, DV, true, false, false, PAD>(p, a, a, c, S, km, (T*)dq, nullptr, nullptr,
+                                                            tokscal, total_rows, nullptr, nullptr, chunk,
+                                                            nchunks, st);
+  return launch_bwd_a<T, DK, DV, false, false, false, PAD>(p, a, a, c, S, km, (T*)dq, nullptr, nullptr,
+                                                           tokscal, total_rows, nullptr, nullptr, chunk,
+                                                           nchunks, st);
+}
+
+template <typename T, bool PAD>
+static int run_bwd_tokens_dims(const Prob& p, const void* q, const void* dout, const float* S,
+                               const float* km, void* dq, float* tokscal, int64_t total_rows, int chunk,
+                               int nchunks, hipStream_t st) {
+  const int DK = tiled_dim(p.DK), DV = tiled_dim(p.DV);
+  if (DK == 64 && DV == 128)
+    return launch_bwd_tokens<T, 64, 128, PAD>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
+  if (DK == 128 && DV == 64)
+    return launch_bwd_tokens<T, 128, 64, PAD>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
+  return launch_bwd_tokens<T, 128, 128, PAD>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
 }
 
 template <typename T>
 static int run_bwd_tokens(const Prob& p, const void* q, const void* dout, const float* S,
                           const float* km, void* dq, float* tokscal, int64_t total_rows,
                           hipStream_t st) {
-  const int big = (p.DK == 128) + (p.DV == 128);
+  const int big = (tiled_dim(p.DK) == 128) + (tiled_dim(p.DV) == 128);
   const int chunk = chunk_for(p, big == 2 ? 1 : 2, 1, 512, 128);
   const int nchunks = (int)cdiv64(p.L, chunk);
-  if (p.DK == 64 && p.DV == 128)
-    return launch_bwd_tokens<T, 64, 128>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
-  if (p.DK == 128 && p.DV == 64)
-    return launch_bwd_tokens<T, 128, 64>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
-  return launch_bwd_tokens<T, 128, 128>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
+  if (padded(p))
+    return run_bwd_tokens_dims<T, true>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
+  return run_bwd_tokens_dims<T, false>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
 }
 
 // token view of the backward alone: dq and the per-row scalars 1/z_t, dz_t

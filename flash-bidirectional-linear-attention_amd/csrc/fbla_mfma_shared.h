@@ -48,11 +48,15 @@ __device__ __forceinline__ int lpt_sequence(const Prob& p, int rank, int* lens /
 // matrix (leading dimension ld), dst_vec (optional) at the block's 64 entries of the vector.
 // Register r of accumulator (a,b) is row 2*m + a, column 2*pp + b with
 // m = 8*(r/4) + 4*kb + r%4 (PAIRED: lanes own feature pairs, the 16-bit kernels) or row
-// 32*a + m, column 32*b + pp (lanes own single features, the fp32 kernels).  Must be reached by all waves of the workgroup.
+// 32*a + m, column 32*b + pp (lanes own single features, the fp32 kernels).  Only the first
+// `rows_ok` rows and `cols_ok` columns of the block are stored (a head dim that is not a
+// multiple of 64 leaves the rest of its last block as padding).  Must be reached by all waves
+// of the workgroup.
 template <int G, bool PAIRED = true>
 __device__ __forceinline__ void reduce_store_block(f32x16 (&acc)[2][2], float (&ks)[2], float* red,
                                                    float* dst, int ld, float* dst_vec, float mscale,
-                                                   float vscale, int g, int lane) {
+                                                   float vscale, int g, int lane, int rows_ok = 64,
+                                                   int cols_ok = 64) {
   const int pp = lane & 31, kb = lane >> 5;
   auto spill = [&]() {
 #pragma unroll
@@ -99,14 +103,15 @@ __device__ __forceinline__ void reduce_store_block(f32x16 (&acc)[2][2], float (&
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = 8 * (r >> 2) + 4 * kb + (r & 3);
-        if constexpr (PAIRED) dst[(2 * m + a) * ld + 2 * pp + b] = acc[a][b][r] * mscale;
-        else dst[(32 * a + m) * ld + 32 * b + pp] = acc[a][b][r] * mscale;
+        const int row = PAIRED ? 2 * m + a : 32 * a + m, col = PAIRED ? 2 * pp + b : 32 * b + pp;
+        if (row < rows_ok && col < cols_ok) dst[row * ld + col] = acc[a][b][r] * mscale;
       }
   if (dst_vec) {
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
       const float tot = ks[a] + __shfl_xor(ks[a], 32);
-      if (kb == 0) dst_vec[PAIRED ? 2 * pp + a : 32 * a + pp] = tot * vscale;
+      const int row = PAIRED ? 2 * pp + a : 32 * a + pp;
+      if (kb == 0 && row < rows_ok) dst_vec[row] = tot * vscale;
     }
   }
 }

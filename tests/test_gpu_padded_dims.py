@@ -1,0 +1,90 @@
+"""Head dims that are multiples of 8 but not 64 or 128 (the MLLA / RALA blocks use 32, the
+PolaFormer block 2d x d/2) run on the matrix-core kernels with the last 64-wide block of a
+head partly empty.  Forward and backward of every operator family against the float64
+oracle, dense and packed, with sequence lengths that take the single-chunk path, the
+path with several chunks per head, ragged tiles and one-token sequences."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_parity, make_qkv, np64, parity_errors
+from oracle import closed_form as cf
+
+pytestmark = pytest.mark.gpu
+
+HEAD_DIMS = [(32, 32), (16, 16), (8, 8), (24, 40), (64, 32), (32, 64), (128, 32), (64, 16), (72, 72),
+             (96, 128), (120, 8), (128, 104), (48, 48)]
+LENGTHS = [1, 17, 300, 2500]
+
+
+def _check_dense(variant, B, H, L, DK, DV, dtype, seed):
+    from flash_bla.ops.linear_attn.decoupled import decoupled_la
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    from flash_bla.ops.simple_la.fused import simple_la
+    q, k, v, do, qr, kr = make_qkv((B, H, L, DK), (B, H, L, DV), dtype, seed, n_extra=2)
+    normalize = variant != "simple"
+    scale = 1.0 / L if normalize else DK ** -0.5
+    kw = dict(q_rope=np64(qr), k_rope=np64(kr)) if variant == "decoupled" else {}
+    ref = cf.dense_backward(np64(q), np64(k), np64(v), np64(do), scale, 1e-6, normalize, **kw)
+    tensors = (q, k, qr, kr, v) if variant == "decoupled" else (q, k, v)
+    leaves = [t.cuda().requires_grad_() for t in tensors]
+    op = {"linear": linear_attention, "simple": simple_la, "decoupled": decoupled_la}[variant]
+    names = ["dq", "dk", "dq_rope", "dk_rope", "dv"] if variant == "decoupled" else ["dq", "dk", "dv"]
+    o = op(*leaves)
+    o.backward(do.cuda())
+    errs = {"o": parity_errors(o, ref["o"], dtype)}
+    for name, t in zip(names, leaves):
+        errs[name] = parity_errors(t.grad, ref[name], dtype, ref.get(name + "_mag"))
+    bad = {n: e for n, e in errs.items() if not e[2]}
+    assert not bad, f"{variant} {dtype} B{B} H{H} L{L} DK{DK} DV{DV}: {errs}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dims", HEAD_DIMS)
+def test_dense_linear_attention(dims, dtype):
+    for i, L in enumerate(LENGTHS):
+        _check_dense("linear", 2, 3, L, dims[0], dims[1], dtype, 10 * i + dims[0])
+
+
+@pytest.mark.parametrize("dims", HEAD_DIMS)
+def test_dense_simple_la(dims):
+    for i, L in enumerate(LENGTHS[1:]):
+        _check_dense("simple", 1, 2, L, dims[0], dims[1], torch.float16, 20 * i + dims[1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dims", [(32, 32), (16, 16), (8, 24), (64, 32), (40, 64), (96, 32)])
+def test_dense_decoupled(dims, dtype):
+    for i, L in enumerate(LENGTHS):
+        _check_dense("decoupled", 2, 2, L, dims[0], dims[1], dtype, 30 * i + dims[0])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dims", [(32, 32), (16, 16), (48, 48), (96, 96), (32, 64), (128, 40), (8, 72)])
+def test_packed(dims, dtype):
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    DK, DV = dims
+    H = 5
+    lengths = [300, 1, 0, 17, 1200, 64, 33]
+    T = sum(lengths)
+    q, k, v, do = make_qkv((T, H, DK), (T, H, DV), dtype, DK + DV)
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lengths)]), dtype=torch.int32).cuda()
+    leaves = [t.cuda().requires_grad_() for t in (q, k, v)]
+    o = varlen_linear_attention(*leaves, cu, max(lengths))
+    o.backward(do.cuda())
+    ref = cf.varlen_backward(np64(q), np64(k), np64(v), np64(do), cu.cpu().numpy())
+    tag = f"{dtype} DK{DK} DV{DV}"
+    assert_parity(o, ref["o"], dtype, f"o {tag}")
+    for name, t in zip(("dq", "dk", "dv"), leaves):
+        for b, e in zip(cu[:-1].tolist(), cu[1:].tolist()):
+            if e > b:
+                floor = ref[name + "_mag"][b:e] if name + "_mag" in ref else None
+                assert_parity(t.grad[b:e], ref[name][b:e], dtype, f"{name}[{b}:{e}] {tag}", floor)
+
+
+def test_many_chunks_per_head():
+    """One head, long sequence: several chunks per head in every kernel, partials summed by the
+    consumers."""
+    _check_dense("linear", 1, 1, 20000, 32, 32, torch.float16, 7)
+    _check_dense("linear", 1, 1, 9000, 128, 32, torch.bfloat16, 8)
+    _check_dense("decoupled", 1, 1, 9000, 32, 32, torch.float16, 9)
