@@ -1,4 +1,6 @@
-// MFMA kernels for 16-bit inputs (fp16 / bf16) with head dims in {64, 128}.
+// MFMA kernels for 16-bit inputs (fp16 / bf16).  A head is tiled into 64-wide blocks:
+// head dims 64 and 128 exactly, every other multiple of 8 up to 128 as the next of the two
+// with the rest of its last block as zero padding (the PAD variants of the kernels).
 //
 // Every wave is an independent worker: it streams its own 16- or 32-token
 // sub-tiles, keeps fp32 accumulators in registers and touches LDS only through

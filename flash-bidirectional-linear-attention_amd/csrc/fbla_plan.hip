@@ -1,7 +1,7 @@
 // The plan: which kernels run, in which order, for each entry point, and how the
 // caller's workspace is carved up.  MFMA kernels are used for the shapes they
-// cover (16-bit inputs with head dims 64 / 128, fp32 inputs with 64 x 64 heads);
-// everything else runs on the generic kernels.
+// cover (16-bit inputs with head dims that are multiples of 8 up to 128, fp32 inputs
+// with 64 x 64 heads); everything else runs on the generic kernels.
 //
 // forward :  state partials -> fixed-order reduce (S, km) -> output rows
 // backward:  S^T -> pass A (dq, partial dS/dkm) -> reduce (s dS, its transpose, dkm/L)
