@@ -382,6 +382,28 @@ def other_configs(dev, flush):
     _report("decoupled_la B2-H16-T16384-D64 bf16 (benchmark_decoupled_la.py shape)", 6 * nb, 16 * nb, f, s, flush)
     del q, k, v, do, qr, kr
 
+    # head dims of the layer callers: MLLA / RALA blocks (decoupled, D=32: mlla.py:88, rala.py:74),
+    # PolaFormer (DK = 2d, DV = d/2: polaformer.py:75-90)
+    def feats(B, H, T, D, seed):
+        g = torch.Generator(device=dev).manual_seed(seed)
+        return (F.elu(torch.randn((B, H, T, D), generator=g, device=dev)) + 1).half().requires_grad_()
+
+    for name, B, H, T, DK, DV, dec in (("decoupled_la B64-H2-T3136-D32 fp16 (MLLA stage 1)", 64, 2, 3136, 32, 32, True),
+                                       ("decoupled_la B8-H16-T4096-D32 fp16", 8, 16, 4096, 32, 32, True),
+                                       ("linear_attn B8-H16-T4096-D32 fp16", 8, 16, 4096, 32, 32, False),
+                                       ("linear_attn B8-H16-T4096-DK128-DV32 fp16 (PolaFormer)", 8, 16, 4096, 128, 32, False)):
+        q, k = feats(B, H, T, DK, 1), feats(B, H, T, DK, 2)
+        v = torch.randn(B, H, T, DV, device=dev).half().requires_grad_()
+        do = torch.randn(B, H, T, DV, device=dev).half()
+        nqk, nv = q.numel() * 2, v.numel() * 2
+        if dec:
+            qr, kr = feats(B, H, T, DK, 3), feats(B, H, T, DK, 4)
+            f, s = run(decoupled_la, (q, k, qr, kr, v), do)
+            _report(name, 4 * nqk + 2 * nv, 11 * nqk + 5 * nv, f, s, flush)
+        else:
+            f, s = run(linear_attention, (q, k, v), do)
+            _report(name, 2 * nqk + 2 * nv, 6 * nqk + 5 * nv, f, s, flush)
+
     varlen_config(dev, flush)
 
 

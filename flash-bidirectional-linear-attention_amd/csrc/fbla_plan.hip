@@ -6,6 +6,8 @@
 // forward :  state partials -> fixed-order reduce (S, km) -> output rows
 // backward:  S^T -> pass A (dq, partial dS/dkm) -> reduce (s dS, its transpose, dkm/L)
 //            -> pass B (dk, dv)
+#include <stdlib.h>
+
 #include "fbla_kernels.h"
 
 namespace fbla {
@@ -42,7 +44,11 @@ static bool fold_reduce(const Prob& p, int reduce_nchunks, int DR, int DC) {
   const int64_t rows_nchunks = cdiv64(p.L, mfma::rows_chunk(p, DR, DC));
   const double extra = (double)p.N * p.H * (double)(rows_nchunks - 1) * reduce_nchunks *
                        ((double)p.DK * p.DV + p.DK) * sizeof(float);
-  return extra <= 16.0e6;
+  static const double limit = [] {
+    const char* v = getenv("FBLA_FOLD_MAX_MB");
+    return v && atof(v) > 0 ? atof(v) * 1e6 : 16.0e6;
+  }();
+  return extra <= limit;
 }
 
 size_t fwd_workspace_bytes(const Prob& p, int dtype) { return partial_bytes(p, fwd_chunk(p, dtype)); }
