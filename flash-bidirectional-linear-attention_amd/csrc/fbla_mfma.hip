@@ -42,6 +42,15 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
 
+// tiles in flight per wave in the rows kernel (128 x 128 heads run one 8-wave workgroup per
+// CU and have the registers for a deeper queue)
+#ifndef FBLA_ROWS_PF128
+#define FBLA_ROWS_PF128 1
+#endif
+#ifndef FBLA_ROWS_PF
+#define FBLA_ROWS_PF 1
+#endif
+
 template <typename T> struct Ops;
 
 template <> struct Ops<_Float16> {
@@ -485,37 +494,61 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
                                                float mscale = 1.f, float* mat_out = nullptr,
                                                int dr = DR, int dc = DC) {
   constexpr int KS = DR / 16;
-  constexpr int kPer = DR * DC / (4 * NT);  // float4 loads per thread
+  constexpr int kUnits = DR * DC / (8 * NT);  // units per thread
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  // one coalesced sweep over the matrix as it lies in memory; values stay in registers
-  f32x4 vals[kPer];
-  float mx = 0.f;
-  const bool c_fast = ld_c == 1;  // memory index = r*dc + c, else c*dr + r
-  // where this thread's i-th group of four operand elements lies in memory (-1: padding)
-  auto mem_index = [&](int i) {
-    const int e = 4 * (tid + NT * i);
-    if constexpr (!PAD) return e;
-    const int r = c_fast ? e / DC : e % DR, cc = c_fast ? e % DC : e / DR;
-    if (r >= dr || cc >= dc) return -1;
-    return c_fast ? r * dc + cc : cc * dr + r;
-  };
+  // A unit is eight consecutive rows r = 8*rg .. 8*rg+7 of one column cc: the eight values of
+  // one lane of one fragment, i.e. one 16-byte LDS write each for the hi and the lo part.
+  // Consecutive threads take consecutive memory: neighbouring columns when the column index
+  // runs fastest in memory (index r*dc + cc), neighbouring row groups otherwise (cc*dr + r).
+  const bool c_fast = ld_c == 1;
+  float vals[kUnits][8];
+  int first[kUnits];  // memory index of the unit's first element, -1 for padding
 #pragma unroll
-  for (int i = 0; i < kPer; ++i) vals[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < kUnits; ++i) {
+    const int u = tid + NT * i;
+    const int rg = c_fast ? u / DC : u % (DR / 8), cc = c_fast ? u % DC : u / (DR / 8);
+    first[i] = (PAD && (8 * rg >= dr || cc >= dc)) ? -1 : (c_fast ? 8 * rg * dc + cc : cc * dr + 8 * rg);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) vals[i][j] = 0.f;
+  }
+  const int rstep = c_fast ? dc : 1;  // memory distance of consecutive rows
   for (int c = 0; c < nsum; ++c) {
+    const float* src = mat + (int64_t)c * sum_stride;
 #pragma unroll
-    for (int i = 0; i < kPer; ++i) {
-      const int idx = mem_index(i);
-      if (!PAD || idx >= 0) vals[i] += *reinterpret_cast<const f32x4*>(mat + (int64_t)c * sum_stride + idx);
+    for (int i = 0; i < kUnits; ++i) {
+      if (PAD && first[i] < 0) continue;
+      if (c_fast) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) vals[i][j] += src[first[i] + j * rstep];
+      } else {
+        const f32x4 a = *reinterpret_cast<const f32x4*>(src + first[i]);
+        const f32x4 b = *reinterpret_cast<const f32x4*>(src + first[i] + 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          vals[i][j] += a[j];
+          vals[i][4 + j] += b[j];
+        }
+      }
     }
   }
+  float mx = 0.f;
 #pragma unroll
-  for (int i = 0; i < kPer; ++i) {
-    vals[i] *= mscale;
-    const int idx = mem_index(i);
-    if (mat_out && (!PAD || idx >= 0)) *reinterpret_cast<f32x4*>(mat_out + idx) = vals[i];
+  for (int i = 0; i < kUnits; ++i) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) mx = fmaxf(mx, fabsf(vals[i][j]));
+    for (int j = 0; j < 8; ++j) {
+      vals[i][j] *= mscale;
+      mx = fmaxf(mx, fabsf(vals[i][j]));
+    }
+    if (mat_out && !(PAD && first[i] < 0)) {
+      if (c_fast) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) mat_out[first[i] + j * rstep] = vals[i][j];
+      } else {
+        *reinterpret_cast<f32x4*>(mat_out + first[i]) = f32x4{vals[i][0], vals[i][1], vals[i][2], vals[i][3]};
+        *reinterpret_cast<f32x4*>(mat_out + first[i] + 4) = f32x4{vals[i][4], vals[i][5], vals[i][6], vals[i][7]};
+      }
+    }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
@@ -530,24 +563,25 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
     frexpf(mx, &e);
     norm = ldexpf(1.f, 4 - e);
   }
-  uint16_t* op16 = reinterpret_cast<uint16_t*>(lds_opnd);
 #pragma unroll
-  for (int i = 0; i < kPer; ++i)
+  for (int i = 0; i < kUnits; ++i) {
+    const int u = tid + NT * i;
+    const int rg = c_fast ? u / DC : u % (DR / 8), cc = c_fast ? u % DC : u / (DR / 8);
+    const int kbA = rg / (DR / 16), ks = rg % (DR / 16);
+    const int kbC = cc / (DC / 2), rem = cc % (DC / 2);
+    const int b = rem >> 4, m = 8 * ((rem & 15) >> 2) + 4 * kbC + (rem & 3);
+    const int f = b * KS + ks, l = m + 32 * kbA;
+    u32x4 whi, wlo;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int e = 4 * (tid + NT * i) + j;
-      const int r = c_fast ? e / DC : e % DR;
-      const int cc = c_fast ? e % DC : e / DR;
-      const int kbA = r / (DR / 2), s = (r % (DR / 2)) >> 3, i8 = r & 7;
-      const int kbC = cc / (DC / 2), rem = cc % (DC / 2);
-      const int b = rem >> 4, m = 8 * ((rem & 15) >> 2) + 4 * kbC + (rem & 3);
-      const int f = b * KS + s, l = m + 32 * kbA;
-      const float val = vals[i][j] * norm;
-      const T hi = (T)val;
-      const T lo = (T)(val - (float)hi);
-      op16[((2 * f + 0) * 64 + l) * 8 + i8] = __builtin_bit_cast(uint16_t, hi);
-      op16[((2 * f + 1) * 64 + l) * 8 + i8] = __builtin_bit_cast(uint16_t, lo);
+      const float v0 = vals[i][2 * j] * norm, v1 = vals[i][2 * j + 1] * norm;
+      const T h0 = (T)v0, h1 = (T)v1;
+      whi[j] = pack2<T>((float)h0, (float)h1);
+      wlo[j] = pack2<T>(v0 - (float)h0, v1 - (float)h1);
     }
+    *reinterpret_cast<u32x4*>(lds_opnd + ((2 * f + 0) * 64 + l) * 16) = whi;
+    *reinterpret_cast<u32x4*>(lds_opnd + ((2 * f + 1) * 64 + l) * 16) = wlo;
+  }
   return 1.f / norm;
 }
 
@@ -602,7 +636,8 @@ template <int DR, int DC, bool DEN, int WAVES> struct RowsLayout {
 // products of backward pass B): workgroups [0, wgs_per_job) run job0, the rest job1.
 // PAD = true: rows are dr (x) and dc (out) elements long in memory, multiples of 8 below the
 // template's DR, DC; the staged tiles keep the padded width, with zeros in the padding.
-template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD = false>
+template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD = false,
+          int PF = (DR == 128 && DC == 128) ? FBLA_ROWS_PF128 : FBLA_ROWS_PF>
 __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, RowsJob job1,
                                                           int wgs_per_job, int chunk, int nchunks,
                                                           int dr_true, int dc_true) {
@@ -677,12 +712,15 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
     }
   };
 
+  // PF register sets hold the tiles in flight: a tile is requested PF tiles ahead of its use
   int t0 = t_begin + 32 * wave;
-  u32x4 xr[XI], xd[XI];
-  if (t0 < t_end) {
-    load_tile(xr, x, t0);
-    if constexpr (DEN) load_tile(xd, xden, t0);
-  }
+  u32x4 xr[PF][XI], xd[DEN ? PF : 1][XI];
+#pragma unroll
+  for (int f = 0; f < PF; ++f)
+    if (t0 + 32 * WAVES * f < t_end) {
+      load_tile(xr[f], x, t0 + 32 * WAVES * f);
+      if constexpr (DEN) load_tile(xd[f], xden, t0 + 32 * WAVES * f);
+    }
 
   // ---- prologue: matrix operand fragments, km pairs, addvec ----
   // Either the finished matrix / vectors are given, or the per-chunk partials of
@@ -716,14 +754,16 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
   __syncthreads();
 
   // ---- main loop ----
-  while (t0 < t_end) {
+  // one tile: its rows move from the register set to the staging area, the set is refilled
+  // with the tile PF steps ahead, then the tile is multiplied and stored
+  auto tile_step = [&](u32x4(&xcur)[XI], u32x4(&dcur)[XI]) {
     wave_sync();  // previous tile's staging reads are done
-    stash_tile(xr, stage);
-    if constexpr (DEN) stash_tile(xd, stage_den);
-    const int tn = t0 + 32 * WAVES;
+    stash_tile(xcur, stage);
+    if constexpr (DEN) stash_tile(dcur, stage_den);
+    const int tn = t0 + 32 * WAVES * PF;
     if (tn < t_end) {
-      load_tile(xr, x, tn);
-      if constexpr (DEN) load_tile(xd, xden, tn);
+      load_tile(xcur, x, tn);
+      if constexpr (DEN) load_tile(dcur, xden, tn);
     }
     wave_sync();
 
@@ -784,7 +824,12 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
         *reinterpret_cast<u32x4*>(out + (row0 + (int64_t)tok * rstride) * dc + ch * 8) = w;
       }
     }
-    t0 = tn;
+    t0 += 32 * WAVES;
+  };
+  while (t0 < t_end) {
+#pragma unroll
+    for (int f = 0; f < PF; ++f)
+      if (t0 < t_end) tile_step(xr[f], xd[DEN ? f : 0]);
   }
 }
 
