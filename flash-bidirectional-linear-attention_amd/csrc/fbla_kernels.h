@@ -84,6 +84,9 @@ struct RowsJob {
 };
 bool supported(const Prob& p, int dtype);
 bool bwd_a_supported(const Prob& p, int dtype);
+// dense 32 x 32 heads: the row-parallel kernels take two tokens per row and need the finished
+// matrices (no partial sums in their prologue)
+bool pair_mode(const Prob& p, int dtype);
 int state_chunk(const Prob& p);
 int bwd_a_chunk(const Prob& p);
 int rows_chunk(const Prob& p, int DR, int DC);
@@ -114,7 +117,6 @@ int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* 
           hipStream_t st, float* fin_mat = nullptr, float* fin_vec = nullptr);
 }  // namespace mfma
 
-// Piecewise (PISA) attention, forward only (fbla_piecewise.hip).
 namespace mfma32 {
 // fp32 inputs on v_mfma_f32_32x32x2_f32: 64 x 64 heads, not decoupled.  Called through the
 // mfma:: entry points, which dispatch on the dtype.
@@ -127,6 +129,7 @@ int bwd_tokens(const Prob& p, const float* q, const float* dout, const float* S,
                float* tokscal, int64_t total_rows, hipStream_t st);
 }  // namespace mfma32
 
+// Piecewise (PISA) attention, forward only (fbla_piecewise.hip).
 namespace piecewise {
 size_t chunk_reduce_workspace_bytes(int64_t BH, int64_t T, int K, int V, int chunk, int dtype,
                                     bool per_chunk);

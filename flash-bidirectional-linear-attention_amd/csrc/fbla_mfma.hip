@@ -487,7 +487,9 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
 // also written there in memory order.
 // PAD = true: the matrix in memory is dr x dc (multiples of 8, at most DR x DC); the
 // operand's remaining rows and columns are zero.
-template <typename T, int DR, int DC, int NT = kThreads, bool PAD = false>
+// PAIR = true (DR = DC = 64): the matrix in memory is 32 x 32 and the operand is
+// blockdiag(M, M): a 64-wide row then holds two independent 32-wide rows.
+template <typename T, int DR, int DC, int NT = kThreads, bool PAD = false, bool PAIR = false>
 __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* lds_max,
                                                const float* __restrict__ mat, int ld_r, int ld_c,
                                                int nsum = 1, int64_t sum_stride = 0,
@@ -508,16 +510,22 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
   for (int i = 0; i < kUnits; ++i) {
     const int u = tid + NT * i;
     const int rg = c_fast ? u / DC : u % (DR / 8), cc = c_fast ? u % DC : u / (DR / 8);
-    first[i] = (PAD && (8 * rg >= dr || cc >= dc)) ? -1 : (c_fast ? 8 * rg * dc + cc : cc * dr + 8 * rg);
+    if constexpr (PAIR) {
+      const int r8 = 8 * (rg % 4), c32 = cc % 32;
+      first[i] = (rg / 4 != cc / 32) ? -1 : (c_fast ? r8 * 32 + c32 : c32 * 32 + r8);
+    } else {
+      first[i] = (PAD && (8 * rg >= dr || cc >= dc)) ? -1 : (c_fast ? 8 * rg * dc + cc : cc * dr + 8 * rg);
+    }
 #pragma unroll
     for (int j = 0; j < 8; ++j) vals[i][j] = 0.f;
   }
-  const int rstep = c_fast ? dc : 1;  // memory distance of consecutive rows
+  constexpr bool kHoles = PAD || PAIR;  // some units are not backed by memory
+  const int rstep = c_fast ? (PAIR ? 32 : dc) : 1;  // memory distance of consecutive rows
   for (int c = 0; c < nsum; ++c) {
     const float* src = mat + (int64_t)c * sum_stride;
 #pragma unroll
     for (int i = 0; i < kUnits; ++i) {
-      if (PAD && first[i] < 0) continue;
+      if (kHoles && first[i] < 0) continue;
       if (c_fast) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) vals[i][j] += src[first[i] + j * rstep];
@@ -540,7 +548,7 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
       vals[i][j] *= mscale;
       mx = fmaxf(mx, fabsf(vals[i][j]));
     }
-    if (mat_out && !(PAD && first[i] < 0)) {
+    if (mat_out && !(kHoles && first[i] < 0)) {
       if (c_fast) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) mat_out[first[i] + j * rstep] = vals[i][j];
@@ -589,18 +597,21 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
 // `src` may be the vector part of the first of `nsum` partials (see build_operand);
 // the sum times `vscale` is the vector.  It is stored as pairs (when `pairs`), as
 // fp32 in LDS (when `f32`) and to memory (when `vec_out`).
-// The LDS copies hold DP >= D entries (DP = 0 stands for D), zero past the first D.
+// The LDS copies hold DP >= D entries (DP = 0 stands for D), zero past the first D, or
+// (repeat) the D entries over and over.
 template <typename T, int NT = kThreads>
 __device__ __forceinline__ void build_vec(uint32_t* pairs, float* f32, const float* __restrict__ src,
                                           int D, int nsum = 1, int64_t sum_stride = 0,
-                                          float vscale = 1.f, float* vec_out = nullptr, int DP = 0) {
+                                          float vscale = 1.f, float* vec_out = nullptr, int DP = 0,
+                                          bool repeat = false) {
   if (DP == 0) DP = D;
   for (int e = threadIdx.x; e < DP / 2; e += NT) {
     float a = 0.f, b = 0.f;
-    const bool real = 2 * e < D;
+    const bool real = repeat || 2 * e < D;
+    const int se = repeat ? (2 * e) % D : 2 * e;
     for (int c = 0; real && c < nsum; ++c) {
-      a += src[(int64_t)c * sum_stride + 2 * e];
-      b += src[(int64_t)c * sum_stride + 2 * e + 1];
+      a += src[(int64_t)c * sum_stride + se];
+      b += src[(int64_t)c * sum_stride + se + 1];
     }
     a *= vscale;
     b *= vscale;
@@ -613,7 +624,7 @@ __device__ __forceinline__ void build_vec(uint32_t* pairs, float* f32, const flo
       f32[2 * e] = a;
       f32[2 * e + 1] = b;
     }
-    if (vec_out && real) {
+    if (vec_out && real && 2 * e < D) {
       vec_out[2 * e] = a;
       vec_out[2 * e + 1] = b;
     }
@@ -636,12 +647,18 @@ template <int DR, int DC, bool DEN, int WAVES> struct RowsLayout {
 // products of backward pass B): workgroups [0, wgs_per_job) run job0, the rest job1.
 // PAD = true: rows are dr (x) and dc (out) elements long in memory, multiples of 8 below the
 // template's DR, DC; the staged tiles keep the padded width, with zeros in the padding.
+// PAIR = true (dense tensors, 32 x 32 heads, DR = DC = 64): a 64-wide row of the kernel is two
+// consecutive tokens of the head, the operand is blockdiag(M, M), and because a lane's z and
+// its output features both belong to one half of the row, the halves never mix: the kernel
+// streams full 128-byte rows at the cost of multiplying zeros.  `chunk` counts row pairs; an
+// odd length leaves the second half of the last pair out.  No partial sums in the prologue.
 template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD = false,
-          int PF = (DR == 128 && DC == 128) ? FBLA_ROWS_PF128 : FBLA_ROWS_PF>
+          int PF = (DR == 128 && DC == 128) ? FBLA_ROWS_PF128 : FBLA_ROWS_PF, bool PAIR = false>
 __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, RowsJob job1,
                                                           int wgs_per_job, int chunk, int nchunks,
                                                           int dr_true, int dc_true) {
-  const int dr = PAD ? dr_true : DR, dc = PAD ? dc_true : DC;
+  static_assert(!PAIR || (DR == 64 && DC == 64 && !PAD), "pair mode: two 32-wide rows per 64-wide row");
+  const int dr = PAD ? dr_true : (PAIR ? 32 : DR), dc = PAD ? dc_true : (PAIR ? 32 : DC);
   const int dpk = PAD ? (p.DK <= 64 ? 64 : 128) : p.DK;  // padded length of the km / dkm vector
   using LY = RowsLayout<DR, DC, DEN, WAVES>;
   const bool second = (int)blockIdx.x >= wgs_per_job;
@@ -666,8 +683,9 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
   int64_t bos, row0, rstride;
   int len;
   seq_range(p, n, bos, len);
+  const int nrows = PAIR ? (len + 1) >> 1 : len;  // rows of this kernel
   const int t_begin = c * chunk;
-  if (t_begin >= len) {
+  if (t_begin >= nrows) {
     if (c == 0 && job.pnchunks > 0) {  // empty sequence: its state is zero
       if (job.mat_out)
         for (int e = threadIdx.x; e < dr * dc; e += NT) job.mat_out[(int64_t)nh * dr * dc + e] = 0.f;
@@ -676,8 +694,19 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
     }
     return;
   }
-  const int t_end = min(len, t_begin + chunk);
+  const int t_end = min(nrows, t_begin + chunk);
   row_base(p, n, h, bos, row0, rstride);
+  // element offset of 16-byte piece `ch` of row `tok` (rows of `rowlen` elements), or -1 when
+  // the piece does not exist
+  auto piece = [&](int tok, int ch, int rowlen) -> int64_t {
+    if constexpr (PAIR) {
+      if (tok >= t_end || 2 * tok + (ch >> 2) >= len) return -1;
+      return (row0 + 2 * (int64_t)tok) * 32 + ch * 8;
+    } else {
+      if (tok >= t_end || (PAD && ch * 8 >= rowlen)) return -1;
+      return (row0 + (int64_t)tok * rstride) * rowlen + ch * 8;
+    }
+  };
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const T* x = (const T*)job.x;
@@ -696,9 +725,9 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
 #pragma unroll
     for (int i = 0; i < XI; ++i) {
       const int q = lane + 64 * i, row = q / XCH, ch = q % XCH;
-      const int tok = tok0 + row;
-      if (tok < t_end && (!PAD || ch * 8 < dr)) {
-        dst[i] = *reinterpret_cast<const u32x4*>(src + (row0 + (int64_t)tok * rstride) * dr + ch * 8);
+      const int64_t off = piece(tok0 + row, ch, dr);
+      if (off >= 0) {
+        dst[i] = *reinterpret_cast<const u32x4*>(src + off);
       } else {
         dst[i] = u32x4{0u, 0u, 0u, 0u};
       }
@@ -745,11 +774,12 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
     if (!job.vec_is_add)
       for (int e = tid; e < DC; e += NT) lds_add[e] = 0.f;
   } else {
-    denorm = build_operand<T, DR, DC, NT, PAD>(lds_opnd, lds_max, job.mat + (int64_t)nh * dr * dc, job.ld_r,
-                                               job.ld_c, 1, 0, 1.f, nullptr, dr, dc);
-    if constexpr (NORM) build_vec<T, NT>(lds_km, nullptr, job.km + (int64_t)nh * dr, dr, 1, 0, 1.f, nullptr, DR);
+    denorm = build_operand<T, DR, DC, NT, PAD, PAIR>(lds_opnd, lds_max, job.mat + (int64_t)nh * dr * dc,
+                                                     job.ld_r, job.ld_c, 1, 0, 1.f, nullptr, dr, dc);
+    if constexpr (NORM)
+      build_vec<T, NT>(lds_km, nullptr, job.km + (int64_t)nh * dr, dr, 1, 0, 1.f, nullptr, DR, PAIR);
     for (int e = tid; e < DC; e += NT)
-      lds_add[e] = (job.addvec && e < dc) ? job.addvec[(int64_t)nh * dc + e] : 0.f;
+      lds_add[e] = (job.addvec && (PAIR || e < dc)) ? job.addvec[(int64_t)nh * dc + (PAIR ? e % 32 : e)] : 0.f;
   }
   __syncthreads();
 
@@ -797,7 +827,7 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
     }
     float rs = denorm;
     if constexpr (NORM) {
-      z += __shfl_xor(z, 32);
+      if constexpr (!PAIR) z += __shfl_xor(z, 32);  // pair mode: each half row has its own z
       rs = denorm / (z + p.eps);
     }
     wave_sync();  // all lanes have read their x chunks; staging is reused for out
@@ -818,10 +848,10 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
 #pragma unroll
     for (int i = 0; i < OI; ++i) {
       const int q = lane + 64 * i, row = q / OCH, ch = q % OCH;
-      const int tok = t0 + row;
-      if (tok < t_end && (!PAD || ch * 8 < dc)) {
+      const int64_t off = piece(t0 + row, ch, dc);
+      if (off >= 0) {
         const u32x4 w = *reinterpret_cast<const u32x4*>(stage + swz<OROWB>(row, ch));
-        *reinterpret_cast<u32x4*>(out + (row0 + (int64_t)tok * rstride) * dc + ch * 8) = w;
+        *reinterpret_cast<u32x4*>(out + off) = w;
       }
     }
     t0 += 32 * WAVES;
@@ -864,7 +894,7 @@ template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struc
   static constexpr int KS = DV / 16, NB = DK / 32;
   static constexpr int kOpnd = NB * KS * 2 * 1024;
   static constexpr int kQ = 32 * DK * 2, kG = 32 * DV * 2;
-  static constexpr int kWave = kQ + kG + (NORM && FUSED && LO ? kG : 0) + (DEN ? kQ : 0) + 128;  // + dz[32]
+  static constexpr int kWave = kQ + kG + (NORM && FUSED && LO ? kG : 0) + (DEN ? kQ : 0) + 256;  // + dz[64]
   static constexpr int kKmPairs = kOpnd + kWaves * kWave;
   static constexpr int kKmF = kKmPairs + DK * 4;
   static constexpr int kMax = kKmF + DK * 4;
@@ -877,7 +907,12 @@ template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struc
 // ([2][total rows]) for scaled_state_kernel, and no partials.
 // PAD = true: head dims p.DK, p.DV (multiples of 8) below the template's DK, DV, as in the
 // other kernels: true row lengths in memory, zero padding in the staged tiles and operands.
-template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true, bool PAD = false>
+// PAIR = true (dense tensors, 32 x 32 heads, DK = DV = 64, FUSED): two consecutive tokens per
+// 64-wide row as in the rows kernel; the token view never mixes the halves of a row, the
+// feature view accumulates blockdiag-shaped sums whose two diagonal 32 x 32 blocks are added
+// before the store.  `chunk` counts row pairs.
+template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true, bool PAD = false,
+          bool PAIR = false>
 __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const T* __restrict__ dout,
     const float* __restrict__ S, const float* __restrict__ km, T* __restrict__ dqn,
@@ -886,7 +921,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
   using LY = BwdALayout<DK, DV, NORM, DEN, FUSED, LO>;
   constexpr int KS = LY::KS, NB = LY::NB;
   constexpr int CK = DK / 32, CV = DV / 32;
-  const int dk = PAD ? p.DK : DK, dv = PAD ? p.DV : DV;
+  static_assert(!PAIR || (DK == 64 && DV == 64 && FUSED && !PAD), "pair mode: two 32-wide rows per 64-wide row");
+  const int dk = PAD ? p.DK : (PAIR ? 32 : DK), dv = PAD ? p.DV : (PAIR ? 32 : DV);
   constexpr int QROWB = DK * 2, GROWB = DV * 2;
   constexpr int QCH = QROWB / 16, GCH = GROWB / 16;
   constexpr int QI = 32 * QCH / 64, GI = 32 * GCH / 64;
@@ -899,8 +935,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
   int64_t bos, row0, rstride;
   int len;
   seq_range(p, n, bos, len);
+  const int nrows = PAIR ? (len + 1) >> 1 : len;  // rows of this kernel
   const int t_begin = c * chunk;
-  if (t_begin >= len) {
+  if (t_begin >= nrows) {
     if (fin_mat && c == 0) {  // empty sequence: no gradient flows through its state
       for (int e = threadIdx.x; e < dk * dv; e += kThreads) fin_mat[(int64_t)nh * dk * dv + e] = 0.f;
       if (fin_vec)
@@ -908,8 +945,19 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     }
     return;
   }
-  const int t_end = min(len, t_begin + chunk);
+  const int t_end = min(nrows, t_begin + chunk);
   row_base(p, n, h, bos, row0, rstride);
+  // element offset of 16-byte piece `ch` of row `tok` (rows of `rowlen` elements), or -1 when
+  // the piece does not exist
+  auto piece = [&](int tok, int ch, int rowlen) -> int64_t {
+    if constexpr (PAIR) {
+      if (tok >= t_end || 2 * tok + (ch >> 2) >= len) return -1;
+      return (row0 + 2 * (int64_t)tok) * 32 + ch * 8;
+    } else {
+      if (tok >= t_end || (PAD && ch * 8 >= rowlen)) return -1;
+      return (row0 + (int64_t)tok * rstride) * rowlen + ch * 8;
+    }
+  };
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int ntok = lane & 31, kb = lane >> 5;
@@ -939,20 +987,16 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
 #pragma unroll
     for (int i = 0; i < QI; ++i) {
       const int q = lane + 64 * i, row = q / QCH, ch = q % QCH;
-      const int tok = tok0 + row;
-      dst[i] = (tok < t_end && (!PAD || ch * 8 < dk))
-                   ? *reinterpret_cast<const u32x4*>(src + (row0 + (int64_t)tok * rstride) * dk + ch * 8)
-                   : u32x4{0u, 0u, 0u, 0u};
+      const int64_t off = piece(tok0 + row, ch, dk);
+      dst[i] = off >= 0 ? *reinterpret_cast<const u32x4*>(src + off) : u32x4{0u, 0u, 0u, 0u};
     }
   };
   auto load_g = [&](u32x4(&dst)[GI], const T* src, int tok0) {
 #pragma unroll
     for (int i = 0; i < GI; ++i) {
       const int q = lane + 64 * i, row = q / GCH, ch = q % GCH;
-      const int tok = tok0 + row;
-      dst[i] = (tok < t_end && (!PAD || ch * 8 < dv))
-                   ? *reinterpret_cast<const u32x4*>(src + (row0 + (int64_t)tok * rstride) * dv + ch * 8)
-                   : u32x4{0u, 0u, 0u, 0u};
+      const int64_t off = piece(tok0 + row, ch, dv);
+      dst[i] = off >= 0 ? *reinterpret_cast<const u32x4*>(src + off) : u32x4{0u, 0u, 0u, 0u};
     }
   };
   auto stash_q = [&](const u32x4(&src)[QI], unsigned char* dstb) {
@@ -973,10 +1017,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
 #pragma unroll
     for (int i = 0; i < QI; ++i) {
       const int q = lane + 64 * i, row = q / QCH, ch = q % QCH;
-      const int tok = tok0 + row;
-      if (tok < t_end && (!PAD || ch * 8 < dk))
-        *reinterpret_cast<u32x4*>(dst + (row0 + (int64_t)tok * rstride) * dk + ch * 8) =
-            *reinterpret_cast<const u32x4*>(srcb + swz<QROWB>(row, ch));
+      const int64_t off = piece(tok0 + row, ch, dk);
+      if (off >= 0)
+        *reinterpret_cast<u32x4*>(dst + off) = *reinterpret_cast<const u32x4*>(srcb + swz<QROWB>(row, ch));
     }
   };
 
@@ -989,10 +1032,10 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
   }
 
   // g_t = dO_t S^T: contraction over dv, M(r = dv, c = dk) = S[c][r]
-  const float denorm = build_operand<T, DV, DK, kThreads, PAD>(lds_opnd, lds_max, S + (int64_t)nh * dk * dv, 1,
-                                                               dv, 1, 0, 1.f, nullptr, dv, dk);
+  const float denorm = build_operand<T, DV, DK, kThreads, PAD, PAIR>(
+      lds_opnd, lds_max, S + (int64_t)nh * dk * dv, 1, dv, 1, 0, 1.f, nullptr, dv, dk);
   if constexpr (NORM) {
-    build_vec<T>(km_pairs, kmf, km + (int64_t)nh * dk, dk, 1, 0, 1.f, nullptr, DK);
+    build_vec<T>(km_pairs, kmf, km + (int64_t)nh * dk, dk, 1, 0, 1.f, nullptr, DK, PAIR);
   }
   __syncthreads();
 
@@ -1046,16 +1089,18 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
           z = Ops<T>::dot2(qz[i], kl[i], z);
         }
       }
-      P += __shfl_xor(P, 32);
-      z += __shfl_xor(z, 32);
-      if (t0 + ntok < t_end) {
+      if constexpr (!PAIR) {  // pair mode: each half row is a token of its own
+        P += __shfl_xor(P, 32);
+        z += __shfl_xor(z, 32);
+      }
+      if (PAIR ? (t0 + ntok < t_end && 2 * (t0 + ntok) + kb < len) : (t0 + ntok < t_end)) {
         rz = 1.f / (z + p.eps);
         dz = -(P * denorm) * rz * rz;
       } else {
         rz = 0.f;  // padding rows contribute nothing
       }
       if constexpr (FUSED) {
-        if (kb == 0) dzs[ntok] = dz;
+        if (PAIR || kb == 0) dzs[32 * (PAIR ? kb : 0) + ntok] = dz;
       } else {
         if (kb == 0 && t0 + ntok < t_end) {
           const int64_t row = row0 + (int64_t)(t0 + ntok) * rstride;
@@ -1134,7 +1179,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
         if constexpr (DEN) lds_rows<CK>(qw, qdt, tok0, ntok);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const float dzj = dzs[tok0 + j];
+          const float dzj = dzs[(PAIR ? 32 * (ntok >> 4) : 0) + tok0 + j];  // lanes 16.. hold the second halves
 #pragma unroll
           for (int c2 = 0; c2 < CK / 2; ++c2) {
             dkm[2 * c2] = fmaf(dzj, Ops<T>::lo(qw.w[j][c2]), dkm[2 * c2]);
@@ -1167,7 +1212,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : dst + dk * dv;
     const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
     const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
-    reduce_store_block<4>(acc, dkm, red, dst, dv, dst_vec, mscale, vscale, wave, lane, dk, dv);
+    reduce_store_block<4, true, PAIR>(acc, dkm, red, dst, dv, dst_vec, mscale, vscale, wave, lane, dk, dv);
   }
 }
 
@@ -1178,6 +1223,12 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
 // it, the padded variants (PAD) when it is not one of the two.
 static int tiled_dim(int d) { return d <= 64 ? 64 : 128; }
 static bool padded(const Prob& p) { return p.DK != tiled_dim(p.DK) || p.DV != tiled_dim(p.DV); }
+
+// Dense tensors with 32 x 32 heads: the row-parallel kernels take two tokens per 64-wide row
+// (PAIR variants) instead of padding every row to 64.
+bool pair_mode(const Prob& p, int dtype) {
+  return (dtype == kF16 || dtype == kBF16) && !p.cu && p.DK == 32 && p.DV == 32;
+}
 
 // 16-bit inputs with head dims that are multiples of 8 (16-byte row pieces) up to 128; the
 // decoupled operator up to 64 x 64.
@@ -1304,11 +1355,12 @@ template <typename K> static int reserve_lds(K kernel, int bytes, bool& done) {
   return kOk;
 }
 
-template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD>
+template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD, bool PAIR = false>
 static int launch_rows_k(const Prob& p, const RowsJob& job, const RowsJob* job2, int chunk,
                          int nchunks, int dr, int dc, hipStream_t st) {
   using LY = RowsLayout<DR, DC, DEN, WAVES>;
-  auto kernel = rows_kernel<T, DR, DC, NORM, DEN, WAVES, PAD>;
+  constexpr int PF = (DR == 128 && DC == 128) ? FBLA_ROWS_PF128 : FBLA_ROWS_PF;
+  auto kernel = rows_kernel<T, DR, DC, NORM, DEN, WAVES, PAD, PF, PAIR>;
   static thread_local bool configured = false;
   int rc = reserve_lds(kernel, LY::kTotal, configured);
   if (rc != kOk) return rc;
@@ -1336,6 +1388,20 @@ static int launch_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, i
   return kErrUnsupported;
 }
 
+// two tokens per row: chunks are counted in row pairs
+template <typename T>
+static int launch_rows_pair(const Prob& p, const RowsJob& job, const RowsJob* job2, hipStream_t st) {
+  Prob pw = p;
+  pw.L = (p.L + 1) / 2;
+  const int chunk = rows_chunk(pw, 64, 64);
+  const int nchunks = (int)cdiv64(pw.L, chunk);
+  const bool norm = job.xden != nullptr;
+  const bool den = norm && job.xden != job.x;
+  if (!norm) return launch_rows_k<T, 64, 64, false, false, 4, false, true>(p, job, job2, chunk, nchunks, 32, 32, st);
+  if (!den) return launch_rows_k<T, 64, 64, true, false, 4, false, true>(p, job, job2, chunk, nchunks, 32, 32, st);
+  return launch_rows_k<T, 64, 64, true, true, 4, false, true>(p, job, job2, chunk, nchunks, 32, 32, st);
+}
+
 template <typename T, bool PAD>
 static int run_rows_dims(const Prob& p, const RowsJob& job, const RowsJob* job2, int dr, int dc,
                          hipStream_t st) {
@@ -1349,6 +1415,7 @@ static int run_rows_dims(const Prob& p, const RowsJob& job, const RowsJob* job2,
 template <typename T>
 static int run_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, int dr, int dc,
                     hipStream_t st) {
+  if (pair_mode(p, kF16) && job.pnchunks == 0) return launch_rows_pair<T>(p, job, job2, st);
   if (padded(p)) return run_rows_dims<T, true>(p, job, job2, dr, dc, st);
   return run_rows_dims<T, false>(p, job, job2, dr, dc, st);
 }
@@ -1397,7 +1464,7 @@ int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, in
   return run_rows<__bf16>(p, job0, &job1, DR, DC, st);
 }
 
-template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool PAD>
+template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool PAD, bool PAIR = false>
 static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, const float* S,
                         const float* km, T* dqn, T* dqd, float* partial, float* tokscal,
                         int64_t total_rows, float* fm, float* fv, int chunk, int nchunks,
@@ -1413,7 +1480,7 @@ static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, 
                               (int)sizeof(float) * 64 * ((DK / 32) * (DV / 32) * 16 + DK / 32),
                 "reduction buffer must fit in the tile area");
   static_assert(LY::kTotal <= 160 * 1024, "LDS budget of one workgroup");
-  auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN, FUSED, LO, PAD>;
+  auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN, FUSED, LO, PAD, PAIR>;
   static thread_local bool configured = false;  // per instantiation
   int rc = reserve_lds(kernel, LY::kTotal, configured);
   if (rc != kOk) return rc;
@@ -1423,23 +1490,26 @@ static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, 
   return kOk;
 }
 
-template <typename T, bool PAD>
+template <typename T, bool PAD, bool PAIR = false>
 static int run_bwd_a_pad(const Prob& p, const void* qn, const void* qd, const void* dout, const float* S,
                          const float* km, void* dqn, void* dqd, float* partial, float* fm, float* fv,
                          int chunk, int nchunks, hipStream_t st) {
   const T *a = (const T*)qn, *b = (const T*)qd, *c = (const T*)dout;
   T *x = (T*)dqn, *y = (T*)dqd;
   if (!(p.flags & kNormalize))
-    return launch_bwd_a<T, 64, 64, false, false, true, PAD>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+    return launch_bwd_a<T, 64, 64, false, false, true, PAD, PAIR>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
   if (p.flags & kDecoupled)
-    return launch_bwd_a<T, 64, 64, true, true, true, PAD>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
-  return launch_bwd_a<T, 64, 64, true, false, true, PAD>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+    return launch_bwd_a<T, 64, 64, true, true, true, PAD, PAIR>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+  return launch_bwd_a<T, 64, 64, true, false, true, PAD, PAIR>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
 }
 
 template <typename T>
 static int run_bwd_a(const Prob& p, const void* qn, const void* qd, const void* dout, const float* S,
                      const float* km, void* dqn, void* dqd, float* partial, float* fm, float* fv,
                      int chunk, int nchunks, hipStream_t st) {
+  // pair mode: the chunk (a multiple of 128 tokens) becomes a count of row pairs
+  if (pair_mode(p, kF16))
+    return run_bwd_a_pad<T, false, true>(p, qn, qd, dout, S, km, dqn, dqd, partial, fm, fv, chunk / 2, nchunks, st);
   if (padded(p)) return run_bwd_a_pad<T, true>(p, qn, qd, dout, S, km, dqn, dqd, partial, fm, fv, chunk, nchunks, st);
   return run_bwd_a_pad<T, false>(p, qn, qd, dout, S, km, dqn, dqd, partial, fm, fv, chunk, nchunks, st);
 }

@@ -51,8 +51,10 @@ __device__ __forceinline__ int lpt_sequence(const Prob& p, int rank, int* lens /
 // 32*a + m, column 32*b + pp (lanes own single features, the fp32 kernels).  Only the first
 // `rows_ok` rows and `cols_ok` columns of the block are stored (a head dim that is not a
 // multiple of 64 leaves the rest of its last block as padding).  Must be reached by all waves
-// of the workgroup.
-template <int G, bool PAIRED = true>
+// of the workgroup.  FOLD = true (PAIRED only): the block holds two 32 x 32 sums on its diagonal
+// (rows and columns 0..31 and 32..63) whose sum is stored as a 32 x 32 matrix (rows_ok =
+// cols_ok = 32), and likewise the two halves of the vector.
+template <int G, bool PAIRED = true, bool FOLD = false>
 __device__ __forceinline__ void reduce_store_block(f32x16 (&acc)[2][2], float (&ks)[2], float* red,
                                                    float* dst, int ld, float* dst_vec, float mscale,
                                                    float vscale, int g, int lane, int rows_ok = 64,
@@ -96,6 +98,17 @@ __device__ __forceinline__ void reduce_store_block(f32x16 (&acc)[2][2], float (&
     if (g == 0) absorb();
   }
   if (g != 0) return;
+  if constexpr (FOLD) {
+    // row + 32 is register r + 8, column + 32 is lane + 16
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int r = 0; r < 8; ++r) acc[a][b][r] += __shfl_down(acc[a][b][r + 8], 16);
+      ks[a] += __shfl_down(ks[a], 16);
+    }
+  }
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll

@@ -78,7 +78,7 @@ int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
     else
       generic::state_partial(p, dtype, kn, a.v, a.k, partial, chunk, nchunks, st);
   }
-  const bool fold = fast && !direct && dtype != kF32 && fold_reduce(p, nchunks, p.DK, p.DV);
+  const bool fold = fast && !direct && dtype != kF32 && !mfma::pair_mode(p, dtype) && fold_reduce(p, nchunks, p.DK, p.DV);
   if (!fold && !direct && (phases & kPhaseFwdReduce))
     generic::state_reduce(p, partial, chunk, nchunks, a.s, nullptr, a.km, st);
   if (phases & kPhaseFwdOutput) {
@@ -147,7 +147,7 @@ int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
       generic::bwd_a(p, dtype, qn, a.q, a.dout, a.s, St, a.km, dqn, dqd, partial, chunk, nchunks, st);
     }
   }
-  const bool fold = fast && !direct && dtype != kF32 && fold_reduce(p, nchunks, p.DV, p.DK);
+  const bool fold = fast && !direct && dtype != kF32 && !mfma::pair_mode(p, dtype) && fold_reduce(p, nchunks, p.DV, p.DK);
   if (!fold && !direct && (phases & kPhaseBwdReduce))
     generic::state_reduce(p, partial, chunk, nchunks, dS, fast ? nullptr : dSt, dkm, st);
   if (phases & kPhaseBwdB) {
