@@ -892,9 +892,11 @@ __device__ __forceinline__ void lds_rows(RowWords<C>& dst, const unsigned char* 
 
 template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struct BwdALayout {
   static constexpr int KS = DV / 16, NB = DK / 32;
+  static constexpr bool kBig = FUSED && DK == 128 && DV == 128;  // no staged lo part (LDS budget)
   static constexpr int kOpnd = NB * KS * 2 * 1024;
   static constexpr int kQ = 32 * DK * 2, kG = 32 * DV * 2;
-  static constexpr int kWave = kQ + kG + (NORM && FUSED && LO ? kG : 0) + (DEN ? kQ : 0) + 256;  // + dz[64]
+  static constexpr int kWave =
+      kQ + kG + (NORM && FUSED && LO && !kBig ? kG : 0) + (DEN ? kQ : 0) + 256;  // + dz[64] (or dz[32], 1/z[32])
   static constexpr int kKmPairs = kOpnd + kWaves * kWave;
   static constexpr int kKmF = kKmPairs + DK * 4;
   static constexpr int kMax = kKmF + DK * 4;
@@ -911,9 +913,15 @@ template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struc
 // 64-wide row as in the rows kernel; the token view never mixes the halves of a row, the
 // feature view accumulates blockdiag-shaped sums whose two diagonal 32 x 32 blocks are added
 // before the store.  `chunk` counts row pairs.
+// FUSED at 128 x 128 (one workgroup per CU, 134 KiB of LDS): dS does not fit one wave, so each
+// of the four waves owns one 64 x 64 block of it and walks the tiles of all four waves.  Per
+// step of 128 tokens: every wave runs the token view of its own 32-token tile and leaves 1/z_t
+// and dz_t in LDS; barrier; every wave multiplies its block over the four tiles, scaling and
+// splitting dO rows into hi + lo on the fly (there is no room to stage a lo copy); barrier;
+// every wave stages and stores the dq of its tile.
 template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true, bool PAD = false,
           bool PAIR = false>
-__global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
+__global__ __launch_bounds__(kThreads, (FUSED && DK == 128 && DV == 128) ? 1 : 2) void bwd_a_kernel(
     Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const T* __restrict__ dout,
     const float* __restrict__ S, const float* __restrict__ km, T* __restrict__ dqn,
     T* __restrict__ dqd, float* __restrict__ partial, float* __restrict__ tokscal,
@@ -921,6 +929,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
   using LY = BwdALayout<DK, DV, NORM, DEN, FUSED, LO>;
   constexpr int KS = LY::KS, NB = LY::NB;
   constexpr int CK = DK / 32, CV = DV / 32;
+  constexpr bool BIG = LY::kBig;
+  static_assert(!FUSED || BIG || (DK == 64 && DV == 64), "fused pass A: 64 x 64 or 128 x 128 tiles");
+  static_assert(!BIG || !DEN, "no decoupled variant at 128 x 128");
   static_assert(!PAIR || (DK == 64 && DV == 64 && FUSED && !PAD), "pair mode: two 32-wide rows per 64-wide row");
   const int dk = PAD ? p.DK : (PAIR ? 32 : DK), dv = PAD ? p.DV : (PAIR ? 32 : DV);
   constexpr int QROWB = DK * 2, GROWB = DV * 2;
@@ -966,22 +977,21 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
   unsigned char* qt = smem + LY::kOpnd + wave * LY::kWave;
   unsigned char* gt = qt + LY::kQ;             // dO, later dO/z (hi part)
   unsigned char* gl = gt + LY::kG;             // dO/z (lo part), NORM && FUSED only
-  unsigned char* qdt = gl + (NORM && FUSED && LO ? LY::kG : 0);  // plain q, DEN only
+  unsigned char* qdt = gl + (NORM && FUSED && LO && !LY::kBig ? LY::kG : 0);  // plain q, DEN only
   float* dzs = reinterpret_cast<float*>(qdt + (DEN ? LY::kQ : 0));
   uint32_t* km_pairs = reinterpret_cast<uint32_t*>(smem + LY::kKmPairs);
   float* kmf = reinterpret_cast<float*>(smem + LY::kKmF);
   float* lds_max = reinterpret_cast<float*>(smem + LY::kMax);
 
-  f32x16 acc[FUSED ? CK : 1][FUSED ? CV : 1];
+  constexpr int AK = FUSED ? 2 : 1, AV = FUSED ? 2 : 1;  // one 64 x 64 block of dS per wave
+  f32x16 acc[AK][AV];
 #pragma unroll
-  for (int a = 0; a < (FUSED ? CK : 1); ++a)
+  for (int a = 0; a < AK; ++a)
 #pragma unroll
-    for (int b = 0; b < (FUSED ? CV : 1); ++b)
+    for (int b = 0; b < AV; ++b)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-  float dkm[CK];
-#pragma unroll
-  for (int a = 0; a < CK; ++a) dkm[a] = 0.f;
+  float dkm[2] = {0.f, 0.f};
 
   auto load_q = [&](u32x4(&dst)[QI], const T* src, int tok0) {
 #pragma unroll
@@ -1025,7 +1035,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
 
   int t0 = t_begin + 32 * wave;
   u32x4 rq[QI], rg[GI], rd[QI];
-  if (t0 < t_end) {
+  if (LY::kBig || t0 < t_end) {
     load_q(rq, qn, t0);
     load_g(rg, dout, t0);
     if constexpr (DEN) load_q(rd, qd, t0);
@@ -1039,13 +1049,15 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
   }
   __syncthreads();
 
-  while (t0 < t_end) {
+  // BIG: all waves make the same number of steps (a wave whose tile lies past the end works
+  // on zeros), because the steps contain workgroup barriers
+  while (BIG ? t0 - 32 * wave < t_end : t0 < t_end) {
     wave_sync();  // the previous sub-tile's staged dq has been read out
     stash_q(rq, qt);
     stash_g(rg, gt);
     if constexpr (DEN) stash_q(rd, qdt);
     const int tn = t0 + 32 * kWaves;
-    if (tn < t_end) {
+    if (BIG || tn < t_end) {
       load_q(rq, qn, tn);
       load_g(rg, dout, tn);
       if constexpr (DEN) load_q(rd, qd, tn);
@@ -1101,6 +1113,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
       }
       if constexpr (FUSED) {
         if (PAIR || kb == 0) dzs[32 * (PAIR ? kb : 0) + ntok] = dz;
+        if (BIG && kb == 0) dzs[32 + ntok] = rz;
       } else {
         if (kb == 0 && t0 + ntok < t_end) {
           const int64_t row = row0 + (int64_t)(t0 + ntok) * rstride;
@@ -1130,7 +1143,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
       }
     }
     // dO / z as hi + lo, in place over this lane's own chunks of the dO tile
-    if constexpr (NORM && FUSED) {
+    if constexpr (NORM && FUSED && !BIG) {
 #pragma unroll
       for (int ch = 0; ch < GCH / 2; ++ch) {
         const int off = swz<GROWB>(ntok, (GCH / 2) * kb + ch);
@@ -1147,10 +1160,72 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
         if constexpr (LO) *reinterpret_cast<u32x4*>(gl + off) = wl;
       }
     }
-    wave_sync();
+    if constexpr (BIG) __syncthreads();  // all four tiles and their scalars are staged
+    else wave_sync();
 
     // ---- feature view: two k-steps of 16 tokens ----
-    if constexpr (FUSED) {
+    if constexpr (BIG) {
+      const int bk = wave >> 1, bv = wave & 1;
+#pragma unroll
+      for (int u = 0; u < kWaves; ++u) {
+        const unsigned char* qtu = smem + LY::kOpnd + u * LY::kWave;
+        const unsigned char* gtu = qtu + LY::kQ;
+        const float* scal = reinterpret_cast<const float*>(gtu + LY::kG);  // dz[32], 1/z[32]
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          const int tok0 = 16 * ks + 8 * kb;
+          RowWords<2> qw, gw;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            qw.w[j][0] = *reinterpret_cast<const uint32_t*>(qtu + swz<QROWB>(tok0 + j, 8 * bk + (ntok >> 2)) +
+                                                            ((ntok & 3) << 2));
+            gw.w[j][0] = *reinterpret_cast<const uint32_t*>(gtu + swz<GROWB>(tok0 + j, 8 * bv + (ntok >> 2)) +
+                                                            ((ntok & 3) << 2));
+          }
+          u32x4 A[2], Bh[2];
+          transpose_rows<2>(qw, A);
+          if constexpr (NORM) {
+            RowWords<2> vh, vl;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float rzj = scal[32 + tok0 + j];
+              const float x0 = Ops<T>::lo(gw.w[j][0]) * rzj, x1 = Ops<T>::hi(gw.w[j][0]) * rzj;
+              const T h0 = (T)x0, h1 = (T)x1;
+              vh.w[j][0] = pack2<T>((float)h0, (float)h1);
+              if constexpr (LO) vl.w[j][0] = pack2<T>(x0 - (float)h0, x1 - (float)h1);
+            }
+            transpose_rows<2>(vh, Bh);
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+              for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bh[b], acc[a][b]);
+            if constexpr (LO) {
+              u32x4 Bl[2];
+              transpose_rows<2>(vl, Bl);
+#pragma unroll
+              for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bl[b], acc[a][b]);
+            }
+            if (bv == 0) {  // one of the two waves of a key-feature block sums dkm
+#pragma unroll
+              for (int j = 0; j < 8; ++j) {
+                const float dzj = scal[tok0 + j];
+                dkm[0] = fmaf(dzj, Ops<T>::lo(qw.w[j][0]), dkm[0]);
+                dkm[1] = fmaf(dzj, Ops<T>::hi(qw.w[j][0]), dkm[1]);
+              }
+            }
+          } else {
+            transpose_rows<2>(gw, Bh);
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+              for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bh[b], acc[a][b]);
+          }
+        }
+      }
+      __syncthreads();  // every wave has read every tile: they can take the dq now
+    } else if constexpr (FUSED) {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       const int tok0 = 16 * ks + 8 * kb;
@@ -1212,7 +1287,14 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : dst + dk * dv;
     const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
     const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
-    reduce_store_block<4, true, PAIR>(acc, dkm, red, dst, dv, dst_vec, mscale, vscale, wave, lane, dk, dv);
+    if constexpr (BIG) {  // every wave stores the block it owns
+      const int bk = wave >> 1, bv = wave & 1;
+      reduce_store_block<1>(acc, dkm, red, dst + (64 * bk) * dv + 64 * bv, dv,
+                            (dst_vec && bv == 0) ? dst_vec + 64 * bk : nullptr, mscale, vscale, 0, lane,
+                            dk - 64 * bk, dv - 64 * bv);
+    } else {
+      reduce_store_block<4, true, PAIR>(acc, dkm, red, dst, dv, dst_vec, mscale, vscale, wave, lane, dk, dv);
+    }
   }
 }
 
@@ -1240,9 +1322,10 @@ bool supported(const Prob& p, int dtype) {
   return true;
 }
 
-// The fused backward pass A exists for heads up to 64 x 64.
+// The fused backward pass A exists for heads tiled as 64 x 64 and as 128 x 128 (the latter
+// not for the decoupled operator, which `supported` already limits to 64 x 64).
 bool bwd_a_supported(const Prob& p, int dtype) {
-  return dtype != kF32 && supported(p, dtype) && p.DK <= 64 && p.DV <= 64;
+  return dtype != kF32 && supported(p, dtype) && tiled_dim(p.DK) == tiled_dim(p.DV);
 }
 
 // Number of compute units of the current device (256 on MI355X; also the value
@@ -1288,6 +1371,8 @@ int state_chunk(const Prob& p) {
 
 int bwd_a_chunk(const Prob& p) {
   static const int per_cu = knob("FBLA_BWDA_WGS_PER_CU", 2);
+  // 128 x 128: one workgroup per CU, steps of 128 tokens
+  if (tiled_dim(p.DK) == 128) return chunk_for(p, 1, 1, 512, 128);
   return chunk_for(p, per_cu, 1, 256, 128);
 }
 
@@ -1499,6 +1584,13 @@ static int run_bwd_a_pad(const Prob& p, const void* qn, const void* qd, const vo
                          int chunk, int nchunks, hipStream_t st) {
   const T *a = (const T*)qn, *b = (const T*)qd, *c = (const T*)dout;
   T *x = (T*)dqn, *y = (T*)dqd;
+  if constexpr (!PAIR) {
+    if (tiled_dim(p.DK) == 128) {
+      if (!(p.flags & kNormalize))
+        return launch_bwd_a<T, 128, 128, false, false, true, PAD>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+      return launch_bwd_a<T, 128, 128, true, false, true, PAD>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+    }
+  }
   if (!(p.flags & kNormalize))
     return launch_bwd_a<T, 64, 64, false, false, true, PAD, PAIR>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
   if (p.flags & kDecoupled)
