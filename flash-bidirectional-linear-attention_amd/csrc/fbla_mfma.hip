@@ -892,11 +892,9 @@ __device__ __forceinline__ void lds_rows(RowWords<C>& dst, const unsigned char* 
 
 template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struct BwdALayout {
   static constexpr int KS = DV / 16, NB = DK / 32;
-  static constexpr bool kBig = FUSED && DK == 128 && DV == 128;  // no staged lo part (LDS budget)
   static constexpr int kOpnd = NB * KS * 2 * 1024;
   static constexpr int kQ = 32 * DK * 2, kG = 32 * DV * 2;
-  static constexpr int kWave =
-      kQ + kG + (NORM && FUSED && LO && !kBig ? kG : 0) + (DEN ? kQ : 0) + 256;  // + dz[64] (or dz[32], 1/z[32])
+  static constexpr int kWave = kQ + kG + (NORM && FUSED && LO ? kG : 0) + (DEN ? kQ : 0) + 256;  // + dz[64]
   static constexpr int kKmPairs = kOpnd + kWaves * kWave;
   static constexpr int kKmF = kKmPairs + DK * 4;
   static constexpr int kMax = kKmF + DK * 4;
@@ -913,15 +911,9 @@ template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struc
 // 64-wide row as in the rows kernel; the token view never mixes the halves of a row, the
 // feature view accumulates blockdiag-shaped sums whose two diagonal 32 x 32 blocks are added
 // before the store.  `chunk` counts row pairs.
-// FUSED at 128 x 128 (one workgroup per CU, 134 KiB of LDS): dS does not fit one wave, so each
-// of the four waves owns one 64 x 64 block of it and walks the tiles of all four waves.  Per
-// step of 128 tokens: every wave runs the token view of its own 32-token tile and leaves 1/z_t
-// and dz_t in LDS; barrier; every wave multiplies its block over the four tiles, scaling and
-// splitting dO rows into hi + lo on the fly (there is no room to stage a lo copy); barrier;
-// every wave stages and stores the dq of its tile.
 template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true, bool PAD = false,
           bool PAIR = false>
-__global__ __launch_bounds__(kThreads, (FUSED && DK == 128 && DV == 128) ? 1 : 2) void bwd_a_kernel(
+__global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const T* __restrict__ dout,
     const float* __restrict__ S, const float* __restrict__ km, T* __restrict__ dqn,
     T* __restrict__ dqd, float* __restrict__ partial, float* __restrict__ tokscal,
@@ -929,9 +921,7 @@ __global__ __launch_bounds__(kThreads, (FUSED && DK == 128 && DV == 128) ? 1 : 2
   using LY = BwdALayout<DK, DV, NORM, DEN, FUSED, LO>;
   constexpr int KS = LY::KS, NB = LY::NB;
   constexpr int CK = DK / 32, CV = DV / 32;
-  constexpr bool BIG = LY::kBig;
-  static_assert(!FUSED || BIG || (DK == 64 && DV == 64), "fused pass A: 64 x 64 or 128 x 128 tiles");
-  static_assert(!BIG || !DEN, "no decoupled variant at 128 x 128");
+  static_assert(!FUSED || (DK == 64 && DV == 64), "the fused form exists for 64 x 64 tiles (128 x 128: bwd_a128_kernel)");
   static_assert(!PAIR || (DK == 64 && DV == 64 && FUSED && !PAD), "pair mode: two 32-wide rows per 64-wide row");
   const int dk = PAD ? p.DK : (PAIR ? 32 : DK), dv = PAD ? p.DV : (PAIR ? 32 : DV);
   constexpr int QROWB = DK * 2, GROWB = DV * 2;
@@ -977,7 +967,7 @@ __global__ __launch_bounds__(kThreads, (FUSED && DK == 128 && DV == 128) ? 1 : 2
   unsigned char* qt = smem + LY::kOpnd + wave * LY::kWave;
   unsigned char* gt = qt + LY::kQ;             // dO, later dO/z (hi part)
   unsigned char* gl = gt + LY::kG;             // dO/z (lo part), NORM && FUSED only
-  unsigned char* qdt = gl + (NORM && FUSED && LO && !LY::kBig ? LY::kG : 0);  // plain q, DEN only
+  unsigned char* qdt = gl + (NORM && FUSED && LO ? LY::kG : 0);  // plain q, DEN only
   float* dzs = reinterpret_cast<float*>(qdt + (DEN ? LY::kQ : 0));
   uint32_t* km_pairs = reinterpret_cast<uint32_t*>(smem + LY::kKmPairs);
   float* kmf = reinterpret_cast<float*>(smem + LY::kKmF);
@@ -1035,7 +1025,7 @@ __global__ __launch_bounds__(kThreads, (FUSED && DK == 128 && DV == 128) ? 1 : 2
 
   int t0 = t_begin + 32 * wave;
   u32x4 rq[QI], rg[GI], rd[QI];
-  if (LY::kBig || t0 < t_end) {
+  if (t0 < t_end) {
     load_q(rq, qn, t0);
     load_g(rg, dout, t0);
     if constexpr (DEN) load_q(rd, qd, t0);
@@ -1049,15 +1039,13 @@ __global__ __launch_bounds__(kThreads, (FUSED && DK == 128 && DV == 128) ? 1 : 2
   }
   __syncthreads();
 
-  // BIG: all waves make the same number of steps (a wave whose tile lies past the end works
-  // on zeros), because the steps contain workgroup barriers
-  while (BIG ? t0 - 32 * wave < t_end : t0 < t_end) {
+  while (t0 < t_end) {
     wave_sync();  // the previous sub-tile's staged dq has been read out
     stash_q(rq, qt);
     stash_g(rg, gt);
     if constexpr (DEN) stash_q(rd, qdt);
     const int tn = t0 + 32 * kWaves;
-    if (BIG || tn < t_end) {
+    if (tn < t_end) {
       load_q(rq, qn, tn);
       load_g(rg, dout, tn);
       if constexpr (DEN) load_q(rd, qd, tn);
@@ -1113,7 +1101,6 @@ __global__ __launch_bounds__(kThreads, (FUSED && DK == 128 && DV == 128) ? 1 : 2
       }
       if constexpr (FUSED) {
         if (PAIR || kb == 0) dzs[32 * (PAIR ? kb : 0) + ntok] = dz;
-        if (BIG && kb == 0) dzs[32 + ntok] = rz;
       } else {
         if (kb == 0 && t0 + ntok < t_end) {
           const int64_t row = row0 + (int64_t)(t0 + ntok) * rstride;
@@ -1143,7 +1130,7 @@ __global__ __launch_bounds__(kThreads, (FUSED && DK == 128 && DV == 128) ? 1 : 2
       }
     }
     // dO / z as hi + lo, in place over this lane's own chunks of the dO tile
-    if constexpr (NORM && FUSED && !BIG) {
+    if constexpr (NORM && FUSED) {
 #pragma unroll
       for (int ch = 0; ch < GCH / 2; ++ch) {
         const int off = swz<GROWB>(ntok, (GCH / 2) * kb + ch);
@@ -1160,72 +1147,10 @@ __global__ __launch_bounds__(kThreads, (FUSED && DK == 128 && DV == 128) ? 1 : 2
         if constexpr (LO) *reinterpret_cast<u32x4*>(gl + off) = wl;
       }
     }
-    if constexpr (BIG) __syncthreads();  // all four tiles and their scalars are staged
-    else wave_sync();
+    wave_sync();
 
     // ---- feature view: two k-steps of 16 tokens ----
-    if constexpr (BIG) {
-      const int bk = wave >> 1, bv = wave & 1;
-#pragma unroll
-      for (int u = 0; u < kWaves; ++u) {
-        const unsigned char* qtu = smem + LY::kOpnd + u * LY::kWave;
-        const unsigned char* gtu = qtu + LY::kQ;
-        const float* scal = reinterpret_cast<const float*>(gtu + LY::kG);  // dz[32], 1/z[32]
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-          const int tok0 = 16 * ks + 8 * kb;
-          RowWords<2> qw, gw;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            qw.w[j][0] = *reinterpret_cast<const uint32_t*>(qtu + swz<QROWB>(tok0 + j, 8 * bk + (ntok >> 2)) +
-                                                            ((ntok & 3) << 2));
-            gw.w[j][0] = *reinterpret_cast<const uint32_t*>(gtu + swz<GROWB>(tok0 + j, 8 * bv + (ntok >> 2)) +
-                                                            ((ntok & 3) << 2));
-          }
-          u32x4 A[2], Bh[2];
-          transpose_rows<2>(qw, A);
-          if constexpr (NORM) {
-            RowWords<2> vh, vl;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              const float rzj = scal[32 + tok0 + j];
-              const float x0 = Ops<T>::lo(gw.w[j][0]) * rzj, x1 = Ops<T>::hi(gw.w[j][0]) * rzj;
-              const T h0 = (T)x0, h1 = (T)x1;
-              vh.w[j][0] = pack2<T>((float)h0, (float)h1);
-              if constexpr (LO) vl.w[j][0] = pack2<T>(x0 - (float)h0, x1 - (float)h1);
-            }
-            transpose_rows<2>(vh, Bh);
-#pragma unroll
-            for (int a = 0; a < 2; ++a)
-#pragma unroll
-              for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bh[b], acc[a][b]);
-            if constexpr (LO) {
-              u32x4 Bl[2];
-              transpose_rows<2>(vl, Bl);
-#pragma unroll
-              for (int a = 0; a < 2; ++a)
-#pragma unroll
-                for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bl[b], acc[a][b]);
-            }
-            if (bv == 0) {  // one of the two waves of a key-feature block sums dkm
-#pragma unroll
-              for (int j = 0; j < 8; ++j) {
-                const float dzj = scal[tok0 + j];
-                dkm[0] = fmaf(dzj, Ops<T>::lo(qw.w[j][0]), dkm[0]);
-                dkm[1] = fmaf(dzj, Ops<T>::hi(qw.w[j][0]), dkm[1]);
-              }
-            }
-          } else {
-            transpose_rows<2>(gw, Bh);
-#pragma unroll
-            for (int a = 0; a < 2; ++a)
-#pragma unroll
-              for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bh[b], acc[a][b]);
-          }
-        }
-      }
-      __syncthreads();  // every wave has read every tile: they can take the dq now
-    } else if constexpr (FUSED) {
+    if constexpr (FUSED) {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       const int tok0 = 16 * ks + 8 * kb;
@@ -1287,14 +1212,291 @@ __global__ __launch_bounds__(kThreads, (FUSED && DK == 128 && DV == 128) ? 1 : 2
     float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : dst + dk * dv;
     const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
     const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
-    if constexpr (BIG) {  // every wave stores the block it owns
-      const int bk = wave >> 1, bv = wave & 1;
-      reduce_store_block<1>(acc, dkm, red, dst + (64 * bk) * dv + 64 * bv, dv,
-                            (dst_vec && bv == 0) ? dst_vec + 64 * bk : nullptr, mscale, vscale, 0, lane,
-                            dk - 64 * bk, dv - 64 * bv);
-    } else {
-      reduce_store_block<4, true, PAIR>(acc, dkm, red, dst, dv, dst_vec, mscale, vscale, wave, lane, dk, dv);
+    reduce_store_block<4, true, PAIR>(acc, dkm, red, dst, dv, dst_vec, mscale, vscale, wave, lane, dk, dv);
+  }
+}
+
+// ===========================================================================
+// backward pass A, heads tiled 128 x 128
+// ===========================================================================
+// dS (128 x 128 fp32) does not fit one wave and the 64 KiB matrix operand leaves LDS for four
+// 32-token tiles only, so one workgroup of eight waves shares a step of 128 tokens:
+//   token view    wave w takes tile u = w % 4 and the output half hf = w / 4 of g = dO S^T (two
+//                 of the four 32-column blocks); the partial q~.g and q.km sums of the two
+//                 halves meet in LDS, then both waves know 1/z_t and dz_t and pack their half
+//                 of dq;
+//   feature view  wave w owns block w % 4 of dS (64 x 64) over the tiles 2*(w/4), 2*(w/4)+1;
+//                 dO rows are scaled by 1/z_t and split into hi + lo on the fly (no LDS left
+//                 for a staged copy); the two waves of a block are summed at the end;
+//   dq            goes back through the q tile so that whole rows are stored.
+// The steps are separated by workgroup barriers; all waves make the same number of steps (a
+// tile past the end of the chunk is all zeros).
+struct BwdA128Layout {
+  static constexpr int kOpnd = 4 * 8 * 2 * 1024;  // 4 blocks x 8 k-steps x (hi, lo) fragments
+  static constexpr int kTile = 2 * 32 * 256;      // q tile | dO tile
+  static constexpr int kTiles = kOpnd;
+  static constexpr int kPz = kTiles + 4 * kTile;  // [tile][half][32] partial (q~.g, q.km)
+  static constexpr int kScal = kPz + 4 * 2 * 32 * 8;  // [tile] dz[32], 1/z[32]
+  static constexpr int kKmPairs = kScal + 4 * 64 * 4;
+  static constexpr int kKmF = kKmPairs + 128 * 4;
+  static constexpr int kMax = kKmF + 128 * 4;
+  static constexpr int kLpt = kMax + 64;
+  static constexpr int kTotal = kLpt + (kLptMax + 1) * 4;
+  // the final two-wave reduction reuses the tile area
+  static_assert(kKmPairs - kTiles >= 4 * 64 * 66 * 4, "reduction buffers of the four blocks");
+  static_assert(kTotal <= 160 * 1024, "LDS of one CU");
+};
+
+template <typename T, bool NORM, bool PAD>
+__global__ __launch_bounds__(512, 1) void bwd_a128_kernel(
+    Prob p, const T* __restrict__ qn, const T* __restrict__ dout, const float* __restrict__ S,
+    const float* __restrict__ km, T* __restrict__ dqn, float* __restrict__ partial, float* fin_mat,
+    float* fin_vec, int chunk, int nchunks) {
+  using LY = BwdA128Layout;
+  constexpr bool LO = !std::is_same<T, _Float16>::value;  // see launch_bwd_a
+  constexpr int KS = 8, ROWB = 256, NT = 512;
+  const int dk = PAD ? p.DK : 128, dv = PAD ? p.DV : 128;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int wg_nh = blockIdx.x / nchunks, c = blockIdx.x - wg_nh * nchunks;
+  const int h = wg_nh % p.H;
+  const int n = lpt_sequence(p, wg_nh / p.H, reinterpret_cast<int*>(smem + LY::kLpt));
+  const int nh = n * p.H + h;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t_begin = c * chunk;
+  if (t_begin >= len) {
+    if (fin_mat && c == 0) {  // empty sequence: no gradient flows through its state
+      for (int e = threadIdx.x; e < dk * dv; e += NT) fin_mat[(int64_t)nh * dk * dv + e] = 0.f;
+      if (fin_vec)
+        for (int e = threadIdx.x; e < dk; e += NT) fin_vec[(int64_t)nh * dk + e] = 0.f;
     }
+    return;
+  }
+  const int t_end = min(len, t_begin + chunk);
+  row_base(p, n, h, bos, row0, rstride);
+  auto piece = [&](int tok, int ch, int rowlen) -> int64_t {
+    if (tok >= t_end || (PAD && ch * 8 >= rowlen)) return -1;
+    return (row0 + (int64_t)tok * rstride) * rowlen + ch * 8;
+  };
+
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int ntok = lane & 31, kb = lane >> 5;
+  const int u = wave & 3, hf = wave >> 2;  // token view: tile, output half; feature view: block, tile pair
+  unsigned char* lds_opnd = smem;
+  unsigned char* qt = smem + LY::kTiles + u * LY::kTile;
+  unsigned char* gt = qt + LY::kTile / 2;
+  float* pz = reinterpret_cast<float*>(smem + LY::kPz);
+  float* scal = reinterpret_cast<float*>(smem + LY::kScal) + 64 * u;
+  uint32_t* km_pairs = reinterpret_cast<uint32_t*>(smem + LY::kKmPairs);
+  float* kmf = reinterpret_cast<float*>(smem + LY::kKmF);
+  float* lds_max = reinterpret_cast<float*>(smem + LY::kMax);
+
+  // a wave moves the half of its tile's 512 16-byte pieces given by hf (rows 16*hf .. 16*hf+15)
+  auto load_half = [&](u32x4(&dst)[4], const T* src, int tok0, int rowlen) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = 256 * hf + lane + 64 * i;
+      const int64_t off = piece(tok0 + (q >> 4), q & 15, rowlen);
+      dst[i] = off >= 0 ? *reinterpret_cast<const u32x4*>(src + off) : u32x4{0u, 0u, 0u, 0u};
+    }
+  };
+  auto stash_half = [&](const u32x4(&src)[4], unsigned char* dstb) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = 256 * hf + lane + 64 * i;
+      *reinterpret_cast<u32x4*>(dstb + swz<ROWB>(q >> 4, q & 15)) = src[i];
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  float dkm[2] = {0.f, 0.f};
+
+  u32x4 rq[4], rg[4];
+  load_half(rq, qn, t_begin + 32 * u, dk);
+  load_half(rg, dout, t_begin + 32 * u, dv);
+
+  // g_t = dO_t S^T: contraction over dv, M(r = dv, c = dk) = S[c][r]
+  const float denorm = build_operand<T, 128, 128, NT, PAD>(lds_opnd, lds_max, S + (int64_t)nh * dk * dv, 1, dv,
+                                                          1, 0, 1.f, nullptr, dv, dk);
+  if constexpr (NORM) build_vec<T, NT>(km_pairs, kmf, km + (int64_t)nh * dk, dk, 1, 0, 1.f, nullptr, 128);
+
+  for (int base = t_begin; base < t_end; base += 128) {
+    const int t0 = base + 32 * u;
+    __syncthreads();  // operand built / the previous step's dq has left the tiles
+    stash_half(rq, qt);
+    stash_half(rg, gt);
+    load_half(rq, qn, t0 + 128, dk);
+    load_half(rg, dout, t0 + 128, dv);
+    __syncthreads();
+
+    // ---- token view: output blocks 2*hf, 2*hf+1; this lane: columns 64*kb + 32*hf + 0..31
+    f32x16 g[2];
+#pragma unroll
+    for (int bb = 0; bb < 2; ++bb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) g[bb][r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const u32x4 bq = *reinterpret_cast<const u32x4*>(gt + swz<ROWB>(ntok, KS * kb + s));
+#pragma unroll
+      for (int bb = 0; bb < 2; ++bb) {
+        const int f = (2 * hf + bb) * KS + s;
+        const u32x4 ah = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * f + 0) * 64 + lane) * 16);
+        const u32x4 al = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * f + 1) * 64 + lane) * 16);
+        g[bb] = Ops<T>::mma(ah, bq, g[bb]);
+        g[bb] = Ops<T>::mma(al, bq, g[bb]);
+      }
+    }
+    float rz = 1.f, dz = 0.f;
+    if constexpr (NORM) {
+      float P = 0.f, z = 0.f;
+#pragma unroll
+      for (int ch = 0; ch < 4; ++ch) {
+        const u32x4 qw = *reinterpret_cast<const u32x4*>(qt + swz<ROWB>(ntok, 8 * kb + 4 * hf + ch));
+        const u32x4 kh = *reinterpret_cast<const u32x4*>(&km_pairs[32 * kb + 16 * hf + 4 * ch]);
+        const u32x4 kl = *reinterpret_cast<const u32x4*>(&km_pairs[64 + 32 * kb + 16 * hf + 4 * ch]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int c0 = 8 * ch + 2 * i;
+          P = fmaf(Ops<T>::lo(qw[i]), g[c0 >> 4][c0 & 15], P);
+          P = fmaf(Ops<T>::hi(qw[i]), g[c0 >> 4][(c0 & 15) + 1], P);
+          z = Ops<T>::dot2(qw[i], kh[i], z);
+          z = Ops<T>::dot2(qw[i], kl[i], z);
+        }
+      }
+      P += __shfl_xor(P, 32);
+      z += __shfl_xor(z, 32);
+      if (kb == 0) {
+        pz[2 * ((2 * u + hf) * 32 + ntok)] = P;
+        pz[2 * ((2 * u + hf) * 32 + ntok) + 1] = z;
+      }
+      __syncthreads();
+      P += pz[2 * ((2 * u + 1 - hf) * 32 + ntok)];
+      z += pz[2 * ((2 * u + 1 - hf) * 32 + ntok) + 1];
+      if (t0 + ntok < t_end) {
+        rz = 1.f / (z + p.eps);
+        dz = -(P * denorm) * rz * rz;
+      } else {
+        rz = 0.f;  // padding rows contribute nothing
+      }
+      if (hf == 0 && kb == 0) {
+        scal[ntok] = dz;
+        scal[32 + ntok] = rz;
+      }
+    }
+    uint32_t dqp[16];
+    {
+      const float gs = denorm * rz;
+#pragma unroll
+      for (int c2 = 0; c2 < 16; ++c2) {
+        const int c0 = 2 * c2;
+        float v0 = g[c0 >> 4][c0 & 15] * gs, v1 = g[c0 >> 4][(c0 & 15) + 1] * gs;
+        if constexpr (NORM) {
+          v0 = fmaf(dz, kmf[64 * kb + 32 * hf + c0], v0);
+          v1 = fmaf(dz, kmf[64 * kb + 32 * hf + c0 + 1], v1);
+        }
+        dqp[c2] = pack2<T>(v0, v1);
+      }
+    }
+    __syncthreads();  // all four tiles and their scalars are complete
+
+    // ---- feature view: block u = (bk, bv) of dS over the tiles 2*hf, 2*hf+1
+    {
+      const int bk = u >> 1, bv = u & 1;
+#pragma unroll 1
+      for (int uu = 0; uu < 2; ++uu) {
+        const unsigned char* qtu = smem + LY::kTiles + (2 * hf + uu) * LY::kTile;
+        const unsigned char* gtu = qtu + LY::kTile / 2;
+        const float* sc = reinterpret_cast<const float*>(smem + LY::kScal) + 64 * (2 * hf + uu);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          const int tok0 = 16 * ks + 8 * kb;
+          RowWords<2> qw, gw;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            qw.w[j][0] = *reinterpret_cast<const uint32_t*>(qtu + swz<ROWB>(tok0 + j, 8 * bk + (ntok >> 2)) +
+                                                            ((ntok & 3) << 2));
+            gw.w[j][0] = *reinterpret_cast<const uint32_t*>(gtu + swz<ROWB>(tok0 + j, 8 * bv + (ntok >> 2)) +
+                                                            ((ntok & 3) << 2));
+          }
+          u32x4 A[2], Bh[2];
+          transpose_rows<2>(qw, A);
+          if constexpr (NORM) {
+            RowWords<2> vh, vl;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float rzj = sc[32 + tok0 + j];
+              const float x0 = Ops<T>::lo(gw.w[j][0]) * rzj, x1 = Ops<T>::hi(gw.w[j][0]) * rzj;
+              const T h0 = (T)x0, h1 = (T)x1;
+              vh.w[j][0] = pack2<T>((float)h0, (float)h1);
+              if constexpr (LO) vl.w[j][0] = pack2<T>(x0 - (float)h0, x1 - (float)h1);
+            }
+            transpose_rows<2>(vh, Bh);
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+              for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bh[b], acc[a][b]);
+            if constexpr (LO) {
+              u32x4 Bl[2];
+              transpose_rows<2>(vl, Bl);
+#pragma unroll
+              for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bl[b], acc[a][b]);
+            }
+            if (bv == 0) {  // the waves of one value half of a key block sum dkm
+#pragma unroll
+              for (int j = 0; j < 8; ++j) {
+                const float dzj = sc[tok0 + j];
+                dkm[0] = fmaf(dzj, Ops<T>::lo(qw.w[j][0]), dkm[0]);
+                dkm[1] = fmaf(dzj, Ops<T>::hi(qw.w[j][0]), dkm[1]);
+              }
+            }
+          } else {
+            transpose_rows<2>(gw, Bh);
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+              for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bh[b], acc[a][b]);
+          }
+        }
+      }
+    }
+    __syncthreads();  // every wave has read every tile: they can take the dq now
+#pragma unroll
+    for (int ch = 0; ch < 4; ++ch)
+      *reinterpret_cast<u32x4*>(qt + swz<ROWB>(ntok, 8 * kb + 4 * hf + ch)) =
+          u32x4{dqp[4 * ch], dqp[4 * ch + 1], dqp[4 * ch + 2], dqp[4 * ch + 3]};
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = 256 * hf + lane + 64 * i;
+      const int64_t off = piece(t0 + (q >> 4), q & 15, dk);
+      if (off >= 0)
+        *reinterpret_cast<u32x4*>(dqn + off) = *reinterpret_cast<const u32x4*>(qt + swz<ROWB>(q >> 4, q & 15));
+    }
+  }
+
+  __syncthreads();  // the tiles become the reduction buffers
+  {
+    const int bk = u >> 1, bv = u & 1;
+    float* red = reinterpret_cast<float*>(smem + LY::kTiles) + u * 64 * 66;
+    float* dst = fin_mat ? fin_mat + (int64_t)nh * dk * dv
+                         : partial + ((int64_t)nh * nchunks + c) * (dk * dv + dk);
+    float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : dst + dk * dv;
+    const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
+    const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
+    reduce_store_block<2>(acc, dkm, red, dst + (64 * bk) * dv + 64 * bv, dv,
+                          (dst_vec && bv == 0) ? dst_vec + 64 * bk : nullptr, mscale, vscale, hf, lane,
+                          dk - 64 * bk, dv - 64 * bv);
   }
 }
 
@@ -1578,6 +1780,19 @@ static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, 
   return kOk;
 }
 
+template <typename T, bool NORM, bool PAD>
+static int launch_bwd_a128(const Prob& p, const T* q, const T* dout, const float* S, const float* km, T* dq,
+                           float* partial, float* fm, float* fv, int chunk, int nchunks, hipStream_t st) {
+  using LY = BwdA128Layout;
+  auto kernel = bwd_a128_kernel<T, NORM, PAD>;
+  static thread_local bool configured = false;  // per instantiation
+  int rc = reserve_lds(kernel, LY::kTotal, configured);
+  if (rc != kOk) return rc;
+  const unsigned grid = (unsigned)((int64_t)p.N * p.H * nchunks);
+  kernel<<<dim3(grid), dim3(512), LY::kTotal, st>>>(p, q, dout, S, km, dq, partial, fm, fv, chunk, nchunks);
+  return kOk;
+}
+
 template <typename T, bool PAD, bool PAIR = false>
 static int run_bwd_a_pad(const Prob& p, const void* qn, const void* qd, const void* dout, const float* S,
                          const float* km, void* dqn, void* dqd, float* partial, float* fm, float* fv,
@@ -1587,8 +1802,8 @@ static int run_bwd_a_pad(const Prob& p, const void* qn, const void* qd, const vo
   if constexpr (!PAIR) {
     if (tiled_dim(p.DK) == 128) {
       if (!(p.flags & kNormalize))
-        return launch_bwd_a<T, 128, 128, false, false, true, PAD>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
-      return launch_bwd_a<T, 128, 128, true, false, true, PAD>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+        return launch_bwd_a128<T, false, PAD>(p, a, c, S, km, x, partial, fm, fv, chunk, nchunks, st);
+      return launch_bwd_a128<T, true, PAD>(p, a, c, S, km, x, partial, fm, fv, chunk, nchunks, st);
     }
   }
   if (!(p.flags & kNormalize))
