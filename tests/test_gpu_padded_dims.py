@@ -88,3 +88,16 @@ def test_many_chunks_per_head():
     _check_dense("linear", 1, 1, 20000, 32, 32, torch.float16, 7)
     _check_dense("linear", 1, 1, 9000, 128, 32, torch.bfloat16, 8)
     _check_dense("decoupled", 1, 1, 9000, 32, 32, torch.float16, 9)
+
+
+def test_heads_tiled_128_by_128():
+    """The 128 x 128 backward kernel (eight waves share a step of 128 tokens): several chunks per
+    head, lengths that leave one to three of a step's four tiles empty, the unnormalised
+    operator, head dims below 128 in both tiles."""
+    _check_dense("linear", 1, 1, 9000, 128, 128, torch.bfloat16, 11)
+    _check_dense("linear", 2, 3, 33, 128, 128, torch.float16, 12)
+    _check_dense("linear", 2, 3, 200, 128, 128, torch.bfloat16, 13)
+    _check_dense("simple", 1, 2, 3000, 128, 128, torch.float16, 14)
+    _check_dense("simple", 1, 2, 97, 128, 128, torch.bfloat16, 15)
+    _check_dense("linear", 1, 1, 5000, 96, 120, torch.float16, 16)
+    _check_dense("linear", 3, 2, 129, 72, 128, torch.bfloat16, 17)
