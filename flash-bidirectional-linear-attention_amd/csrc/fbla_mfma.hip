@@ -709,6 +709,7 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
   };
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const bool has_add = job.addvec != nullptr || job.vec_is_add;  // the same for all lanes
   const T* x = (const T*)job.x;
   const T* xden = (const T*)job.xden;
   T* out = (T*)job.out;
@@ -803,21 +804,40 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[b][r] = 0.f;
     float z = 0.f;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const u32x4 bq = *reinterpret_cast<const u32x4*>(stage + swz<XROWB>(ntok, KS * kb + s));
+    // the LDS reads of k-step s+1 are issued before the MFMAs of step s, so that their latency
+    // runs under the multiplications (two register sets, static indices after unrolling)
+    struct Step {
+      u32x4 bq, bd, kh, kl, ah[NB], al[NB];
+    } st[2];
+    auto fetch_step = [&](int s, Step& f) {
+      f.bq = *reinterpret_cast<const u32x4*>(stage + swz<XROWB>(ntok, KS * kb + s));
 #pragma unroll
       for (int b = 0; b < NB; ++b) {
-        const u32x4 ah = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * (b * KS + s) + 0) * 64 + lane) * 16);
-        const u32x4 al = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * (b * KS + s) + 1) * 64 + lane) * 16);
-        acc[b] = Ops<T>::mma(ah, bq, acc[b]);
-        acc[b] = Ops<T>::mma(al, bq, acc[b]);
+        f.ah[b] = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * (b * KS + s) + 0) * 64 + lane) * 16);
+        f.al[b] = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * (b * KS + s) + 1) * 64 + lane) * 16);
+      }
+      if constexpr (NORM) {
+        if constexpr (DEN) f.bd = *reinterpret_cast<const u32x4*>(stage_den + swz<XROWB>(ntok, KS * kb + s));
+        f.kh = *reinterpret_cast<const u32x4*>(&lds_km[(DR / 4) * kb + 4 * s]);
+        f.kl = *reinterpret_cast<const u32x4*>(&lds_km[DR / 2 + (DR / 4) * kb + 4 * s]);
+      }
+    };
+    fetch_step(0, st[0]);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      if (s + 1 < KS) fetch_step(s + 1, st[(s + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);  // keep the reads above ahead of the MFMAs below
+      const Step& f = st[s & 1];
+      const u32x4 bq = f.bq;
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        acc[b] = Ops<T>::mma(f.ah[b], bq, acc[b]);
+        acc[b] = Ops<T>::mma(f.al[b], bq, acc[b]);
       }
       if constexpr (NORM) {
         u32x4 bd = bq;
-        if constexpr (DEN) bd = *reinterpret_cast<const u32x4*>(stage_den + swz<XROWB>(ntok, KS * kb + s));
-        const u32x4 kh = *reinterpret_cast<const u32x4*>(&lds_km[(DR / 4) * kb + 4 * s]);
-        const u32x4 kl = *reinterpret_cast<const u32x4*>(&lds_km[DR / 2 + (DR / 4) * kb + 4 * s]);
+        if constexpr (DEN) bd = f.bd;
+        const u32x4 kh = f.kh, kl = f.kl;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           z = Ops<T>::dot2(bd[i], kh[i], z);
@@ -831,28 +851,45 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
       rs = denorm / (z + p.eps);
     }
     wave_sync();  // all lanes have read their x chunks; staging is reused for out
+    if (has_add) {  // only the dk job of the backward adds a row (dkm / L)
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      u32x4 w0, w1;
-      const float* av = &lds_add[(DC / 2) * kb + 16 * b];
+      for (int b = 0; b < NB; ++b) {
+        u32x4 w0, w1;
+        const float* av = &lds_add[(DC / 2) * kb + 16 * b];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        w0[i] = pack2<T>(fmaf(acc[b][2 * i], rs, av[2 * i]), fmaf(acc[b][2 * i + 1], rs, av[2 * i + 1]));
-        w1[i] = pack2<T>(fmaf(acc[b][8 + 2 * i], rs, av[8 + 2 * i]),
-                         fmaf(acc[b][8 + 2 * i + 1], rs, av[8 + 2 * i + 1]));
+        for (int i = 0; i < 4; ++i) {
+          w0[i] = pack2<T>(fmaf(acc[b][2 * i], rs, av[2 * i]), fmaf(acc[b][2 * i + 1], rs, av[2 * i + 1]));
+          w1[i] = pack2<T>(fmaf(acc[b][8 + 2 * i], rs, av[8 + 2 * i]),
+                           fmaf(acc[b][8 + 2 * i + 1], rs, av[8 + 2 * i + 1]));
+        }
+        *reinterpret_cast<u32x4*>(stage + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b)) = w0;
+        *reinterpret_cast<u32x4*>(stage + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b + 1)) = w1;
       }
-      *reinterpret_cast<u32x4*>(stage + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b)) = w0;
-      *reinterpret_cast<u32x4*>(stage + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b + 1)) = w1;
+    } else {
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        u32x4 w0, w1;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          w0[i] = pack2<T>(acc[b][2 * i] * rs, acc[b][2 * i + 1] * rs);
+          w1[i] = pack2<T>(acc[b][8 + 2 * i] * rs, acc[b][8 + 2 * i + 1] * rs);
+        }
+        *reinterpret_cast<u32x4*>(stage + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b)) = w0;
+        *reinterpret_cast<u32x4*>(stage + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b + 1)) = w1;
+      }
     }
     wave_sync();
+    u32x4 wout[OI];  // all LDS reads first (one wait), then the stores
+#pragma unroll
+    for (int i = 0; i < OI; ++i) {
+      const int q = lane + 64 * i;
+      wout[i] = *reinterpret_cast<const u32x4*>(stage + swz<OROWB>(q / OCH, q % OCH));
+    }
 #pragma unroll
     for (int i = 0; i < OI; ++i) {
       const int q = lane + 64 * i, row = q / OCH, ch = q % OCH;
       const int64_t off = piece(t0 + row, ch, dc);
-      if (off >= 0) {
-        const u32x4 w = *reinterpret_cast<const u32x4*>(stage + swz<OROWB>(row, ch));
-        *reinterpret_cast<u32x4*>(out + off) = w;
-      }
+      if (off >= 0) *reinterpret_cast<u32x4*>(out + off) = wout[i];
     }
     t0 += 32 * WAVES;
   };
