@@ -62,6 +62,7 @@ static Prob make_prob(const int32_t* cu, int64_t N, int64_t H, int64_t L, int64_
   p.N = (int)N;
   p.H = (int)H;
   p.L = (int)L;
+  p.Lk = 0;
   p.T = T;
   p.DK = DK;
   p.DV = DV;
@@ -163,6 +164,62 @@ int fbla_la_bwd(const void* q, const void* k, const void* v, const void* q_rope,
   Prob p = make_prob(nullptr, B, H, L, B * L, DK, DV, flags, scale, eps);
   BwdArgs a{q, k, v, q_rope, k_rope, dout, s, km, dq, dk, dv, dq_rope, dk_rope, workspace,
             workspace_bytes_};
+  return run_bwd(what, p, dtype, a, (hipStream_t)stream);
+}
+
+static int check_cross(const char* what, int64_t Lk, int flags) {
+  if (Lk <= 0 || Lk > 0x7fffffffLL / 2) {
+    set_error("%s: the number of keys must be positive and fit 32-bit indexing, got %lld", what, (long long)Lk);
+    return kErrBadArg;
+  }
+  if (flags & (kDecoupled | kDefaultScale)) {
+    set_error("%s: not available for the decoupled operator or with a per-sequence default scale", what);
+    return kErrBadArg;
+  }
+  return kOk;
+}
+
+size_t fbla_la_cross_workspace_bytes(int pass, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int DK, int DV,
+                                     int dtype, int flags) {
+  const char* what = "fbla_la_cross_workspace_bytes";
+  if (check_dims(what, B, H, Lq, DK, DV, dtype, flags) != kOk || check_cross(what, Lk, flags) != kOk) return 0;
+  Prob p = make_prob(nullptr, B, H, Lq, B * Lq, DK, DV, flags, 1.f, 0.f);
+  p.Lk = (int)Lk;
+  return workspace_bytes(p, dtype, pass);
+}
+
+int fbla_la_cross_fwd(const void* q, const void* k, const void* v, void* o, float* s, float* km,
+                      void* workspace, size_t workspace_bytes_, int64_t B, int64_t H, int64_t Lq, int64_t Lk,
+                      int DK, int DV, int dtype, int flags, float scale, float eps, void* stream) {
+  const char* what = "fbla_la_cross_fwd";
+  int rc = check_dims(what, B, H, Lq, DK, DV, dtype, flags);
+  if (rc == kOk) rc = check_cross(what, Lk, flags);
+  if (rc != kOk) return rc;
+  if (B * H > 0 && Lq > 0 && (!q || !k || !v || !o || !s || ((flags & kNormalize) && !km))) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  Prob p = make_prob(nullptr, B, H, Lq, B * Lq, DK, DV, flags, scale, eps);
+  p.Lk = (int)Lk;
+  FwdArgs a{q, k, v, nullptr, nullptr, o, s, km, workspace, workspace_bytes_};
+  return run_fwd(what, p, dtype, a, (hipStream_t)stream);
+}
+
+int fbla_la_cross_bwd(const void* q, const void* k, const void* v, const void* dout, const float* s,
+                      const float* km, void* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes_,
+                      int64_t B, int64_t H, int64_t Lq, int64_t Lk, int DK, int DV, int dtype, int flags,
+                      float scale, float eps, void* stream) {
+  const char* what = "fbla_la_cross_bwd";
+  int rc = check_dims(what, B, H, Lq, DK, DV, dtype, flags);
+  if (rc == kOk) rc = check_cross(what, Lk, flags);
+  if (rc != kOk) return rc;
+  if (B * H > 0 && Lq > 0 && (!q || !k || !v || !dout || !s || ((flags & kNormalize) && !km) || !dq || !dk || !dv)) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  Prob p = make_prob(nullptr, B, H, Lq, B * Lq, DK, DV, flags, scale, eps);
+  p.Lk = (int)Lk;
+  BwdArgs a{q, k, v, nullptr, nullptr, dout, s, km, dq, dk, dv, nullptr, nullptr, workspace, workspace_bytes_};
   return run_bwd(what, p, dtype, a, (hipStream_t)stream);
 }
 

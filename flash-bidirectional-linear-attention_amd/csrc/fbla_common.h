@@ -24,6 +24,9 @@ enum Flags : int {
 struct Prob {
   const int32_t* cu;
   int N, H, L;  // L: dense length, or max_seqlen upper bound when packed
+  int Lk;       // dense only: number of key / value tokens when it differs from L (the number of
+                // queries), else 0.  Only the plan looks at it: kernels get a problem whose L is
+                // the length of the side they walk.
   int64_t T;    // total tokens (dense: N*L)
   int DK, DV;
   float scale;

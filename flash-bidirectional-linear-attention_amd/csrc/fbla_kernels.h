@@ -81,6 +81,7 @@ struct RowsJob {
   bool vec_is_add = false;
   float* mat_out = nullptr;
   float* vec_out = nullptr;
+  float add_scale = 1.f;  // factor on addvec (queries / keys when their numbers differ)
 };
 bool supported(const Prob& p, int dtype);
 bool bwd_a_supported(const Prob& p, int dtype);

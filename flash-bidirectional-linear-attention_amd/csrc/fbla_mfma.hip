@@ -780,7 +780,9 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
     if constexpr (NORM)
       build_vec<T, NT>(lds_km, nullptr, job.km + (int64_t)nh * dr, dr, 1, 0, 1.f, nullptr, DR, PAIR);
     for (int e = tid; e < DC; e += NT)
-      lds_add[e] = (job.addvec && (PAIR || e < dc)) ? job.addvec[(int64_t)nh * dc + (PAIR ? e % 32 : e)] : 0.f;
+      lds_add[e] = (job.addvec && (PAIR || e < dc))
+                       ? job.addvec[(int64_t)nh * dc + (PAIR ? e % 32 : e)] * job.add_scale
+                       : 0.f;
   }
   __syncthreads();
 

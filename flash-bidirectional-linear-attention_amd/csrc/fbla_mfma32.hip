@@ -225,7 +225,8 @@ struct Rows32Job {
   const float* mat;     // operand M, element (r, c) at mat[nh*4096 + r*ld_r + c*ld_c]
   int ld_r, ld_c;
   const float* km;      // [NH, 64] mean key (NORM / TOKENS with the denominator)
-  const float* addvec;  // [NH, 64] added to every output row, or null
+  const float* addvec;  // [NH, 64] added (times add_scale) to every output row, or null
+  float add_scale;
   float* out;           // [rows, 64]
   float* tokscal;       // TOKENS: [2][total rows]: 1/z_t, dz_t
   int64_t total_rows;
@@ -289,7 +290,7 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
   build_operand32(frag, job.mat + (int64_t)nh * D * D, job.ld_r, job.ld_c, 1.f);
   for (int e = tid; e < D; e += kThreads) {
     kmv[e] = (NORM || TOKENS) && job.km ? job.km[(int64_t)nh * D + e] : 0.f;
-    addv[e] = job.addvec ? job.addvec[(int64_t)nh * D + e] : 0.f;
+    addv[e] = job.addvec ? job.addvec[(int64_t)nh * D + e] * job.add_scale : 0.f;
   }
   __syncthreads();
   const bool with_den = (NORM || TOKENS) && job.km != nullptr;
@@ -442,6 +443,7 @@ static Rows32Job convert(const mfma::RowsJob& j) {
   r.ld_c = j.ld_c;
   r.km = j.km;
   r.addvec = j.addvec;
+  r.add_scale = j.add_scale;
   r.out = (float*)j.out;
   r.tokscal = nullptr;
   r.total_rows = 0;
@@ -468,6 +470,7 @@ int bwd_tokens(const Prob& p, const float* q, const float* dout, const float* S,
   j.ld_c = D;
   j.km = (p.flags & kNormalize) ? km : nullptr;
   j.addvec = nullptr;
+  j.add_scale = 1.f;
   j.out = dq;
   j.tokscal = tokscal;
   j.total_rows = total_rows;

@@ -6,12 +6,36 @@
 // forward :  state partials -> fixed-order reduce (S, km) -> output rows
 // backward:  S^T -> pass A (dq, partial dS/dkm) -> reduce (s dS, its transpose, dkm/L)
 //            -> pass B (dk, dv)
+//
+// A dense problem may have fewer (or more) keys than queries (Prob::Lk): the state kernel and
+// pass B then walk the Lk key / value tokens, the output kernel and pass A the L query tokens,
+// each with a problem of its own length.  The reductions stay separate kernels (or direct
+// stores) in that case, and dkm, which pass A leaves divided by the number of queries, is
+// rescaled to dkm / Lk where pass B adds it.  MFMA path only.
 #include <stdlib.h>
 
 #include "fbla_kernels.h"
 
 namespace fbla {
 namespace plan {
+
+// true when keys and queries differ in number
+static bool cross(const Prob& p) { return !p.cu && p.Lk > 0 && p.Lk != p.L; }
+// the problem as the kernels of one side see it
+static Prob query_side(const Prob& p) {
+  Prob s = p;
+  s.Lk = 0;
+  return s;
+}
+static Prob key_side(const Prob& p) {
+  Prob s = p;
+  if (cross(p)) {
+    s.L = p.Lk;
+    s.T = (int64_t)p.N * p.Lk;
+  }
+  s.Lk = 0;
+  return s;
+}
 
 static size_t state_bytes(const Prob& p) {
   return align_up((size_t)p.N * p.H * p.DK * p.DV * sizeof(float), 256);
@@ -51,15 +75,35 @@ static bool fold_reduce(const Prob& p, int reduce_nchunks, int DR, int DC) {
   return extra <= limit;
 }
 
-size_t fwd_workspace_bytes(const Prob& p, int dtype) { return partial_bytes(p, fwd_chunk(p, dtype)); }
+size_t fwd_workspace_bytes(const Prob& pc, int dtype) {
+  const Prob p = key_side(pc);
+  return partial_bytes(p, fwd_chunk(p, dtype));
+}
 
 // partials | S^T | s*dS | (s*dS)^T | dkm/L | per-row scalars
-size_t bwd_workspace_bytes(const Prob& p, int dtype) {
+size_t bwd_workspace_bytes(const Prob& pc, int dtype) {
+  const Prob p = query_side(pc);
   return partial_bytes(p, bwd_chunk(p, dtype)) + 3 * state_bytes(p) + vec_bytes(p) +
          tokscal_bytes(p, dtype);
 }
 
-int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
+static int check_cross(const Prob& p, int dtype) {
+  if (!cross(p)) return kOk;
+  if ((p.flags & kDecoupled) || !mfma::supported(key_side(p), dtype)) {
+    set_error("different numbers of queries and keys need the matrix-core kernels (16-bit inputs with "
+              "head dims that are multiples of 8, or fp32 inputs with 64 x 64 heads) and are not "
+              "available for the decoupled operator");
+    return kErrUnsupported;
+  }
+  return kOk;
+}
+
+int forward(const Prob& pc, int dtype, const FwdArgs& a, hipStream_t st) {
+  int rc_cross = check_cross(pc, dtype);
+  if (rc_cross != kOk) return rc_cross;
+  const bool is_cross = cross(pc);
+  const Prob p = key_side(pc);    // state kernel, reduce
+  const Prob pq = query_side(pc);  // output kernel
   const bool dec = p.flags & kDecoupled;
   const bool normalize = p.flags & kNormalize;
   const void* qn = dec ? a.q_rope : a.q;
@@ -78,7 +122,8 @@ int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
     else
       generic::state_partial(p, dtype, kn, a.v, a.k, partial, chunk, nchunks, st);
   }
-  const bool fold = fast && !direct && dtype != kF32 && !mfma::pair_mode(p, dtype) && fold_reduce(p, nchunks, p.DK, p.DV);
+  const bool fold = fast && !direct && !is_cross && dtype != kF32 && !mfma::pair_mode(p, dtype) &&
+                    fold_reduce(p, nchunks, p.DK, p.DV);
   if (!fold && !direct && (phases & kPhaseFwdReduce))
     generic::state_reduce(p, partial, chunk, nchunks, a.s, nullptr, a.km, st);
   if (phases & kPhaseFwdOutput) {
@@ -91,7 +136,7 @@ int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
         job.mat_out = a.s;
         job.vec_out = a.km;
       }
-      int rc = mfma::rows(p, dtype, job, p.DK, p.DV, st);
+      int rc = mfma::rows(pq, dtype, job, p.DK, p.DV, st);
       if (rc != kOk) return rc;
     } else {
       generic::output(p, dtype, qn, a.q, a.s, a.km, a.o, st);
@@ -100,7 +145,12 @@ int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
   return kOk;
 }
 
-int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
+int backward(const Prob& pc, int dtype, const BwdArgs& a, hipStream_t st) {
+  int rc_cross = check_cross(pc, dtype);
+  if (rc_cross != kOk) return rc_cross;
+  const bool is_cross = cross(pc);
+  const Prob p = query_side(pc);  // pass A, reduce
+  const Prob pk = key_side(pc);   // pass B
   const bool dec = p.flags & kDecoupled;
   const bool normalize = p.flags & kNormalize;
   const void* qn = dec ? a.q_rope : a.q;
@@ -147,7 +197,8 @@ int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
       generic::bwd_a(p, dtype, qn, a.q, a.dout, a.s, St, a.km, dqn, dqd, partial, chunk, nchunks, st);
     }
   }
-  const bool fold = fast && !direct && dtype != kF32 && !mfma::pair_mode(p, dtype) && fold_reduce(p, nchunks, p.DV, p.DK);
+  const bool fold = fast && !direct && !is_cross && dtype != kF32 && !mfma::pair_mode(p, dtype) &&
+                    fold_reduce(p, nchunks, p.DV, p.DK);
   if (!fold && !direct && (phases & kPhaseBwdReduce))
     generic::state_reduce(p, partial, chunk, nchunks, dS, fast ? nullptr : dSt, dkm, st);
   if (phases & kPhaseBwdB) {
@@ -164,12 +215,14 @@ int backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
         jk.vec_is_add = !dec && normalize;
         jk.vec_out = dec ? dkm : nullptr;
       }
+      // dkm arrives divided by the number of queries; the formula wants dkm / (number of keys)
+      if (is_cross) jk.add_scale = (float)p.L / (float)pk.L;
       int rc;
       if (p.DK == p.DV) {  // same shape: one launch
-        rc = mfma::rows2(p, dtype, jk, jv, p.DV, p.DK, st);
+        rc = mfma::rows2(pk, dtype, jk, jv, p.DV, p.DK, st);
       } else {
-        rc = mfma::rows(p, dtype, jk, p.DV, p.DK, st);
-        if (rc == kOk) rc = mfma::rows(p, dtype, jv, p.DK, p.DV, st);
+        rc = mfma::rows(pk, dtype, jk, p.DV, p.DK, st);
+        if (rc == kOk) rc = mfma::rows(pk, dtype, jv, p.DK, p.DV, st);
       }
       if (rc != kOk) return rc;
       if (dec) generic::broadcast_rows(p, dtype, dkm, dkd, st);

@@ -29,6 +29,9 @@ _SIGNATURES = {
     "fbla_la_workspace_bytes": (_sz, [_i32, _i64, _i64, _i64, _i32, _i32, _i32, _i32]),
     "fbla_la_fwd": (_i32, [_vp] * 9 + [_sz, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_la_bwd": (_i32, [_vp] * 14 + [_sz, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
+    "fbla_la_cross_workspace_bytes": (_sz, [_i32, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32]),
+    "fbla_la_cross_fwd": (_i32, [_vp] * 7 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
+    "fbla_la_cross_bwd": (_i32, [_vp] * 10 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_varlen_workspace_bytes": (_sz, [_i32, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32]),
     "fbla_varlen_fwd": (_i32, [_vp] * 8 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_varlen_bwd": (_i32, [_vp] * 11 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
@@ -100,16 +103,25 @@ def _require_gpu(*tensors):
 
 
 def la_fwd(q, k, v, q_rope, k_rope, scale, eps, flags):
-    """Dense forward: returns (o, s, km).  Tensors must be contiguous [B,H,L,D]."""
+    """Dense forward: returns (o, s, km).  Tensors must be contiguous [B,H,L,D]; k and v may have
+    another number of tokens than q (not with the decoupled operator)."""
     _require_gpu(q, k, v, q_rope, k_rope)
     L = lib()
     B, H, T, DK = q.shape
-    DV = v.shape[-1]
+    Tk, DV = k.shape[-2], v.shape[-1]
     code = dtype_code(q)
     dev = q.device
-    o = torch.empty_like(v)
+    o = torch.empty(B, H, T, DV, dtype=v.dtype, device=dev)
     s = torch.empty(B, H, DK, DV, dtype=torch.float32, device=dev)
     km = torch.empty(B, H, DK, dtype=torch.float32, device=dev)
+    if Tk != T:
+        with torch.cuda.device(dev):
+            ws = _workspace(L.fbla_la_cross_workspace_bytes(0, B, H, T, Tk, DK, DV, code, flags), dev)
+            rc = L.fbla_la_cross_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(s), _ptr(km), _ptr(ws),
+                                     ws.numel(), B, H, T, Tk, DK, DV, code, flags, float(scale), float(eps),
+                                     _stream(dev))
+        _check(rc, "fbla_la_cross_fwd")
+        return o, s, km
     with torch.cuda.device(dev):
         ws = _workspace(L.fbla_la_workspace_bytes(0, B, H, T, DK, DV, code, flags), dev)
         rc = L.fbla_la_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(q_rope), _ptr(k_rope), _ptr(o), _ptr(s),
@@ -124,12 +136,20 @@ def la_bwd(q, k, v, q_rope, k_rope, do, s, km, scale, eps, flags):
     _require_gpu(q, k, v, do)
     L = lib()
     B, H, T, DK = q.shape
-    DV = v.shape[-1]
+    Tk, DV = k.shape[-2], v.shape[-1]
     code = dtype_code(q)
     dev = q.device
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dqr = torch.empty_like(q_rope) if flags & DECOUPLED else None
     dkr = torch.empty_like(k_rope) if flags & DECOUPLED else None
+    if Tk != T:
+        with torch.cuda.device(dev):
+            ws = _workspace(L.fbla_la_cross_workspace_bytes(1, B, H, T, Tk, DK, DV, code, flags), dev)
+            rc = L.fbla_la_cross_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(s), _ptr(km), _ptr(dq),
+                                     _ptr(dk), _ptr(dv), _ptr(ws), ws.numel(), B, H, T, Tk, DK, DV, code,
+                                     flags, float(scale), float(eps), _stream(dev))
+        _check(rc, "fbla_la_cross_bwd")
+        return dq, dk, dv, None, None
     with torch.cuda.device(dev):
         ws = _workspace(L.fbla_la_workspace_bytes(1, B, H, T, DK, DV, code, flags), dev)
         rc = L.fbla_la_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(q_rope), _ptr(k_rope), _ptr(do), _ptr(s),

@@ -9,11 +9,17 @@ def check_dense(name, q, k, v, extra=()):
     for t in tensors:
         if not isinstance(t, torch.Tensor) or t.ndim != 4:
             raise ValueError(f"{name}: tensors must have shape (B, H, L, D)")
-    if q.shape != k.shape or any(t.shape != q.shape for t in extra):
-        raise ValueError(f"{name}: q and k (and their rope versions) must have identical shapes, "
-                         f"got {[tuple(t.shape) for t in (q, k) + tuple(extra)]}")
-    if q.shape[:3] != v.shape[:3]:
-        raise ValueError(f"{name}: q, k, and v must have matching batch, head and token dimensions")
+    if extra:
+        if q.shape != k.shape or any(t.shape != q.shape for t in extra):
+            raise ValueError(f"{name}: q and k (and their rope versions) must have identical shapes, "
+                             f"got {[tuple(t.shape) for t in (q, k) + tuple(extra)]}")
+    elif q.shape[:2] != k.shape[:2] or q.shape[-1] != k.shape[-1]:
+        # k and v may be shorter or longer than q (the PVT-style blocks reduce the keys spatially;
+        # the reference reads one length from q, linear_attn/fused.py:355, and runs out of bounds)
+        raise ValueError(f"{name}: q and k must agree in batch, head and feature dimensions, "
+                         f"got {tuple(q.shape)} and {tuple(k.shape)}")
+    if k.shape[:3] != v.shape[:3]:
+        raise ValueError(f"{name}: k and v must have matching batch, head and token dimensions")
     if any(t.device != q.device for t in tensors):
         raise ValueError(f"{name}: all tensors must be on the same device")
     if any(t.dtype != q.dtype for t in tensors):

@@ -94,6 +94,24 @@ int fbla_la_bwd(const void* q, const void* k, const void* v, const void* q_rope,
                 size_t workspace_bytes, int64_t B, int64_t H, int64_t L, int DK, int DV, int dtype,
                 int flags, float scale, float eps, void* stream);
 
+/* Dense problems with Lk key / value tokens and Lq query tokens per (batch, head), Lk != Lq:
+ * q, dq: [B,H,Lq,DK]; k, dk: [B,H,Lk,DK]; v, dv: [B,H,Lk,DV]; o, dout: [B,H,Lq,DV]; km is the mean
+ * over the Lk keys.  The reference has no counterpart: its dense kernels take one length from q
+ * (linear_attn/fused.py:355) and read k, v out of bounds when the PVT-style blocks
+ * (layers/focused_la.py:55,73-75, layers/polaformer.py) shorten the keys with sr_ratio > 1.
+ * Flags as for fbla_la_fwd without FBLA_DECOUPLED; matrix-core shapes only (16-bit inputs with
+ * head dims that are multiples of 8, fp32 inputs with 64 x 64 heads), else FBLA_ERR_UNSUPPORTED. */
+size_t fbla_la_cross_workspace_bytes(int pass, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int DK,
+                                     int DV, int dtype, int flags);
+int fbla_la_cross_fwd(const void* q, const void* k, const void* v, void* o, float* s, float* km,
+                      void* workspace, size_t workspace_bytes, int64_t B, int64_t H, int64_t Lq,
+                      int64_t Lk, int DK, int DV, int dtype, int flags, float scale, float eps,
+                      void* stream);
+int fbla_la_cross_bwd(const void* q, const void* k, const void* v, const void* dout, const float* s,
+                      const float* km, void* dq, void* dk, void* dv, void* workspace,
+                      size_t workspace_bytes, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int DK,
+                      int DV, int dtype, int flags, float scale, float eps, void* stream);
+
 /* Workspace for the packed (variable-length) entry points. */
 size_t fbla_varlen_workspace_bytes(int pass, int64_t total_tokens, int64_t N, int64_t H,
                                    int64_t max_seqlen, int DK, int DV, int dtype, int flags);

@@ -1,0 +1,80 @@
+"""Keys and values with another number of tokens than the queries (dense operators): the
+PVT-style blocks reduce k, v spatially (`sr_ratio > 1`), the reference's kernels take one
+length from q and run out of bounds there (linear_attn/fused.py:355).  Forward and backward
+against the float64 oracle; the error paths of the shapes without matrix-core kernels."""
+import pytest
+import torch
+
+from helpers import make_qkv, np64, parity_errors
+from oracle import closed_form as cf
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = [(256, 64), (64, 256), (1000, 37), (5, 300), (3000, 750), (1, 8), (9000, 2250)]
+
+
+def _check(variant, B, H, lq, lk, DK, DV, dtype, seed):
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    from flash_bla.ops.simple_la.fused import simple_la
+    q, _, _, do = make_qkv((B, H, lq, DK), (B, H, lq, DV), dtype, seed)
+    _, k, v, _ = make_qkv((B, H, lk, DK), (B, H, lk, DV), dtype, seed + 1)
+    normalize = variant == "linear"
+    scale = 1.0 / lk if normalize else DK ** -0.5
+    ref = cf.dense_backward(np64(q), np64(k), np64(v), np64(do), scale, 1e-6, normalize)
+    leaves = [t.cuda().requires_grad_() for t in (q, k, v)]
+    o = (linear_attention if normalize else simple_la)(*leaves)
+    assert o.shape == (B, H, lq, DV) and o.dtype == dtype
+    o.backward(do.cuda())
+    errs = {"o": parity_errors(o, ref["o"], dtype)}
+    for name, t in zip(("dq", "dk", "dv"), leaves):
+        assert t.grad.shape == t.shape
+        errs[name] = parity_errors(t.grad, ref[name], dtype, ref.get(name + "_mag"))
+    bad = {n: e for n, e in errs.items() if not e[2]}
+    assert not bad, f"{variant} {dtype} B{B} H{H} Lq{lq} Lk{lk} DK{DK} DV{DV}: {errs}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dims", [(64, 64), (32, 32), (128, 128), (128, 32), (64, 128), (48, 72)])
+def test_linear_attention_16bit(dims, dtype):
+    for i, (lq, lk) in enumerate(LENGTHS):
+        _check("linear", 2, 3, lq, lk, dims[0], dims[1], dtype, 50 * i + dims[0])
+
+
+@pytest.mark.parametrize("dims", [(64, 64), (32, 32), (128, 128), (64, 16)])
+def test_simple_la_16bit(dims):
+    for i, (lq, lk) in enumerate(LENGTHS[:5]):
+        _check("simple", 1, 2, lq, lk, dims[0], dims[1], torch.float16, 70 * i + dims[1])
+
+
+def test_fp32_64_by_64():
+    for i, (lq, lk) in enumerate(LENGTHS):
+        _check("linear", 2, 2, lq, lk, 64, 64, torch.float32, 90 + i)
+    _check("simple", 1, 2, 300, 77, 64, 64, torch.float32, 99)
+
+
+def test_default_scale_is_one_over_the_number_of_keys():
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    q, _, _, _ = make_qkv((1, 2, 40, 64), (1, 2, 40, 64), torch.float16, 1)
+    _, k, v, _ = make_qkv((1, 2, 10, 64), (1, 2, 10, 64), torch.float16, 2)
+    a = linear_attention(q.cuda(), k.cuda(), v.cuda())
+    b = linear_attention(q.cuda(), k.cuda(), v.cuda(), scale=0.1)
+    assert torch.equal(a, b)
+
+
+def test_shapes_without_matrix_core_kernels_are_refused():
+    from flash_bla.ops.linear_attn.decoupled import decoupled_la
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    q = torch.rand(1, 2, 40, 20, device="cuda", dtype=torch.float16)   # 20 is not a multiple of 8
+    k = torch.rand(1, 2, 10, 20, device="cuda", dtype=torch.float16)
+    with pytest.raises(ValueError, match="matrix-core"):
+        linear_attention(q, k, k)
+    q32 = torch.rand(1, 2, 40, 32, device="cuda")
+    k32 = torch.rand(1, 2, 10, 32, device="cuda")
+    with pytest.raises(ValueError, match="matrix-core"):
+        linear_attention(q32, k32, k32)
+    # the library is still usable
+    assert linear_attention(q32, q32, q32).shape == q32.shape
+    q64 = torch.rand(1, 2, 40, 64, device="cuda", dtype=torch.float16)
+    k64 = torch.rand(1, 2, 10, 64, device="cuda", dtype=torch.float16)
+    with pytest.raises(ValueError, match="identical shapes"):
+        decoupled_la(q64, k64, q64, k64, k64)

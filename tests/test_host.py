@@ -82,8 +82,10 @@ def test_dense_ops_refuse_cpu_tensors():
     q = torch.rand(1, 2, 8, 4)
     with pytest.raises(ValueError, match="GPU"):
         linear_attention(q, q, q)
-    with pytest.raises(ValueError, match="identical shapes"):
+    with pytest.raises(ValueError, match="must agree"):
         linear_attention(q, q[..., :2], q)
+    with pytest.raises(ValueError, match="k and v"):
+        linear_attention(q, q[:, :, :4], q)   # shorter keys are allowed, but v must follow k
 
 
 @pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "*.npz"))), ids=os.path.basename)

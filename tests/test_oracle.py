@@ -116,6 +116,27 @@ def test_closed_form_backward_matches_autograd(variant):
         np.testing.assert_allclose(g["dk_rope"], np64(krl.grad), rtol=1e-9, atol=1e-11)
 
 
+@pytest.mark.parametrize("normalize", [True, False])
+def test_fewer_or_more_keys_than_queries(normalize):
+    """k, v with another number of tokens than q (the PVT-style blocks shorten the keys): the
+    closed form against the O(Lq Lk) double sum written out, and its gradients against autograd."""
+    for lq, lk in ((23, 9), (5, 31)):
+        q, _, _, do, _, _ = _dense_inputs(2, 2, lq, 8, 6, n_extra=2)
+        _, k, v, _, _, _ = _dense_inputs(2, 2, lk, 8, 6, n_extra=2)
+        scale, eps = 0.07, 1e-6
+        g = cf.dense_backward(np64(q), np64(k), np64(v), np64(do), scale, eps, normalize)
+        w = np.einsum("bhik,bhjk->bhij", np64(q), np64(k))          # q_i . k_j
+        num = scale * np.einsum("bhij,bhjv->bhiv", w, np64(v))
+        ref = num / (w.mean(-1, keepdims=True) + eps) if normalize else num
+        np.testing.assert_allclose(g["o"], ref, rtol=1e-11, atol=1e-13)
+        ql, kl, vl = (t.clone().requires_grad_() for t in (q, k, v))
+        o = tr.naive_linear_attn(ql, kl, vl, scale) if normalize else tr.naive_simple_la(ql, kl, vl, scale)
+        o.backward(do)
+        np.testing.assert_allclose(g["o"], np64(o), rtol=1e-11, atol=1e-13)
+        for name, leaf in (("dq", ql), ("dk", kl), ("dv", vl)):
+            np.testing.assert_allclose(g[name], np64(leaf.grad), rtol=1e-9, atol=1e-11)
+
+
 def test_gradcheck_torch_ref():
     q, k, v, _ = _dense_inputs(1, 1, 7, 3, 2)
     args = [t.clone().requires_grad_() for t in (q, k, v)]
