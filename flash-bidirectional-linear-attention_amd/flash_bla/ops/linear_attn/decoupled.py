@@ -53,6 +53,14 @@ def decoupled_la(
         scale: defaults to `1 / L` (decoupled.py:539-540)
         eps: constant added to the denominator.
     """
+    # RoPE modules hand back fp32 features next to 16-bit q, k (layers/mlla.py:32-36 of the
+    # reference): they are rounded to the type of q here (the kernels read one element type);
+    # the cast is differentiable, so their gradients come back in fp32.
+    if isinstance(q, torch.Tensor) and isinstance(q_rope, torch.Tensor) and isinstance(k_rope, torch.Tensor):
+        if q_rope.dtype != q.dtype and q_rope.is_floating_point():
+            q_rope = q_rope.to(q.dtype)
+        if k_rope.dtype != q.dtype and k_rope.is_floating_point():
+            k_rope = k_rope.to(q.dtype)
     check_dense("decoupled_la", q, k, v, extra=(q_rope, k_rope))
     if scale is None:
         scale = k.shape[-2] ** -1.0

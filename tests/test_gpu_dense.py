@@ -158,3 +158,22 @@ def test_matrix_core_paths_at_awkward_lengths(variant, L, dtype):
     """64 x 64 heads run on the MFMA kernels for all three dtypes; their token loops work in
     tiles of 16 and 32 tokens with a moved-back last tile and a checked path below one tile."""
     _check_dense(variant, 1, 3, L, 64, 64, dtype, seed=L)
+
+
+def test_decoupled_takes_fp32_rotary_features_next_to_16bit_inputs():
+    """RoPE modules return fp32 (layers/mlla.py:32-36 of the reference): the rotary tensors are
+    rounded to the type of q, their gradients come back in fp32."""
+    from flash_bla.ops.linear_attn.decoupled import decoupled_la
+    q, k, v, do, qr, kr = make_qkv((2, 2, 300, 32), (2, 2, 300, 32), torch.float32, 5, n_extra=2)
+    h = lambda t: t.half()
+    ref = cf.dense_backward(np64(h(q)), np64(h(k)), np64(h(v)), np64(h(do)), 1.0 / 300, 1e-6, True,
+                            q_rope=np64(h(qr)), k_rope=np64(h(kr)))
+    leaves = [h(q).cuda().requires_grad_(), h(k).cuda().requires_grad_(), qr.cuda().requires_grad_(),
+              kr.cuda().requires_grad_(), h(v).cuda().requires_grad_()]
+    o = decoupled_la(*leaves)
+    assert o.dtype == torch.float16
+    o.backward(h(do).cuda())
+    assert leaves[2].grad.dtype == torch.float32 and leaves[3].grad.dtype == torch.float32
+    assert_parity(o, ref["o"], torch.float16, "o")
+    for name, t in zip(("dq", "dk", "dq_rope", "dk_rope", "dv"), leaves):
+        assert_parity(t.grad, ref[name], torch.float16, name, ref.get(name + "_mag"))
