@@ -451,11 +451,17 @@ def layer_config(dev, flush):
             t_fast = do_bench(lambda: layer(x, mode="triton"), flush)
             t_torch = do_bench(lambda: layer(x, mode="torch"), flush)
             t_op = do_bench(lambda: linear_attention(q, k, v, eps=1e-4), flush)
+            from flash_bla.utils import CapturedForward
+            graphed = CapturedForward(layer, x, mode="triton")
+            t_graph = do_bench(lambda: graphed(x), flush)
+            graph_equal = bool(torch.equal(graphed(x), layer(x, mode="triton")))
             err = (layer(x, mode="triton").float() - layer(x, mode="torch").float()).abs().max().item()
             ref = layer(x, mode="torch").float().abs().max().item()
         nb = 4 * q.numel() * 2
         print(json.dumps({"config": f"C4 LinFusion layer fwd B2-L{L}-C{C}-{heads}x64 fp16",
-                          "layer_ms": round(t_fast[0], 5), "layer_torch_mode_ms": round(t_torch[0], 5),
+                          "layer_ms": round(t_fast[0], 5), "layer_hip_graph_ms": round(t_graph[0], 5),
+                          "hip_graph_equals_eager": graph_equal,
+                          "layer_torch_mode_ms": round(t_torch[0], 5),
                           "op_ms": round(t_op[0], 5), "op_gbps": round(nb / t_op[0] / 1e6, 1),
                           "modes_max_abs_diff_over_max": round(err / ref, 6)}), file=sys.stderr, flush=True)
 

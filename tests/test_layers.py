@@ -88,3 +88,21 @@ def test_linfusion_sdxl_shapes_fp16(tokens, channels, heads):
         ref = layer.float()(x.float(), mode='torch')
     assert_close("o", ref, out.float(), 0.06)
     assert (out.float() - ref).abs().max() <= 5e-3 * ref.abs().max()
+
+
+@pytest.mark.gpu
+def test_captured_forward_replays_the_block_bit_for_bit():
+    """The LinFusion block's inference forward recorded into a HIP graph: replays on new inputs,
+    with eager work in between, equal the eager block bit for bit."""
+    from flash_bla.utils import CapturedForward
+    torch.manual_seed(3)
+    layer = GeneralizedLinearAttention(640, heads=10, dim_head=64).to("cuda", torch.float16).eval()
+    x = torch.randn(2, 1024, 640, device="cuda", dtype=torch.float16)
+    graphed = CapturedForward(layer, x, mode="triton")
+    for i in range(4):
+        xi = torch.randn(2, 1024, 640, device="cuda", dtype=torch.float16)
+        with torch.no_grad():
+            eager = layer(xi, mode="triton")
+            torch.cuda.synchronize()
+            got = graphed(xi).clone()
+        assert torch.equal(got, eager), f"replay {i}"
