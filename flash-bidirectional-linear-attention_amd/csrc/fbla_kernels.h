@@ -119,13 +119,13 @@ int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* 
 }  // namespace mfma
 
 namespace mfma32 {
-// fp32 inputs on v_mfma_f32_32x32x2_f32: 64 x 64 heads, not decoupled.  Called through the
-// mfma:: entry points, which dispatch on the dtype.
+// fp32 inputs on v_mfma_f32_32x32x2_f32: head dims that are multiples of 4 up to 64, not
+// decoupled.  Called through the mfma:: entry points, which dispatch on the dtype.
 bool supported(const Prob& p);
 void state(const Prob& p, const float* kn, const float* v, const float* kd, float* partial,
            const float* tokscal, int64_t total_rows, int chunk, int nchunks, hipStream_t st, float* fin_mat,
            float* fin_vec);
-int rows(const Prob& p, const mfma::RowsJob& job, const mfma::RowsJob* job2, hipStream_t st);
+int rows(const Prob& p, const mfma::RowsJob& job, const mfma::RowsJob* job2, int dr, int dc, hipStream_t st);
 int bwd_tokens(const Prob& p, const float* q, const float* dout, const float* S, const float* km, float* dq,
                float* tokscal, int64_t total_rows, hipStream_t st);
 }  // namespace mfma32

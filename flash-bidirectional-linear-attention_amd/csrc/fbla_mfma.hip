@@ -1780,7 +1780,7 @@ void scaled_state(const Prob& p, int dtype, const void* qn, const void* dout, co
 }
 
 int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {
-  if (dtype == kF32) return mfma32::rows(p, job, nullptr, st);
+  if (dtype == kF32) return mfma32::rows(p, job, nullptr, DR, DC, st);
   if (dtype == kF16) return run_rows<_Float16>(p, job, nullptr, DR, DC, st);
   return run_rows<__bf16>(p, job, nullptr, DR, DC, st);
 }
@@ -1788,7 +1788,7 @@ int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream
 // two jobs of the same shape and normalisation mode in one launch
 int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, int DR, int DC,
           hipStream_t st) {
-  if (dtype == kF32) return mfma32::rows(p, job0, &job1, st);
+  if (dtype == kF32) return mfma32::rows(p, job0, &job1, DR, DC, st);
   if (dtype == kF16) return run_rows<_Float16>(p, job0, &job1, DR, DC, st);
   return run_rows<__bf16>(p, job0, &job1, DR, DC, st);
 }

@@ -1,6 +1,8 @@
-// MFMA kernels for fp32 inputs, 64 x 64 heads (dense and packed layouts, with or
-// without the denominator; the decoupled operator and other head sizes stay on the
-// shape-generic kernels).  v_mfma_f32_32x32x2_f32 computes in fp32 throughout, so
+// MFMA kernels for fp32 inputs, heads tiled 64 x 64: head dims that are multiples of 4 (16-byte
+// row pieces) up to 64, smaller ones with zero padding (PAD variants: true row lengths in memory,
+// missing features read as zero, outputs and state in their true shapes).  Dense and packed
+// layouts, with or without the denominator; the decoupled operator and larger heads stay on
+// the shape-generic kernels.  v_mfma_f32_32x32x2_f32 computes in fp32 throughout, so
 // there is no operand splitting here: A lane l holds A[m = l%32][k = l/32], B lane l
 // holds B[k = l/32][n = l%32], C register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32].
 // One instruction covers two values of the contraction index and takes 64 cycles:
@@ -48,13 +50,14 @@ __device__ __forceinline__ f32x16 mma(float a, float b, f32x16 c) {
 // Lane l = (f = l%32, kb = l/32).  A 16-token tile is eight k-steps; in k-step s the lane
 // holds feature 32a + f of token 2s + kb for the key blocks a = 0, 1 and the value blocks
 // b = 0, 1.  Four waves take interleaved tiles; two register buffers alternate.
-template <bool SPLIT_KD, bool SCALED>
+template <bool SPLIT_KD, bool SCALED, bool PAD>
 __global__ __launch_bounds__(kThreads, 2) void state32_kernel(
     Prob p, const float* __restrict__ kn, const float* __restrict__ v, const float* __restrict__ kd,
     float* __restrict__ partial, const float* __restrict__ tokscal, int64_t total_rows, float* fin_mat,
     float* fin_vec, int chunk, int nchunks) {
   __shared__ float red[64 * 66];
   __shared__ int lpt_lens[kLptMax + 1];
+  const int dk = PAD ? p.DK : D, dv = PAD ? p.DV : D;  // row lengths in memory
   const int wg_nh = blockIdx.x / nchunks, c = blockIdx.x - wg_nh * nchunks;
   const int h = wg_nh % p.H;
   const int n = lpt_sequence(p, wg_nh / p.H, lpt_lens);
@@ -65,9 +68,9 @@ __global__ __launch_bounds__(kThreads, 2) void state32_kernel(
   const int t_begin = c * chunk;
   if (t_begin >= len) {
     if (fin_mat && c == 0) {  // empty sequence: its state is zero
-      for (int e = threadIdx.x; e < D * D; e += kThreads) fin_mat[(int64_t)nh * D * D + e] = 0.f;
+      for (int e = threadIdx.x; e < dk * dv; e += kThreads) fin_mat[(int64_t)nh * dk * dv + e] = 0.f;
       if (fin_vec)
-        for (int e = threadIdx.x; e < D; e += kThreads) fin_vec[(int64_t)nh * D + e] = 0.f;
+        for (int e = threadIdx.x; e < dk; e += kThreads) fin_vec[(int64_t)nh * dk + e] = 0.f;
     }
     return;
   }
@@ -76,6 +79,17 @@ __global__ __launch_bounds__(kThreads, 2) void state32_kernel(
 
   const int g = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int f = lane & 31, kb = lane >> 5;
+  // this lane's two key and two value features; one past the head dim is read from column 0
+  // and replaced by zero
+  bool kok[2], vok[2];
+  int kcol[2], vcol[2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    kok[a] = !PAD || f + 32 * a < dk;
+    vok[a] = !PAD || f + 32 * a < dv;
+    kcol[a] = kok[a] ? f + 32 * a : 0;
+    vcol[a] = vok[a] ? f + 32 * a : 0;
+  }
 
   f32x16 acc[2][2];
 #pragma unroll
@@ -91,24 +105,27 @@ __global__ __launch_bounds__(kThreads, 2) void state32_kernel(
     float d[SPLIT_KD ? 8 : 1][2];
     float rz[SCALED ? 8 : 1], dz[SCALED ? 8 : 1];
   };
-  const uint32_t step = (uint32_t)(rstride * D);
-  const uint32_t voff = (uint32_t)kb * step + (uint32_t)f;
+  const uint32_t kstep = (uint32_t)(rstride * dk), vstep = (uint32_t)(rstride * dv);
   // A tile that would cross the end of the chunk is moved back so that it ends there; the
   // rows it shares with the previous tile are zeroed before use.
   auto fetch = [&](Buf& b, int tok) {
     const int tb = min(tok, t_end - 16);
     const int64_t row = row0 + (int64_t)tb * rstride;
-    const float* kp = kn + row * D;
-    const float* vp = v + row * D;
-    const float* dp = kd + row * D;
+    const float* kp = kn + row * dk;
+    const float* vp = v + row * dv;
+    const float* dp = kd + row * dk;
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-      const size_t ro = (size_t)(2 * s) * step;
+      const size_t kro = (size_t)(2 * s + kb) * kstep, vro = (size_t)(2 * s + kb) * vstep;
 #pragma unroll
       for (int a = 0; a < 2; ++a) {
-        b.k[s][a] = kp[ro + voff + 32 * a];
-        b.v[s][a] = vp[ro + voff + 32 * a];
-        if constexpr (SPLIT_KD) b.d[s][a] = dp[ro + voff + 32 * a];
+        const float kx = kp[kro + kcol[a]], vx = vp[vro + vcol[a]];
+        b.k[s][a] = kok[a] ? kx : 0.f;
+        b.v[s][a] = vok[a] ? vx : 0.f;
+        if constexpr (SPLIT_KD) {
+          const float dx = dp[kro + kcol[a]];
+          b.d[s][a] = kok[a] ? dx : 0.f;
+        }
       }
       if constexpr (SCALED) {
         const int64_t r = row + (int64_t)(2 * s + kb) * rstride;
@@ -125,9 +142,9 @@ __global__ __launch_bounds__(kThreads, 2) void state32_kernel(
       const int64_t r = row0 + (int64_t)t * rstride;
 #pragma unroll
       for (int a = 0; a < 2; ++a) {
-        b.k[s][a] = ok ? kn[r * D + 32 * a + f] : 0.f;
-        b.v[s][a] = ok ? v[r * D + 32 * a + f] : 0.f;
-        if constexpr (SPLIT_KD) b.d[s][a] = ok ? kd[r * D + 32 * a + f] : 0.f;
+        b.k[s][a] = ok && kok[a] ? kn[r * dk + kcol[a]] : 0.f;
+        b.v[s][a] = ok && vok[a] ? v[r * dv + vcol[a]] : 0.f;
+        if constexpr (SPLIT_KD) b.d[s][a] = ok && kok[a] ? kd[r * dk + kcol[a]] : 0.f;
       }
       if constexpr (SCALED) {
         b.rz[s] = ok ? tokscal[r] : 0.f;
@@ -187,12 +204,12 @@ __global__ __launch_bounds__(kThreads, 2) void state32_kernel(
     }
   }
 
-  float* mat = fin_mat ? fin_mat + (int64_t)nh * D * D
-                       : partial + ((int64_t)nh * nchunks + c) * (D * D + D);
-  float* vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * D : nullptr) : mat + D * D;
+  float* mat = fin_mat ? fin_mat + (int64_t)nh * dk * dv
+                       : partial + ((int64_t)nh * nchunks + c) * (dk * dv + dk);
+  float* vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : mat + dk * dv;
   const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
   const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
-  reduce_store_block<4, false>(acc, ks, red, mat, D, vec, mscale, vscale, g, lane);
+  reduce_store_block<4, false>(acc, ks, red, mat, dv, vec, mscale, vscale, g, lane, dk, dv);
 }
 
 // ===========================================================================
@@ -207,15 +224,17 @@ __global__ __launch_bounds__(kThreads, 2) void state32_kernel(
 //
 // Operand fragments in LDS: frag[((b*8 + s/4)*64 + lane)*4 + s%4] = M[r(s,kb)][sigma(b,m)],
 // lane = m + 32*kb.  M is read as mat[r*ld_r + c*ld_c] times mscale.
+// The matrix in memory is dr x dc; rows and columns past that are zero in the operand.
 __device__ __forceinline__ void build_operand32(float* frag, const float* __restrict__ mat, int ld_r,
-                                                int ld_c, float mscale) {
+                                                int ld_c, float mscale, int dr, int dc) {
   for (int e = threadIdx.x; e < D * D; e += blockDim.x) {
     // walk the matrix along its contiguous direction
     const int r = ld_c == 1 ? e / D : e % D, cc = ld_c == 1 ? e % D : e / D;
     const int s = 2 * (r >> 2) + (r & 1), kb = (r >> 1) & 1;
     const int kbp = cc >> 5, b = (cc >> 4) & 1, gq = (cc >> 2) & 3, j = cc & 3;
     const int m = 8 * gq + 4 * kbp + j;
-    frag[((b * 8 + (s >> 2)) * 64 + m + 32 * kb) * 4 + (s & 3)] = mat[(int64_t)r * ld_r + (int64_t)cc * ld_c] * mscale;
+    const float val = (r < dr && cc < dc) ? mat[(int64_t)r * ld_r + (int64_t)cc * ld_c] * mscale : 0.f;
+    frag[((b * 8 + (s >> 2)) * 64 + m + 32 * kb) * 4 + (s & 3)] = val;
   }
 }
 
@@ -230,6 +249,7 @@ struct Rows32Job {
   float* out;           // [rows, 64]
   float* tokscal;       // TOKENS: [2][total rows]: 1/z_t, dz_t
   int64_t total_rows;
+  int dr, dc;           // row lengths of x and out in memory (<= 64, multiples of 4)
 };
 
 struct Rows32Layout {
@@ -245,7 +265,7 @@ struct Rows32Layout {
 // view of backward pass A: g = x_t M (x = dO, M = S^T), P = q_t . g, z = q_t . km + eps,
 // dz = -P / z^2, out = dq_t = g / z + dz km (without the denominator: out = g), and the
 // per-row scalars 1/z_t, dz_t go to tokscal.
-template <bool NORM, bool TOKENS>
+template <bool NORM, bool TOKENS, bool PAD>
 __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0, Rows32Job job1,
                                                           int wgs_per_job, int chunk, int nchunks) {
   using LY = Rows32Layout;
@@ -268,6 +288,7 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ntok = lane & 31, kb = lane >> 5;
+  const int dr = PAD ? job.dr : D, dc = PAD ? job.dc : D;
   float* frag = reinterpret_cast<float*>(smem);
   unsigned char* stage = smem + LY::kFrag + wave * LY::kStage;
   float* kmv = reinterpret_cast<float*>(smem + LY::kKm);
@@ -279,18 +300,20 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
     for (int i = 0; i < 8; ++i) {
       const int q = lane + 64 * i, row = q >> 4, ch = q & 15;
       const int tok = tok0 + row;
-      dst[i] = tok < t_end ? *reinterpret_cast<const f32x4*>(src + (row0 + (int64_t)tok * rstride) * D + ch * 4)
-                           : f32x4{0.f, 0.f, 0.f, 0.f};
+      dst[i] = (tok < t_end && (!PAD || ch * 4 < dr))
+                   ? *reinterpret_cast<const f32x4*>(src + (row0 + (int64_t)tok * rstride) * dr + ch * 4)
+                   : f32x4{0.f, 0.f, 0.f, 0.f};
     }
   };
   int t0 = t_begin + 32 * wave;
   f32x4 xr[8];
   if (t0 < t_end) load_tile(xr, job.x, t0);
 
-  build_operand32(frag, job.mat + (int64_t)nh * D * D, job.ld_r, job.ld_c, 1.f);
+  build_operand32(frag, job.mat + (int64_t)nh * dr * dc, job.ld_r, job.ld_c, 1.f, dr, dc);
+  const int dkm = NORM ? dr : dc;  // length of km: the contracted side (output) or q's (token view)
   for (int e = tid; e < D; e += kThreads) {
-    kmv[e] = (NORM || TOKENS) && job.km ? job.km[(int64_t)nh * D + e] : 0.f;
-    addv[e] = job.addvec ? job.addvec[(int64_t)nh * D + e] * job.add_scale : 0.f;
+    kmv[e] = (NORM || TOKENS) && job.km && e < dkm ? job.km[(int64_t)nh * dkm + e] : 0.f;
+    addv[e] = job.addvec && e < dc ? job.addvec[(int64_t)nh * dc + e] * job.add_scale : 0.f;
   }
   __syncthreads();
   const bool with_den = (NORM || TOKENS) && job.km != nullptr;
@@ -343,13 +366,14 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
       if (with_den) {
         // q row half of this lane straight from global memory (a full 128-byte line per lane)
         const int tok = min(t0 + ntok, t_end - 1);
-        const float* qrow = job.xden + (row0 + (int64_t)tok * rstride) * D + 32 * kb;
+        const float* qrow = job.xden + (row0 + (int64_t)tok * rstride) * dc + 32 * kb;
         float P = 0.f, zz = 0.f;
 #pragma unroll
         for (int b = 0; b < 2; ++b)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const f32x4 qv = *reinterpret_cast<const f32x4*>(qrow + 16 * b + 4 * i);
+            f32x4 qv = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (!PAD || 32 * kb + 16 * b + 4 * i < dc) qv = *reinterpret_cast<const f32x4*>(qrow + 16 * b + 4 * i);
             const f32x4 kv = *reinterpret_cast<const f32x4*>(kmv + 32 * kb + 16 * b + 4 * i);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -388,8 +412,8 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
     for (int i = 0; i < 8; ++i) {
       const int q = lane + 64 * i, row = q >> 4, ch = q & 15;
       const int tok = t0 + row;
-      if (tok < t_end)
-        *reinterpret_cast<f32x4*>(job.out + (row0 + (int64_t)tok * rstride) * D + ch * 4) =
+      if (tok < t_end && (!PAD || ch * 4 < dc))
+        *reinterpret_cast<f32x4*>(job.out + (row0 + (int64_t)tok * rstride) * dc + ch * 4) =
             *reinterpret_cast<const f32x4*>(stage + swz<256>(row, ch));
     }
     t0 = tn;
@@ -400,22 +424,30 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
 // host side
 // ===========================================================================
 bool supported(const Prob& p) {
-  return p.DK == D && p.DV == D && !(p.flags & kDecoupled);
+  return p.DK >= 4 && p.DV >= 4 && p.DK <= D && p.DV <= D && p.DK % 4 == 0 && p.DV % 4 == 0 &&
+         !(p.flags & kDecoupled);
 }
+static bool padded(const Prob& p) { return p.DK != D || p.DV != D; }
 
 void state(const Prob& p, const float* kn, const float* v, const float* kd, float* partial,
            const float* tokscal, int64_t total_rows, int chunk, int nchunks, hipStream_t st, float* fin_mat,
            float* fin_vec) {
   const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(kThreads);
-  if (tokscal)
-    state32_kernel<false, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks);
-  else
-    state32_kernel<false, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks);
+  if (padded(p)) {
+    if (tokscal)
+      state32_kernel<false, true, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks);
+    else
+      state32_kernel<false, false, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks);
+  } else if (tokscal) {
+    state32_kernel<false, true, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks);
+  } else {
+    state32_kernel<false, false, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks);
+  }
 }
 
-template <bool NORM, bool TOKENS>
-static int launch_rows(const Prob& p, const Rows32Job& j0, const Rows32Job* j1, hipStream_t st) {
-  auto kernel = rows32_kernel<NORM, TOKENS>;
+template <bool NORM, bool TOKENS, bool PAD>
+static int launch_rows_k(const Prob& p, const Rows32Job& j0, const Rows32Job* j1, hipStream_t st) {
+  auto kernel = rows32_kernel<NORM, TOKENS, PAD>;
   static thread_local bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -434,7 +466,13 @@ static int launch_rows(const Prob& p, const Rows32Job& j0, const Rows32Job* j1, 
   return kOk;
 }
 
-static Rows32Job convert(const mfma::RowsJob& j) {
+template <bool NORM, bool TOKENS>
+static int launch_rows(const Prob& p, const Rows32Job& j0, const Rows32Job* j1, hipStream_t st) {
+  if (padded(p)) return launch_rows_k<NORM, TOKENS, true>(p, j0, j1, st);
+  return launch_rows_k<NORM, TOKENS, false>(p, j0, j1, st);
+}
+
+static Rows32Job convert(const mfma::RowsJob& j, int dr, int dc) {
   Rows32Job r;
   r.x = (const float*)j.x;
   r.xden = (const float*)j.xden;
@@ -447,14 +485,17 @@ static Rows32Job convert(const mfma::RowsJob& j) {
   r.out = (float*)j.out;
   r.tokscal = nullptr;
   r.total_rows = 0;
+  r.dr = dr;
+  r.dc = dc;
   return r;
 }
 
-int rows(const Prob& p, const mfma::RowsJob& job, const mfma::RowsJob* job2, hipStream_t st) {
-  const Rows32Job a = convert(job);
+// dr, dc: the contracted and the output head dim of the job (of both jobs when there are two)
+int rows(const Prob& p, const mfma::RowsJob& job, const mfma::RowsJob* job2, int dr, int dc, hipStream_t st) {
+  const Rows32Job a = convert(job, dr, dc);
   if (job.xden) return launch_rows<true, false>(p, a, nullptr, st);
   if (job2) {
-    const Rows32Job b = convert(*job2);
+    const Rows32Job b = convert(*job2, dr, dc);
     return launch_rows<false, false>(p, a, &b, st);
   }
   return launch_rows<false, false>(p, a, nullptr, st);
@@ -467,7 +508,9 @@ int bwd_tokens(const Prob& p, const float* q, const float* dout, const float* S,
   j.xden = q;
   j.mat = S;  // M(r = dv, c = dk) = S[c][r]
   j.ld_r = 1;
-  j.ld_c = D;
+  j.ld_c = p.DV;
+  j.dr = p.DV;
+  j.dc = p.DK;
   j.km = (p.flags & kNormalize) ? km : nullptr;
   j.addvec = nullptr;
   j.add_scale = 1.f;

@@ -1,7 +1,7 @@
 // The plan: which kernels run, in which order, for each entry point, and how the
 // caller's workspace is carved up.  MFMA kernels are used for the shapes they
 // cover (16-bit inputs with head dims that are multiples of 8 up to 128, fp32 inputs
-// with 64 x 64 heads); everything else runs on the generic kernels.
+// with head dims that are multiples of 4 up to 64); everything else runs on the generic kernels.
 //
 // forward :  state partials -> fixed-order reduce (S, km) -> output rows
 // backward:  S^T -> pass A (dq, partial dS/dkm) -> reduce (s dS, its transpose, dkm/L)
@@ -91,7 +91,7 @@ static int check_cross(const Prob& p, int dtype) {
   if (!cross(p)) return kOk;
   if ((p.flags & kDecoupled) || !mfma::supported(key_side(p), dtype)) {
     set_error("different numbers of queries and keys need the matrix-core kernels (16-bit inputs with "
-              "head dims that are multiples of 8, or fp32 inputs with 64 x 64 heads) and are not "
+              "head dims that are multiples of 8, or fp32 inputs with head dims up to 64) and are not "
               "available for the decoupled operator");
     return kErrUnsupported;
   }

@@ -46,10 +46,13 @@ def test_simple_la_16bit(dims):
         _check("simple", 1, 2, lq, lk, dims[0], dims[1], torch.float16, 70 * i + dims[1])
 
 
-def test_fp32_64_by_64():
+def test_fp32():
     for i, (lq, lk) in enumerate(LENGTHS):
         _check("linear", 2, 2, lq, lk, 64, 64, torch.float32, 90 + i)
+        _check("linear", 1, 2, lq, lk, 32, 32, torch.float32, 190 + i)
     _check("simple", 1, 2, 300, 77, 64, 64, torch.float32, 99)
+    _check("simple", 1, 2, 300, 77, 48, 20, torch.float32, 98)
+    _check("linear", 2, 1, 77, 300, 12, 64, torch.float32, 97)
 
 
 def test_default_scale_is_one_over_the_number_of_keys():
@@ -68,8 +71,8 @@ def test_shapes_without_matrix_core_kernels_are_refused():
     k = torch.rand(1, 2, 10, 20, device="cuda", dtype=torch.float16)
     with pytest.raises(ValueError, match="matrix-core"):
         linear_attention(q, k, k)
-    q32 = torch.rand(1, 2, 40, 32, device="cuda")
-    k32 = torch.rand(1, 2, 10, 32, device="cuda")
+    q32 = torch.rand(1, 2, 40, 128, device="cuda")   # fp32: head dims up to 64 only
+    k32 = torch.rand(1, 2, 10, 128, device="cuda")
     with pytest.raises(ValueError, match="matrix-core"):
         linear_attention(q32, k32, k32)
     # the library is still usable

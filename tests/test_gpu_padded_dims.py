@@ -101,3 +101,31 @@ def test_heads_tiled_128_by_128():
     _check_dense("simple", 1, 2, 97, 128, 128, torch.bfloat16, 15)
     _check_dense("linear", 1, 1, 5000, 96, 120, torch.float16, 16)
     _check_dense("linear", 3, 2, 129, 72, 128, torch.bfloat16, 17)
+
+
+@pytest.mark.parametrize("dims", [(32, 32), (16, 16), (4, 4), (24, 40), (64, 32), (32, 64), (60, 12), (48, 48)])
+def test_fp32_head_dims_up_to_64(dims):
+    """fp32 inputs: head dims that are multiples of 4 up to 64 run on the fp32 matrix instructions."""
+    for i, L in enumerate(LENGTHS):
+        _check_dense("linear", 2, 3, L, dims[0], dims[1], torch.float32, 40 * i + dims[0])
+    _check_dense("simple", 1, 2, 700, dims[0], dims[1], torch.float32, 41 + dims[1])
+
+
+def test_fp32_packed_small_heads():
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    for DK, DV in ((32, 32), (16, 48), (64, 8)):
+        H = 3
+        lengths = [300, 1, 0, 17, 1200, 64, 33]
+        T = sum(lengths)
+        q, k, v, do = make_qkv((T, H, DK), (T, H, DV), torch.float32, DK + DV)
+        cu = torch.tensor(np.concatenate([[0], np.cumsum(lengths)]), dtype=torch.int32).cuda()
+        leaves = [t.cuda().requires_grad_() for t in (q, k, v)]
+        o = varlen_linear_attention(*leaves, cu, max(lengths))
+        o.backward(do.cuda())
+        ref = cf.varlen_backward(np64(q), np64(k), np64(v), np64(do), cu.cpu().numpy())
+        assert_parity(o, ref["o"], torch.float32, f"o DK{DK} DV{DV}")
+        for name, t in zip(("dq", "dk", "dv"), leaves):
+            for b, e in zip(cu[:-1].tolist(), cu[1:].tolist()):
+                if e > b:
+                    floor = ref[name + "_mag"][b:e] if name + "_mag" in ref else None
+                    assert_parity(t.grad[b:e], ref[name][b:e], torch.float32, f"{name}[{b}:{e}] DK{DK} DV{DV}", floor)
