@@ -104,14 +104,16 @@ void state_with_block_stats(const Prob& p, int dtype, const void* k, const void*
 int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st);
 int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, int DR, int DC,
           hipStream_t st);
-// two-kernel form of backward pass A for head dims above 64 (not decoupled):
+// two-kernel form of backward pass A (16-bit heads tiled 64 x 128 / 128 x 64, fp32 inputs):
+// qn / dqn are the rows of the numerator and their gradient (q_rope, dq_rope when decoupled, which
+// only the fp32 kernels support here; then qd = q, dqd = dq), otherwise qn == qd and dqd is unused.
 // bwd_tokens writes dq and tokscal = [1/z_t | dz_t] per (token, head) row, scaled_state
 // accumulates the partials of dS = sum_t q_t^T (dO_t / z_t) and dkm = sum_t dz_t q_t
-int bwd_tokens(const Prob& p, int dtype, const void* q, const void* dout, const float* S,
-               const float* km, void* dq, float* tokscal, int64_t total_rows, hipStream_t st);
-void scaled_state(const Prob& p, int dtype, const void* qn, const void* dout, const float* tokscal,
-                  int64_t total_rows, float* partial, int chunk, int nchunks, hipStream_t st,
-                  float* fin_mat = nullptr, float* fin_vec = nullptr);
+int bwd_tokens(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout, const float* S,
+               const float* km, void* dqn, void* dqd, float* tokscal, int64_t total_rows, hipStream_t st);
+void scaled_state(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout,
+                  const float* tokscal, int64_t total_rows, float* partial, int chunk, int nchunks,
+                  hipStream_t st, float* fin_mat = nullptr, float* fin_vec = nullptr);
 // backward pass A: dq~ (and dq when decoupled) + per-chunk partials of dS and dkm
 int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout, const float* S,
           const float* km, void* dqn, void* dqd, float* partial, int chunk, int nchunks,
@@ -126,8 +128,8 @@ void state(const Prob& p, const float* kn, const float* v, const float* kd, floa
            const float* tokscal, int64_t total_rows, int chunk, int nchunks, hipStream_t st, float* fin_mat,
            float* fin_vec);
 int rows(const Prob& p, const mfma::RowsJob& job, const mfma::RowsJob* job2, int dr, int dc, hipStream_t st);
-int bwd_tokens(const Prob& p, const float* q, const float* dout, const float* S, const float* km, float* dq,
-               float* tokscal, int64_t total_rows, hipStream_t st);
+int bwd_tokens(const Prob& p, const float* qn, const float* qd, const float* dout, const float* S,
+               const float* km, float* dqn, float* dqd, float* tokscal, int64_t total_rows, hipStream_t st);
 }  // namespace mfma32
 
 // Piecewise (PISA) attention, forward only (fbla_piecewise.hip).

@@ -1766,12 +1766,12 @@ void state_with_block_stats(const Prob& p, int dtype, const void* k, const void*
   else run_state<__bf16>(p, k, v, k, partial, nullptr, 0, nullptr, nullptr, chunk, nchunks, bs, st);
 }
 
-void scaled_state(const Prob& p, int dtype, const void* qn, const void* dout, const float* tokscal,
-                  int64_t total_rows, float* partial, int chunk, int nchunks, hipStream_t st,
-                  float* fin_mat, float* fin_vec) {
+void scaled_state(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout,
+                  const float* tokscal, int64_t total_rows, float* partial, int chunk, int nchunks,
+                  hipStream_t st, float* fin_mat, float* fin_vec) {
   const BlockStats none{nullptr, nullptr, 0};
   if (dtype == kF32)
-    return mfma32::state(p, (const float*)qn, (const float*)dout, (const float*)qn, partial, tokscal,
+    return mfma32::state(p, (const float*)qn, (const float*)dout, (const float*)qd, partial, tokscal,
                          total_rows, chunk, nchunks, st, fin_mat, fin_vec);
   if (dtype == kF16)
     run_state<_Float16>(p, qn, dout, qn, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, none, st);
@@ -1910,12 +1910,13 @@ static int run_bwd_tokens(const Prob& p, const void* q, const void* dout, const 
 }
 
 // token view of the backward alone: dq and the per-row scalars 1/z_t, dz_t
-int bwd_tokens(const Prob& p, int dtype, const void* q, const void* dout, const float* S,
-               const float* km, void* dq, float* tokscal, int64_t total_rows, hipStream_t st) {
+int bwd_tokens(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout, const float* S,
+               const float* km, void* dqn, void* dqd, float* tokscal, int64_t total_rows, hipStream_t st) {
   if (dtype == kF32)
-    return mfma32::bwd_tokens(p, (const float*)q, (const float*)dout, S, km, (float*)dq, tokscal, total_rows, st);
-  if (dtype == kF16) return run_bwd_tokens<_Float16>(p, q, dout, S, km, dq, tokscal, total_rows, st);
-  return run_bwd_tokens<__bf16>(p, q, dout, S, km, dq, tokscal, total_rows, st);
+    return mfma32::bwd_tokens(p, (const float*)qn, (const float*)qd, (const float*)dout, S, km, (float*)dqn,
+                              (float*)dqd, tokscal, total_rows, st);
+  if (dtype == kF16) return run_bwd_tokens<_Float16>(p, qn, dout, S, km, dqn, tokscal, total_rows, st);
+  return run_bwd_tokens<__bf16>(p, qn, dout, S, km, dqn, tokscal, total_rows, st);
 }
 
 }  // namespace mfma

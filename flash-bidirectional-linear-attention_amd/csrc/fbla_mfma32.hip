@@ -1,8 +1,8 @@
 // MFMA kernels for fp32 inputs, heads tiled 64 x 64: head dims that are multiples of 4 (16-byte
 // row pieces) up to 64, smaller ones with zero padding (PAD variants: true row lengths in memory,
 // missing features read as zero, outputs and state in their true shapes).  Dense and packed
-// layouts, with or without the denominator; the decoupled operator and larger heads stay on
-// the shape-generic kernels.  v_mfma_f32_32x32x2_f32 computes in fp32 throughout, so
+// layouts, with or without the denominator, plain and decoupled (numerator from the rotary
+// features, denominator from the plain ones); larger heads stay on the shape-generic kernels.  v_mfma_f32_32x32x2_f32 computes in fp32 throughout, so
 // there is no operand splitting here: A lane l holds A[m = l%32][k = l/32], B lane l
 // holds B[k = l/32][n = l%32], C register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32].
 // One instruction covers two values of the contraction index and takes 64 cycles:
@@ -177,7 +177,7 @@ __global__ __launch_bounds__(kThreads, 2) void state32_kernel(
       for (int a = 0; a < 2; ++a) {
 #pragma unroll
         for (int bb = 0; bb < 2; ++bb) acc[a][bb] = mma(b.k[s][a], vv[bb], acc[a][bb]);
-        if constexpr (SCALED) ks[a] = fmaf(b.dz[s], b.k[s][a], ks[a]);
+        if constexpr (SCALED) ks[a] = fmaf(b.dz[s], SPLIT_KD ? b.d[s][a] : b.k[s][a], ks[a]);
         else ks[a] += SPLIT_KD ? b.d[s][a] : b.k[s][a];
       }
     }
@@ -240,7 +240,9 @@ __device__ __forceinline__ void build_operand32(float* frag, const float* __rest
 
 struct Rows32Job {
   const float* x;       // [rows, 64] B operand
-  const float* xden;    // NORM: rows for the denominator (== x here); TOKENS: q
+  const float* xnum;    // TOKENS: the rows q~ of the numerator (q_rope when decoupled, else q)
+  float* out2;          // TOKENS, decoupled: dq = dz km (out then holds dq~ = g / z)
+  const float* xden;    // NORM: rows for the denominator (x itself unless decoupled); TOKENS: q
   const float* mat;     // operand M, element (r, c) at mat[nh*4096 + r*ld_r + c*ld_c]
   int ld_r, ld_c;
   const float* km;      // [NH, 64] mean key (NORM / TOKENS with the denominator)
@@ -262,10 +264,12 @@ struct Rows32Layout {
 };
 
 // NORM: rowscale = 1 / (x_t . km + eps).  TOKENS (implies the job's q in xden): the token
-// view of backward pass A: g = x_t M (x = dO, M = S^T), P = q_t . g, z = q_t . km + eps,
+// view of backward pass A: g = x_t M (x = dO, M = S^T), P = q~_t . g, z = q_t . km + eps,
 // dz = -P / z^2, out = dq_t = g / z + dz km (without the denominator: out = g), and the
-// per-row scalars 1/z_t, dz_t go to tokscal.
-template <bool NORM, bool TOKENS, bool PAD>
+// per-row scalars 1/z_t, dz_t go to tokscal.  DEN (decoupled): the denominator rows are not
+// the multiplied rows; they are read straight from global memory (NORM: z; TOKENS: z from q,
+// P from q~ = q_rope, and the two gradients go to out = dq~ and out2 = dq).
+template <bool NORM, bool TOKENS, bool PAD, bool DEN>
 __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0, Rows32Job job1,
                                                           int wgs_per_job, int chunk, int nchunks) {
   using LY = Rows32Layout;
@@ -347,7 +351,7 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[b] = mma(a4[e], xv[e], acc[b]);
       }
-      if constexpr (NORM) {
+      if constexpr (NORM && !DEN) {
         const f32x2 k01 = *reinterpret_cast<const f32x2*>(kmv + 8 * sg + 2 * kb);
         const f32x2 k23 = *reinterpret_cast<const f32x2*>(kmv + 8 * sg + 4 + 2 * kb);
         z = fmaf(x01[0], k01[0], z);
@@ -359,6 +363,18 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
     // this lane: token ntok, output features 32*kb + 16*b + r
     float rs = 1.f, dz = 0.f;
     if constexpr (NORM) {
+      if constexpr (DEN) {  // this lane's half of the plain row: one 128-byte line
+        const int tok = min(t0 + ntok, t_end - 1);
+        const float* drow = job.xden + (row0 + (int64_t)tok * rstride) * dr + 32 * kb;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          if (PAD && 32 * kb + 4 * i >= dr) continue;
+          const f32x4 dv4 = *reinterpret_cast<const f32x4*>(drow + 4 * i);
+          const f32x4 kv = *reinterpret_cast<const f32x4*>(kmv + 32 * kb + 4 * i);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) z = fmaf(dv4[j], kv[j], z);
+        }
+      }
       z += __shfl_xor(z, 32);
       rs = 1.f / (z + p.eps);
     }
@@ -366,18 +382,24 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
       if (with_den) {
         // q row half of this lane straight from global memory (a full 128-byte line per lane)
         const int tok = min(t0 + ntok, t_end - 1);
-        const float* qrow = job.xden + (row0 + (int64_t)tok * rstride) * dc + 32 * kb;
+        const int64_t roff = (row0 + (int64_t)tok * rstride) * dc + 32 * kb;
+        const float* qrow = job.xden + roff;   // plain q: the denominator
+        const float* nrow = job.xnum + roff;   // q~: the numerator
         float P = 0.f, zz = 0.f;
 #pragma unroll
         for (int b = 0; b < 2; ++b)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            f32x4 qv = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (!PAD || 32 * kb + 16 * b + 4 * i < dc) qv = *reinterpret_cast<const f32x4*>(qrow + 16 * b + 4 * i);
+            f32x4 qv = f32x4{0.f, 0.f, 0.f, 0.f}, nv = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (!PAD || 32 * kb + 16 * b + 4 * i < dc) {
+              qv = *reinterpret_cast<const f32x4*>(qrow + 16 * b + 4 * i);
+              nv = qv;
+              if constexpr (DEN) nv = *reinterpret_cast<const f32x4*>(nrow + 16 * b + 4 * i);
+            }
             const f32x4 kv = *reinterpret_cast<const f32x4*>(kmv + 32 * kb + 16 * b + 4 * i);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-              P = fmaf(qv[j], acc[b][4 * i + j], P);
+              P = fmaf(nv[j], acc[b][4 * i + j], P);
               zz = fmaf(qv[j], kv[j], zz);
             }
           }
@@ -402,7 +424,7 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           float o = fmaf(acc[b][4 * i + j], rs, addv[c0 + j]);
-          if constexpr (TOKENS) o = fmaf(dz, kmv[c0 + j], o);
+          if constexpr (TOKENS && !DEN) o = fmaf(dz, kmv[c0 + j], o);
           w[j] = o;
         }
         *reinterpret_cast<f32x4*>(stage + swz<256>(ntok, c0 >> 2)) = w;
@@ -416,6 +438,26 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
         *reinterpret_cast<f32x4*>(job.out + (row0 + (int64_t)tok * rstride) * dc + ch * 4) =
             *reinterpret_cast<const f32x4*>(stage + swz<256>(row, ch));
     }
+    if constexpr (TOKENS && DEN) {  // the second gradient, dq = dz km, through the same tile
+      wave_sync();
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int c0 = 32 * kb + 16 * b + 4 * i;
+          *reinterpret_cast<f32x4*>(stage + swz<256>(ntok, c0 >> 2)) =
+              f32x4{dz * kmv[c0], dz * kmv[c0 + 1], dz * kmv[c0 + 2], dz * kmv[c0 + 3]};
+        }
+      wave_sync();
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int q = lane + 64 * i, row = q >> 4, ch = q & 15;
+        const int tok = t0 + row;
+        if (tok < t_end && (!PAD || ch * 4 < dc))
+          *reinterpret_cast<f32x4*>(job.out2 + (row0 + (int64_t)tok * rstride) * dc + ch * 4) =
+              *reinterpret_cast<const f32x4*>(stage + swz<256>(row, ch));
+      }
+    }
     t0 = tn;
   }
 }
@@ -424,8 +466,7 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
 // host side
 // ===========================================================================
 bool supported(const Prob& p) {
-  return p.DK >= 4 && p.DV >= 4 && p.DK <= D && p.DV <= D && p.DK % 4 == 0 && p.DV % 4 == 0 &&
-         !(p.flags & kDecoupled);
+  return p.DK >= 4 && p.DV >= 4 && p.DK <= D && p.DV <= D && p.DK % 4 == 0 && p.DV % 4 == 0;
 }
 static bool padded(const Prob& p) { return p.DK != D || p.DV != D; }
 
@@ -433,21 +474,26 @@ void state(const Prob& p, const float* kn, const float* v, const float* kd, floa
            const float* tokscal, int64_t total_rows, int chunk, int nchunks, hipStream_t st, float* fin_mat,
            float* fin_vec) {
   const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(kThreads);
-  if (padded(p)) {
-    if (tokscal)
-      state32_kernel<false, true, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks);
-    else
-      state32_kernel<false, false, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks);
-  } else if (tokscal) {
-    state32_kernel<false, true, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks);
-  } else {
-    state32_kernel<false, false, false><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fin_mat, fin_vec, chunk, nchunks);
+  auto go = [&](auto kernel) {
+    kernel<<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, tokscal ? total_rows : 0, fin_mat, fin_vec, chunk, nchunks);
+  };
+  // kd != kn: the decoupled operator (vector part from the plain rows)
+  const int variant = (kd != kn ? 4 : 0) + (tokscal ? 2 : 0) + (padded(p) ? 1 : 0);
+  switch (variant) {
+    case 0: go(state32_kernel<false, false, false>); break;
+    case 1: go(state32_kernel<false, false, true>); break;
+    case 2: go(state32_kernel<false, true, false>); break;
+    case 3: go(state32_kernel<false, true, true>); break;
+    case 4: go(state32_kernel<true, false, false>); break;
+    case 5: go(state32_kernel<true, false, true>); break;
+    case 6: go(state32_kernel<true, true, false>); break;
+    default: go(state32_kernel<true, true, true>); break;
   }
 }
 
-template <bool NORM, bool TOKENS, bool PAD>
+template <bool NORM, bool TOKENS, bool PAD, bool DEN>
 static int launch_rows_k(const Prob& p, const Rows32Job& j0, const Rows32Job* j1, hipStream_t st) {
-  auto kernel = rows32_kernel<NORM, TOKENS, PAD>;
+  auto kernel = rows32_kernel<NORM, TOKENS, PAD, DEN>;
   static thread_local bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -466,15 +512,17 @@ static int launch_rows_k(const Prob& p, const Rows32Job& j0, const Rows32Job* j1
   return kOk;
 }
 
-template <bool NORM, bool TOKENS>
+template <bool NORM, bool TOKENS, bool DEN = false>
 static int launch_rows(const Prob& p, const Rows32Job& j0, const Rows32Job* j1, hipStream_t st) {
-  if (padded(p)) return launch_rows_k<NORM, TOKENS, true>(p, j0, j1, st);
-  return launch_rows_k<NORM, TOKENS, false>(p, j0, j1, st);
+  if (padded(p)) return launch_rows_k<NORM, TOKENS, true, DEN>(p, j0, j1, st);
+  return launch_rows_k<NORM, TOKENS, false, DEN>(p, j0, j1, st);
 }
 
 static Rows32Job convert(const mfma::RowsJob& j, int dr, int dc) {
   Rows32Job r;
   r.x = (const float*)j.x;
+  r.xnum = nullptr;
+  r.out2 = nullptr;
   r.xden = (const float*)j.xden;
   r.mat = j.mat;
   r.ld_r = j.ld_r;
@@ -493,6 +541,7 @@ static Rows32Job convert(const mfma::RowsJob& j, int dr, int dc) {
 // dr, dc: the contracted and the output head dim of the job (of both jobs when there are two)
 int rows(const Prob& p, const mfma::RowsJob& job, const mfma::RowsJob* job2, int dr, int dc, hipStream_t st) {
   const Rows32Job a = convert(job, dr, dc);
+  if (job.xden && job.xden != job.x) return launch_rows<true, false, true>(p, a, nullptr, st);
   if (job.xden) return launch_rows<true, false>(p, a, nullptr, st);
   if (job2) {
     const Rows32Job b = convert(*job2, dr, dc);
@@ -501,11 +550,15 @@ int rows(const Prob& p, const mfma::RowsJob& job, const mfma::RowsJob* job2, int
   return launch_rows<false, false>(p, a, nullptr, st);
 }
 
-int bwd_tokens(const Prob& p, const float* q, const float* dout, const float* S, const float* km, float* dq,
-               float* tokscal, int64_t total_rows, hipStream_t st) {
+// qn / dqn: the rows of the numerator and their gradient (q_rope, dq_rope when decoupled, then
+// qd = q and dqd = dq; otherwise qn == qd and dqd is not used)
+int bwd_tokens(const Prob& p, const float* qn, const float* qd, const float* dout, const float* S,
+               const float* km, float* dqn, float* dqd, float* tokscal, int64_t total_rows, hipStream_t st) {
   Rows32Job j;
   j.x = dout;
-  j.xden = q;
+  j.xnum = qn;
+  j.out2 = dqd;
+  j.xden = qd;
   j.mat = S;  // M(r = dv, c = dk) = S[c][r]
   j.ld_r = 1;
   j.ld_c = p.DV;
@@ -514,9 +567,10 @@ int bwd_tokens(const Prob& p, const float* q, const float* dout, const float* S,
   j.km = (p.flags & kNormalize) ? km : nullptr;
   j.addvec = nullptr;
   j.add_scale = 1.f;
-  j.out = dq;
+  j.out = dqn;
   j.tokscal = tokscal;
   j.total_rows = total_rows;
+  if (p.flags & kDecoupled) return launch_rows<false, true, true>(p, j, nullptr, st);
   return launch_rows<false, true>(p, j, nullptr, st);
 }
 

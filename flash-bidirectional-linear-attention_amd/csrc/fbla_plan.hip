@@ -186,10 +186,10 @@ int backward(const Prob& pc, int dtype, const BwdArgs& a, hipStream_t st) {
     } else if (fast) {
       // head dims above 64: token view and feature view as two kernels
       const int64_t rows = p.T * p.H;
-      int rc = mfma::bwd_tokens(p, dtype, a.q, a.dout, a.s, a.km, a.dq, tokscal, rows, st);
+      int rc = mfma::bwd_tokens(p, dtype, qn, a.q, a.dout, a.s, a.km, dqn, dqd, tokscal, rows, st);
       if (rc != kOk) return rc;
       if (normalize)
-        mfma::scaled_state(p, dtype, a.q, a.dout, tokscal, rows, partial, chunk, nchunks, st, fm, fv);
+        mfma::scaled_state(p, dtype, qn, a.q, a.dout, tokscal, rows, partial, chunk, nchunks, st, fm, fv);
       else
         mfma::state(p, dtype, a.q, a.dout, a.q, partial, chunk, nchunks, st, fm, fv);
     } else {

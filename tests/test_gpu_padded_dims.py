@@ -129,3 +129,10 @@ def test_fp32_packed_small_heads():
                 if e > b:
                     floor = ref[name + "_mag"][b:e] if name + "_mag" in ref else None
                     assert_parity(t.grad[b:e], ref[name][b:e], torch.float32, f"{name}[{b}:{e}] DK{DK} DV{DV}", floor)
+
+
+@pytest.mark.parametrize("dims", [(32, 32), (64, 64), (16, 40), (64, 32), (4, 60)])
+def test_fp32_decoupled(dims):
+    """The decoupled operator in fp32 (the MLLA / RALA blocks without autocast)."""
+    for i, L in enumerate(LENGTHS + [5000]):
+        _check_dense("decoupled", 2, 2, L, dims[0], dims[1], torch.float32, 60 * i + dims[1])
