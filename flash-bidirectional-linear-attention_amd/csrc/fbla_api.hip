@@ -4,6 +4,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <initializer_list>
+
 #include "../../include/flash_bla_hip.h"
 #include "fbla_kernels.h"
 
@@ -55,6 +57,16 @@ static int check_dims(const char* what, int64_t N, int64_t H, int64_t L, int DK,
   return kOk;
 }
 
+// The kernels move 16-byte pieces of rows.
+static int check_aligned(const char* what, std::initializer_list<const void*> ptrs) {
+  for (const void* ptr : ptrs)
+    if (reinterpret_cast<uintptr_t>(ptr) & 15) {
+      set_error("%s: tensor pointers must be 16-byte aligned", what);
+      return kErrBadArg;
+    }
+  return kOk;
+}
+
 static Prob make_prob(const int32_t* cu, int64_t N, int64_t H, int64_t L, int64_t T, int DK, int DV,
                       int flags, float scale, float eps) {
   Prob p;
@@ -78,6 +90,8 @@ static size_t workspace_bytes(const Prob& p, int dtype, int pass) {
 
 static int run_fwd(const char* what, const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
   if ((int64_t)p.N * p.H == 0 || p.L == 0) return kOk;
+  if (check_aligned(what, {a.q, a.k, a.v, a.q_rope, a.k_rope, a.o, a.s, a.km, a.workspace}) != kOk)
+    return kErrBadArg;
   const size_t need = workspace_bytes(p, dtype, 0);
   if (a.workspace_bytes < need || (need && !a.workspace)) {
     set_error("%s: workspace too small (%zu < %zu bytes)", what, a.workspace_bytes, need);
@@ -90,6 +104,9 @@ static int run_fwd(const char* what, const Prob& p, int dtype, const FwdArgs& a,
 
 static int run_bwd(const char* what, const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
   if ((int64_t)p.N * p.H == 0 || p.L == 0) return kOk;
+  if (check_aligned(what, {a.q, a.k, a.v, a.q_rope, a.k_rope, a.dout, a.s, a.km, a.dq, a.dk, a.dv, a.dq_rope,
+                           a.dk_rope, a.workspace}) != kOk)
+    return kErrBadArg;
   const size_t need = workspace_bytes(p, dtype, 1);
   if (a.workspace_bytes < need || (need && !a.workspace)) {
     set_error("%s: workspace too small (%zu < %zu bytes)", what, a.workspace_bytes, need);

@@ -95,6 +95,13 @@ def _workspace(nbytes, device):
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
 
 
+def _aligned(*tensors):
+    """The kernels move 16-byte pieces: a tensor whose storage offset leaves its first element off
+    a 16-byte boundary (a view into a larger buffer) is copied to fresh, aligned memory."""
+    return tuple(t if t is None or t.data_ptr() % 16 == 0 else t.clone(memory_format=torch.contiguous_format)
+                 for t in tensors)
+
+
 def _require_gpu(*tensors):
     for t in tensors:
         if t is not None and not t.is_cuda:
@@ -106,6 +113,7 @@ def la_fwd(q, k, v, q_rope, k_rope, scale, eps, flags):
     """Dense forward: returns (o, s, km).  Tensors must be contiguous [B,H,L,D]; k and v may have
     another number of tokens than q (not with the decoupled operator)."""
     _require_gpu(q, k, v, q_rope, k_rope)
+    q, k, v, q_rope, k_rope = _aligned(q, k, v, q_rope, k_rope)
     L = lib()
     B, H, T, DK = q.shape
     Tk, DV = k.shape[-2], v.shape[-1]
@@ -134,6 +142,7 @@ def la_fwd(q, k, v, q_rope, k_rope, scale, eps, flags):
 def la_bwd(q, k, v, q_rope, k_rope, do, s, km, scale, eps, flags):
     """Dense backward: returns (dq, dk, dv, dq_rope, dk_rope)."""
     _require_gpu(q, k, v, do)
+    q, k, v, q_rope, k_rope, do, s, km = _aligned(q, k, v, q_rope, k_rope, do, s, km)
     L = lib()
     B, H, T, DK = q.shape
     Tk, DV = k.shape[-2], v.shape[-1]
@@ -163,6 +172,7 @@ def la_bwd(q, k, v, q_rope, k_rope, do, s, km, scale, eps, flags):
 def varlen_fwd(q, k, v, cu_seqlens, max_seqlen, scale, eps):
     """Packed forward: returns (o, s, km).  Tensors contiguous [T,H,D]."""
     _require_gpu(q, k, v, cu_seqlens)
+    q, k, v, cu_seqlens = _aligned(q, k, v, cu_seqlens)
     L = lib()
     T, H, DK = q.shape
     DV = v.shape[-1]
@@ -186,6 +196,7 @@ def varlen_fwd(q, k, v, cu_seqlens, max_seqlen, scale, eps):
 def varlen_bwd(q, k, v, cu_seqlens, max_seqlen, do, s, km, scale, eps):
     """Packed backward: returns (dq, dk, dv)."""
     _require_gpu(q, k, v, do, cu_seqlens)
+    q, k, v, do, cu_seqlens, s, km = _aligned(q, k, v, do, cu_seqlens, s, km)
     L = lib()
     T, H, DK = q.shape
     DV = v.shape[-1]
@@ -208,6 +219,7 @@ def chunk_reduce(q, k, v, chunk, with_norm=False, p_norm=2.0):
     """Block statistics of piecewise attention.  q,k:[B,H,T,K] v:[B,H,T,V] contiguous.
     Returns fp32 (qc, kc, vc, h, h_norm or None)."""
     _require_gpu(q, k, v)
+    q, k, v = _aligned(q, k, v)
     L = lib()
     B, H, T, K = k.shape
     V = v.shape[-1]
@@ -230,6 +242,7 @@ def chunk_reduce(q, k, v, chunk, with_norm=False, p_norm=2.0):
 def select_blocks(qc, kc, bias, top_k, scale):
     """Indices (int32, ascending) of the top_k key blocks per query block; qc, kc fp32 [B,H,NT,K]."""
     _require_gpu(qc, kc, bias)
+    qc, kc, bias = _aligned(qc, kc, bias)
     L = lib()
     B, H, NT, K = qc.shape
     dev = qc.device
@@ -250,6 +263,7 @@ def piecewise_supported(q, v, block):
 def piecewise_fwd(q, k, v, kc, vc, h, indices, block, scale):
     """Piecewise attention forward; indices int32 [B,H,NT,NS]; kc, vc, h fp32 from chunk_reduce."""
     _require_gpu(q, k, v, kc, vc, h, indices)
+    q, k, v, kc, vc, h, indices = _aligned(q, k, v, kc, vc, h, indices)
     L = lib()
     B, H, T, K = q.shape
     V = v.shape[-1]

@@ -117,3 +117,32 @@ def test_error_is_per_thread_and_does_not_poison():
     q, k, v, do = (t.to(dev) for t in make_qkv(shape, shape, torch.float16, seed=3)[:4])
     o, *_ = _step(hip, q, k, v, do, 1.0 / 256)
     assert torch.isfinite(o).all()
+
+
+def test_views_off_a_16_byte_boundary():
+    """A contiguous view that starts 2 bytes into a buffer: the bindings copy it to aligned memory
+    (the kernels move 16-byte pieces); the C entry point itself refuses such a pointer."""
+    import ctypes
+    from flash_bla import _hip
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    B, H, L, D = 1, 2, 100, 64
+    n = B * H * L * D
+    bufs = [torch.rand(n + 8, device="cuda", dtype=torch.float16) + 0.5 for _ in range(3)]
+    q, k, v = (b[1:1 + n].view(B, H, L, D) for b in bufs)
+    assert q.data_ptr() % 16 != 0 and q.is_contiguous()
+    ref = linear_attention(q.clone(), k.clone(), v.clone())
+    leaves = [t.detach().requires_grad_() for t in (q, k, v)]
+    out = linear_attention(*leaves)
+    assert torch.equal(out, ref)
+    out.backward(torch.ones_like(out))
+    assert all(torch.isfinite(t.grad).all() for t in leaves)
+    lib = _hip.lib()
+    o = torch.empty(B, H, L, D, device="cuda", dtype=torch.float16)
+    s = torch.empty(B, H, D, D, device="cuda")
+    km = torch.empty(B, H, D, device="cuda")
+    ws = torch.empty(lib.fbla_la_workspace_bytes(0, B, H, L, D, D, _hip.F16, _hip.NORMALIZE) + 16, device="cuda",
+                     dtype=torch.uint8)
+    rc = lib.fbla_la_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), None, None, o.data_ptr(), s.data_ptr(),
+                         km.data_ptr(), ws.data_ptr(), ws.numel(), B, H, L, D, D, _hip.F16, _hip.NORMALIZE,
+                         ctypes.c_float(0.01), ctypes.c_float(1e-6), None)
+    assert rc == -1 and b"aligned" in lib.fbla_last_error()
