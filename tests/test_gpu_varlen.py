@@ -144,3 +144,26 @@ def test_varlen_golden_fixtures(path, dtype):
         for b, e in zip(d["cu_seqlens"][:-1], d["cu_seqlens"][1:]):
             floor = d["ref_" + name + "_mag"][b:e] if "ref_" + name + "_mag" in d else None
             assert_parity(t.grad[b:e], d["ref_" + name][b:e], dtype, name, floor)
+
+
+@pytest.mark.parametrize("nseq", [1024, 1025, 3000])
+def test_varlen_many_short_sequences(nseq):
+    """Around and beyond the number of sequences whose lengths the kernels rank in LDS for the
+    longest-first walk (1024): beyond it the sequences are walked in index order."""
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    rng = np.random.default_rng(nseq)
+    lengths = rng.integers(0, 40, nseq).tolist()
+    lengths[7] = 900   # one long sequence among the short ones
+    T, H, D = sum(lengths), 2, 64
+    q, k, v, do = make_qkv((T, H, D), (T, H, D), torch.bfloat16, nseq)
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lengths)]), dtype=torch.int32).cuda()
+    leaves = [t.cuda().requires_grad_() for t in (q, k, v)]
+    o = varlen_linear_attention(*leaves, cu, max(lengths))
+    o.backward(do.cuda())
+    ref = cf.varlen_backward(np64(q), np64(k), np64(v), np64(do), cu.cpu().numpy())
+    assert_parity(o, ref["o"], torch.bfloat16, "o")
+    # gradients sequence by sequence would be 3000 comparisons: compare the long one and the whole
+    b, e = int(cu[7]), int(cu[8])
+    for name, t in zip(("dq", "dk", "dv"), leaves):
+        assert_parity(t.grad[b:e], ref[name][b:e], torch.bfloat16, f"{name} long", ref.get(name + "_mag", ref[name])[b:e])
+        assert_parity(t.grad, ref[name], torch.bfloat16, name, ref.get(name + "_mag"))
