@@ -71,6 +71,7 @@ static Prob make_prob(const int32_t* cu, int64_t N, int64_t H, int64_t L, int64_
                       int flags, float scale, float eps) {
   Prob p;
   p.cu = cu;
+  p.perm = nullptr;
   p.N = (int)N;
   p.H = (int)H;
   p.L = (int)L;

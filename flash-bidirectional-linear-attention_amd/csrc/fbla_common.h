@@ -21,8 +21,16 @@ enum Flags : int {
 // One problem instance.  Dense: cu == nullptr, N = batch, every sequence has L
 // tokens and tensors are [N,H,L,D].  Packed: cu = int32[N+1] on the device and
 // tensors are [T_total,H,D].
+// Packed batches are walked longest sequence first.  Up to kRankInline sequences every
+// workgroup ranks the lengths itself (in LDS, a fraction of a microsecond); up to kRankMax a
+// small kernel writes the order once per call (Prob::perm); beyond that the order is the
+// index order.
+constexpr int kRankInline = 128;
+constexpr int kRankMax = 1 << 16;
+
 struct Prob {
   const int32_t* cu;
+  const int32_t* perm;  // packed: perm[r] = index of the sequence with the r-th largest length, or null
   int N, H, L;  // L: dense length, or max_seqlen upper bound when packed
   int Lk;       // dense only: number of key / value tokens when it differs from L (the number of
                 // queries), else 0.  Only the plan looks at it: kernels get a problem whose L is

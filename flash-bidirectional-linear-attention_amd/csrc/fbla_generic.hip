@@ -556,5 +556,31 @@ void broadcast_rows(const Prob& p, int dtype, const float* vec, void* out, hipSt
   else broadcast_rows_kernel<float><<<grid, block, 0, st>>>(p, vec, (float*)out, ntiles);
 }
 
+// One thread per sequence j counts the sequences that come before it in the order (longer,
+// or as long with a smaller index); the lengths pass through LDS in tiles of the block size.
+__global__ __launch_bounds__(256) void rank_sequences_kernel(const int32_t* __restrict__ cu, int N,
+                                                             int32_t* __restrict__ perm) {
+  __shared__ int tile[256];
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  const int lj = j < N ? cu[j + 1] - cu[j] : 0;
+  int r = 0;
+  for (int base = 0; base < N; base += 256) {
+    const int i = base + threadIdx.x;
+    tile[threadIdx.x] = i < N ? cu[i + 1] - cu[i] : -1;
+    __syncthreads();
+    const int cnt = min(256, N - base);
+    for (int t = 0; t < cnt; ++t) {
+      const int li = tile[t];
+      r += (li > lj) || (li == lj && base + t < j);
+    }
+    __syncthreads();
+  }
+  if (j < N) perm[r] = j;
+}
+
+void rank_sequences(const Prob& p, int32_t* perm, hipStream_t st) {
+  rank_sequences_kernel<<<dim3((unsigned)((p.N + 255) / 256)), dim3(256), 0, st>>>(p.cu, p.N, perm);
+}
+
 }  // namespace generic
 }  // namespace fbla

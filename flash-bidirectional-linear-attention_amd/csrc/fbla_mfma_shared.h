@@ -22,11 +22,14 @@ __device__ __forceinline__ void wave_sync() {
 // Packed sequences have different lengths, and workgroups are dispatched in index
 // order: handing out the longest sequences first (LPT) keeps the last round of
 // workgroups short.  Returns the index of the sequence with the `rank`-th largest
-// length (ties by index); the identity for dense problems, a single sequence, or
-// more sequences than the LDS table holds.  Called by all threads of the workgroup.
-constexpr int kLptMax = 1024;
+// length (ties by index): from the order a kernel wrote before (p.perm), else ranked here
+// in LDS (quadratic in the number of sequences: small batches only); the identity for dense
+// problems, a single sequence, or when neither applies.  Called by all threads of the workgroup.
+constexpr int kLptMax = kRankInline;
 __device__ __forceinline__ int lpt_sequence(const Prob& p, int rank, int* lens /* [kLptMax + 1] */) {
-  if (!p.cu || p.N < 2 || p.N > kLptMax) return rank;
+  if (!p.cu || p.N < 2) return rank;
+  if (p.perm) return __builtin_amdgcn_readfirstlane(p.perm[rank]);
+  if (p.N > kLptMax) return rank;
   const int nthreads = blockDim.x;
   for (int i = threadIdx.x; i < p.N; i += nthreads) lens[i] = p.cu[i + 1] - p.cu[i];
   __syncthreads();

@@ -836,9 +836,11 @@ int select_blocks(const float* qc, const float* kc, const float* bias, int32_t* 
 static Prob dense_prob(int64_t BH, int64_t T, int K, int V) {
   Prob p;
   p.cu = nullptr;
+  p.perm = nullptr;
   p.N = (int)BH;
   p.H = 1;
   p.L = (int)T;
+  p.Lk = 0;
   p.T = BH * T;
   p.DK = K;
   p.DV = V;

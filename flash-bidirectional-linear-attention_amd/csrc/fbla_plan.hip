@@ -75,17 +75,36 @@ static bool fold_reduce(const Prob& p, int reduce_nchunks, int DR, int DC) {
   return extra <= limit;
 }
 
-size_t fwd_workspace_bytes(const Prob& pc, int dtype) {
+// the walking order of a packed batch with too many sequences to rank inside every workgroup
+static size_t perm_bytes(const Prob& p) {
+  return (p.cu && p.N > kRankInline && p.N <= kRankMax) ? align_up((size_t)p.N * sizeof(int32_t), 256) : 0;
+}
+// Writes the order behind the first `used` bytes of the workspace and returns the problem with it.
+static Prob with_order(const Prob& p, void* workspace, size_t used, hipStream_t st) {
+  Prob r = p;
+  if (perm_bytes(p)) {
+    int32_t* perm = reinterpret_cast<int32_t*>((char*)workspace + used);
+    generic::rank_sequences(p, perm, st);
+    r.perm = perm;
+  }
+  return r;
+}
+
+static size_t fwd_used_bytes(const Prob& pc, int dtype) {
   const Prob p = key_side(pc);
   return partial_bytes(p, fwd_chunk(p, dtype));
 }
-
-// partials | S^T | s*dS | (s*dS)^T | dkm/L | per-row scalars
-size_t bwd_workspace_bytes(const Prob& pc, int dtype) {
+static size_t bwd_used_bytes(const Prob& pc, int dtype) {
   const Prob p = query_side(pc);
   return partial_bytes(p, bwd_chunk(p, dtype)) + 3 * state_bytes(p) + vec_bytes(p) +
          tokscal_bytes(p, dtype);
 }
+
+// partials | walking order
+size_t fwd_workspace_bytes(const Prob& pc, int dtype) { return fwd_used_bytes(pc, dtype) + perm_bytes(pc); }
+
+// partials | S^T | s*dS | (s*dS)^T | dkm/L | per-row scalars | walking order
+size_t bwd_workspace_bytes(const Prob& pc, int dtype) { return bwd_used_bytes(pc, dtype) + perm_bytes(pc); }
 
 static int check_cross(const Prob& p, int dtype) {
   if (!cross(p)) return kOk;
@@ -98,9 +117,10 @@ static int check_cross(const Prob& p, int dtype) {
   return kOk;
 }
 
-int forward(const Prob& pc, int dtype, const FwdArgs& a, hipStream_t st) {
-  int rc_cross = check_cross(pc, dtype);
+int forward(const Prob& pc_, int dtype, const FwdArgs& a, hipStream_t st) {
+  int rc_cross = check_cross(pc_, dtype);
   if (rc_cross != kOk) return rc_cross;
+  const Prob pc = with_order(pc_, a.workspace, fwd_used_bytes(pc_, dtype), st);
   const bool is_cross = cross(pc);
   const Prob p = key_side(pc);    // state kernel, reduce
   const Prob pq = query_side(pc);  // output kernel
@@ -145,9 +165,10 @@ int forward(const Prob& pc, int dtype, const FwdArgs& a, hipStream_t st) {
   return kOk;
 }
 
-int backward(const Prob& pc, int dtype, const BwdArgs& a, hipStream_t st) {
-  int rc_cross = check_cross(pc, dtype);
+int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
+  int rc_cross = check_cross(pc_, dtype);
   if (rc_cross != kOk) return rc_cross;
+  const Prob pc = with_order(pc_, a.workspace, bwd_used_bytes(pc_, dtype), st);
   const bool is_cross = cross(pc);
   const Prob p = query_side(pc);  // pass A, reduce
   const Prob pk = key_side(pc);   // pass B
