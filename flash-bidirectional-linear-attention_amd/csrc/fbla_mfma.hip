@@ -1593,12 +1593,32 @@ static int knob(const char* name, int dflt) {
 // Tokens per workgroup for a kernel of which `wgs_per_cu` workgroups fit on a CU:
 // the grid is sized to at most `rounds` full rounds of resident workgroups, with
 // all workgroups doing the same amount of work (no ragged last round).
-static int chunk_for(const Prob& p, int wgs_per_cu, int rounds, int min_chunk, int align) {
+// Packed batches: the grid is laid out for the longest sequence, so a batch with one very
+// long sequence among short ones would leave that sequence to one workgroup per head.  When
+// the longest sequence is more than four times a workgroup's fair share of all tokens, the
+// chunk shrinks to twice that share (the workgroups of the chunks a short sequence does not
+// have exit at once).  `reduction`: the kernel writes a partial per chunk, whose storage grows
+// with the number of chunks of the longest sequence times all (sequence, head) pairs: the
+// number of chunks is then also kept within 1 GiB of partials (reserved, only the chunks
+// that exist are written and read) and 64.
+static int chunk_for(const Prob& p, int wgs_per_cu, int rounds, int min_chunk, int align, bool reduction) {
   const int64_t nh = (int64_t)p.N * p.H;
   const int64_t slots = (int64_t)cu_count() * wgs_per_cu * rounds;
   int64_t nchunks = slots / (nh > 0 ? nh : 1);
   if (nchunks < 1) nchunks = 1;
   int64_t chunk = cdiv64(p.L, nchunks);
+  if (p.cu && nh > 0) {
+    const int64_t fair = cdiv64(p.T * p.H, slots);
+    if (p.L > 4 * fair && chunk > 2 * fair) {
+      chunk = 2 * fair;
+      if (reduction) {
+        const int64_t level_bytes = nh * ((int64_t)p.DK * p.DV + p.DK) * (int64_t)sizeof(float);
+        int64_t levels = (1LL << 30) / (level_bytes > 0 ? level_bytes : 1);
+        levels = levels < 1 ? 1 : (levels > 64 ? 64 : levels);
+        if (chunk < cdiv64(p.L, levels)) chunk = cdiv64(p.L, levels);
+      }
+    }
+  }
   if (chunk < min_chunk) chunk = min_chunk;
   chunk = cdiv64(chunk, align) * align;
   return (int)chunk;
@@ -1607,14 +1627,14 @@ static int chunk_for(const Prob& p, int wgs_per_cu, int rounds, int min_chunk, i
 // Reduction kernels (state, backward pass A): one round of resident workgroups.
 int state_chunk(const Prob& p) {
   static const int per_cu = knob("FBLA_STATE_WGS_PER_CU", 2);
-  return chunk_for(p, per_cu, 1, 256, 64);
+  return chunk_for(p, per_cu, 1, 256, 64, true);
 }
 
 int bwd_a_chunk(const Prob& p) {
   static const int per_cu = knob("FBLA_BWDA_WGS_PER_CU", 2);
   // 128 x 128: one workgroup per CU, steps of 128 tokens
-  if (tiled_dim(p.DK) == 128) return chunk_for(p, 1, 1, 512, 128);
-  return chunk_for(p, per_cu, 1, 256, 128);
+  if (tiled_dim(p.DK) == 128) return chunk_for(p, 1, 1, 512, 128, true);
+  return chunk_for(p, per_cu, 1, 256, 128, true);
 }
 
 // Row-parallel kernels: long enough chunks to amortise the operand prologue.
@@ -1628,7 +1648,7 @@ int rows_chunk(const Prob& p, int DR, int DC) {
   const int big = (tiled_dim(DR) == 128) + (tiled_dim(DC) == 128);
   const int rounds = p.cu ? packed_rounds : (big == 2 ? 1 : big == 1 ? (dense_rounds + 1) / 2 : dense_rounds);
   const int per_cu = big == 0 ? per_cu_knob : (big == 1 ? 2 : 1);
-  return chunk_for(p, per_cu, rounds, 512, big == 2 ? 256 : 128);
+  return chunk_for(p, per_cu, rounds, 512, big == 2 ? 256 : 128, false);
 }
 
 template <typename T, int DK, int DV, bool PAD>
@@ -1902,7 +1922,7 @@ static int run_bwd_tokens(const Prob& p, const void* q, const void* dout, const 
                           const float* km, void* dq, float* tokscal, int64_t total_rows,
                           hipStream_t st) {
   const int big = (tiled_dim(p.DK) == 128) + (tiled_dim(p.DV) == 128);
-  const int chunk = chunk_for(p, big == 2 ? 1 : 2, 1, 512, 128);
+  const int chunk = chunk_for(p, big == 2 ? 1 : 2, 1, 512, 128, false);
   const int nchunks = (int)cdiv64(p.L, chunk);
   if (padded(p))
     return run_bwd_tokens_dims<T, true>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);

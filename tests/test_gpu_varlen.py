@@ -167,3 +167,25 @@ def test_varlen_many_short_sequences(nseq):
     for name, t in zip(("dq", "dk", "dv"), leaves):
         assert_parity(t.grad[b:e], ref[name][b:e], torch.bfloat16, f"{name} long", ref.get(name + "_mag", ref[name])[b:e])
         assert_parity(t.grad, ref[name], torch.bfloat16, name, ref.get(name + "_mag"))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=str)
+@pytest.mark.parametrize("D", [64, 128, 32])
+def test_varlen_one_long_sequence_among_short_ones(D, dtype):
+    """A skewed batch: the long sequence is split over many workgroups (chunks that the short
+    sequences do not have), its partial sums are reduced in chunk order."""
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    lengths = [20] * 17 + [9000] + [35] * 30 + [0, 1]
+    T, H = sum(lengths), 3
+    q, k, v, do = make_qkv((T, H, D), (T, H, D), dtype, D)
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lengths)]), dtype=torch.int32).cuda()
+    leaves = [t.cuda().requires_grad_() for t in (q, k, v)]
+    o = varlen_linear_attention(*leaves, cu, max(lengths))
+    o.backward(do.cuda())
+    ref = cf.varlen_backward(np64(q), np64(k), np64(v), np64(do), cu.cpu().numpy())
+    assert_parity(o, ref["o"], dtype, "o")
+    for name, t in zip(("dq", "dk", "dv"), leaves):
+        for b, e in zip(cu[:-1].tolist(), cu[1:].tolist()):
+            if e > b:
+                floor = ref[name + "_mag"][b:e] if name + "_mag" in ref else None
+                assert_parity(t.grad[b:e], ref[name][b:e], dtype, f"{name}[{b}:{e}]", floor)
