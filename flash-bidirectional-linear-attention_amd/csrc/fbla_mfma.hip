@@ -1914,7 +1914,8 @@ static int run_bwd_tokens_dims(const Prob& p, const void* q, const void* dout, c
     return launch_bwd_tokens<T, 64, 128, PAD>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
   if (DK == 128 && DV == 64)
     return launch_bwd_tokens<T, 128, 64, PAD>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
-  return launch_bwd_tokens<T, 128, 128, PAD>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
+  set_error("the token view alone exists for heads tiled 64 x 128 and 128 x 64");  // others: fused pass A
+  return kErrUnsupported;
 }
 
 template <typename T>
