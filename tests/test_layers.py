@@ -58,8 +58,6 @@ GPU_CASES = {
 def test_fast_mode_matches_torch_mode(name, dtype):
     torch.manual_seed(1)
     make, shape, extra = GPU_CASES[name]
-    if dtype == torch.float16 and name in ("mlla", "rala"):
-        pytest.skip("the rotary features of these blocks are fp32 (mlla.py:32-36)")
     if dtype == torch.float32 and name == "pola_sr2":
         pytest.skip("fewer keys than queries in fp32 needs 64 x 64 heads; this block has 128 x 32")
     layer = make().to("cuda", dtype)
