@@ -34,6 +34,30 @@ namespace mfma {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+// Streaming accesses.  Every token row is read once per kernel and every output row written
+// once, so the rows bypass the caches' retention ("nt" on the instruction): a kernel that
+// starts behind the dirty lines of its predecessor's output then does not wait for their
+// write-back on every fill.  One bit per access class, so each can be switched separately.
+#ifndef FBLA_NT
+#define FBLA_NT 31
+#endif
+constexpr int kNtStateLoad = 1, kNtRowsLoad = 2, kNtRowsStore = 4, kNtPassALoad = 8, kNtPassAStore = 16;
+template <typename V, int BIT>
+__device__ __forceinline__ V load_stream(const void* src) {
+  if constexpr ((FBLA_NT & BIT) != 0) {
+    return __builtin_nontemporal_load(reinterpret_cast<const V*>(src));
+  } else {
+    return *reinterpret_cast<const V*>(src);
+  }
+}
+template <int BIT>
+__device__ __forceinline__ void store_row16(void* dst, u32x4 w) {
+  if constexpr ((FBLA_NT & BIT) != 0) {
+    __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(dst));
+  } else {
+    *reinterpret_cast<u32x4*>(dst) = w;
+  }
+}
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
@@ -121,9 +145,9 @@ __device__ __forceinline__ void load_rows(RowWords<C>& dst, const T* __restrict_
   for (int j = 0; j < 8; ++j) {
     const char* row = base + (size_t)((uint32_t)j * step_b);
     if constexpr (C == 2) {
-      dst.w[j][0] = *reinterpret_cast<const uint32_t*>(row + voff_b);
+      dst.w[j][0] = load_stream<uint32_t, kNtStateLoad>(row + voff_b);
     } else {
-      u32x2 x = *reinterpret_cast<const u32x2*>(row + voff_b);
+      u32x2 x = load_stream<u32x2, kNtStateLoad>(row + voff_b);
       dst.w[j][0] = x[0];
       dst.w[j][1] = x[1];
     }
@@ -728,7 +752,7 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
       const int q = lane + 64 * i, row = q / XCH, ch = q % XCH;
       const int64_t off = piece(tok0 + row, ch, dr);
       if (off >= 0) {
-        dst[i] = *reinterpret_cast<const u32x4*>(src + off);
+        dst[i] = load_stream<u32x4, kNtRowsLoad>(src + off);
       } else {
         dst[i] = u32x4{0u, 0u, 0u, 0u};
       }
@@ -891,7 +915,7 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
     for (int i = 0; i < OI; ++i) {
       const int q = lane + 64 * i, row = q / OCH, ch = q % OCH;
       const int64_t off = piece(t0 + row, ch, dc);
-      if (off >= 0) *reinterpret_cast<u32x4*>(out + off) = wout[i];
+      if (off >= 0) store_row16<kNtRowsStore>(out + off, wout[i]);
     }
     t0 += 32 * WAVES;
   };
@@ -1027,7 +1051,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     for (int i = 0; i < QI; ++i) {
       const int q = lane + 64 * i, row = q / QCH, ch = q % QCH;
       const int64_t off = piece(tok0 + row, ch, dk);
-      dst[i] = off >= 0 ? *reinterpret_cast<const u32x4*>(src + off) : u32x4{0u, 0u, 0u, 0u};
+      dst[i] = off >= 0 ? load_stream<u32x4, kNtPassALoad>(src + off) : u32x4{0u, 0u, 0u, 0u};
     }
   };
   auto load_g = [&](u32x4(&dst)[GI], const T* src, int tok0) {
@@ -1035,7 +1059,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     for (int i = 0; i < GI; ++i) {
       const int q = lane + 64 * i, row = q / GCH, ch = q % GCH;
       const int64_t off = piece(tok0 + row, ch, dv);
-      dst[i] = off >= 0 ? *reinterpret_cast<const u32x4*>(src + off) : u32x4{0u, 0u, 0u, 0u};
+      dst[i] = off >= 0 ? load_stream<u32x4, kNtPassALoad>(src + off) : u32x4{0u, 0u, 0u, 0u};
     }
   };
   auto stash_q = [&](const u32x4(&src)[QI], unsigned char* dstb) {
@@ -1058,7 +1082,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
       const int q = lane + 64 * i, row = q / QCH, ch = q % QCH;
       const int64_t off = piece(tok0 + row, ch, dk);
       if (off >= 0)
-        *reinterpret_cast<u32x4*>(dst + off) = *reinterpret_cast<const u32x4*>(srcb + swz<QROWB>(row, ch));
+        store_row16<kNtPassAStore>(dst + off, *reinterpret_cast<const u32x4*>(srcb + swz<QROWB>(row, ch)));
     }
   };
 
@@ -1338,7 +1362,7 @@ __global__ __launch_bounds__(512, 1) void bwd_a128_kernel(
     for (int i = 0; i < 4; ++i) {
       const int q = 256 * hf + lane + 64 * i;
       const int64_t off = piece(tok0 + (q >> 4), q & 15, rowlen);
-      dst[i] = off >= 0 ? *reinterpret_cast<const u32x4*>(src + off) : u32x4{0u, 0u, 0u, 0u};
+      dst[i] = off >= 0 ? load_stream<u32x4, kNtPassALoad>(src + off) : u32x4{0u, 0u, 0u, 0u};
     }
   };
   auto stash_half = [&](const u32x4(&src)[4], unsigned char* dstb) {
@@ -1520,7 +1544,7 @@ __global__ __launch_bounds__(512, 1) void bwd_a128_kernel(
       const int q = 256 * hf + lane + 64 * i;
       const int64_t off = piece(t0 + (q >> 4), q & 15, dk);
       if (off >= 0)
-        *reinterpret_cast<u32x4*>(dqn + off) = *reinterpret_cast<const u32x4*>(qt + swz<ROWB>(q >> 4, q & 15));
+        store_row16<kNtPassAStore>(dqn + off, *reinterpret_cast<const u32x4*>(qt + swz<ROWB>(q >> 4, q & 15)));
     }
   }
 
