@@ -35,10 +35,10 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # the 256 MiB device copy of the same run reads 256 MiB and the counter shows
 # 128.0 MiB; WRITE_SIZE shows 256.0 MiB for it (factor 1.0).
 MEASURED_TRAFFIC = {
-    "fwd_state": int((2 * 256.1 + 8.1) * 2 ** 20),
+    "fwd_state": int((2 * 256.7 + 8.1) * 2 ** 20),
     "fwd_output": int((2 * 136.2 + 256.0) * 2 ** 20),
     "bwd_pass_a": int((2 * 260.2 + 264.1) * 2 ** 20),
-    "bwd_pass_b": int((2 * 272.2 + 512.0) * 2 ** 20),
+    "bwd_pass_b": int((2 * 264.7 + 512.0) * 2 ** 20),
 }
 
 PHASES = {  # name -> (phase bit, tensors read+written once, entry point)
@@ -167,8 +167,9 @@ def kernel_times(q, k, v, do, n=20):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=200,
+                    help="untimed steps first: a few milliseconds of work do not bring the GPU to its steady clocks")
     ap.add_argument("--T", type=int, default=16384)
     ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16", "fp32"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -240,7 +241,7 @@ def main():
     parity = parity_spot_check(q.detach(), k.detach(), v.detach(), do, o, (q.grad, k.grad, v.grad))
 
     flush = torch.empty(256 << 20, dtype=torch.int8, device=dev)
-    for _ in range(3):
+    for _ in range(args.warmup):
         fwd_only()
     fwd_loop_ms = timed_loop(fwd_only, args.steps)  # back-to-back, no cache-flush write in between
     fwd_q = do_bench(fwd_only, flush)

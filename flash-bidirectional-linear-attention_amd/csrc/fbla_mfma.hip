@@ -34,29 +34,19 @@ namespace mfma {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-// Streaming accesses.  Every token row is read once per kernel and every output row written
-// once, so the rows bypass the caches' retention ("nt" on the instruction): a kernel that
-// starts behind the dirty lines of its predecessor's output then does not wait for their
-// write-back on every fill.  One bit per access class, so each can be switched separately.
+// Which accesses carry the streaming hint (stream_load / stream_store), one bit per class so
+// that each can be switched separately.
 #ifndef FBLA_NT
 #define FBLA_NT 31
 #endif
 constexpr int kNtStateLoad = 1, kNtRowsLoad = 2, kNtRowsStore = 4, kNtPassALoad = 8, kNtPassAStore = 16;
 template <typename V, int BIT>
 __device__ __forceinline__ V load_stream(const void* src) {
-  if constexpr ((FBLA_NT & BIT) != 0) {
-    return __builtin_nontemporal_load(reinterpret_cast<const V*>(src));
-  } else {
-    return *reinterpret_cast<const V*>(src);
-  }
+  return stream_load<(FBLA_NT & BIT) != 0, V>(src);
 }
 template <int BIT>
 __device__ __forceinline__ void store_row16(void* dst, u32x4 w) {
-  if constexpr ((FBLA_NT & BIT) != 0) {
-    __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(dst));
-  } else {
-    *reinterpret_cast<u32x4*>(dst) = w;
-  }
+  stream_store<(FBLA_NT & BIT) != 0>(dst, w);
 }
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -1672,7 +1662,8 @@ int rows_chunk(const Prob& p, int DR, int DC) {
   const int big = (tiled_dim(DR) == 128) + (tiled_dim(DC) == 128);
   const int rounds = p.cu ? packed_rounds : (big == 2 ? 1 : big == 1 ? (dense_rounds + 1) / 2 : dense_rounds);
   const int per_cu = big == 0 ? per_cu_knob : (big == 1 ? 2 : 1);
-  return chunk_for(p, per_cu, rounds, 512, big == 2 ? 256 : 128, false);
+  static const int min_chunk = knob("FBLA_ROWS_MIN_CHUNK", 512);
+  return chunk_for(p, per_cu, rounds, min_chunk, big == 2 ? 256 : 128, false);
 }
 
 template <typename T, int DK, int DV, bool PAD>

@@ -30,10 +30,17 @@ using mfma::f32x16;
 using mfma::kLptMax;
 using mfma::lpt_sequence;
 using mfma::reduce_store_block;
+using mfma::stream_load;
+using mfma::stream_store;
 using mfma::swz;
 using mfma::wave_sync;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+// streaming hint per access class: 1 = state kernel loads, 2 = rows kernel tile loads,
+// 4 = rows kernel stores
+#ifndef FBLA_NT32
+#define FBLA_NT32 7
+#endif
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kThreads = 256;
@@ -119,11 +126,12 @@ __global__ __launch_bounds__(kThreads, 2) void state32_kernel(
       const size_t kro = (size_t)(2 * s + kb) * kstep, vro = (size_t)(2 * s + kb) * vstep;
 #pragma unroll
       for (int a = 0; a < 2; ++a) {
-        const float kx = kp[kro + kcol[a]], vx = vp[vro + vcol[a]];
+        const float kx = stream_load<(FBLA_NT32 & 1) != 0, float>(kp + kro + kcol[a]);
+        const float vx = stream_load<(FBLA_NT32 & 1) != 0, float>(vp + vro + vcol[a]);
         b.k[s][a] = kok[a] ? kx : 0.f;
         b.v[s][a] = vok[a] ? vx : 0.f;
         if constexpr (SPLIT_KD) {
-          const float dx = dp[kro + kcol[a]];
+          const float dx = stream_load<(FBLA_NT32 & 1) != 0, float>(dp + kro + kcol[a]);
           b.d[s][a] = kok[a] ? dx : 0.f;
         }
       }
@@ -305,7 +313,7 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
       const int q = lane + 64 * i, row = q >> 4, ch = q & 15;
       const int tok = tok0 + row;
       dst[i] = (tok < t_end && (!PAD || ch * 4 < dr))
-                   ? *reinterpret_cast<const f32x4*>(src + (row0 + (int64_t)tok * rstride) * dr + ch * 4)
+                   ? stream_load<(FBLA_NT32 & 2) != 0, f32x4>(src + (row0 + (int64_t)tok * rstride) * dr + ch * 4)
                    : f32x4{0.f, 0.f, 0.f, 0.f};
     }
   };
@@ -435,8 +443,8 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
       const int q = lane + 64 * i, row = q >> 4, ch = q & 15;
       const int tok = t0 + row;
       if (tok < t_end && (!PAD || ch * 4 < dc))
-        *reinterpret_cast<f32x4*>(job.out + (row0 + (int64_t)tok * rstride) * dc + ch * 4) =
-            *reinterpret_cast<const f32x4*>(stage + swz<256>(row, ch));
+        stream_store<(FBLA_NT32 & 4) != 0>(job.out + (row0 + (int64_t)tok * rstride) * dc + ch * 4,
+                                           *reinterpret_cast<const f32x4*>(stage + swz<256>(row, ch)));
     }
     if constexpr (TOKENS && DEN) {  // the second gradient, dq = dz km, through the same tile
       wave_sync();
@@ -454,8 +462,8 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
         const int q = lane + 64 * i, row = q >> 4, ch = q & 15;
         const int tok = t0 + row;
         if (tok < t_end && (!PAD || ch * 4 < dc))
-          *reinterpret_cast<f32x4*>(job.out2 + (row0 + (int64_t)tok * rstride) * dc + ch * 4) =
-              *reinterpret_cast<const f32x4*>(stage + swz<256>(row, ch));
+          stream_store<(FBLA_NT32 & 4) != 0>(job.out2 + (row0 + (int64_t)tok * rstride) * dc + ch * 4,
+                                             *reinterpret_cast<const f32x4*>(stage + swz<256>(row, ch)));
       }
     }
     t0 = tn;

@@ -10,6 +10,27 @@ namespace mfma {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
+// Streaming accesses.  Every token row is read once per kernel and every output row written
+// once, so the rows bypass the caches' retention ("nt" on the instruction): a kernel that
+// starts behind the dirty lines of its predecessor's output then does not wait for their
+// write-back on every fill.
+template <bool NT, typename V>
+__device__ __forceinline__ V stream_load(const void* src) {
+  if constexpr (NT) {
+    return __builtin_nontemporal_load(reinterpret_cast<const V*>(src));
+  } else {
+    return *reinterpret_cast<const V*>(src);
+  }
+}
+template <bool NT, typename V>
+__device__ __forceinline__ void stream_store(void* dst, V w) {
+  if constexpr (NT) {
+    __builtin_nontemporal_store(w, reinterpret_cast<V*>(dst));
+  } else {
+    *reinterpret_cast<V*>(dst) = w;
+  }
+}
+
 // Orders this wave's LDS traffic: everything written before is visible to every
 // lane of the wave after (LDS executes a wave's instructions in order; this keeps
 // the compiler from moving accesses across the point).
