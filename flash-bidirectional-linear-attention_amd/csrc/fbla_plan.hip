@@ -77,7 +77,8 @@ static bool fold_reduce(const Prob& p, int reduce_nchunks, int DR, int DC) {
 
 // the walking order of a packed batch with too many sequences to rank inside every workgroup
 static size_t perm_bytes(const Prob& p) {
-  return (p.cu && p.N > kRankInline && p.N <= kRankMax) ? align_up((size_t)p.N * sizeof(int32_t), 256) : 0;
+  static const int inline_max = [] { const char* v = getenv("FBLA_RANK_INLINE"); return v ? atoi(v) : kRankInline; }();
+  return (p.cu && p.N > inline_max && p.N >= 2 && p.N <= kRankMax) ? align_up((size_t)p.N * sizeof(int32_t), 256) : 0;
 }
 // Writes the order behind the first `used` bytes of the workspace and returns the problem with it.
 static Prob with_order(const Prob& p, void* workspace, size_t used, hipStream_t st) {
