@@ -1662,7 +1662,12 @@ int rows_chunk(const Prob& p, int DR, int DC) {
   const int big = (tiled_dim(DR) == 128) + (tiled_dim(DC) == 128);
   const int rounds = p.cu ? packed_rounds : (big == 2 ? 1 : big == 1 ? (dense_rounds + 1) / 2 : dense_rounds);
   const int per_cu = big == 0 ? per_cu_knob : (big == 1 ? 2 : 1);
-  static const int min_chunk = knob("FBLA_ROWS_MIN_CHUNK", 512);
+  static const int min_chunk_knob = knob("FBLA_ROWS_MIN_CHUNK", 512);
+  // a problem too small to give every CU a workgroup: shorter chunks (the operand build of the
+  // extra workgroups costs less than the idle CUs)
+  int min_chunk = min_chunk_knob;
+  const int64_t nh = (int64_t)p.N * p.H;
+  while (min_chunk > 128 && big < 2 && nh * cdiv64(p.L, min_chunk) < cu_count()) min_chunk /= 2;
   return chunk_for(p, per_cu, rounds, min_chunk, big == 2 ? 256 : 128, false);
 }
 
