@@ -90,7 +90,8 @@ bool bwd_a_supported(const Prob& p, int dtype);
 // dense 32 x 32 heads: the row-parallel kernels take two tokens per row and need the finished
 // matrices (no partial sums in their prologue)
 bool pair_mode(const Prob& p, int dtype);
-int state_chunk(const Prob& p);
+// block_stats: the launch that also writes piecewise attention's block statistics
+int state_chunk(const Prob& p, bool block_stats = false);
 int bwd_a_chunk(const Prob& p);
 int rows_chunk(const Prob& p, int DR, int DC);
 // fin_mat / fin_vec (only with nchunks == 1): store the finished, scaled matrix [N*H,DK,DV] and

@@ -485,6 +485,192 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
 }
 
 // ===========================================================================
+// state kernel for heads tiled 128 x 128 (plain operator: no rotary keys, no row scaling,
+// no block statistics)
+// ===========================================================================
+// Every wave holds the whole 128 x 128 state (256 accumulator registers, which is why one
+// workgroup of four waves has a CU to itself) and the waves take interleaved steps of two
+// 16-token tiles.  Each row is therefore read by exactly one wave; in state_kernel's split by
+// 64 x 64 blocks every 128-byte half of a row is read by two waves, and with streaming loads
+// the second read is often served by HBM again.  A lane owns four adjacent features of k and
+// of v (one 8-byte load per row and tensor: 32 loads per step, so that "all but the newest
+// step" still fits the 6-bit counter of outstanding loads), which makes accumulator (a, b),
+// register r of lane (pp, kb) the element S[4 m + a][4 pp + b], m = 8 (r / 4) + 4 kb + r % 4.
+template <typename T, bool PAD>
+__global__ __launch_bounds__(kThreads, 1) void state128_kernel(Prob p, const T* __restrict__ kn,
+                                                               const T* __restrict__ v,
+                                                               float* __restrict__ partial,
+                                                               float* __restrict__ fin_mat,
+                                                               float* __restrict__ fin_vec, int chunk,
+                                                               int nchunks) {
+  const int dk = PAD ? p.DK : 128, dv = PAD ? p.DV : 128;  // row lengths in memory
+  constexpr int G = kWaves, TILES = 2, kStep = 16 * TILES;
+  __shared__ float red[64 * 65];  // one quarter of a wave's sums: [value][lane]
+  __shared__ int lpt_lens[kLptMax + 1];
+  const int wg_nh = blockIdx.x / nchunks, c = blockIdx.x - wg_nh * nchunks;
+  const int h = wg_nh % p.H;
+  const int n = lpt_sequence(p, wg_nh / p.H, lpt_lens);
+  const int nh = n * p.H + h;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t_begin = c * chunk;
+  if (t_begin >= len) {
+    if (fin_mat && c == 0) {  // empty sequence: its state is zero
+      for (int e = threadIdx.x; e < dk * dv; e += kThreads) fin_mat[(int64_t)nh * dk * dv + e] = 0.f;
+      if (fin_vec)
+        for (int e = threadIdx.x; e < dk; e += kThreads) fin_vec[(int64_t)nh * dk + e] = 0.f;
+    }
+    return;
+  }
+  const int t_end = min(len, t_begin + chunk);
+  row_base(p, n, h, bos, row0, rstride);
+
+  const int g = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int pp = lane & 31, kb = lane >> 5;
+  // this lane's four features, and whether they exist (head dims are multiples of 8)
+  const bool k_ok = !PAD || 4 * pp < dk, v_ok = !PAD || 4 * pp < dv;
+  const int kcol0 = k_ok ? 4 * pp : 0, vcol0 = v_ok ? 4 * pp : 0;
+  const uint32_t k_keep = k_ok ? ~0u : 0u, v_keep = v_ok ? ~0u : 0u;
+  const uint32_t kstep = (uint32_t)(rstride * dk), vstep = (uint32_t)(rstride * dv);
+  const uint32_t kvoff = (uint32_t)(8 * kb) * kstep + (uint32_t)kcol0;
+  const uint32_t vvoff = (uint32_t)(8 * kb) * vstep + (uint32_t)vcol0;
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  float ks[4] = {0.f, 0.f, 0.f, 0.f};
+
+  struct Buf {
+    RowWords<4> k[TILES], v[TILES];
+  };
+  // as in state_kernel: a tile that would cross the end of the chunk is moved back so that it
+  // ends there, and the rows it shares with the tile before it are zeroed before use
+  auto fetch = [&](Buf& b, int tok) {
+#pragma unroll
+    for (int u = 0; u < TILES; ++u) {
+      const int tb = min(tok + 16 * u, t_end - 16);
+      const int64_t row = row0 + (int64_t)tb * rstride;
+      load_rows<T, 4>(b.k[u], kn + row * dk, kstep, kvoff);
+      load_rows<T, 4>(b.v[u], v + row * dv, vstep, vvoff);
+    }
+  };
+  auto fetch_checked = [&](Buf& b, int tok) {  // chunk shorter than a tile
+#pragma unroll
+    for (int u = 0; u < TILES; ++u) {
+      const int rows = t_end - (tok + 16 * u);
+      const int64_t row = row0 + (int64_t)(tok + 16 * u) * rstride;
+      load_rows_checked<T, 4>(b.k[u], kn + row * dk, kstep, 8 * kb, kcol0, rows);
+      load_rows_checked<T, 4>(b.v[u], v + row * dv, vstep, 8 * kb, vcol0, rows);
+    }
+  };
+  auto compute = [&](Buf& b, int tok, bool checked) {
+#pragma unroll
+    for (int u = 0; u < TILES; ++u) {
+      if constexpr (PAD) {
+        keep_rows<4>(b.k[u], k_keep);
+        keep_rows<4>(b.v[u], v_keep);
+      }
+      if (!checked && tok + kStep > t_end) {  // last step of the chunk: some tiles were moved back
+        const int lo = min(16, tok + 16 * u - min(tok + 16 * u, t_end - 16));
+        mask_rows<4>(b.k[u], 8 * kb, lo);
+      }
+      u32x4 A[4], B[4];
+      transpose_rows<4>(b.k[u], A);
+      transpose_rows<4>(b.v[u], B);
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb) acc[a][bb] = Ops<T>::mma(A[a], B[bb], acc[a][bb]);
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ks[a] = Ops<T>::dot2(A[a][i], Ops<T>::kOnes, ks[a]);
+    }
+  };
+  int t0 = t_begin + kStep * g;
+  if (t_end - t_begin < 16) {
+    if (t0 < t_end) {
+      Buf b0;
+      fetch_checked(b0, t0);
+      compute(b0, t0, true);
+    }
+  } else if (t0 < t_end) {
+    Buf b0, b1;
+    fetch(b0, t0);
+    while (true) {
+      int tn = t0 + kStep * G;
+      fetch(b1, tn);
+      compute(b0, t0, false);
+      t0 = tn;
+      if (t0 >= t_end) break;
+      tn = t0 + kStep * G;
+      fetch(b0, tn);
+      compute(b1, t0, false);
+      t0 = tn;
+      if (t0 >= t_end) break;
+    }
+  }
+
+  // Fixed-order sum over the four waves, a quarter of the state (accumulator row a: 64
+  // registers) at a time through LDS: 2 -> 0, 3 -> 1, 1 -> 0 with the roles rotated by a, so
+  // that quarter a ends in wave a and the four quarters are stored by four waves.  One chunk
+  // per (sequence, head): the sum is final and is stored scaled where the reduce kernel would
+  // have put it; otherwise this chunk's partial is stored.
+  float* mat = fin_mat ? fin_mat + (int64_t)nh * dk * dv
+                       : partial + ((int64_t)nh * nchunks + c) * (dk * dv + dk);
+  float* vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : mat + dk * dv;
+  const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
+  const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int role = (g + G - a) & (G - 1);
+    auto spill = [&]() {
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) red[(b * 16 + r) * 64 + lane] = acc[a][b][r];
+      red[64 * 64 + lane] = ks[a];
+    };
+    auto absorb = [&]() {
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] += red[(b * 16 + r) * 64 + lane];
+      ks[a] += red[64 * 64 + lane];
+    };
+    if (role == 2) spill();
+    __syncthreads();
+    if (role == 0) absorb();
+    __syncthreads();
+    if (role == 3) spill();
+    __syncthreads();
+    if (role == 1) absorb();
+    __syncthreads();
+    if (role == 1) spill();
+    __syncthreads();
+    if (role == 0) {
+      absorb();
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = 4 * (8 * (r >> 2) + 4 * kb + (r & 3)) + a;
+        if (row < dk && 4 * pp < dv)
+          *reinterpret_cast<f32x4*>(mat + row * dv + 4 * pp) =
+              f32x4{acc[a][0][r] * mscale, acc[a][1][r] * mscale, acc[a][2][r] * mscale, acc[a][3][r] * mscale};
+      }
+      const float tot = ks[a] + __shfl_xor(ks[a], 32);
+      if (vec && kb == 0 && 4 * pp + a < dk) vec[4 * pp + a] = tot * vscale;
+    }
+    __syncthreads();  // `red` is reused by the next quarter
+  }
+}
+
+// ===========================================================================
 // rows kernel: out_t = (x_t M) * rowscale_t + addvec
 // ===========================================================================
 // LDS layout of a DR x DC matrix operand M: fragment f = (b*KS + s)*2 + hl holds,
@@ -1639,8 +1825,15 @@ static int chunk_for(const Prob& p, int wgs_per_cu, int rounds, int min_chunk, i
 }
 
 // Reduction kernels (state, backward pass A): one round of resident workgroups.
-int state_chunk(const Prob& p) {
+// 128 x 128 states of the plain operator: state128_kernel, one workgroup per CU
+static bool whole_state_per_wave(const Prob& p) {
+  static const int on = knob("FBLA_STATE128", 1);  // 2 = off (A/B comparisons)
+  return on == 1 && tiled_dim(p.DK) == 128 && tiled_dim(p.DV) == 128 && !(p.flags & kDecoupled);
+}
+
+int state_chunk(const Prob& p, bool block_stats) {
   static const int per_cu = knob("FBLA_STATE_WGS_PER_CU", 2);
+  if (!block_stats && whole_state_per_wave(p)) return chunk_for(p, 1, 1, 256, 64, true);
   return chunk_for(p, per_cu, 1, 256, 64, true);
 }
 
@@ -1680,6 +1873,12 @@ static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, fl
   // same tokens and so have half as many bytes in flight per token (packed batches with a
   // few long sequences finish 9 % sooner)
   constexpr int TL = (DK == 128 && DV == 128) ? 2 : 1;
+  if constexpr (DK == 128 && DV == 128) {
+    if (!bs.kc && !tokscal && whole_state_per_wave(p)) {
+      state128_kernel<T, PAD><<<grid, block, 0, st>>>(p, kn, v, partial, fm, fv, chunk, nchunks);
+      return;
+    }
+  }
   if (bs.kc) {
     if constexpr (!PAD)
       state_kernel<T, DK, DV, false, 1, false, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);

@@ -854,7 +854,7 @@ static Prob dense_prob(int64_t BH, int64_t T, int K, int V) {
 // wanted (one partial per chunk), else whatever fills the machine
 static int state_chunk_for(const Prob& p, int dtype, int chunk, bool per_chunk) {
   if (per_chunk) return chunk;
-  return mfma::supported(p, dtype) ? mfma::state_chunk(p) : generic::state_chunk(p);
+  return mfma::supported(p, dtype) ? mfma::state_chunk(p, true) : generic::state_chunk(p);
 }
 
 size_t chunk_reduce_workspace_bytes(int64_t BH, int64_t T, int K, int V, int chunk, int dtype,
