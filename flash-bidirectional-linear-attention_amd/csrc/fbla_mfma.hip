@@ -1825,16 +1825,21 @@ static int chunk_for(const Prob& p, int wgs_per_cu, int rounds, int min_chunk, i
 }
 
 // Reduction kernels (state, backward pass A): one round of resident workgroups.
-// 128 x 128 states of the plain operator: state128_kernel, one workgroup per CU
-static bool whole_state_per_wave(const Prob& p) {
+// 128 x 128 states of the plain operator: state128_kernel, one workgroup per CU, when that
+// leaves a workgroup at least 1024 tokens.  Its four waves each sum the whole state over a
+// quarter of the tokens and add the four sums at the end; with fewer tokens that addition
+// costs more than state_kernel's second read of every row.
+static int whole_state_chunk(const Prob& p) {
   static const int on = knob("FBLA_STATE128", 1);  // 2 = off (A/B comparisons)
-  return on == 1 && tiled_dim(p.DK) == 128 && tiled_dim(p.DV) == 128 && !(p.flags & kDecoupled);
+  if (on != 1 || tiled_dim(p.DK) != 128 || tiled_dim(p.DV) != 128 || (p.flags & kDecoupled)) return 0;
+  const int chunk = chunk_for(p, 1, 1, 256, 64, true);
+  return chunk >= 1024 ? chunk : 0;
 }
 
 int state_chunk(const Prob& p, bool block_stats) {
   static const int per_cu = knob("FBLA_STATE_WGS_PER_CU", 2);
-  if (!block_stats && whole_state_per_wave(p)) return chunk_for(p, 1, 1, 256, 64, true);
-  return chunk_for(p, per_cu, 1, 256, 64, true);
+  const int whole = block_stats ? 0 : whole_state_chunk(p);
+  return whole ? whole : chunk_for(p, per_cu, 1, 256, 64, true);
 }
 
 int bwd_a_chunk(const Prob& p) {
@@ -1874,7 +1879,7 @@ static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, fl
   // few long sequences finish 9 % sooner)
   constexpr int TL = (DK == 128 && DV == 128) ? 2 : 1;
   if constexpr (DK == 128 && DV == 128) {
-    if (!bs.kc && !tokscal && whole_state_per_wave(p)) {
+    if (!bs.kc && !tokscal && whole_state_chunk(p) == chunk) {
       state128_kernel<T, PAD><<<grid, block, 0, st>>>(p, kn, v, partial, fm, fv, chunk, nchunks);
       return;
     }

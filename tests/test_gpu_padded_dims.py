@@ -103,6 +103,54 @@ def test_heads_tiled_128_by_128():
     _check_dense("linear", 3, 2, 129, 72, 128, torch.bfloat16, 17)
 
 
+@pytest.mark.parametrize("dims,dtype,L", [((128, 128), torch.bfloat16, 1030), ((96, 120), torch.float16, 1100),
+                                           ((128, 72), torch.bfloat16, 2049)])
+def test_whole_state_per_wave_dense(dims, dtype, L):
+    """256 heads of more than 1024 tokens with a state tiled 128 x 128: the state kernel in which
+    every wave keeps the whole state.  A few heads are checked against the oracle."""
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    DK, DV = dims
+    B, H = 16, 16
+    g = torch.Generator().manual_seed(DK + L)
+    q = (torch.nn.functional.elu(torch.randn(B, H, L, DK, generator=g)) + 1).to(dtype)
+    k = (torch.nn.functional.elu(torch.randn(B, H, L, DK, generator=g)) + 1).to(dtype)
+    v = torch.randn(B, H, L, DV, generator=g).to(dtype)
+    do = torch.randn(B, H, L, DV, generator=g).to(dtype)
+    leaves = [t.cuda().requires_grad_() for t in (q, k, v)]
+    o = linear_attention(*leaves)
+    o.backward(do.cuda())
+    for b, h in ((0, 0), (7, 9), (15, 15)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        ref = cf.dense_backward(np64(q[sl]), np64(k[sl]), np64(v[sl]), np64(do[sl]), 1.0 / L, 1e-6, True)
+        tag = f"{dtype} DK{DK} DV{DV} head ({b},{h})"
+        assert_parity(o[sl], ref["o"], dtype, f"o {tag}")
+        for name, t in zip(("dq", "dk", "dv"), leaves):
+            assert_parity(t.grad[sl], ref[name], dtype, f"{name} {tag}", ref.get(name + "_mag"))
+
+
+def test_whole_state_per_wave_packed():
+    """The same kernel on a packed batch: 320 (sequence, head) pairs, the longest sequence above
+    1024 tokens, among them sequences shorter than one tile, of one token and empty ones."""
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    H, DK, DV, dtype = 8, 128, 128, torch.bfloat16
+    lengths = [1500, 1024, 1, 0, 17, 2100, 15, 16, 33, 700] * 4
+    T = sum(lengths)
+    q, k, v, do = make_qkv((T, H, DK), (T, H, DV), dtype, 77)
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lengths)]), dtype=torch.int32).cuda()
+    leaves = [t.cuda().requires_grad_() for t in (q, k, v)]
+    o = varlen_linear_attention(*leaves, cu, max(lengths))
+    o.backward(do.cuda())
+    for h in (0, 5):
+        hs = slice(h, h + 1)
+        ref = cf.varlen_backward(np64(q[:, hs]), np64(k[:, hs]), np64(v[:, hs]), np64(do[:, hs]), cu.cpu().numpy())
+        assert_parity(o[:, hs], ref["o"], dtype, f"o head {h}")
+        for name, t in zip(("dq", "dk", "dv"), leaves):
+            for b, e in zip(cu[:-1].tolist(), cu[1:].tolist()):
+                if e > b:
+                    floor = ref[name + "_mag"][b:e] if name + "_mag" in ref else None
+                    assert_parity(t.grad[b:e, hs], ref[name][b:e], dtype, f"{name}[{b}:{e}] head {h}", floor)
+
+
 @pytest.mark.parametrize("dims", [(32, 32), (16, 16), (4, 4), (24, 40), (64, 32), (32, 64), (60, 12), (48, 48)])
 def test_fp32_head_dims_up_to_64(dims):
     """fp32 inputs: head dims that are multiples of 4 up to 64 run on the fp32 matrix instructions."""
