@@ -232,7 +232,8 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
   __shared__ float red[G > 1 ? NB * 64 * 66 : 1];  // per-group reduction buffers, [value][lane]
 
   __shared__ int lpt_lens[kLptMax + 1];
-  const int wg_nh = blockIdx.x / nchunks, c = blockIdx.x - wg_nh * nchunks;
+  const int wg_item = packed_item(p, blockIdx.x, p.H * nchunks);
+  const int wg_nh = wg_item / nchunks, c = wg_item - wg_nh * nchunks;
   const int h = wg_nh % p.H;
   const int n = lpt_sequence(p, wg_nh / p.H, lpt_lens);
   const int nh = n * p.H + h;
@@ -507,7 +508,8 @@ __global__ __launch_bounds__(kThreads, 1) void state128_kernel(Prob p, const T* 
   constexpr int G = kWaves, TILES = 2, kStep = 16 * TILES;
   __shared__ float red[64 * 65];  // one quarter of a wave's sums: [value][lane]
   __shared__ int lpt_lens[kLptMax + 1];
-  const int wg_nh = blockIdx.x / nchunks, c = blockIdx.x - wg_nh * nchunks;
+  const int wg_item = packed_item(p, blockIdx.x, p.H * nchunks);
+  const int wg_nh = wg_item / nchunks, c = wg_item - wg_nh * nchunks;
   const int h = wg_nh % p.H;
   const int n = lpt_sequence(p, wg_nh / p.H, lpt_lens);
   const int nh = n * p.H + h;
@@ -876,7 +878,8 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
   float* lds_add = reinterpret_cast<float*>(smem + LY::kAdd);
   float* lds_max = reinterpret_cast<float*>(smem + LY::kMax);
 
-  const int wg_nh = wg / nchunks, c = wg - wg_nh * nchunks;
+  const int wg_item = packed_item(p, wg, p.H * nchunks);
+  const int wg_nh = wg_item / nchunks, c = wg_item - wg_nh * nchunks;
   const int h = wg_nh % p.H;
   const int n = lpt_sequence(p, wg_nh / p.H, reinterpret_cast<int*>(smem + LY::kLpt));
   const int nh = n * p.H + h;
@@ -1168,7 +1171,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
   constexpr int QI = 32 * QCH / 64, GI = 32 * GCH / 64;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
-  const int wg_nh = blockIdx.x / nchunks, c = blockIdx.x - wg_nh * nchunks;
+  const int wg_item = packed_item(p, blockIdx.x, p.H * nchunks);
+  const int wg_nh = wg_item / nchunks, c = wg_item - wg_nh * nchunks;
   const int h = wg_nh % p.H;
   const int n = lpt_sequence(p, wg_nh / p.H, reinterpret_cast<int*>(smem + LY::kLpt));
   const int nh = n * p.H + h;
@@ -1497,7 +1501,8 @@ __global__ __launch_bounds__(512, 1) void bwd_a128_kernel(
   const int dk = PAD ? p.DK : 128, dv = PAD ? p.DV : 128;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
-  const int wg_nh = blockIdx.x / nchunks, c = blockIdx.x - wg_nh * nchunks;
+  const int wg_item = packed_item(p, blockIdx.x, p.H * nchunks);
+  const int wg_nh = wg_item / nchunks, c = wg_item - wg_nh * nchunks;
   const int h = wg_nh % p.H;
   const int n = lpt_sequence(p, wg_nh / p.H, reinterpret_cast<int*>(smem + LY::kLpt));
   const int nh = n * p.H + h;
@@ -1993,8 +1998,25 @@ static int run_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, int 
   return run_rows_dims<T, false>(p, job, job2, dr, dc, st);
 }
 
-void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,
+// Packed batches, which kernels keep the workgroups of a sequence on one XCD (packed_item):
+// bit 0 the state kernels, bit 1 the row-parallel kernels, bit 2 backward pass A.  The
+// row-parallel kernels gain (their stores come in 128-byte pieces a token row apart, and the
+// pieces of the other heads are then written at about the same time: forward output 89 -> 82 us,
+// pass B 152 -> 145 us at 64 sequences, H=16, D=64; 3-7 % of forward and backward from 16 to
+// 256 sequences); the reductions lose a little of the longest-first balance and gain nothing,
+// and so do the row-parallel kernels with 128-wide tiles (one or two workgroups per CU, several
+// rounds of them).
+static bool small_tiles(int DR, int DC) { return tiled_dim(DR) == 64 && tiled_dim(DC) == 64; }
+static Prob xcd_ordered(const Prob& p, int kernel_bit) {
+  static const int mask = [] { const char* v = getenv("FBLA_XCD_ORDER"); return v ? atoi(v) : 2; }();
+  Prob r = p;
+  if (p.cu && (mask & kernel_bit)) r.flags |= kXcdOrder;
+  return r;
+}
+
+void state(const Prob& p_, int dtype, const void* kn, const void* v, const void* kd, float* partial,
            int chunk, int nchunks, hipStream_t st, float* fin_mat, float* fin_vec) {
+  const Prob p = xcd_ordered(p_, 1);
   const BlockStats none{nullptr, nullptr, 0};
   if (dtype == kF32)
     return mfma32::state(p, (const float*)kn, (const float*)v, (const float*)kd, partial, nullptr, 0, chunk,
@@ -2023,15 +2045,17 @@ void scaled_state(const Prob& p, int dtype, const void* qn, const void* qd, cons
     run_state<__bf16>(p, qn, dout, qn, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, none, st);
 }
 
-int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {
+int rows(const Prob& p_, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {
+  const Prob p = small_tiles(DR, DC) ? xcd_ordered(p_, 2) : p_;
   if (dtype == kF32) return mfma32::rows(p, job, nullptr, DR, DC, st);
   if (dtype == kF16) return run_rows<_Float16>(p, job, nullptr, DR, DC, st);
   return run_rows<__bf16>(p, job, nullptr, DR, DC, st);
 }
 
 // two jobs of the same shape and normalisation mode in one launch
-int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, int DR, int DC,
+int rows2(const Prob& p_, int dtype, const RowsJob& job0, const RowsJob& job1, int DR, int DC,
           hipStream_t st) {
+  const Prob p = small_tiles(DR, DC) ? xcd_ordered(p_, 2) : p_;
   if (dtype == kF32) return mfma32::rows(p, job0, &job1, DR, DC, st);
   if (dtype == kF16) return run_rows<_Float16>(p, job0, &job1, DR, DC, st);
   return run_rows<__bf16>(p, job0, &job1, DR, DC, st);
@@ -2107,9 +2131,10 @@ static int run_bwd_a(const Prob& p, const void* qn, const void* qd, const void* 
   return run_bwd_a_pad<T, false>(p, qn, qd, dout, S, km, dqn, dqd, partial, fm, fv, chunk, nchunks, st);
 }
 
-int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout, const float* S,
+int bwd_a(const Prob& p_, int dtype, const void* qn, const void* qd, const void* dout, const float* S,
           const float* km, void* dqn, void* dqd, float* partial, int chunk, int nchunks,
           hipStream_t st, float* fin_mat, float* fin_vec) {
+  const Prob p = xcd_ordered(p_, 4);
   if (dtype == kF16)
     return run_bwd_a<_Float16>(p, qn, qd, dout, S, km, dqn, dqd, partial, fin_mat, fin_vec, chunk, nchunks, st);
   return run_bwd_a<__bf16>(p, qn, qd, dout, S, km, dqn, dqd, partial, fin_mat, fin_vec, chunk, nchunks, st);

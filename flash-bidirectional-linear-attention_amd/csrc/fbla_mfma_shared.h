@@ -40,6 +40,20 @@ __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Workgroups are dispatched round-robin over the eight XCDs (workgroup i runs on XCD i % 8).
+// In a packed batch the heads of one token sit next to each other in memory, so the workgroups
+// of one sequence (its heads and chunks: `per_seq` of them) should run at the same time and
+// behind the same L2: workgroup i takes item j of XCD x = i % 8, j = i / 8, and the XCDs take
+// the sequences (in walking order) round-robin.  Sequences beyond the last multiple of eight
+// keep the plain order.  Returns the item index (sequence rank * per_seq + item within it).
+__device__ __forceinline__ int packed_item(const Prob& p, int wg, int per_seq) {
+  if (!(p.flags & kXcdOrder)) return wg;
+  const int full = (p.N / 8) * 8 * per_seq;
+  if (wg >= full) return wg;
+  const int xcd = wg & 7, j = wg >> 3;
+  return ((j / per_seq) * 8 + xcd) * per_seq + j % per_seq;
+}
+
 // Packed sequences have different lengths, and workgroups are dispatched in index
 // order: handing out the longest sequences first (LPT) keeps the last round of
 // workgroups short.  Returns the index of the sequence with the `rank`-th largest
