@@ -189,3 +189,28 @@ def test_varlen_one_long_sequence_among_short_ones(D, dtype):
             if e > b:
                 floor = ref[name + "_mag"][b:e] if name + "_mag" in ref else None
                 assert_parity(t.grad[b:e], ref[name][b:e], dtype, f"{name}[{b}:{e}]", floor)
+
+
+@pytest.mark.parametrize("nseq", [8, 9, 17, 40])
+def test_varlen_sequences_dealt_to_the_xcds(nseq):
+    """From eight sequences on, the row-parallel kernels deal the sequences out to the eight XCDs
+    and walk a sequence's heads and chunks as consecutive workgroups of one XCD; sequences past the
+    last multiple of eight keep the plain order.  Long sequences (several chunks each) next to
+    short and empty ones."""
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    rng = np.random.default_rng(nseq)
+    lengths = rng.integers(0, 300, nseq).tolist()
+    lengths[1], lengths[nseq - 1], lengths[nseq // 2] = 7000, 2500, 0
+    T, H, D, dtype = sum(lengths), 5, 64, torch.bfloat16
+    q, k, v, do = make_qkv((T, H, D), (T, H, D), dtype, 300 + nseq)
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lengths)]), dtype=torch.int32).cuda()
+    leaves = [t.cuda().requires_grad_() for t in (q, k, v)]
+    o = varlen_linear_attention(*leaves, cu, max(lengths))
+    o.backward(do.cuda())
+    ref = cf.varlen_backward(np64(q), np64(k), np64(v), np64(do), cu.cpu().numpy())
+    assert_parity(o, ref["o"], dtype, "o")
+    for name, t in zip(("dq", "dk", "dv"), leaves):
+        for b, e in zip(cu[:-1].tolist(), cu[1:].tolist()):
+            if e > b:
+                floor = ref[name + "_mag"][b:e] if name + "_mag" in ref else None
+                assert_parity(t.grad[b:e], ref[name][b:e], dtype, f"{name}[{b}:{e}]", floor)
