@@ -392,4 +392,38 @@ int fbla_select_blocks(const float* qc, const float* kc, const float* bias, int3
   return check_launch(what);
 }
 
+int fbla_elu1_fwd(const void* x0, void* y0, int64_t n0, const void* x1, void* y1, int64_t n1, int dtype,
+                  void* stream) {
+  const char* what = "fbla_elu1_fwd";
+  if (n0 < 0 || n1 < 0 || (dtype != kF16 && dtype != kBF16 && dtype != kF32)) {
+    set_error("%s: bad sizes or dtype (n0=%lld n1=%lld dtype=%d)", what, (long long)n0, (long long)n1, dtype);
+    return kErrBadArg;
+  }
+  if ((n0 > 0 && (!x0 || !y0)) || (n1 > 0 && (!x1 || !y1))) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  if (check_aligned(what, {n0 > 0 ? x0 : nullptr, n0 > 0 ? y0 : nullptr, n1 > 0 ? x1 : nullptr,
+                           n1 > 0 ? y1 : nullptr}) != kOk)
+    return kErrBadArg;
+  feature::elu1_fwd(x0, y0, n0, x1, y1, n1, dtype, (hipStream_t)stream);
+  return check_launch(what);
+}
+
+int fbla_elu1_bwd(const void* x, const void* dy, void* dx, int64_t n, int dtype, void* stream) {
+  const char* what = "fbla_elu1_bwd";
+  if (n < 0 || (dtype != kF16 && dtype != kBF16 && dtype != kF32)) {
+    set_error("%s: bad size or dtype (n=%lld dtype=%d)", what, (long long)n, dtype);
+    return kErrBadArg;
+  }
+  if (n == 0) return kOk;
+  if (!x || !dy || !dx) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  if (check_aligned(what, {x, dy, dx}) != kOk) return kErrBadArg;
+  feature::elu1_bwd(x, dy, dx, n, dtype, (hipStream_t)stream);
+  return check_launch(what);
+}
+
 }  // extern "C"

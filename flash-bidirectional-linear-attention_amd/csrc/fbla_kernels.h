@@ -135,6 +135,15 @@ int bwd_tokens(const Prob& p, const float* qn, const float* qd, const float* dou
                const float* km, float* dqn, float* dqd, float* tokscal, int64_t total_rows, hipStream_t st);
 }  // namespace mfma32
 
+// The callers' feature map elu(x) + 1 and its derivative (fbla_feature.hip).
+namespace feature {
+// y0 = elu(x0) + 1 over n0 elements and y1 = elu(x1) + 1 over n1 elements, one launch
+void elu1_fwd(const void* x0, void* y0, int64_t n0, const void* x1, void* y1, int64_t n1, int dtype,
+              hipStream_t st);
+// dx = g * (x > 0 ? 1 : exp(x))
+void elu1_bwd(const void* x, const void* g, void* dx, int64_t n, int dtype, hipStream_t st);
+}  // namespace feature
+
 // Piecewise (PISA) attention, forward only (fbla_piecewise.hip).
 namespace piecewise {
 size_t chunk_reduce_workspace_bytes(int64_t BH, int64_t T, int K, int V, int chunk, int dtype,

@@ -285,7 +285,6 @@ typedef uint32_t u32x2p __attribute__((ext_vector_type(2)));
 template <typename T, int K, int V>
 __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) {
   using LY = Attn32Layout<K, V>;
-  constexpr int KCH = K / 8;                 // 16-byte chunks per K tile row
   constexpr int KS = K / 16;                 // k-steps of the score product
   constexpr int MB = V / 32;                 // 32-row blocks of O^T
   constexpr int OLD = 64 * (V / 8) / kThreads;

@@ -40,6 +40,8 @@ _SIGNATURES = {
     "fbla_select_blocks": (_i32, [_vp] * 4 + [_i64, _i64, _i32, _i32, _f32, _vp]),
     "fbla_piecewise_workspace_bytes": (_sz, [_i64, _i64, _i32, _i32, _i32, _i32]),
     "fbla_piecewise_fwd": (_i32, [_vp] * 9 + [_sz, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
+    "fbla_elu1_fwd": (_i32, [_vp, _vp, _i64, _vp, _vp, _i64, _i32, _vp]),
+    "fbla_elu1_bwd": (_i32, [_vp, _vp, _vp, _i64, _i32, _vp]),
 }
 
 
@@ -278,3 +280,31 @@ def piecewise_fwd(q, k, v, kc, vc, h, indices, block, scale):
                                   float(scale), code, _stream(dev))
     _check(rc, "fbla_piecewise_fwd")
     return o
+
+
+def elu1_fwd(x0, x1=None):
+    """elu(x) + 1 of one or two contiguous tensors in one launch: returns the new tensor(s)."""
+    _require_gpu(x0, x1)
+    x0, x1 = _aligned(x0, x1)
+    L = lib()
+    y0 = torch.empty_like(x0)
+    y1 = torch.empty_like(x1) if x1 is not None else None
+    if x1 is not None and (x1.dtype != x0.dtype or x1.device != x0.device):
+        raise ValueError("elu1_fwd: both tensors must have the same dtype and device")
+    with torch.cuda.device(x0.device):
+        rc = L.fbla_elu1_fwd(_ptr(x0), _ptr(y0), x0.numel(), _ptr(x1), _ptr(y1),
+                             x1.numel() if x1 is not None else 0, dtype_code(x0), _stream(x0.device))
+    _check(rc, "fbla_elu1_fwd")
+    return y0 if x1 is None else (y0, y1)
+
+
+def elu1_bwd(x, dy):
+    """dy * d(elu(x) + 1)/dx for contiguous tensors of the same shape and dtype."""
+    _require_gpu(x, dy)
+    x, dy = _aligned(x, dy)
+    L = lib()
+    dx = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = L.fbla_elu1_bwd(_ptr(x), _ptr(dy), _ptr(dx), x.numel(), dtype_code(x), _stream(x.device))
+    _check(rc, "fbla_elu1_bwd")
+    return dx

@@ -4,6 +4,7 @@ import torch
 import torch.nn as nn
 
 from flash_bla.layers._common import check_mode, merge_heads, split_heads, torch_linear_attention
+from flash_bla.ops.feature_map import elu_plus_one
 from flash_bla.ops.linear_attn.decoupled import decoupled_la
 
 
@@ -39,7 +40,11 @@ class MambaLikeLinearAttention(nn.Module):
         fast = check_mode(mode)
         b, n, c = x.shape
         side = int(n ** 0.5)
-        q, k = (self.elu(t) + 1.0 for t in self.qk(x).chunk(2, dim=-1))
+        qk = self.qk(x)
+        if fast:  # one launch over the joint projection
+            q, k = elu_plus_one(qk).chunk(2, dim=-1)
+        else:
+            q, k = (self.elu(t) + 1.0 for t in qk.chunk(2, dim=-1))
         rot = [self.rope(t.reshape(b, side, side, c)).reshape(b, n, c).to(x.dtype) for t in (q, k)]
         q, k, v, q_rope, k_rope = (split_heads(t, self.num_heads) for t in (q, k, x, *rot))
         if fast:

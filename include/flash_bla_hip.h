@@ -177,6 +177,18 @@ int fbla_piecewise_fwd(const void* q, const void* k, const void* v, const float*
                        size_t workspace_bytes, int64_t BH, int64_t T, int K, int V, int block, int NS,
                        float scale, int dtype, void* stream);
 
+/* The feature map of the reference's blocks, phi(x) = elu(x) + 1, for the queries and the
+ * keys in one launch.  Replaces the two elementwise torch kernels per tensor of
+ * flash_bla/layers/linfusion.py:88-89, mlla.py:74-75 and rala.py:52-53 (`F.elu(x) + 1.0`), with
+ * torch's rounding (elu in fp32 rounded to the element type, then + 1 rounded again).
+ * x0/y0 hold n0 elements, x1/y1 n1 (either count may be 0); y may alias x.  Any dtype of the
+ * FBLA_* element types; pointers 16-byte aligned. */
+int fbla_elu1_fwd(const void* x0, void* y0, int64_t n0, const void* x1, void* y1, int64_t n1, int dtype,
+                  void* stream);
+
+/* Its derivative: dx = dy * (x > 0 ? 1 : exp(x)), what autograd computes for `F.elu(x) + 1.0`. */
+int fbla_elu1_bwd(const void* x, const void* dy, void* dx, int64_t n, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
