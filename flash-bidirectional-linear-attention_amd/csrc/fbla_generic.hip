@@ -367,7 +367,7 @@ template <typename T>
 __global__ __launch_bounds__(kThreads) void bwd_b_kernel(
     Prob p, const T* __restrict__ kn, const T* __restrict__ v, const float* __restrict__ dS,
     const float* __restrict__ dSt, const float* __restrict__ dkm, T* __restrict__ dkn,
-    T* __restrict__ dkd, T* __restrict__ dv, int ntiles) {
+    T* __restrict__ dkd, T* __restrict__ dv, int ntiles, float dkm_scale) {
   __shared__ float Ks[kTile * kLd];
   __shared__ float Vs[kTile * kLd];
   const int nh = blockIdx.x / ntiles, tile = blockIdx.x - nh * ntiles;
@@ -402,7 +402,7 @@ __global__ __launch_bounds__(kThreads) void bwd_b_kernel(
       const int cc = lane + 32 * j;
       if (cc >= DK) continue;
       float g = acc[i][j];
-      const float den = normalize ? dkmh[cc] : 0.f;
+      const float den = normalize ? dkmh[cc] * dkm_scale : 0.f;
       if (split) {
         dkd[roff + cc] = from_f32<T>(den);
       } else {
@@ -515,17 +515,18 @@ void bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void*
 
 template <typename T>
 static void bwd_b_t(const Prob& p, const void* kn, const void* v, const float* dS, const float* dSt,
-                    const float* dkm, void* dkn, void* dkd, void* dv, hipStream_t st) {
+                    const float* dkm, void* dkn, void* dkd, void* dv, float dkm_scale, hipStream_t st) {
   const int ntiles = (int)cdiv64(p.L, kTile);
   bwd_b_kernel<T><<<dim3((unsigned)((int64_t)p.N * p.H * ntiles)), dim3(kThreads), 0, st>>>(
-      p, (const T*)kn, (const T*)v, dS, dSt, dkm, (T*)dkn, (T*)dkd, (T*)dv, ntiles);
+      p, (const T*)kn, (const T*)v, dS, dSt, dkm, (T*)dkn, (T*)dkd, (T*)dv, ntiles, dkm_scale);
 }
 
 void bwd_b(const Prob& p, int dtype, const void* kn, const void* v, const float* dS,
-           const float* dSt, const float* dkm, void* dkn, void* dkd, void* dv, hipStream_t st) {
-  if (dtype == kF16) bwd_b_t<_Float16>(p, kn, v, dS, dSt, dkm, dkn, dkd, dv, st);
-  else if (dtype == kBF16) bwd_b_t<__bf16>(p, kn, v, dS, dSt, dkm, dkn, dkd, dv, st);
-  else bwd_b_t<float>(p, kn, v, dS, dSt, dkm, dkn, dkd, dv, st);
+           const float* dSt, const float* dkm, void* dkn, void* dkd, void* dv, hipStream_t st,
+           float dkm_scale) {
+  if (dtype == kF16) bwd_b_t<_Float16>(p, kn, v, dS, dSt, dkm, dkn, dkd, dv, dkm_scale, st);
+  else if (dtype == kBF16) bwd_b_t<__bf16>(p, kn, v, dS, dSt, dkm, dkn, dkd, dv, dkm_scale, st);
+  else bwd_b_t<float>(p, kn, v, dS, dSt, dkm, dkn, dkd, dv, dkm_scale, st);
 }
 
 template <typename T>

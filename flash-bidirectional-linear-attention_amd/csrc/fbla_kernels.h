@@ -57,8 +57,11 @@ void output(const Prob& p, int dtype, const void* qn, const void* qd, const floa
 void bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout,
            const float* S, const float* St, const float* km, void* dqn, void* dqd, float* partial,
            int chunk, int nchunks, hipStream_t st);
+// dkm_scale: the vector arrives divided by the number of queries; with another number of keys
+// the formula wants it divided by that (factor Lq / Lk)
 void bwd_b(const Prob& p, int dtype, const void* kn, const void* v, const float* dS,
-           const float* dSt, const float* dkm, void* dkn, void* dkd, void* dv, hipStream_t st);
+           const float* dSt, const float* dkm, void* dkn, void* dkd, void* dv, hipStream_t st,
+           float dkm_scale = 1.f);
 void broadcast_rows(const Prob& p, int dtype, const float* vec, void* out, hipStream_t st);
 // perm[r] = index of the sequence with the r-th largest length (ties by index)
 void rank_sequences(const Prob& p, int32_t* perm, hipStream_t st);

@@ -109,10 +109,8 @@ size_t bwd_workspace_bytes(const Prob& pc, int dtype) { return bwd_used_bytes(pc
 
 static int check_cross(const Prob& p, int dtype) {
   if (!cross(p)) return kOk;
-  if ((p.flags & kDecoupled) || !mfma::supported(key_side(p), dtype)) {
-    set_error("different numbers of queries and keys need the matrix-core kernels (16-bit inputs with "
-              "head dims that are multiples of 8, or fp32 inputs with head dims up to 64) and are not "
-              "available for the decoupled operator");
+  if (p.flags & kDecoupled) {
+    set_error("different numbers of queries and keys are not available for the decoupled operator");
     return kErrUnsupported;
   }
   return kOk;
@@ -160,7 +158,7 @@ int forward(const Prob& pc_, int dtype, const FwdArgs& a, hipStream_t st) {
       int rc = mfma::rows(pq, dtype, job, p.DK, p.DV, st);
       if (rc != kOk) return rc;
     } else {
-      generic::output(p, dtype, qn, a.q, a.s, a.km, a.o, st);
+      generic::output(pq, dtype, qn, a.q, a.s, a.km, a.o, st);
     }
   }
   return kOk;
@@ -249,7 +247,8 @@ int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
       if (rc != kOk) return rc;
       if (dec) generic::broadcast_rows(p, dtype, dkm, dkd, st);
     } else {
-      generic::bwd_b(p, dtype, kn, a.v, dS, dSt, dkm, dkn, dkd, a.dv, st);
+      generic::bwd_b(pk, dtype, kn, a.v, dS, dSt, dkm, dkn, dkd, a.dv, st,
+                     is_cross ? (float)p.L / (float)pk.L : 1.f);
     }
   }
   return kOk;

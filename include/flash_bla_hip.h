@@ -99,9 +99,8 @@ int fbla_la_bwd(const void* q, const void* k, const void* v, const void* q_rope,
  * over the Lk keys.  The reference has no counterpart: its dense kernels take one length from q
  * (linear_attn/fused.py:355) and read k, v out of bounds when the PVT-style blocks
  * (layers/focused_la.py:55,73-75, layers/polaformer.py) shorten the keys with sr_ratio > 1.
- * Flags as for fbla_la_fwd without FBLA_DECOUPLED; matrix-core shapes only (16-bit inputs with
- * head dims that are multiples of 8, fp32 inputs with head dims that are multiples of 4 up to 64),
- * else FBLA_ERR_UNSUPPORTED. */
+ * Flags as for fbla_la_fwd without FBLA_DECOUPLED (FBLA_ERR_UNSUPPORTED with it); every dtype
+ * and head dim of fbla_la_fwd. */
 size_t fbla_la_cross_workspace_bytes(int pass, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int DK,
                                      int DV, int dtype, int flags);
 int fbla_la_cross_fwd(const void* q, const void* k, const void* v, void* o, float* s, float* km,

@@ -1,7 +1,7 @@
 """Keys and values with another number of tokens than the queries (dense operators): the
 PVT-style blocks reduce k, v spatially (`sr_ratio > 1`), the reference's kernels take one
 length from q and run out of bounds there (linear_attn/fused.py:355).  Forward and backward
-against the float64 oracle; the error paths of the shapes without matrix-core kernels."""
+against the float64 oracle, on the matrix-core kernels and on the shape-generic ones."""
 import pytest
 import torch
 
@@ -64,19 +64,20 @@ def test_default_scale_is_one_over_the_number_of_keys():
     assert torch.equal(a, b)
 
 
-def test_shapes_without_matrix_core_kernels_are_refused():
+def test_shapes_of_the_generic_kernels():
+    """Head dims that are not multiples of 8 (4 in fp32) and fp32 heads above 64 run on the
+    shape-generic kernels, with another number of keys than queries as well."""
+    for i, (lq, lk) in enumerate(LENGTHS[:4]):
+        _check("linear", 1, 2, lq, lk, 20, 20, torch.float16, 300 + i)
+        _check("linear", 2, 1, lq, lk, 17, 13, torch.bfloat16, 310 + i)
+        _check("simple", 1, 2, lq, lk, 100, 36, torch.float16, 320 + i)
+        _check("linear", 1, 2, lq, lk, 128, 128, torch.float32, 330 + i)
+        _check("linear", 1, 1, lq, lk, 128, 32, torch.float32, 340 + i)
+        _check("simple", 1, 2, lq, lk, 6, 70, torch.float32, 350 + i)
+
+
+def test_the_decoupled_operator_is_refused():
     from flash_bla.ops.linear_attn.decoupled import decoupled_la
-    from flash_bla.ops.linear_attn.fused import linear_attention
-    q = torch.rand(1, 2, 40, 20, device="cuda", dtype=torch.float16)   # 20 is not a multiple of 8
-    k = torch.rand(1, 2, 10, 20, device="cuda", dtype=torch.float16)
-    with pytest.raises(ValueError, match="matrix-core"):
-        linear_attention(q, k, k)
-    q32 = torch.rand(1, 2, 40, 128, device="cuda")   # fp32: head dims up to 64 only
-    k32 = torch.rand(1, 2, 10, 128, device="cuda")
-    with pytest.raises(ValueError, match="matrix-core"):
-        linear_attention(q32, k32, k32)
-    # the library is still usable
-    assert linear_attention(q32, q32, q32).shape == q32.shape
     q64 = torch.rand(1, 2, 40, 64, device="cuda", dtype=torch.float16)
     k64 = torch.rand(1, 2, 10, 64, device="cuda", dtype=torch.float16)
     with pytest.raises(ValueError, match="identical shapes"):
