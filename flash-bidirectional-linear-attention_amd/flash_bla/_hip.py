@@ -89,8 +89,34 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device):
+    """Handle of torch's current stream on `device` (the raw getter saves the Stream object: these
+    wrappers are on the host-bound path of small problems)."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _Here:
+    """No-op context: the tensors' device is already the current one."""
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_HERE = _Here()
+
+
+def _on(device):
+    """Context that makes `device` current for the launch (kernels run on the current device)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _HERE
+    return torch.cuda.device(device)
 
 
 def _workspace(nbytes, device):
@@ -125,14 +151,14 @@ def la_fwd(q, k, v, q_rope, k_rope, scale, eps, flags):
     s = torch.empty(B, H, DK, DV, dtype=torch.float32, device=dev)
     km = torch.empty(B, H, DK, dtype=torch.float32, device=dev)
     if Tk != T:
-        with torch.cuda.device(dev):
+        with _on(dev):
             ws = _workspace(L.fbla_la_cross_workspace_bytes(0, B, H, T, Tk, DK, DV, code, flags), dev)
             rc = L.fbla_la_cross_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(s), _ptr(km), _ptr(ws),
                                      ws.numel(), B, H, T, Tk, DK, DV, code, flags, float(scale), float(eps),
                                      _stream(dev))
         _check(rc, "fbla_la_cross_fwd")
         return o, s, km
-    with torch.cuda.device(dev):
+    with _on(dev):
         ws = _workspace(L.fbla_la_workspace_bytes(0, B, H, T, DK, DV, code, flags), dev)
         rc = L.fbla_la_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(q_rope), _ptr(k_rope), _ptr(o), _ptr(s),
                            _ptr(km), _ptr(ws), ws.numel(), B, H, T, DK, DV, code, flags,
@@ -154,14 +180,14 @@ def la_bwd(q, k, v, q_rope, k_rope, do, s, km, scale, eps, flags):
     dqr = torch.empty_like(q_rope) if flags & DECOUPLED else None
     dkr = torch.empty_like(k_rope) if flags & DECOUPLED else None
     if Tk != T:
-        with torch.cuda.device(dev):
+        with _on(dev):
             ws = _workspace(L.fbla_la_cross_workspace_bytes(1, B, H, T, Tk, DK, DV, code, flags), dev)
             rc = L.fbla_la_cross_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(s), _ptr(km), _ptr(dq),
                                      _ptr(dk), _ptr(dv), _ptr(ws), ws.numel(), B, H, T, Tk, DK, DV, code,
                                      flags, float(scale), float(eps), _stream(dev))
         _check(rc, "fbla_la_cross_bwd")
         return dq, dk, dv, None, None
-    with torch.cuda.device(dev):
+    with _on(dev):
         ws = _workspace(L.fbla_la_workspace_bytes(1, B, H, T, DK, DV, code, flags), dev)
         rc = L.fbla_la_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(q_rope), _ptr(k_rope), _ptr(do), _ptr(s),
                            _ptr(km), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dqr), _ptr(dkr), _ptr(ws),
@@ -185,7 +211,7 @@ def varlen_fwd(q, k, v, cu_seqlens, max_seqlen, scale, eps):
     o = torch.empty_like(v)
     s = torch.empty(N, H, DK, DV, dtype=torch.float32, device=dev)
     km = torch.empty(N, H, DK, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         ws = _workspace(L.fbla_varlen_workspace_bytes(0, T, N, H, max_seqlen, DK, DV, code, flags), dev)
         rc = L.fbla_varlen_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(cu_seqlens), _ptr(o), _ptr(s),
                                _ptr(km), _ptr(ws), ws.numel(), T, N, H, max_seqlen, DK, DV, code,
@@ -207,7 +233,7 @@ def varlen_bwd(q, k, v, cu_seqlens, max_seqlen, do, s, km, scale, eps):
     dev = q.device
     flags = NORMALIZE | (DEFAULT_SCALE if scale is None else 0)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    with torch.cuda.device(dev):
+    with _on(dev):
         ws = _workspace(L.fbla_varlen_workspace_bytes(1, T, N, H, max_seqlen, DK, DV, code, flags), dev)
         rc = L.fbla_varlen_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(cu_seqlens), _ptr(do), _ptr(s),
                                _ptr(km), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws.numel(), T, N,
@@ -232,7 +258,7 @@ def chunk_reduce(q, k, v, chunk, with_norm=False, p_norm=2.0):
     qc, kc = torch.empty(B, H, NT, K, **f32), torch.empty(B, H, NT, K, **f32)
     vc, h = torch.empty(B, H, NT, V, **f32), torch.empty(B, H, K, V, **f32)
     h_norm = torch.empty(B, H, NT, **f32) if with_norm else None
-    with torch.cuda.device(dev):
+    with _on(dev):
         ws = _workspace(L.fbla_chunk_reduce_workspace_bytes(B * H, T, K, V, chunk, code, int(with_norm)), dev)
         rc = L.fbla_chunk_reduce(_ptr(q), _ptr(k), _ptr(v), _ptr(qc), _ptr(kc), _ptr(vc), _ptr(h),
                                  _ptr(h_norm), _ptr(ws), ws.numel(), B * H, T, K, V, chunk,
@@ -249,7 +275,7 @@ def select_blocks(qc, kc, bias, top_k, scale):
     B, H, NT, K = qc.shape
     dev = qc.device
     idx = torch.empty(B, H, NT, top_k, dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on(dev):
         rc = L.fbla_select_blocks(_ptr(qc), _ptr(kc), _ptr(bias), _ptr(idx), B * H, NT, K, top_k,
                                   float(scale), _stream(dev))
     _check(rc, "fbla_select_blocks")
@@ -273,7 +299,7 @@ def piecewise_fwd(q, k, v, kc, vc, h, indices, block, scale):
     code = dtype_code(q)
     dev = q.device
     o = torch.empty_like(v)
-    with torch.cuda.device(dev):
+    with _on(dev):
         ws = _workspace(L.fbla_piecewise_workspace_bytes(B * H, T, K, V, block, code), dev)
         rc = L.fbla_piecewise_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(kc), _ptr(vc), _ptr(h), _ptr(indices),
                                   _ptr(o), _ptr(ws), ws.numel(), B * H, T, K, V, block, NS,
@@ -291,7 +317,7 @@ def elu1_fwd(x0, x1=None):
     y1 = torch.empty_like(x1) if x1 is not None else None
     if x1 is not None and (x1.dtype != x0.dtype or x1.device != x0.device):
         raise ValueError("elu1_fwd: both tensors must have the same dtype and device")
-    with torch.cuda.device(x0.device):
+    with _on(x0.device):
         rc = L.fbla_elu1_fwd(_ptr(x0), _ptr(y0), x0.numel(), _ptr(x1), _ptr(y1),
                              x1.numel() if x1 is not None else 0, dtype_code(x0), _stream(x0.device))
     _check(rc, "fbla_elu1_fwd")
@@ -304,7 +330,7 @@ def elu1_bwd(x, dy):
     x, dy = _aligned(x, dy)
     L = lib()
     dx = torch.empty_like(x)
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = L.fbla_elu1_bwd(_ptr(x), _ptr(dy), _ptr(dx), x.numel(), dtype_code(x), _stream(x.device))
     _check(rc, "fbla_elu1_bwd")
     return dx
