@@ -399,6 +399,7 @@ int fbla_elu1_fwd(const void* x0, void* y0, int64_t n0, const void* x1, void* y1
     set_error("%s: bad sizes or dtype (n0=%lld n1=%lld dtype=%d)", what, (long long)n0, (long long)n1, dtype);
     return kErrBadArg;
   }
+  if (n0 == 0 && n1 == 0) return kOk;
   if ((n0 > 0 && (!x0 || !y0)) || (n1 > 0 && (!x1 || !y1))) {
     set_error("%s: null tensor pointer", what);
     return kErrBadArg;

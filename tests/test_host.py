@@ -88,6 +88,27 @@ def test_dense_ops_refuse_cpu_tensors():
         linear_attention(q, q[:, :, :4], q)   # shorter keys are allowed, but v must follow k
 
 
+def test_feature_map_refuses_cpu_tensors_and_bad_arguments():
+    from flash_bla.ops.feature_map import elu_plus_one
+    x = torch.rand(4, 8)
+    with pytest.raises(ValueError, match="GPU"):
+        elu_plus_one(x)                          # no CPU path behind the operator
+    with pytest.raises(ValueError, match="same dtype"):
+        elu_plus_one(x, x.double())
+    with pytest.raises(TypeError):
+        elu_plus_one(x.long())
+    with pytest.raises(TypeError):
+        elu_plus_one([1.0, 2.0])
+    L = _hip.lib()
+    assert L.fbla_elu1_fwd(None, None, -1, None, None, 0, _hip.F16, None) == -1   # negative size
+    assert L.fbla_elu1_fwd(None, None, 8, None, None, 0, _hip.F16, None) == -1    # null pointers
+    assert b"null" in L.fbla_last_error()
+    assert L.fbla_elu1_fwd(None, None, 0, None, None, 0, 9, None) == -1           # unknown dtype
+    assert L.fbla_elu1_bwd(None, None, None, 0, _hip.F32, None) == 0              # nothing to do
+    assert L.fbla_elu1_fwd(None, None, 0, None, None, 0, _hip.BF16, None) == 0
+    assert L.fbla_elu1_bwd(None, None, None, 5, _hip.F32, None) == -1
+
+
 @pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "*.npz"))), ids=os.path.basename)
 def test_oracle_reproduces_golden_fixture(path):
     d = np.load(path)
