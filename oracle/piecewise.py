@@ -2,9 +2,11 @@
 
 Test infrastructure only (see oracle/__init__.py).  Written from
 flash_bla/ops/piecewise_attn/kernel.py; the reference ships neither a naive
-implementation nor a test for this operator, so agreement with the reference's
-Triton kernel is "parity unpinned".  What is implemented is the kernel's
-intended mathematics:
+implementation nor a test for this operator; this closed form is pinned by
+softmax-attention special cases and by the independent per-token C evaluation
+oracle/piecewise_tokens.c (tests/test_oracle.py, including a mutation check of
+the first-order coefficient).  What is implemented is the kernel's mathematics
+with one group:
 
   s_ij  = scale * q_i.k_j                    exact scores       (kernel.py:227-228)
   sb_ic = scale * q_i.kc_c                   block-mean scores  (kernel.py:250-251)

@@ -12,6 +12,7 @@ import torch
 
 from helpers import make_qkv, np64
 from oracle import brute, closed_form as cf, piecewise as pw, torch_ref as tr
+from oracle.piecewise_tokens import pisa_tokens
 
 
 def _dense_inputs(B=2, H=3, L=37, DK=16, DV=8, seed=0, n_extra=0):
@@ -226,11 +227,9 @@ def test_piecewise_chunk_reduce_and_selection():
 
 
 def test_piecewise_first_order_term_is_taylor_expansion():
-    # Small scores: exp(s_ij) ~ exp(sb_ic)(1 + s_ij - sb_ic); summed over a chunk the
-    # numerator correction is exp(sb_ic) scale q.(K_c - kc_c)^T V_c, which the kernel
-    # approximates with the global H weighted by G/T.  With one unselected chunk and
-    # the rest selected, G/T * H_total differs from exp(sb)*hc_c, so only check that
-    # the first-order term moves the result towards exact attention on average.
+    # Small scores: exp(s_ij) ~ exp(sb_ic)(1 + s_ij - sb_ic); the first-order term must
+    # move the result towards exact attention (a sanity check; the coefficient itself
+    # is pinned by the three tests below).
     q, k, v = _pw_inputs(T=512, K=8, V=4, seed=9)
     q, k = 0.3 * q, 0.3 * k
     NT = 8
@@ -240,3 +239,81 @@ def test_piecewise_first_order_term_is_taylor_expansion():
     e0 = np.abs(pw.piecewise_forward(q, k, v, idx, 64, first_order=False) - ref).mean()
     e1 = np.abs(pw.piecewise_forward(q, k, v, idx, 64, first_order=True) - ref).mean()
     assert e1 < 0.5 * e0
+
+
+def _pw_ragged_case(T, K, V, block, n_sel, seed, scale=None):
+    q, k, v = _pw_inputs(T=T, K=K, V=V, seed=seed)
+    NT = -(-T // block)
+    rng = np.random.default_rng(seed)
+    idx = np.stack([rng.permutation(NT)[:n_sel] for _ in range(NT)])
+    return q, k, v, idx
+
+
+# The per-token C evaluation (oracle/piecewise_tokens.c) follows the reference kernel
+# step by step in base 2 with the kernel's 9-digit log2(e); the dense numpy closed form
+# uses exp().  The constants differ by 6e-10 relative, which for |score| < 20 bounds the
+# disagreement of the two by ~2e-8; every coefficient mistake below is 1e-3 or more.
+_PW_TOL = 2e-8
+
+
+@pytest.mark.parametrize("T,K,V,block,n_sel,scale", [
+    (200, 16, 8, 64, 1, None),      # ragged last chunk (8 tokens), default scale
+    (333, 24, 12, 32, 3, 0.37),     # other block size, explicit scale != K^-0.5
+    (129, 8, 16, 64, 2, None),      # last chunk of one token
+    (64, 8, 4, 16, 4, 0.5),         # every chunk selected: phases 2 and 3 vanish
+])
+def test_piecewise_closed_form_matches_per_token_c_evaluation(T, K, V, block, n_sel, scale):
+    q, k, v, idx = _pw_ragged_case(T, K, V, block, n_sel, seed=T)
+    o_np = pw.piecewise_forward(q, k, v, idx, block, scale=scale)
+    o_c = pisa_tokens(q, k, v, idx, block, scale=scale)
+    assert np.abs(o_np - o_c).max() <= _PW_TOL * np.abs(o_c).max()
+
+
+def test_piecewise_coefficient_mistakes_are_caught():
+    # The first-order term is additive in the numerator, so a closed form with the term
+    # multiplied by f is  o_0 + f (o_1 - o_0).  Each plausible mistake must be far outside
+    # the tolerance with which the correct closed form matches the per-token evaluation.
+    T, K, V, block, n_sel, scale = 333, 24, 12, 32, 3, 0.37
+    q, k, v, idx = _pw_ragged_case(T, K, V, block, n_sel, seed=T)
+    o_c = pisa_tokens(q, k, v, idx, block, scale=scale)
+    o1 = pw.piecewise_forward(q, k, v, idx, block, scale=scale)
+    o0 = pw.piecewise_forward(q, k, v, idx, block, scale=scale, first_order=False)
+    tol = _PW_TOL * np.abs(o_c).max()
+    assert np.abs(o1 - o_c).max() <= tol
+    mistakes = {
+        "G/(T - selected tokens)": T / (T - n_sel * block),
+        "scale dropped": 1.0 / scale,
+        "x0.7": 0.7,
+        "sign": -1.0,
+        "term missing": 0.0,
+        "G/NT instead of G/T": T / (-(-T // block)),
+    }
+    for name, f in mistakes.items():
+        err = np.abs(o0 + f * (o1 - o0) - o_c).max()
+        assert err > 1e4 * tol, (name, err, tol)
+
+
+def test_piecewise_zero_mean_chunks_isolate_first_order_coefficient():
+    # Keys centred inside every chunk: all chunk means are 0, every mean score is 0,
+    # H = K^T V, and G_i = (number of unselected tokens), independent of q.  Then
+    #   o_i = [ sum_{j sel} e^{s_ij} v_j + sum_{j unsel} v_j
+    #           + (N_unsel/T) scale sum_{all j} (q_i.k_j) v_j ] / [ sum_{j sel} e^{s_ij} + N_unsel ]
+    # evaluated here token by token as (q K^T) V - a different contraction order from the
+    # oracle's q (K^T V) - and without any running maximum.
+    T, K, V, block, scale = 200, 8, 4, 64, 0.41
+    q, k, v = _pw_inputs(T=T, K=K, V=V, seed=21)
+    for lo in range(0, T, block):
+        k[lo:lo + block] -= k[lo:lo + block].mean(0, keepdims=True)
+    idx = np.array([[1], [3], [0], [2]])
+    o = pw.piecewise_forward(q, k, v, idx, block, scale=scale)
+    s = scale * (q @ k.T)                          # [T,T] exact scores
+    lin = (q @ k.T) @ v                            # sum_j (q_i.k_j) v_j
+    for t in range(4):
+        rows = slice(t * block, min(T, (t + 1) * block))
+        sel = np.zeros(T, dtype=bool)
+        sel[idx[t, 0] * block:(idx[t, 0] + 1) * block] = True
+        n_unsel = float((~sel).sum())
+        num = np.exp(s[rows][:, sel]) @ v[sel] + v[~sel].sum(0) + (n_unsel / T) * scale * lin[rows]
+        den = np.exp(s[rows][:, sel]).sum(-1) + n_unsel
+        np.testing.assert_allclose(o[rows], num / den[:, None], rtol=1e-11, atol=1e-13)
+    np.testing.assert_allclose(pisa_tokens(q, k, v, idx, block, scale=scale), o, rtol=1e-7, atol=1e-9)
