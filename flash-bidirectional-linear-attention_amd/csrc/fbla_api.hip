@@ -4,7 +4,9 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <atomic>
 #include <initializer_list>
+#include <mutex>
 
 #include "../../include/flash_bla_hip.h"
 #include "fbla_kernels.h"
@@ -183,6 +185,75 @@ int fbla_la_bwd(const void* q, const void* k, const void* v, const void* q_rope,
   BwdArgs a{q, k, v, q_rope, k_rope, dout, s, km, dq, dk, dv, dq_rope, dk_rope, workspace,
             workspace_bytes_};
   return run_bwd(what, p, dtype, a, (hipStream_t)stream);
+}
+
+// ---- the entry point that allocates nothing ------------------------------------------------
+// Workspace of fbla_la_fwd_static: a fixed array in the library's device image.  Every GPU the
+// library runs on holds its own copy at its own address until the process ends; host code may
+// only use the address hipGetSymbolAddress returns for the current device, never the array's
+// name (which is a host-side stand-in).
+static constexpr size_t kStaticScratchBytes = (size_t)FBLA_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+static constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];  // zero-initialised: not looked up yet
+static std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device (looked up once per device), or null with
+// the error text set.
+static void* static_scratch(const char* what) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("%s: cannot identify the current device (%s)", what,
+              e != hipSuccess ? hipGetErrorString(e) : "device index out of range");
+    return nullptr;
+  }
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr) return ptr;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  ptr = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+  if (ptr) return ptr;
+  e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !ptr) {
+    set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", what, dev, hipGetErrorString(e));
+    return nullptr;
+  }
+  g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  return ptr;
+}
+
+size_t fbla_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int fbla_la_fwd_static(const void* q, const void* k, const void* v, const void* q_rope, const void* k_rope,
+                       void* o, float* s, float* km, int64_t B, int64_t H, int64_t L, int DK, int DV,
+                       int dtype, int flags, float scale, float eps, void* stream) {
+  const char* what = "fbla_la_fwd_static";
+  int rc = check_dims(what, B, H, L, DK, DV, dtype, flags);
+  if (rc != kOk) return rc;
+  if (flags & kDefaultScale) {
+    set_error("%s: FBLA_DEFAULT_SCALE is only valid for the packed entry points", what);
+    return kErrBadArg;
+  }
+  if (B * H * L == 0) return kOk;
+  if (!q || !k || !v || !o || !s || ((flags & kNormalize) && !km) ||
+      ((flags & kDecoupled) && (!q_rope || !k_rope))) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  Prob p = make_prob(nullptr, B, H, L, B * L, DK, DV, flags, scale, eps);
+  const size_t need = workspace_bytes(p, dtype, 0);
+  if (need > kStaticScratchBytes) {
+    set_error("%s: this problem needs %zu bytes of workspace, the built-in scratch holds %zu; "
+              "use fbla_la_fwd with a caller-provided workspace", what, need, kStaticScratchBytes);
+    return kErrWorkspace;
+  }
+  void* ws = static_scratch(what);
+  if (!ws) return kErrLaunch;
+  // Every partial the reductions read is written earlier in the same call, so nothing in the
+  // scratch has to start at zero.
+  FwdArgs a{q, k, v, q_rope, k_rope, o, s, km, ws, kStaticScratchBytes};
+  return run_fwd(what, p, dtype, a, (hipStream_t)stream);
 }
 
 static int check_cross(const char* what, int64_t Lk, int flags) {

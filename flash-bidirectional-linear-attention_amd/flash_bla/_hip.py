@@ -28,6 +28,8 @@ _SIGNATURES = {
     "fbla_set_phase_mask": (None, [ctypes.c_uint]),
     "fbla_la_workspace_bytes": (_sz, [_i32, _i64, _i64, _i64, _i32, _i32, _i32, _i32]),
     "fbla_la_fwd": (_i32, [_vp] * 9 + [_sz, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
+    "fbla_static_scratch_bytes": (_sz, []),
+    "fbla_la_fwd_static": (_i32, [_vp] * 8 + [_i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_la_bwd": (_i32, [_vp] * 14 + [_sz, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_la_cross_workspace_bytes": (_sz, [_i32, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32]),
     "fbla_la_cross_fwd": (_i32, [_vp] * 7 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),

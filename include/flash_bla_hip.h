@@ -94,6 +94,22 @@ int fbla_la_bwd(const void* q, const void* k, const void* v, const void* q_rope,
                 size_t workspace_bytes, int64_t B, int64_t H, int64_t L, int DK, int DV, int dtype,
                 int flags, float scale, float eps, void* stream);
 
+/* Dense forward that allocates nothing.  No counterpart in the reference: it is for callers
+ * that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc) and have no workspace to hand over.  Same arguments,
+ * arithmetic and results as fbla_la_fwd, but the workspace is a fixed array of
+ * FBLA_STATIC_SCRATCH_BYTES inside the library's device image (each GPU the library runs on
+ * holds one copy until the process ends).  A problem whose fbla_la_workspace_bytes(0, ...)
+ * exceeds that returns FBLA_ERR_WORKSPACE.  The call makes no hipMalloc / hipFree and no
+ * allocating library call.  All calls on one GPU share the array: calls that overlap on one
+ * GPU (two streams, two threads) race; serialise them or use fbla_la_fwd. */
+#define FBLA_STATIC_SCRATCH_BYTES (16u << 20)
+size_t fbla_static_scratch_bytes(void);
+int fbla_la_fwd_static(const void* q, const void* k, const void* v, const void* q_rope,
+                       const void* k_rope, void* o, float* s, float* km, int64_t B, int64_t H,
+                       int64_t L, int DK, int DV, int dtype, int flags, float scale, float eps,
+                       void* stream);
+
 /* Dense problems with Lk key / value tokens and Lq query tokens per (batch, head), Lk != Lq:
  * q, dq: [B,H,Lq,DK]; k, dk: [B,H,Lk,DK]; v, dv: [B,H,Lk,DV]; o, dout: [B,H,Lq,DV]; km is the mean
  * over the Lk keys.  The reference has no counterpart: its dense kernels take one length from q
