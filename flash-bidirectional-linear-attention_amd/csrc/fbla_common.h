@@ -17,6 +17,7 @@ enum Flags : int {
   kDecoupled = 2,     // numerator uses q_rope/k_rope, denominator q/k
   kDefaultScale = 4,  // varlen only: scale = 1/len_i per sequence
   kXcdOrder = 256,    // internal (set per launch): packed batches keep a sequence's heads on one XCD
+  kInterleave = 512,  // internal (set per launch): the workgroups of a head take interleaved token steps
 };
 
 // One problem instance.  Dense: cu == nullptr, N = batch, every sequence has L

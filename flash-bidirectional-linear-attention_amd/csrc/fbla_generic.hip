@@ -150,7 +150,7 @@ __global__ __launch_bounds__(kThreads) void state_reduce_kernel(
   const int DK = p.DK, DV = p.DV, E = DK * DV, stride = E + DK;
   const int e = blk * kThreads + threadIdx.x;
   if (e >= stride) return;
-  const int nvalid = len > 0 ? (len + chunk - 1) / chunk : 0;
+  const int nvalid = len > 0 ? min(nchunks, (len + chunk - 1) / chunk) : 0;
   const float* src = partial + (int64_t)nh * nchunks * stride + e;
   // fixed order: chunk 0, 1, 2, ... (four independent loads in flight at a time)
   float a = 0.f;

@@ -97,6 +97,15 @@ bool pair_mode(const Prob& p, int dtype);
 int state_chunk(const Prob& p, bool block_stats = false);
 int bwd_a_chunk(const Prob& p);
 int rows_chunk(const Prob& p, int DR, int DC);
+// Tokens per partial as a reduction must count them (`kernel_bit`: 1 the state kernel, 4 backward
+// pass A): the kernel's chunk, or the step of the interleaved walk when the workgroups of a head
+// take interleaved steps.
+int partial_chunk(const Prob& p, int dtype, int kernel_bit, int chunk);
+// The problem with the interleaved walk switched on for the kernel `kernel_bit` (1 the state
+// kernel, 2 the row-parallel kernels, 4 backward pass A) where it applies: dense 16-bit heads
+// tiled 64 x 64.  Only for callers that treat the partials as an unordered set to be summed
+// (partial_chunk tells how many of them a sequence of a given length has).
+Prob with_interleave(const Prob& p, int dtype, int kernel_bit);
 // fin_mat / fin_vec (only with nchunks == 1): store the finished, scaled matrix [N*H,DK,DV] and
 // vector [N*H,DK] directly instead of a partial (no reduce step needed)
 void state(const Prob& p, int dtype, const void* kn, const void* v, const void* kd, float* partial,

@@ -64,6 +64,16 @@ constexpr int kWaves = 4;
 #ifndef FBLA_ROWS_PF
 #define FBLA_ROWS_PF 1
 #endif
+// register budgets: four waves per SIMD for the 64 x 64 row kernel, three for the fused fp16 pass A
+#ifndef FBLA_ROWS_OCC4
+#define FBLA_ROWS_OCC4 1
+#endif
+#ifndef FBLA_ROWS_FAST
+#define FBLA_ROWS_FAST 3
+#endif
+#ifndef FBLA_BWDA_OCC3
+#define FBLA_BWDA_OCC3 0
+#endif
 
 template <typename T> struct Ops;
 
@@ -107,8 +117,12 @@ template <> struct Ops<__bf16> {
   static constexpr uint32_t kOnes = 0x3f803f80u;
 };
 
+// two floats rounded to T, packed (a in the low half): written as a vector conversion so that
+// the compiler can use the packed / half-writing conversion instructions
 template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b) {
-  return Ops<T>::bits(a) | (Ops<T>::bits(b) << 16);
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef T tx2_t __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{a, b}, tx2_t));
 }
 
 // ===========================================================================
@@ -240,7 +254,12 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
   int64_t bos, row0, rstride;
   int len;
   seq_range(p, n, bos, len);
-  const int t_begin = c * chunk;
+  // Interleaved walk (dense tensors): the nchunks workgroups of a head sweep it together,
+  // workgroup c taking every nchunks-th step of kStep * G tokens, so that at any time they read
+  // one moving window of the head instead of nchunks distant streams.
+  constexpr int kStep = 16 * TILES;
+  const bool il = !STATS && (p.flags & kInterleave) != 0;
+  const int t_begin = il ? c * (kStep * G) : c * chunk;
   if (t_begin >= len) {
     if (fin_mat && c == 0) {  // empty sequence: its state is zero
       for (int e = threadIdx.x; e < dk * dv; e += kThreads) fin_mat[(int64_t)nh * dk * dv + e] = 0.f;
@@ -249,7 +268,8 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
     }
     return;
   }
-  const int t_end = min(len, t_begin + chunk);
+  const int t_end = il ? len : min(len, t_begin + chunk);
+  const int t_stride = kStep * G * (il ? nchunks : 1);
   row_base(p, n, h, bos, row0, rstride);
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -279,7 +299,6 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
   // interleaved.  Two register buffers alternate (the loop is unrolled by two so that no
   // copy is needed): the loads of the next step are issued, unconditionally, before the
   // current step is multiplied.
-  constexpr int kStep = 16 * TILES;
   struct Buf {
     RowWords<CK> k[TILES];
     RowWords<CV> v[TILES];
@@ -447,10 +466,12 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
   // token walk: single tiles interleaved over the G waves, or (STATS) whole 64-token blocks
   auto next = [&](int t) {
     if constexpr (STATS) return ((t + 16) & 63) ? t + 16 : t + 16 + 64 * (G - 1);
-    else return t + kStep * G;
+    else return t + t_stride;
   };
   int t0 = t_begin + (STATS ? 64 : kStep) * g;
-  if (t_end - t_begin < 16) {
+  // fewer rows than one tile: in the interleaved walk a moved-back tile may reach into the
+  // steps of other workgroups (it zeroes what it shares), so only the sequence length matters
+  if (il ? len < 16 : t_end - t_begin < 16) {
     if (t0 < t_end) {
       Buf b0;
       fetch_checked(b0, t0);
@@ -856,7 +877,7 @@ template <int DR, int DC, bool DEN, int WAVES> struct RowsLayout {
 // odd length leaves the second half of the last pair out.  No partial sums in the prologue.
 template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD = false,
           int PF = (DR == 128 && DC == 128) ? FBLA_ROWS_PF128 : FBLA_ROWS_PF, bool PAIR = false>
-__global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, RowsJob job1,
+__global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64 && !DEN) ? 4 : 1) void rows_kernel(Prob p, RowsJob job0, RowsJob job1,
                                                           int wgs_per_job, int chunk, int nchunks,
                                                           int dr_true, int dc_true) {
   static_assert(!PAIR || (DR == 64 && DC == 64 && !PAD), "pair mode: two 32-wide rows per 64-wide row");
@@ -887,7 +908,11 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
   int len;
   seq_range(p, n, bos, len);
   const int nrows = PAIR ? (len + 1) >> 1 : len;  // rows of this kernel
-  const int t_begin = c * chunk;
+  // interleaved walk: the nchunks workgroups of a head take every nchunks-th step of
+  // 32 * WAVES rows (one moving window per head instead of nchunks distant streams)
+  const bool il = (p.flags & kInterleave) != 0;
+  const int t_begin = il ? c * (32 * WAVES) : c * chunk;
+  const int t_stride = 32 * WAVES * (il ? nchunks : 1);
   if (t_begin >= nrows) {
     if (c == 0 && job.pnchunks > 0) {  // empty sequence: its state is zero
       if (job.mat_out)
@@ -897,7 +922,7 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
     }
     return;
   }
-  const int t_end = min(nrows, t_begin + chunk);
+  const int t_end = il ? nrows : min(nrows, t_begin + chunk);
   row_base(p, n, h, bos, row0, rstride);
   // element offset of 16-byte piece `ch` of row `tok` (rows of `rowlen` elements), or -1 when
   // the piece does not exist
@@ -911,7 +936,7 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
     }
   };
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const bool has_add = job.addvec != nullptr || job.vec_is_add;  // the same for all lanes
   const T* x = (const T*)job.x;
   const T* xden = (const T*)job.xden;
@@ -944,15 +969,31 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
       *reinterpret_cast<u32x4*>(dstb + swz<XROWB>(row, ch)) = src[i];
     }
   };
+  // Whole tiles of plain rows (every tile but a ragged last one): a wave-uniform tile address
+  // plus one constant byte offset per lane, and a uniform step between the lane's pieces; no
+  // bounds checks and no 64-bit address arithmetic in vector registers.
+  const bool kFast = !PAD && !PAIR && rstride <= (1 << 15);  // lane offsets stay within 32 bits
+  const uint32_t xrow_b = (uint32_t)rstride * (uint32_t)(XROWB), orow_b = (uint32_t)rstride * (uint32_t)(OROWB);
+  const uint32_t xvoff = (uint32_t)(lane / XCH) * xrow_b + (uint32_t)(lane % XCH) * 16u;
+  const uint32_t ovoff = DR == DC ? xvoff : (uint32_t)(lane / OCH) * orow_b + (uint32_t)(lane % OCH) * 16u;
+  const uint32_t xstep = (uint32_t)(64 / XCH) * xrow_b, ostep = (uint32_t)(64 / OCH) * orow_b;
+  auto tile_ptr = [&](const void* base, int tok0, int rowlen) -> const char* {
+    return reinterpret_cast<const char*>(base) + ((row0 + (int64_t)tok0 * rstride) * rowlen) * (int64_t)sizeof(T);
+  };
+  auto load_tile_full = [&](u32x4(&dst)[XI], const T* src, int tok0) {
+    const char* tp = tile_ptr(src, tok0, DR);
+#pragma unroll
+    for (int i = 0; i < XI; ++i) dst[i] = load_stream<u32x4, kNtRowsLoad>(tp + (size_t)(xvoff + (uint32_t)i * xstep));
+  };
 
   // PF register sets hold the tiles in flight: a tile is requested PF tiles ahead of its use
   int t0 = t_begin + 32 * wave;
   u32x4 xr[PF][XI], xd[DEN ? PF : 1][XI];
 #pragma unroll
   for (int f = 0; f < PF; ++f)
-    if (t0 + 32 * WAVES * f < t_end) {
-      load_tile(xr[f], x, t0 + 32 * WAVES * f);
-      if constexpr (DEN) load_tile(xd[f], xden, t0 + 32 * WAVES * f);
+    if (t0 + t_stride * f < t_end) {
+      load_tile(xr[f], x, t0 + t_stride * f);
+      if constexpr (DEN) load_tile(xd[f], xden, t0 + t_stride * f);
     }
 
   // ---- prologue: matrix operand fragments, km pairs, addvec ----
@@ -963,7 +1004,7 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
   if (job.pnchunks > 0) {
     const int E = dr * dc;
     const int64_t pstride = E + p.DK;
-    const int nsum = (len + job.pchunk - 1) / job.pchunk;
+    const int nsum = min(job.pnchunks, (len + job.pchunk - 1) / job.pchunk);
     const float* part = job.mat + (int64_t)nh * job.pnchunks * pstride;
     const bool writer = c == 0;
     denorm = build_operand<T, DR, DC, NT, PAD>(lds_opnd, lds_max, part, job.ld_r, job.ld_c, nsum, pstride,
@@ -996,8 +1037,11 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
     wave_sync();  // previous tile's staging reads are done
     stash_tile(xcur, stage);
     if constexpr (DEN) stash_tile(dcur, stage_den);
-    const int tn = t0 + 32 * WAVES * PF;
-    if (tn < t_end) {
+    const int tn = t0 + t_stride * PF;
+    if ((FBLA_ROWS_FAST & 1) && !NORM && kFast && tn + 32 <= t_end) {
+      load_tile_full(xcur, x, tn);
+      if constexpr (DEN) load_tile_full(dcur, xden, tn);
+    } else if (tn < t_end) {
       load_tile(xcur, x, tn);
       if constexpr (DEN) load_tile(dcur, xden, tn);
     }
@@ -1090,13 +1134,19 @@ __global__ __launch_bounds__(WAVES * 64) void rows_kernel(Prob p, RowsJob job0, 
       const int q = lane + 64 * i;
       wout[i] = *reinterpret_cast<const u32x4*>(stage + swz<OROWB>(q / OCH, q % OCH));
     }
+    if ((FBLA_ROWS_FAST & 2) && !NORM && kFast && t0 + 32 <= t_end) {
+      char* tp = const_cast<char*>(tile_ptr(out, t0, DC));
 #pragma unroll
-    for (int i = 0; i < OI; ++i) {
-      const int q = lane + 64 * i, row = q / OCH, ch = q % OCH;
-      const int64_t off = piece(t0 + row, ch, dc);
-      if (off >= 0) store_row16<kNtRowsStore>(out + off, wout[i]);
+      for (int i = 0; i < OI; ++i) store_row16<kNtRowsStore>(tp + (size_t)(ovoff + (uint32_t)i * ostep), wout[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < OI; ++i) {
+        const int q = lane + 64 * i, row = q / OCH, ch = q % OCH;
+        const int64_t off = piece(t0 + row, ch, dc);
+        if (off >= 0) store_row16<kNtRowsStore>(out + off, wout[i]);
+      }
     }
-    t0 += 32 * WAVES;
+    t0 += t_stride;
   };
   while (t0 < t_end) {
 #pragma unroll
@@ -1155,7 +1205,7 @@ template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struc
 // before the store.  `chunk` counts row pairs.
 template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true, bool PAD = false,
           bool PAIR = false>
-__global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
+__global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) ? 3 : 2) void bwd_a_kernel(
     Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const T* __restrict__ dout,
     const float* __restrict__ S, const float* __restrict__ km, T* __restrict__ dqn,
     T* __restrict__ dqd, float* __restrict__ partial, float* __restrict__ tokscal,
@@ -1180,7 +1230,10 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
   int len;
   seq_range(p, n, bos, len);
   const int nrows = PAIR ? (len + 1) >> 1 : len;  // rows of this kernel
-  const int t_begin = c * chunk;
+  // interleaved walk: the nchunks workgroups of a head take every nchunks-th step of 128 rows
+  const bool il = FUSED && (p.flags & kInterleave) != 0;
+  const int t_begin = il ? c * (32 * kWaves) : c * chunk;
+  const int t_stride = 32 * kWaves * (il ? nchunks : 1);
   if (t_begin >= nrows) {
     if (fin_mat && c == 0) {  // empty sequence: no gradient flows through its state
       for (int e = threadIdx.x; e < dk * dv; e += kThreads) fin_mat[(int64_t)nh * dk * dv + e] = 0.f;
@@ -1189,7 +1242,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     }
     return;
   }
-  const int t_end = min(nrows, t_begin + chunk);
+  const int t_end = il ? nrows : min(nrows, t_begin + chunk);
   row_base(p, n, h, bos, row0, rstride);
   // element offset of 16-byte piece `ch` of row `tok` (rows of `rowlen` elements), or -1 when
   // the piece does not exist
@@ -1203,7 +1256,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     }
   };
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int ntok = lane & 31, kb = lane >> 5;
 
   unsigned char* lds_opnd = smem;
@@ -1265,6 +1318,35 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
         store_row16<kNtPassAStore>(dst + off, *reinterpret_cast<const u32x4*>(srcb + swz<QROWB>(row, ch)));
     }
   };
+  // Whole tiles of plain rows: a wave-uniform tile address plus one constant byte offset per
+  // lane and a uniform step between the lane's pieces (as in the rows kernel).
+  const bool kFast = !PAD && !PAIR && rstride <= (1 << 15);  // lane offsets stay within 32 bits
+  const uint32_t qrow_b = (uint32_t)rstride * (uint32_t)QROWB, grow_b = (uint32_t)rstride * (uint32_t)GROWB;
+  const uint32_t qvoff = (uint32_t)(lane / QCH) * qrow_b + (uint32_t)(lane % QCH) * 16u;
+  const uint32_t gvoff = (uint32_t)(lane / GCH) * grow_b + (uint32_t)(lane % GCH) * 16u;
+  const uint32_t qstep = (uint32_t)(64 / QCH) * qrow_b, gstep = (uint32_t)(64 / GCH) * grow_b;
+  auto tile_ptr = [&](const void* base, int tok0, int rowlen) -> const char* {
+    return reinterpret_cast<const char*>(base) + ((row0 + (int64_t)tok0 * rstride) * rowlen) * (int64_t)sizeof(T);
+  };
+  auto load_q_full = [&](u32x4(&dst)[QI], const T* src, int tok0) {
+    const char* tp = tile_ptr(src, tok0, DK);
+#pragma unroll
+    for (int i = 0; i < QI; ++i) dst[i] = load_stream<u32x4, kNtPassALoad>(tp + (size_t)(qvoff + (uint32_t)i * qstep));
+  };
+  auto load_g_full = [&](u32x4(&dst)[GI], const T* src, int tok0) {
+    const char* tp = tile_ptr(src, tok0, DV);
+#pragma unroll
+    for (int i = 0; i < GI; ++i) dst[i] = load_stream<u32x4, kNtPassALoad>(tp + (size_t)(gvoff + (uint32_t)i * gstep));
+  };
+  auto store_q_full = [&](const unsigned char* srcb, T* dst, int tok0) {
+    char* tp = const_cast<char*>(tile_ptr(dst, tok0, DK));
+#pragma unroll
+    for (int i = 0; i < QI; ++i) {
+      const int q = lane + 64 * i;
+      store_row16<kNtPassAStore>(tp + (size_t)(qvoff + (uint32_t)i * qstep),
+                                 *reinterpret_cast<const u32x4*>(srcb + swz<QROWB>(q / QCH, q % QCH)));
+    }
+  };
 
   int t0 = t_begin + 32 * wave;
   u32x4 rq[QI], rg[GI], rd[QI];
@@ -1287,8 +1369,12 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
     stash_q(rq, qt);
     stash_g(rg, gt);
     if constexpr (DEN) stash_q(rd, qdt);
-    const int tn = t0 + 32 * kWaves;
-    if (tn < t_end) {
+    const int tn = t0 + t_stride;
+    if (kFast && tn + 32 <= t_end) {
+      load_q_full(rq, qn, tn);
+      load_g_full(rg, dout, tn);
+      if constexpr (DEN) load_q_full(rd, qd, tn);
+    } else if (tn < t_end) {
       load_q(rq, qn, tn);
       load_g(rg, dout, tn);
       if constexpr (DEN) load_q(rd, qd, tn);
@@ -1442,8 +1528,13 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_a_kernel(
             u32x4{dqdp[4 * ch], dqdp[4 * ch + 1], dqdp[4 * ch + 2], dqdp[4 * ch + 3]};
     }
     wave_sync();
-    store_q(qt, dqn, t0);
-    if constexpr (DEN) store_q(qdt, dqd, t0);
+    if (kFast && t0 + 32 <= t_end) {
+      store_q_full(qt, dqn, t0);
+      if constexpr (DEN) store_q_full(qdt, dqd, t0);
+    } else {
+      store_q(qt, dqn, t0);
+      if constexpr (DEN) store_q(qdt, dqd, t0);
+    }
     t0 = tn;
   }
 
@@ -2011,6 +2102,28 @@ static Prob xcd_ordered(const Prob& p, int kernel_bit) {
   static const int mask = [] { const char* v = getenv("FBLA_XCD_ORDER"); return v ? atoi(v) : 2; }();
   Prob r = p;
   if (p.cu && (mask & kernel_bit)) r.flags |= kXcdOrder;
+  return r;
+}
+
+// Dense tensors, 16-bit heads tiled 64 x 64 (not the two-tokens-per-row mode): which kernels let
+// the workgroups of a head take interleaved token steps (bit 0 the state kernel, bit 1 the
+// row-parallel kernels, bit 2 backward pass A).
+static int interleave_mask() {
+  static const int mask = [] { const char* v = getenv("FBLA_ILEAVE"); return v ? atoi(v) : 7; }();
+  return mask;
+}
+bool interleaved(const Prob& p, int dtype, int kernel_bit) {
+  return (interleave_mask() & kernel_bit) && !p.cu && dtype != kF32 && small_tiles(p.DK, p.DV) &&
+         !pair_mode(p, dtype);
+}
+// Tokens per partial as the reduction sees them: workgroup c of an interleaved walk has work
+// when c * granule < len.
+int partial_chunk(const Prob& p, int dtype, int kernel_bit, int chunk) {
+  return interleaved(p, dtype, kernel_bit) ? (kernel_bit == 1 ? 64 : 128) : chunk;
+}
+Prob with_interleave(const Prob& p, int dtype, int kernel_bit) {
+  Prob r = p;
+  if (interleaved(p, dtype, kernel_bit)) r.flags |= kInterleave;
   return r;
 }
 

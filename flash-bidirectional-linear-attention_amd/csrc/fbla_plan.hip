@@ -136,26 +136,28 @@ int forward(const Prob& pc_, int dtype, const FwdArgs& a, hipStream_t st) {
   const bool direct = fast && nchunks == 1;
   if (phases & kPhaseFwdState) {
     if (fast)
-      mfma::state(p, dtype, kn, a.v, a.k, partial, chunk, nchunks, st, direct ? a.s : nullptr,
-                  direct ? a.km : nullptr);
+      mfma::state(mfma::with_interleave(p, dtype, 1), dtype, kn, a.v, a.k, partial, chunk, nchunks, st,
+                  direct ? a.s : nullptr, direct ? a.km : nullptr);
     else
       generic::state_partial(p, dtype, kn, a.v, a.k, partial, chunk, nchunks, st);
   }
   const bool fold = fast && !direct && !is_cross && dtype != kF32 && !mfma::pair_mode(p, dtype) &&
                     fold_reduce(p, nchunks, p.DK, p.DV);
+  // tokens per partial as the consumers of the partials count them
+  const int pchunk = fast ? mfma::partial_chunk(p, dtype, 1, chunk) : chunk;
   if (!fold && !direct && (phases & kPhaseFwdReduce))
-    generic::state_reduce(p, partial, chunk, nchunks, a.s, nullptr, a.km, st);
+    generic::state_reduce(p, partial, pchunk, nchunks, a.s, nullptr, a.km, st);
   if (phases & kPhaseFwdOutput) {
     if (fast) {
       mfma::RowsJob job{qn, normalize ? a.q : nullptr, a.s, p.DV, 1, a.km, nullptr, a.o};
       if (fold) {  // the output kernel sums the partials itself and stores S and km on the way
         job.mat = partial;
-        job.pchunk = chunk;
+        job.pchunk = pchunk;
         job.pnchunks = nchunks;
         job.mat_out = a.s;
         job.vec_out = a.km;
       }
-      int rc = mfma::rows(pq, dtype, job, p.DK, p.DV, st);
+      int rc = mfma::rows(mfma::with_interleave(pq, dtype, 2), dtype, job, p.DK, p.DV, st);
       if (rc != kOk) return rc;
     } else {
       generic::output(pq, dtype, qn, a.q, a.s, a.km, a.o, st);
@@ -200,8 +202,8 @@ int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
   float* fv = direct ? dkm : nullptr;
   if (phases & kPhaseBwdA) {
     if (mfma::bwd_a_supported(p, dtype)) {
-      int rc = mfma::bwd_a(p, dtype, qn, a.q, a.dout, a.s, a.km, dqn, dqd, partial, chunk, nchunks, st,
-                           fm, fv);
+      int rc = mfma::bwd_a(mfma::with_interleave(p, dtype, 4), dtype, qn, a.q, a.dout, a.s, a.km, dqn, dqd,
+                           partial, chunk, nchunks, st, fm, fv);
       if (rc != kOk) return rc;
     } else if (fast) {
       // head dims above 64: token view and feature view as two kernels
@@ -219,8 +221,9 @@ int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
   }
   const bool fold = fast && !direct && !is_cross && dtype != kF32 && !mfma::pair_mode(p, dtype) &&
                     fold_reduce(p, nchunks, p.DV, p.DK);
+  const int pchunk = mfma::bwd_a_supported(p, dtype) ? mfma::partial_chunk(p, dtype, 4, chunk) : chunk;
   if (!fold && !direct && (phases & kPhaseBwdReduce))
-    generic::state_reduce(p, partial, chunk, nchunks, dS, fast ? nullptr : dSt, dkm, st);
+    generic::state_reduce(p, partial, pchunk, nchunks, dS, fast ? nullptr : dSt, dkm, st);
   if (phases & kPhaseBwdB) {
     if (fast) {
       // dk~_t = v_t (s dS)^T (+ dkm/L): contraction over dv, M(r=dv, c=dk) = dS[c][r]
@@ -229,7 +232,7 @@ int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
       mfma::RowsJob jv{kn, nullptr, dS, p.DV, 1, nullptr, nullptr, a.dv};
       if (fold) {  // both kernels sum the pass-A partials themselves (s dS, dkm/L)
         jk.mat = jv.mat = partial;
-        jk.pchunk = jv.pchunk = chunk;
+        jk.pchunk = jv.pchunk = pchunk;
         jk.pnchunks = jv.pnchunks = nchunks;
         jk.addvec = nullptr;
         jk.vec_is_add = !dec && normalize;
@@ -238,11 +241,12 @@ int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
       // dkm arrives divided by the number of queries; the formula wants dkm / (number of keys)
       if (is_cross) jk.add_scale = (float)p.L / (float)pk.L;
       int rc;
+      const Prob pki = mfma::with_interleave(pk, dtype, 2);
       if (p.DK == p.DV) {  // same shape: one launch
-        rc = mfma::rows2(pk, dtype, jk, jv, p.DV, p.DK, st);
+        rc = mfma::rows2(pki, dtype, jk, jv, p.DV, p.DK, st);
       } else {
-        rc = mfma::rows(pk, dtype, jk, p.DV, p.DK, st);
-        if (rc == kOk) rc = mfma::rows(pk, dtype, jv, p.DK, p.DV, st);
+        rc = mfma::rows(pki, dtype, jk, p.DV, p.DK, st);
+        if (rc == kOk) rc = mfma::rows(pki, dtype, jv, p.DK, p.DV, st);
       }
       if (rc != kOk) return rc;
       if (dec) generic::broadcast_rows(p, dtype, dkm, dkd, st);
