@@ -125,3 +125,28 @@ def test_oracle_reproduces_golden_fixture(path):
             if name.endswith("_mag"):
                 got = got.max(axis=-1, keepdims=True)
             np.testing.assert_allclose(got, ref, rtol=1e-12, atol=1e-14)
+
+
+def test_package_torch_formulas_match_the_oracle_restatement():
+    """flash_bla.ops.*.naive are written in their own terms (einsum over a shared helper); the
+    oracle restates the reference line by line.  Same values, fp64, all four functions."""
+    import torch
+    from flash_bla.ops.linear_attn import naive as pkg
+    from flash_bla.ops.simple_la.naive import naive_simple_la
+    from oracle import torch_ref as tr
+    g = torch.Generator().manual_seed(3)
+    q, k, qr, kr = (torch.rand(2, 3, 29, 12, generator=g, dtype=torch.float64) + 0.1 for _ in range(4))
+    v = torch.randn(2, 3, 29, 7, generator=g, dtype=torch.float64)
+    for scale in (None, 0.37):
+        torch.testing.assert_close(pkg.naive_linear_attn(q, k, v, scale), tr.naive_linear_attn(q, k, v, scale),
+                                   rtol=1e-12, atol=1e-14)
+        torch.testing.assert_close(pkg.naive_decoupled_la(q, k, qr, kr, v, scale),
+                                   tr.naive_decoupled_la(q, k, qr, kr, v, scale), rtol=1e-12, atol=1e-14)
+        torch.testing.assert_close(naive_simple_la(q, k, v, scale), tr.naive_simple_la(q, k, v, scale),
+                                   rtol=1e-12, atol=1e-14)
+    cu = torch.tensor([0, 5, 18, 19, 40], dtype=torch.int32)
+    qp, kp = (torch.rand(40, 3, 12, generator=g, dtype=torch.float64) + 0.1 for _ in range(2))
+    vp = torch.randn(40, 3, 7, generator=g, dtype=torch.float64)
+    for scale in (None, 0.2):
+        torch.testing.assert_close(pkg.naive_varlen_linear_attn(qp, kp, vp, cu, scale, 1e-5),
+                                   tr.naive_varlen_linear_attn(qp, kp, vp, cu, scale, 1e-5), rtol=1e-12, atol=1e-14)
