@@ -29,19 +29,26 @@ import torch.nn.functional as F  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
-# HBM bytes per launch of each large kernel at the default workload (B8-H16-D64,
-# T=16384, fp16), from two `rocprofv3 --pmc` runs of `bench.py --probe 3`
-# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch).  FETCH_SIZE is scaled by 2.0:
-# the 256 MiB device copy of the same run reads 256 MiB and the counter shows
-# 128.0 MiB; WRITE_SIZE shows 256.0 MiB for it (factor 1.0).
 CLOCK_RAMP_S = 0.1  # untimed work before the warm-up steps
 
-MEASURED_TRAFFIC = {
-    "fwd_state": int((2 * 256.7 + 8.1) * 2 ** 20),
-    "fwd_output": int((2 * 136.2 + 256.0) * 2 ** 20),
-    "bwd_pass_a": int((2 * 260.2 + 264.1) * 2 ** 20),
-    "bwd_pass_b": int((2 * 264.7 + 512.0) * 2 ** 20),
-}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "linear_attn_fwd_bwd_B8H16T16384D64_fp16_hbm_traffic.md")
+TRAFFIC_ROW = {"fwd_state": "state_kernel", "fwd_output": "rows_kernel NORM", "bwd_pass_a": "bwd_a_kernel",
+               "bwd_pass_b": "rows_kernel x2"}
+
+
+def measured_traffic(kernel):
+    """HBM bytes per launch of `kernel` at the default workload, read from the counter summary
+    under profiles/ (column "HBM MiB" of its table); None when the file or the row is missing."""
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            for line in f:
+                cells = [c.strip() for c in line.split("|")]
+                if len(cells) > 6 and cells[1].startswith(TRAFFIC_ROW[kernel]):
+                    return int(float(cells[5]) * 2 ** 20)
+    except (OSError, ValueError, KeyError):
+        pass
+    return None
+
 
 PHASES = {  # name -> (phase bit, tensors read+written once, entry point)
     "fwd_state": (1, 2, "fwd"),     # reads k, v
@@ -96,33 +103,69 @@ def do_bench(fn, flush, quantiles=(0.5, 0.2, 0.8)):
     return [float(x) for x in torch.quantile(times, torch.tensor(quantiles, dtype=torch.float64))]
 
 
+def _cpu_time(fn, reps):
+    times = []
+    for _ in range(reps + 1):  # the first run warms the allocator and the thread pool
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return sorted(times[1:])[len(times[1:]) // 2]
+
+
+def _cpu_inputs(shape, dtype_round, seed=42):
+    g = torch.Generator().manual_seed(seed)
+    q = F.elu(torch.randn(shape, generator=g)) + 1
+    k = F.elu(torch.randn(shape, generator=g)) + 1
+    v = torch.randn(shape, generator=g)
+    do = torch.randn(shape, generator=g)
+    if dtype_round is not None:  # fp32 math on values already rounded to the GPU workload's type
+        q, k, v, do = (t.to(dtype_round).float() for t in (q, k, v, do))
+    return q, k, v, do
+
+
 def cpu_baseline(T, D, H, sample_batches, reps=3):
-    """Reference torch path (oracle.torch_ref.naive_linear_attn + autograd) on the
-    host cores, fp32 math on fp16-valued inputs, for `sample_batches` of the 8
-    batches of the workload."""
+    """Reference torch path (oracle.torch_ref, the restatement of the reference's naive operators,
+    + autograd) on the host cores.  The headline entry is linear_attn fwd+bwd on `sample_batches`
+    of the 8 batches of the workload; `configs` adds BASELINE config 1 (forward, fp32, 10 runs) and
+    the other lengths of config 2, each on a bounded sample."""
     from oracle import torch_ref
     torch.set_num_threads(os.cpu_count() or 1)
-    g = torch.Generator().manual_seed(42)
-    shape = (sample_batches, H, T, D)
-    q = (F.elu(torch.randn(shape, generator=g)) + 1).half().float().requires_grad_()
-    k = (F.elu(torch.randn(shape, generator=g)) + 1).half().float().requires_grad_()
-    v = torch.randn(shape, generator=g).half().float().requires_grad_()
-    do = torch.randn(shape, generator=g).half().float()
-    times = []
-    for _ in range(reps + 1):
-        q.grad = k.grad = v.grad = None
-        t0 = time.perf_counter()
-        torch_ref.naive_linear_attn(q, k, v).backward(do)
-        times.append(time.perf_counter() - t0)
-    t = sorted(times[1:])[len(times[1:]) // 2]
-    bytes_fp16 = 11 * sample_batches * H * T * D * 2
+    cores = torch.get_num_threads()
+
+    def fwd_bwd_entry(Tn, batches, nreps):
+        q, k, v, do = _cpu_inputs((batches, H, Tn, D), torch.float16)
+        for t in (q, k, v):
+            t.requires_grad_()
+
+        def run():
+            q.grad = k.grad = v.grad = None
+            torch_ref.naive_linear_attn(q, k, v).backward(do)
+        t = _cpu_time(run, nreps)
+        nbytes = 11 * batches * H * Tn * D * 2
+        return {"config": f"C2 linear_attn fwd+bwd T={Tn}", "value": round(nbytes / t / 1e9, 3), "unit": "GB/s",
+                "ms": round(t * 1e3, 3), "reps": nreps,
+                "sample": f"{batches} of 8 batches (B{batches},H{H},T{Tn},D{D}), fp32 math on the fp16-valued "
+                          f"inputs; bytes counted as the fp16 workload's 11 tensor passes"}
+
+    head = fwd_bwd_entry(T, sample_batches, reps)
+    configs = []
+    # BASELINE config 1: the reference's own CPU-runnable case, forward, fp32
+    q, k, v, _ = _cpu_inputs((2, 4, 1024, 64), None)
+    nb1 = 4 * q.numel() * 4
+    with torch.no_grad():
+        for name, fn in (("simple_la", lambda: torch_ref.naive_simple_la(q, k, v)),
+                         ("linear_attn", lambda: torch_ref.naive_linear_attn(q, k, v))):
+            t = _cpu_time(fn, 10)
+            configs.append({"config": f"C1 {name} forward B2-H4-T1024-D64 fp32", "value": round(nb1 / t / 1e9, 3),
+                            "unit": "GB/s", "ms": round(t * 1e3, 3), "reps": 10,
+                            "sample": "the whole config; bytes = 4 fp32 tensor passes"})
+    for Tn, batches, nreps in ((1024, 8, 5), (4096, 8, 3), (32768, 1, 2)):
+        if Tn != T:
+            configs.append(fwd_bwd_entry(Tn, batches, nreps))
     return {
-        "value": round(bytes_fp16 / t / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
-        "kind": "port",
-        "sample": f"linear_attn fwd+bwd, {sample_batches} of 8 batches (B{sample_batches},H{H},T{T},D{D}), "
-                  f"fp32 math on the fp16-valued inputs, median of {reps} runs; "
-                  f"{t * 1e3:.1f} ms per run; bytes counted as the fp16 workload's 11 tensor passes",
-        "ms": round(t * 1e3, 3),
+        "value": head["value"], "unit": "GB/s", "cores": cores, "kind": "port",
+        "sample": f"linear_attn fwd+bwd, {head['sample']}, median of {reps} runs; {head['ms']:.1f} ms per run",
+        "ms": head["ms"], "configs": configs,
     }
 
 
@@ -175,8 +218,11 @@ def main():
     ap.add_argument("--T", type=int, default=16384)
     ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16", "fp32"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--sweep", action="store_true",
-                    help="also print a table over T in {1024,4096,16384,32768} to stderr")
+    ap.add_argument("--no-sweep", action="store_true",
+                    help="skip the table over T in {1024,4096,16384,32768} (the `sweep` list of the JSON line)")
+    ap.add_argument("--sweep", action="store_true", help="accepted for compatibility: the sweep is on by default")
+    ap.add_argument("--tables-md", default=None, metavar="PATH",
+                    help="with --tables: also write the tables as markdown to PATH")
     ap.add_argument("--probe", type=int, default=0, metavar="N",
                     help="counter-collection mode for rocprofv3 --pmc: run N steps of the workload, each "
                          "followed by a 256 MiB device copy of known traffic, then exit")
@@ -260,7 +306,8 @@ def main():
     roofline = {
         "bound": "hbm", "kernel": dom, "achieved": kern[dom]["gbps"], "peak": HBM_PEAK_GBPS,
         "unit": "GB/s", "frac": kern[dom]["frac"],
-        "traffic": MEASURED_TRAFFIC.get(dom) if (T == 16384 and args.dtype == "fp16") else None,
+        "traffic": measured_traffic(dom) if (T == 16384 and args.dtype == "fp16") else None,
+        "traffic_source": os.path.relpath(TRAFFIC_PROFILE, ROOT),
         "alg_bytes_per_launch": kern[dom]["alg_bytes"], "avg_launch_ms": kern[dom]["ms"],
     }
     cpu = None if args.no_cpu else cpu_baseline(T, D, H, sample_batches=2)
@@ -284,7 +331,8 @@ def main():
         "cpu_baseline": cpu,
         "fwd_bwd": {"ms_p50_p20_p80_flushed": [round(x, 5) for x in step_q],
                     "gbps_p50": round(step_bytes / step_q[0] / 1e6, 1),
-                    "frac_of_peak": round(step_bytes / ms_per_step / 1e6 / HBM_PEAK_GBPS, 4)},
+                    "frac_of_peak": round(step_bytes / step_q[0] / 1e6 / HBM_PEAK_GBPS, 4),
+                    "frac_back_to_back": round(step_bytes / ms_per_step / 1e6 / HBM_PEAK_GBPS, 4)},
         "fwd": {"ms_back_to_back": round(fwd_loop_ms, 5),
                 "gbps_back_to_back": round(fwd_bytes / fwd_loop_ms / 1e6, 1),
                 "frac_back_to_back": round(fwd_bytes / fwd_loop_ms / 1e6 / HBM_PEAK_GBPS, 4),
@@ -295,20 +343,22 @@ def main():
         "device_copy_gbps": copy_gbps,
         "parity": parity,
     }
-    if args.sweep:
-        sweep(dtype, dev, flush)
+    if not args.no_sweep:
+        del q, k, v, do, o
+        line["sweep"] = sweep(dtype, dev, flush)
     if args.configs:
         other_configs(dev, flush)
         layer_config(dev, flush)
         piecewise_config(dev, flush)
     if args.tables:
-        reference_tables(dev, flush)
+        reference_tables(dev, flush, args.tables_md)
     print(json.dumps(line), flush=True)
 
 
 def sweep(dtype, dev, flush):
-    """Per-length table (forward and forward+backward, flushed medians) on stderr."""
+    """Per-length rows (forward and forward+backward, flushed medians) of BASELINE config 2."""
     from flash_bla.ops.linear_attn.fused import linear_attention
+    rows = []
     for T in (1024, 4096, 16384, 32768):
         q, k, v, do = make_inputs(8, 16, T, 64, dtype, dev)
         q.requires_grad_(), k.requires_grad_(), v.requires_grad_()
@@ -324,9 +374,12 @@ def sweep(dtype, dev, flush):
 
         f = do_bench(fwd_only, flush)
         s = do_bench(step, flush)
-        print(json.dumps({"T": T, "fwd_ms": round(f[0], 5), "fwd_gbps": round(4 * nbytes / f[0] / 1e6, 1),
-                          "fwd_bwd_ms": round(s[0], 5), "fwd_bwd_gbps": round(11 * nbytes / s[0] / 1e6, 1)}),
-              file=sys.stderr, flush=True)
+        rows.append({"T": T, "fwd_ms": round(f[0], 5), "fwd_gbps": round(4 * nbytes / f[0] / 1e6, 1),
+                     "fwd_frac": round(4 * nbytes / f[0] / 1e6 / HBM_PEAK_GBPS, 4),
+                     "fwd_bwd_ms": round(s[0], 5), "fwd_bwd_gbps": round(11 * nbytes / s[0] / 1e6, 1),
+                     "fwd_bwd_frac": round(11 * nbytes / s[0] / 1e6 / HBM_PEAK_GBPS, 4)})
+        del q, k, v, do
+    return rows
 
 
 def _report(name, nbytes_fwd, nbytes_step, fwd_fn, step_fn, flush, extra=None):
@@ -476,50 +529,89 @@ def layer_config(dev, flush):
                           "modes_max_abs_diff_over_max": round(err / ref, 6)}), file=sys.stderr, flush=True)
 
 
-def reference_tables(dev, flush):
-    """The tables of the reference's benchmark scripts, with the torch formula and torch's
-    scaled_dot_product_attention beside the HIP operators (benchmarks/ops/benchmark_linear_attn.py:
-    B8-H16-D64 fp16 over T; benchmark_varlen_linear_attn.py:20-52: 8 sequences, padded batch
-    against the packed operator at max_seqlen 256/1024/4096)."""
+def reference_tables(dev, flush, md_path=None):
+    """The tables of the reference's three benchmark scripts, columns named as there:
+    benchmarks/ops/benchmark_linear_attn.py (providers torch_la / flash_bla / torch_sdpa, `_fwd` and
+    `_bwd` = forward + backward, T in {1024, 4096, 16384, 32768}; the script runs B2-H16-D64 bf16,
+    the README quotes B8 fp16: both), benchmark_decoupled_la.py:11-62 (B2-H16-D64 bf16) and
+    benchmark_varlen_linear_attn.py:20-86 (8 equal sequences, H16-D64 bf16, the padded dense
+    operator against the packed one, forward and forward + backward).  Flushed medians in ms;
+    gradients are reset before every backward (the scripts let them accumulate in the leaves,
+    which times one more elementwise pass per tensor)."""
+    from flash_bla.ops.linear_attn.decoupled import decoupled_la
     from flash_bla.ops.linear_attn.fused import linear_attention
-    from flash_bla.ops.linear_attn.naive import naive_linear_attn
+    from flash_bla.ops.linear_attn.naive import naive_decoupled_la, naive_linear_attn
     from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
-    for T in (1024, 4096, 16384):
-        q, k, v, do = make_inputs(8, 16, T, 64, torch.float16, dev)
-        for t in (q, k, v):
-            t.requires_grad_()
+    rows = []
 
+    def emit(row):
+        rows.append(row)
+        print(json.dumps(row), file=sys.stderr, flush=True)
+
+    def time_providers(row, providers, leaves, do):
         def bwd_of(fn):
             def step():
-                q.grad = k.grad = v.grad = None
+                for t in leaves:
+                    t.grad = None
                 fn().backward(do)
             return step
-        row = {"table": "linear_attn B8-H16-D64 fp16", "T": T}
-        for name, fn in (("torch_la", lambda: naive_linear_attn(q, k, v)),
-                         ("flash_bla", lambda: linear_attention(q, k, v)),
-                         ("torch_sdpa", lambda: F.scaled_dot_product_attention(q, k, v))):
+        for name, fn in providers:
             with torch.no_grad():
-                row[name + "_fwd_ms"] = round(do_bench(fn, flush)[0], 4)
-            row[name + "_fwd_bwd_ms"] = round(do_bench(bwd_of(fn), flush)[0], 4)
-        print(json.dumps(row), file=sys.stderr, flush=True)
-    g = torch.Generator().manual_seed(42)
+                row[name + "_fwd"] = round(do_bench(fn, flush)[0], 4)
+            row[name + "_bwd"] = round(do_bench(bwd_of(fn), flush)[0], 4)
+
+    lengths = (1024, 4096, 16384, 32768)
+    for B, dtype, tag in ((2, torch.bfloat16, "bf16"), (8, torch.float16, "fp16")):
+        for T in lengths:
+            q, k, v, do = make_inputs(B, 16, T, 64, dtype, dev)
+            leaves = [t.requires_grad_() for t in (q, k, v)]
+            row = {"table": f"linear_attn B{B}-H16-D64 {tag}", "T": T}
+            time_providers(row, (("torch_la", lambda: naive_linear_attn(q, k, v)),
+                                 ("flash_bla", lambda: linear_attention(q, k, v)),
+                                 ("torch_sdpa", lambda: F.scaled_dot_product_attention(q, k, v))), leaves, do)
+            emit(row)
+            del q, k, v, do, leaves
+    for T in lengths:
+        q, k, v, do = make_inputs(2, 16, T, 64, torch.bfloat16, dev)
+        qr, kr, _, _ = make_inputs(2, 16, T, 64, torch.bfloat16, dev, seed=7)
+        leaves = [t.requires_grad_() for t in (q, k, qr, kr, v)]
+        row = {"table": "decoupled_la B2-H16-D64 bf16", "T": T}
+        time_providers(row, (("torch_la", lambda: naive_decoupled_la(q, k, qr, kr, v)),
+                             ("flash_bla", lambda: decoupled_la(q, k, qr, kr, v)),
+                             ("torch_sdpa", lambda: F.scaled_dot_product_attention(q, k, v))), leaves, do)
+        emit(row)
+        del q, k, v, do, qr, kr, leaves
     for max_len in (256, 1024, 4096):
-        lengths = torch.randint(max_len // 4, max_len + 1, (8,), generator=g)
-        lengths[0] = max_len
-        cu = torch.cat([torch.zeros(1, dtype=torch.int32), torch.cumsum(lengths, 0).to(torch.int32)]).to(dev)
-        total = int(lengths.sum())
-        qp = (F.elu(torch.randn(total, 16, 64, device=dev)) + 1).half()
-        kp = (F.elu(torch.randn(total, 16, 64, device=dev)) + 1).half()
-        vp = torch.randn(total, 16, 64, device=dev).half()
-        qd = (F.elu(torch.randn(8, 16, max_len, 64, device=dev)) + 1).half()
-        kd = (F.elu(torch.randn(8, 16, max_len, 64, device=dev)) + 1).half()
-        vd = torch.randn(8, 16, max_len, 64, device=dev).half()
+        cu = (torch.arange(9, dtype=torch.int32) * max_len).to(dev)
+        qd, kd, vd, dod = make_inputs(8, 16, max_len, 64, torch.bfloat16, dev)
+        qp, kp, vp, dop = (t.transpose(1, 2).reshape(8 * max_len, 16, 64).contiguous() for t in (qd, kd, vd, dod))
+        dense, packed = [t.requires_grad_() for t in (qd, kd, vd)], [t.requires_grad_() for t in (qp, kp, vp)]
+
+        def fwdbwd(fn, leaves, do):
+            def step():
+                for t in leaves:
+                    t.grad = None
+                fn().backward(do)
+            return step
+        pad = lambda: linear_attention(qd, kd, vd)  # noqa: E731
+        var = lambda: varlen_linear_attention(qp, kp, vp, cu, max_len)  # noqa: E731
+        row = {"table": "varlen-equal-B8-H16-D64 bf16", "max_seqlen": max_len}
         with torch.no_grad():
-            t_pad = do_bench(lambda: linear_attention(qd, kd, vd), flush)[0]
-            t_var = do_bench(lambda: varlen_linear_attention(qp, kp, vp, cu, max_len), flush)[0]
-        print(json.dumps({"table": "varlen 8 seqs H16 D64 fp16 fwd", "max_seqlen": max_len, "total_tokens": total,
-                          "padded_dense_ms": round(t_pad, 4), "varlen_ms": round(t_var, 4)}),
-              file=sys.stderr, flush=True)
+            row["flash_padded_fwd"] = round(do_bench(pad, flush)[0], 4)
+            row["varlen_fwd"] = round(do_bench(var, flush)[0], 4)
+        row["flash_padded_fwdbwd"] = round(do_bench(fwdbwd(pad, dense, dod), flush)[0], 4)
+        row["varlen_fwdbwd"] = round(do_bench(fwdbwd(var, packed, dop), flush)[0], 4)
+        emit(row)
+    if md_path:
+        with open(md_path, "w") as f:
+            f.write("Flushed medians in ms (`_bwd` columns = forward + backward, as in the reference's scripts).\n")
+            table = None
+            for row in rows:
+                cols = [c for c in row if c != "table"]
+                if row["table"] != table:
+                    table = row["table"]
+                    f.write(f"\n**{table}**\n\n| " + " | ".join(cols) + " |\n|" + "---|" * len(cols) + "\n")
+                f.write("| " + " | ".join(str(row[c]) for c in cols) + " |\n")
 
 
 def piecewise_config(dev, flush):

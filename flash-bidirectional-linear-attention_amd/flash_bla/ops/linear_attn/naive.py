@@ -12,9 +12,9 @@ def _state_attention(q_num, k_num, q_den, k_den, v, scale, eps):
 
     `scale` multiplies v before the contraction so that the state stays in range for
     16-bit inputs."""
-    state = torch.einsum("...tk,...tv->...kv", k_num, v * scale)
-    denom = torch.einsum("...tk,...k->...t", q_den, k_den.mean(dim=-2)) + eps
-    return torch.einsum("...tk,...kv->...tv", q_num, state) / denom.unsqueeze(-1)
+    state = k_num.mT @ (v * scale)                          # [..., K, V]
+    denom = q_den @ k_den.mean(dim=-2).unsqueeze(-1) + eps  # [..., T, 1]
+    return (q_num @ state) / denom
 
 
 def naive_linear_attn(q, k, v, scale=None):

@@ -128,7 +128,7 @@ def test_oracle_reproduces_golden_fixture(path):
 
 
 def test_package_torch_formulas_match_the_oracle_restatement():
-    """flash_bla.ops.*.naive are written in their own terms (einsum over a shared helper); the
+    """flash_bla.ops.*.naive are written in their own terms (one shared helper); the
     oracle restates the reference line by line.  Same values, fp64, all four functions."""
     import torch
     from flash_bla.ops.linear_attn import naive as pkg
