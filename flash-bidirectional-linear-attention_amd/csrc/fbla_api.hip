@@ -400,8 +400,9 @@ int fbla_chunk_reduce(const void* q, const void* k, const void* v, float* qc, fl
 
 size_t fbla_piecewise_workspace_bytes(int64_t BH, int64_t T, int K, int V, int block, int dtype) {
   if (check_dims("fbla_piecewise_workspace_bytes", BH, 1, T, K, V, dtype, 0) != kOk) return 0;
-  if (!piecewise::attention_supported(K, V, block, dtype)) return 0;
-  return piecewise::attention_workspace_bytes(BH, T, K, V);
+  if (piecewise::attention_supported(K, V, block, dtype)) return piecewise::attention_workspace_bytes(BH, T, K, V);
+  // the shape-generic kernel needs no workspace; a token size keeps "0 = not supported"
+  return piecewise::attention_generic_supported(T, K, V, block, dtype) ? 256 : 0;
 }
 
 int fbla_piecewise_fwd(const void* q, const void* k, const void* v, const float* kc, const float* vc,
@@ -411,12 +412,13 @@ int fbla_piecewise_fwd(const void* q, const void* k, const void* v, const float*
   const char* what = "fbla_piecewise_fwd";
   int rc = check_dims(what, BH, 1, T, K, V, dtype, 0);
   if (rc != kOk) return rc;
-  if (!piecewise::attention_supported(K, V, block, dtype)) {
-    set_error("%s: needs fp16/bf16, head dims in {64,128} and 64-token blocks (got K=%d V=%d block=%d dtype=%d)",
-              what, K, V, block, dtype);
+  const bool fast = piecewise::attention_supported(K, V, block, dtype);
+  if (!fast && !piecewise::attention_generic_supported(T, K, V, block, dtype)) {
+    set_error("%s: needs head dims in [1,128], a positive block size and block flags that fit LDS "
+              "(got K=%d V=%d block=%d dtype=%d T=%lld)", what, K, V, block, dtype, (long long)T);
     return kErrUnsupported;
   }
-  const int64_t NT = (T + 63) / 64;
+  const int64_t NT = (T + block - 1) / block;
   if (NS < 1 || NS > NT) {
     set_error("%s: the number of selected blocks must be in [1, %lld], got %d", what, (long long)NT, NS);
     return kErrBadArg;
@@ -425,6 +427,12 @@ int fbla_piecewise_fwd(const void* q, const void* k, const void* v, const float*
   if (!q || !k || !v || !kc || !vc || !h || !indices || !o) {
     set_error("%s: null tensor pointer", what);
     return kErrBadArg;
+  }
+  if (!fast) {
+    rc = piecewise::attention_generic(q, k, v, kc, vc, h, indices, o, BH, T, K, V, block, NS, scale, dtype,
+                                      (hipStream_t)stream);
+    if (rc != kOk) return rc;
+    return check_launch(what);
   }
   const size_t need = piecewise::attention_workspace_bytes(BH, T, K, V);
   if (workspace_bytes_ < need || !workspace) {
@@ -450,7 +458,7 @@ int fbla_select_blocks(const float* qc, const float* kc, const float* bias, int3
     return kErrBadArg;
   }
   if (!piecewise::select_blocks_supported((int)NT, K)) {
-    set_error("%s: needs K in {64,128} and a score row that fits LDS (got K=%d NT=%lld)", what, K,
+    set_error("%s: needs K in [1,128] and a score row that fits LDS (got K=%d NT=%lld)", what, K,
               (long long)NT);
     return kErrUnsupported;
   }

@@ -707,11 +707,13 @@ __device__ __forceinline__ uint32_t order_bits(float x) {
   return b ^ ((b >> 31) ? 0xffffffffu : 0x80000000u);
 }
 
-template <int K>
+// KT = 64 / 128: the head dim; KT = 0: any head dim `Kr`, staged zero-padded to a multiple of 4.
+template <int KT>
 __global__ __launch_bounds__(kThreads) void select_blocks_kernel(
     const float* __restrict__ qc, const float* __restrict__ kc, const float* __restrict__ bias,
-    int32_t* __restrict__ indices, int NT, int NS, float scale) {
-  constexpr int KLD = K + 4;  // padded key rows: 16-byte reads of 16 lanes hit 16 bank groups
+    int32_t* __restrict__ indices, int NT, int NS, float scale, int Kr) {
+  const int K = KT ? KT : ((Kr + 3) & ~3);  // row length in LDS
+  const int KLD = K + 4;  // padded key rows: 16-byte reads of 16 lanes hit 16 bank groups
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   float* qs = reinterpret_cast<float*>(smem);          // [16][K]
   float* kt = qs + kSelRows * K;                       // [64][K + 4]
@@ -721,14 +723,27 @@ __global__ __launch_bounds__(kThreads) void select_blocks_kernel(
   const int r0 = (blockIdx.x % nrt) * kSelRows;
   const int64_t bh = blockIdx.x / nrt;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const float* qh = qc + bh * NT * K;
-  const float* kh = kc + bh * NT * K;
+  const int Km = KT ? KT : Kr;  // row length in memory
+  const float* qh = qc + bh * NT * Km;
+  const float* kh = kc + bh * NT * Km;
   typedef float f4 __attribute__((ext_vector_type(4)));
+  // four consecutive values of a row in memory (scalar loads and zero padding when the head dim
+  // is not one of the two built-in ones)
+  auto load4 = [&](const float* rowp, int c4) -> f4 {
+    if constexpr (KT != 0) {
+      return *reinterpret_cast<const f4*>(rowp + 4 * c4);
+    } else {
+      f4 x;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[i] = 4 * c4 + i < Km ? rowp[4 * c4 + i] : 0.f;
+      return x;
+    }
+  };
 
   for (int e = tid; e < kSelRows * (K / 4); e += kThreads) {
     const int row = e / (K / 4), c4 = e % (K / 4);
     f4 x = f4{0.f, 0.f, 0.f, 0.f};
-    if (r0 + row < NT) x = *reinterpret_cast<const f4*>(qh + (int64_t)(r0 + row) * K + 4 * c4);
+    if (r0 + row < NT) x = load4(qh + (int64_t)(r0 + row) * Km, c4);
     *reinterpret_cast<f4*>(qs + row * K + 4 * c4) = x;
   }
   for (int j0 = 0; j0 < NT; j0 += kSelKeys) {
@@ -736,7 +751,7 @@ __global__ __launch_bounds__(kThreads) void select_blocks_kernel(
     for (int e = tid; e < kSelKeys * (K / 4); e += kThreads) {
       const int row = e / (K / 4), c4 = e % (K / 4);
       f4 x = f4{0.f, 0.f, 0.f, 0.f};
-      if (j0 + row < NT) x = *reinterpret_cast<const f4*>(kh + (int64_t)(j0 + row) * K + 4 * c4);
+      if (j0 + row < NT) x = load4(kh + (int64_t)(j0 + row) * Km, c4);
       *reinterpret_cast<f4*>(kt + row * KLD + 4 * c4) = x;
     }
     __syncthreads();
@@ -803,12 +818,12 @@ __global__ __launch_bounds__(kThreads) void select_blocks_kernel(
 }
 
 size_t select_blocks_lds_bytes(int NT, int K) {
-  const int NTs = (NT + 63) & ~63;
-  return (size_t)(kSelRows * K + kSelKeys * (K + 4) + kSelRows * NTs) * sizeof(float);
+  const int NTs = (NT + 63) & ~63, KP = (K + 3) & ~3;
+  return (size_t)(kSelRows * KP + kSelKeys * (KP + 4) + kSelRows * NTs) * sizeof(float);
 }
 
 bool select_blocks_supported(int NT, int K) {
-  return (K == 64 || K == 128) && select_blocks_lds_bytes(NT, K) <= 160 * 1024;
+  return K >= 1 && K <= 128 && select_blocks_lds_bytes(NT, K) <= 160 * 1024;
 }
 
 int select_blocks(const float* qc, const float* kc, const float* bias, int32_t* indices, int64_t BH,
@@ -825,11 +840,12 @@ int select_blocks(const float* qc, const float* kc, const float* bias, int32_t* 
         return (int)kErrLaunch;
       }
     }
-    kernel<<<grid, block, lds, st>>>(qc, kc, bias, indices, NT, NS, scale);
+    kernel<<<grid, block, lds, st>>>(qc, kc, bias, indices, NT, NS, scale, K);
     return (int)kOk;
   };
   if (K == 64) return run(select_blocks_kernel<64>);
-  return run(select_blocks_kernel<128>);
+  if (K == 128) return run(select_blocks_kernel<128>);
+  return run(select_blocks_kernel<0>);
 }
 
 static Prob dense_prob(int64_t BH, int64_t T, int K, int V) {
@@ -891,9 +907,10 @@ int chunk_reduce(const void* q, const void* k, const void* v, float* qc, float* 
   const int sc = state_chunk_for(p, dtype, chunk, per_chunk);
   const int nparts = (int)cdiv64(T, sc);
   float* partial = (float*)workspace;
-  // 16-bit, MFMA-sized heads, 64-token blocks: k and v are read once, by the state kernel,
+  // 16-bit, head dims 64 / 128 (no padded variant of that kernel), 64-token blocks: k and v are read once, by the state kernel,
   // which also writes their block statistics; q has its own streaming pass
-  const bool fused = mfma::supported(p, dtype) && chunk == 64 && !per_chunk;
+  const bool fused = dtype != kF32 && (K == 64 || K == 128) && (V == 64 || V == 128) && mfma::supported(p, dtype) &&
+                     chunk == 64 && !per_chunk;
   if (dtype == kF16) launch_sums<_Float16>(q, k, v, qc, kc, vc, BH, (int)T, NT, chunk, K, V, fused, st);
   else if (dtype == kBF16) launch_sums<__bf16>(q, k, v, qc, kc, vc, BH, (int)T, NT, chunk, K, V, fused, st);
   else launch_sums<float>(q, k, v, qc, kc, vc, BH, (int)T, NT, chunk, K, V, false, st);
@@ -971,6 +988,202 @@ static int attention_t(const void* q, const void* k, const void* v, const float*
   if (K == 64) return launch_attention<T, 64, 128>(a, v, BH, st);
   if (V == 64) return launch_attention<T, 128, 64>(a, v, BH, st);
   return launch_attention<T, 128, 128>(a, v, BH, st);
+}
+
+// ===========================================================================
+// shape-generic attention kernel
+// ===========================================================================
+// Every head dim up to 128, every block size, fp16 / bf16 / fp32 inputs: what the MFMA kernel
+// (16-bit, head dims 64 / 128, 64-token blocks) does not cover.  Plain fp32 FMAs, correct
+// everywhere and an order of magnitude slower.  One workgroup per (query block, head); the
+// block's queries are handled 64 at a time: four neighbouring lanes share a query, each
+// holding a quarter of the contraction index for the scores (summed with two lane exchanges)
+// and a quarter of the value features for the accumulators.  Keys / values (phase 1), mean
+// keys / value sums (phase 2) and the rows of H (phase 3) pass through LDS 32 at a time,
+// converted to fp32; the softmax statistics are updated once per tile of 32 keys.
+constexpr int kGenQ = 64, kGenTile = 32;
+
+template <typename T> __device__ __forceinline__ float gen_load(const T* p) { return (float)*p; }
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void attention_generic_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ kc,
+    const float* __restrict__ vc, const float* __restrict__ h, const int32_t* __restrict__ indices,
+    T* __restrict__ o, int Tn, int NT, int NS, int K, int V, int BT, float scale) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int KP = K + 1;                   // padded query rows: lanes of different queries hit different banks
+  const int VS = (V + 3) / 4;             // value features per lane (at most 32)
+  float* qs = reinterpret_cast<float*>(smem);        // [64][K + 1]
+  float* kt = qs + kGenQ * KP;                        // [32][K]
+  float* vt = kt + kGenTile * K;                      // [32][V]
+  unsigned char* sel = reinterpret_cast<unsigned char*>(vt + kGenTile * V);  // [NT]
+  const int blk = blockIdx.x % NT;
+  const int64_t bh = blockIdx.x / NT;
+  const int tid = threadIdx.x, qi = tid >> 2, part = tid & 3;
+  const T* qh = q + bh * (int64_t)Tn * K;
+  const T* kh = k + bh * (int64_t)Tn * K;
+  const T* vh = v + bh * (int64_t)Tn * V;
+  const float* kch = kc + bh * (int64_t)NT * K;
+  const float* vch = vc + bh * (int64_t)NT * V;
+  const float* hh = h + bh * (int64_t)K * V;
+  const int32_t* idx = indices + (bh * NT + blk) * (int64_t)NS;
+  const float sm_scale = scale * 1.44269504088896f;
+  const float ninf = -__builtin_huge_valf();
+
+  for (int i = tid; i < NT; i += kThreads) sel[i] = 0;
+  __syncthreads();
+  for (int i = tid; i < NS; i += kThreads) {
+    const int c = idx[i];
+    if (c >= 0 && c < NT) sel[c] = 1;
+  }
+
+  const int q_begin = blk * BT, q_end = min(Tn, q_begin + BT);
+  for (int q0 = q_begin; q0 < q_end; q0 += kGenQ) {
+    __syncthreads();  // the previous pass is done with the tiles; `sel` is complete
+    for (int e = tid; e < kGenQ * K; e += kThreads) {
+      const int row = e / K, d = e - row * K;
+      qs[row * KP + d] = q0 + row < q_end ? gen_load(qh + (int64_t)(q0 + row) * K + d) : 0.f;
+    }
+    const bool active = q0 + qi < q_end;
+    const float* qrow = qs + qi * KP;
+    float acc[32], m = ninf, l = 0.f, g = 0.f;
+#pragma unroll
+    for (int e = 0; e < 32; ++e) acc[e] = 0.f;
+
+    // one tile of up to 32 rows of (keys, values) in LDS, `n_c(j)` tokens behind row j
+    // (1 in phase 1, the chunk length in phase 2; 0 = row does not take part)
+    auto consume = [&](int rows, auto weight, bool linear) {
+      float sc[kGenTile];
+      float tmax = ninf;
+#pragma unroll
+      for (int j = 0; j < kGenTile; ++j) {
+        float a = 0.f;
+        if (j < rows) {
+          for (int d = part; d < K; d += 4) a = fmaf(qrow[d], kt[j * K + d], a);
+          a += __shfl_xor(a, 1);
+          a += __shfl_xor(a, 2);
+        }
+        sc[j] = (j < rows && weight(j) > 0.f) ? a * sm_scale : ninf;
+        tmax = fmaxf(tmax, sc[j]);
+      }
+      if (tmax == ninf) return;  // nothing in this tile for this query (the same for its four lanes)
+      const float m_new = fmaxf(m, tmax);
+      const float alpha = m == ninf ? 0.f : exp2f(m - m_new);
+      l *= alpha;
+      g *= alpha;
+#pragma unroll
+      for (int e = 0; e < 32; ++e) acc[e] *= alpha;
+      m = m_new;
+#pragma unroll
+      for (int j = 0; j < kGenTile; ++j) {
+        if (sc[j] == ninf) continue;
+        const float pj = exp2f(sc[j] - m);
+        if (linear) g += pj * weight(j);
+        else l += pj;
+#pragma unroll
+        for (int e = 0; e < 32; ++e) {
+          const int col = part * VS + e;
+          if (e < VS && col < V) acc[e] = fmaf(pj, vt[j * V + col], acc[e]);
+        }
+      }
+    };
+
+    // ---- phase 1: the selected blocks, token by token ----
+    for (int s_i = 0; s_i < NS; ++s_i) {
+      const int c = idx[s_i];
+      if (c < 0 || c >= NT) continue;
+      const int t_lo = c * BT, t_hi = min(Tn, t_lo + BT);
+      for (int t0 = t_lo; t0 < t_hi; t0 += kGenTile) {
+        const int rows = min(kGenTile, t_hi - t0);
+        __syncthreads();
+        for (int e = tid; e < rows * K; e += kThreads) kt[e] = gen_load(kh + (int64_t)t0 * K + e);
+        for (int e = tid; e < rows * V; e += kThreads) vt[e] = gen_load(vh + (int64_t)t0 * V + e);
+        __syncthreads();
+        if (active) consume(rows, [](int) { return 1.f; }, false);
+      }
+    }
+    // ---- phase 2: every other block through its mean key and value sum ----
+    for (int c0 = 0; c0 < NT; c0 += kGenTile) {
+      const int rows = min(kGenTile, NT - c0);
+      __syncthreads();
+      for (int e = tid; e < rows * K; e += kThreads) kt[e] = kch[(int64_t)c0 * K + e];
+      for (int e = tid; e < rows * V; e += kThreads) vt[e] = vch[(int64_t)c0 * V + e];
+      __syncthreads();
+      if (active)
+        consume(rows, [&](int j) {
+          const int c = c0 + j;
+          return sel[c] ? 0.f : (float)min(BT, Tn - c * BT);
+        }, true);
+    }
+    // ---- phase 3: first-order term (q H) * g / T * scale ----
+    float r[32];
+#pragma unroll
+    for (int e = 0; e < 32; ++e) r[e] = 0.f;
+    for (int d0 = 0; d0 < K; d0 += kGenTile) {
+      const int rows = min(kGenTile, K - d0);
+      __syncthreads();
+      for (int e = tid; e < rows * V; e += kThreads) vt[e] = hh[(int64_t)d0 * V + e];
+      __syncthreads();
+      if (active)
+        for (int j = 0; j < rows; ++j) {
+          const float qd = qrow[d0 + j];
+#pragma unroll
+          for (int e = 0; e < 32; ++e) {
+            const int col = part * VS + e;
+            if (e < VS && col < V) r[e] = fmaf(qd, vt[j * V + col], r[e]);
+          }
+        }
+    }
+    if (active) {
+      const float coeff = g * (1.0f / (float)Tn) * scale;
+      const float inv = 1.0f / (l + g);
+#pragma unroll
+      for (int e = 0; e < 32; ++e) {
+        const int col = part * VS + e;
+        if (e < VS && col < V) o[(bh * Tn + (q0 + qi)) * (int64_t)V + col] = (T)((acc[e] + r[e] * coeff) * inv);
+      }
+    }
+  }
+}
+
+static size_t attention_generic_lds(int NT, int K, int V) {
+  return (size_t)(kGenQ * (K + 1) + kGenTile * K + kGenTile * V) * sizeof(float) + (size_t)((NT + 15) & ~15);
+}
+
+bool attention_generic_supported(int64_t T, int K, int V, int block, int dtype) {
+  if (K < 1 || K > 128 || V < 1 || V > 128 || block < 1) return false;
+  if (dtype != kF16 && dtype != kBF16 && dtype != kF32) return false;
+  return attention_generic_lds((int)cdiv64(T > 0 ? T : 1, block), K, V) <= 160 * 1024;
+}
+
+template <typename T>
+static int attention_generic_t(const void* q, const void* k, const void* v, const float* kc, const float* vc,
+                               const float* h, const int32_t* indices, void* o, int64_t BH, int64_t Tn, int K,
+                               int V, int block, int NS, float scale, hipStream_t st) {
+  const int NT = (int)cdiv64(Tn, block);
+  const int lds = (int)attention_generic_lds(NT, K, V);
+  auto kernel = attention_generic_kernel<T>;
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) {
+      set_error("piecewise attention: cannot reserve %d bytes of LDS: %s", lds, hipGetErrorString(e));
+      return kErrLaunch;
+    }
+  }
+  kernel<<<dim3((unsigned)(BH * NT)), dim3(kThreads), lds, st>>>((const T*)q, (const T*)k, (const T*)v, kc, vc, h,
+                                                              indices, (T*)o, (int)Tn, NT, NS, K, V, block, scale);
+  return kOk;
+}
+
+int attention_generic(const void* q, const void* k, const void* v, const float* kc, const float* vc,
+                      const float* h, const int32_t* indices, void* o, int64_t BH, int64_t T, int K, int V,
+                      int block, int NS, float scale, int dtype, hipStream_t st) {
+  if (dtype == kF16)
+    return attention_generic_t<_Float16>(q, k, v, kc, vc, h, indices, o, BH, T, K, V, block, NS, scale, st);
+  if (dtype == kBF16)
+    return attention_generic_t<__bf16>(q, k, v, kc, vc, h, indices, o, BH, T, K, V, block, NS, scale, st);
+  return attention_generic_t<float>(q, k, v, kc, vc, h, indices, o, BH, T, K, V, block, NS, scale, st);
 }
 
 int attention(const void* q, const void* k, const void* v, const float* kc, const float* vc,

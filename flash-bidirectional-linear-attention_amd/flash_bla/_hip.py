@@ -286,7 +286,7 @@ def select_blocks(qc, kc, bias, top_k, scale):
 
 def piecewise_supported(q, v, block):
     B, H, T, K = q.shape
-    return bool(q.dtype in (torch.float16, torch.bfloat16) and
+    return bool(q.dtype in _DTYPES and
                 lib().fbla_piecewise_workspace_bytes(B * H, T, K, v.shape[-1], block, dtype_code(q)))
 
 

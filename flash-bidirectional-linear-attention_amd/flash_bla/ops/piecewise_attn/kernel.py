@@ -1,12 +1,16 @@
 """Piecewise (PISA) sparse attention, forward only (drop-in for
 flash_bla/ops/piecewise_attn/kernel.py:152-176,295-333).
 
-Key blocks of 64 tokens are ranked per query block by the product of block-mean
+Key blocks of `block_size` tokens are ranked per query block by the product of block-mean
 queries and keys; the top `density` fraction is attended exactly (softmax), every
 other block contributes through its mean key and value sum (zeroth order) plus a
 first-order correction with H = sum_c (K_c - kc_c)^T V_c.  All block statistics
 are kept in fp32 (the reference stores them in the input dtype) and the running
 linear-branch normaliser is rescaled consistently with the running maximum.
+
+Two kernels: fp16 / bf16 inputs with head dims in {64, 128} and 64-token blocks run on the
+MFMA kernel; every other head dim up to 128, every other block size and fp32 inputs run on a
+shape-generic fp32 kernel (correct, about an order of magnitude slower).
 """
 import torch
 
@@ -58,9 +62,10 @@ def piecewise_sparse_attention(q, k, v, density=0.1, block_size=64, scale=None, 
                                indices=None):
     """
     Args:
-        q, k: `(B, H, T, K)`; v: `(B, H, T, V)`; fp16 or bf16, K and V in {64, 128}.
+        q, k: `(B, H, T, K)`; v: `(B, H, T, V)`; fp16, bf16 or fp32, K and V up to 128.
         density: fraction of key blocks attended exactly per query block (at least one).
-        block_size: tokens per block; the HIP kernel is built for 64.
+        block_size: tokens per block (the MFMA kernel is built for 64; other sizes take the
+            shape-generic kernel).
         scale: score scale, default `K ** -0.5`.
         use_bias: rank blocks by softmax(score + log(norm of the block's first-order matrix)).
         indices: optional precomputed selection `(B, H, N, top_k)` (not in the reference;
@@ -71,10 +76,13 @@ def piecewise_sparse_attention(q, k, v, density=0.1, block_size=64, scale=None, 
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     K = k.shape[-1]
     scale = K ** -0.5 if scale is None else scale
+    if block_size < 1:
+        raise ValueError(f"block_size must be positive, got {block_size}")
     if not _hip.piecewise_supported(q, v, block_size):
         raise NotImplementedError(
-            "piecewise_sparse_attention on gfx950 needs fp16/bf16 inputs, head dims in {64, 128} and "
-            f"block_size 64 (got dtype {q.dtype}, K={K}, V={v.shape[-1]}, block_size={block_size})")
+            "piecewise_sparse_attention on gfx950 needs fp16/bf16/fp32 inputs, head dims up to 128 and a "
+            "number of blocks whose selection flags fit LDS "
+            f"(got dtype {q.dtype}, K={K}, V={v.shape[-1]}, block_size={block_size}, T={q.shape[-2]})")
     qc, kc, vc, h, bias = chunk_reduce_fp32(q, k, v, block_size, use_bias)
     if indices is None:
         indices = select_blocks(qc, kc, scale, density, bias)

@@ -174,19 +174,24 @@ int fbla_chunk_reduce(const void* q, const void* k, const void* v, float* qc, fl
  * change the order).  qc, kc: fp32 [BH,NT,K] from fbla_chunk_reduce; indices: int32
  * [BH,NT,NS], written in ascending block order (torch.topk orders by score; the attention
  * result does not depend on the order); ties at the threshold go to the lower block index.
- * K in {64,128}. */
+ * K in [1,128]; the scores of 16 query blocks against all NT key blocks must fit LDS
+ * (NT up to about 2000). */
 int fbla_select_blocks(const float* qc, const float* kc, const float* bias, int32_t* indices,
                        int64_t BH, int64_t NT, int K, int NS, float scale, void* stream);
 
-/* Workspace of fbla_piecewise_fwd; 0 when the shape is not supported. */
+/* Workspace of fbla_piecewise_fwd; 0 when the shape is not supported (a head dim above 128, or so
+ * many blocks that their selection flags do not fit LDS). */
 size_t fbla_piecewise_workspace_bytes(int64_t BH, int64_t T, int K, int V, int block, int dtype);
 
 /* Piecewise attention forward.  Replaces piecewise_sparse_attention_fwd_kernel
- * (kernel.py:189-292): exact softmax attention over the NS selected 64-key blocks of
- * every 64-query block (indices: int32 [BH, NT, NS]), the remaining blocks through
- * their mean key / value sum (zeroth order) and h (first order).  kc, vc, h are the
- * fp32 outputs of fbla_chunk_reduce with chunk = block.  fp16/bf16, K,V in {64,128},
- * block = 64; anything else returns FBLA_ERR_UNSUPPORTED. */
+ * (kernel.py:189-292): exact softmax attention over the NS selected key blocks of every
+ * query block of `block` tokens (indices: int32 [BH, NT, NS], NT = ceil(T / block)), the
+ * remaining blocks through their mean key / value sum (zeroth order) and h (first order).
+ * kc, vc, h are the fp32 outputs of fbla_chunk_reduce with chunk = block.  fp16 / bf16 with
+ * K, V in {64,128} and block = 64 run on the MFMA kernel; every other K, V in [1,128], every
+ * other block size and fp32 inputs run on a shape-generic fp32 kernel (same results to
+ * rounding, about an order of magnitude slower, no workspace used).  The reference takes the
+ * same domain through BK = min(128, next_pow2(K)) (kernel.py:296-308). */
 int fbla_piecewise_fwd(const void* q, const void* k, const void* v, const float* kc, const float* vc,
                        const float* h, const int32_t* indices, void* o, void* workspace,
                        size_t workspace_bytes, int64_t BH, int64_t T, int K, int V, int block, int NS,

@@ -1,7 +1,8 @@
 """GPU parity of the piecewise (PISA) operators against the float64 oracle
-(oracle/piecewise.py).  The reference has neither a naive implementation nor a
-test for this operator: agreement with its Triton kernel is "parity unpinned";
-what is checked here is the mathematics the kernel text defines."""
+(oracle/piecewise.py, the closed form) and against oracle/piecewise_tokens.c (a per-token
+evaluation that follows the reference kernel's phases with one group).  The reference has
+neither a naive implementation nor a test for this operator; the two oracles pin each other
+(tests/test_oracle.py) and what is checked here is the mathematics the kernel text defines."""
 import numpy as np
 import pytest
 import torch
@@ -41,14 +42,55 @@ def test_fused_chunk_reduce(dtype, T, K, V, chunk):
     assert out[3].shape == (1, 3, K, V)
 
 
-def _oracle(q, k, v, indices, scale=None):
+def _oracle(q, k, v, indices, scale=None, block=64):
     B, H = q.shape[:2]
     out = np.zeros(v.shape, dtype=np.float64)
     for b in range(B):
         for h in range(H):
             out[b, h] = pw.piecewise_forward(np64(q)[b, h], np64(k)[b, h], np64(v)[b, h],
-                                             indices[b, h].cpu().numpy(), 64, scale)
+                                             indices[b, h].cpu().numpy(), block, scale)
     return out
+
+
+@pytest.mark.parametrize("T,K,V,block,density,dtype", [
+    (200, 16, 8, 32, 0.3, torch.float32),       # small head dims, ragged last block, fp32
+    (300, 100, 72, 64, 0.25, torch.float16),    # head dims that are not multiples of 16
+    (257, 64, 64, 16, 0.2, torch.bfloat16),     # the MFMA head dims with another block size
+    (400, 128, 128, 128, 0.5, torch.float16),   # 128-token blocks
+    (333, 24, 40, 50, 0.1, torch.float32),      # nothing a power of two
+    (256, 64, 64, 64, 0.25, torch.float32),     # the MFMA shape in fp32
+    (70, 8, 4, 1, 0.05, torch.float32),         # one-token blocks
+    (260, 32, 16, 64, 0.25, torch.bfloat16),    # 16-bit head dims that the state kernel pads
+])
+def test_shape_generic_kernel_matches_oracle_and_per_token_evaluation(T, K, V, block, density, dtype):
+    """Head dims, block sizes and the dtype outside the MFMA kernel's domain run on the
+    shape-generic kernel: against the float64 closed form and, independently, against the
+    per-token C evaluation that follows the reference kernel's phases."""
+    from flash_bla.ops.piecewise_attn.kernel import (chunk_reduce_fp32, piecewise_sparse_attention,
+                                                     select_blocks)
+    from oracle.piecewise_tokens import pisa_tokens
+    q, k, v = _inputs(1, 2, T, K, V, dtype, seed=T + K)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    scale = 0.8 * K ** -0.5
+    qc, kc, vc, h, _ = chunk_reduce_fp32(qd, kd, vd, block)
+    for hd in range(2):
+        rq, rk, rv, _, rH, _ = pw.chunk_reduce(np64(q)[0, hd], np64(k)[0, hd], np64(v)[0, hd], block)
+        assert max_rel_err(qc[0, hd], rq) < 1e-5 and max_rel_err(kc[0, hd], rk) < 1e-5
+        # H = K^T V - sum_c kc_c vc_c^T cancels (to zero for one-token blocks): the scale is K^T V's
+        assert max_rel_err(vc[0, hd], rv) < 1e-5 and max_rel_err(h[0, hd], rH, np64(k)[0, hd].T @ np64(v)[0, hd]) < 2e-5
+    indices = select_blocks(qc, kc, scale, density)
+    NT = -(-T // block)
+    assert indices.shape == (1, 2, NT, max(1, int(density * NT)))
+    o = piecewise_sparse_attention(qd, kd, vd, density=density, block_size=block, scale=scale, indices=indices)
+    assert o.dtype == dtype and o.shape == v.shape
+    ref = _oracle(q, k, v, indices, scale=scale, block=block)
+    floor = _oracle(q, k, v.abs(), indices, scale=scale, block=block)
+    assert_parity(o, ref, dtype, f"T{T} K{K} V{V} block{block}", floor)
+    for hd in range(2):
+        tok = pisa_tokens(np64(q)[0, hd], np64(k)[0, hd], np64(v)[0, hd], indices[0, hd].cpu().numpy(), block, scale)
+        assert_parity(o[0, hd], tok, dtype, f"per-token evaluation, head {hd}", floor[0, hd])
+    o2 = piecewise_sparse_attention(qd, kd, vd, density=density, block_size=block, scale=scale)
+    assert torch.equal(o, o2)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
@@ -70,6 +112,10 @@ def test_piecewise_attention_matches_oracle(dtype, T, K, V, density):
     assert o.dtype == dtype and o.shape == v.shape
     ref = _oracle(q, k, v, indices)
     assert_parity(o, ref, dtype, f"T{T} K{K} V{V}")
+    # independently of the closed form: the per-token C evaluation of the reference kernel's phases
+    from oracle.piecewise_tokens import pisa_tokens
+    tok = pisa_tokens(np64(q)[0, 0], np64(k)[0, 0], np64(v)[0, 0], indices[0, 0].cpu().numpy(), 64)
+    assert_parity(o[0, 0], tok, dtype, f"per-token evaluation T{T} K{K} V{V}")
     # and with its own selection (same code path as select_blocks)
     o2 = piecewise_sparse_attention(qd, kd, vd, density=density)
     assert torch.equal(o, o2)
@@ -100,12 +146,13 @@ def test_use_bias_selection_and_errors():
     q, k, v = _inputs(1, 2, 512, 64, 64, torch.bfloat16, seed=5)
     o = piecewise_sparse_attention(q.cuda(), k.cuda(), v.cuda(), density=0.25, use_bias=True)
     assert torch.isfinite(o).all()
-    with pytest.raises(NotImplementedError):
-        piecewise_sparse_attention(q.cuda().float(), k.cuda().float(), v.cuda().float())
-    with pytest.raises(NotImplementedError):
-        piecewise_sparse_attention(q.cuda(), k.cuda(), v.cuda(), block_size=32)
+    with pytest.raises(ValueError):
+        piecewise_sparse_attention(q.cuda(), k.cuda(), v.cuda(), block_size=0)
     with pytest.raises(ValueError):
         piecewise_sparse_attention(q, k, v)
+    big = torch.zeros(1, 1, 8, 192, dtype=torch.float16, device="cuda")  # head dim above 128
+    with pytest.raises(NotImplementedError):
+        piecewise_sparse_attention(big, big, big)
 
 
 @pytest.mark.parametrize("NT,K,top_density", [(256, 128, 0.25), (37, 64, 0.3), (1, 64, 1.0), (130, 128, 0.01),
