@@ -24,6 +24,10 @@ for _p in (ROOT, os.path.join(ROOT, "flash-bidirectional-linear-attention_amd"),
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
+# the per-kernel timings below launch single kernels through the library's phase mask, which the
+# library only honours in a process that asked for it
+os.environ.setdefault("FBLA_ALLOW_PHASE_MASK", "1")
+
 import torch  # noqa: E402
 import torch.nn.functional as F  # noqa: E402
 

@@ -3,6 +3,7 @@
 // replaces are in include/flash_bla_hip.h.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 
 #include <atomic>
 #include <initializer_list>
@@ -128,7 +129,12 @@ extern "C" {
 
 int fbla_version(void) { return 100; }
 
-void fbla_set_phase_mask(unsigned mask) { g_phase_mask = mask ? mask : kPhaseAll; }
+// Only honoured when the process opted in through the environment: a caller cannot switch kernels
+// off by accident, and a mask left set by a profiling script that died cannot outlive its process.
+void fbla_set_phase_mask(unsigned mask) {
+  static const bool allowed = [] { const char* v = getenv("FBLA_ALLOW_PHASE_MASK"); return v && v[0] == '1'; }();
+  g_phase_mask = (allowed && mask) ? mask : kPhaseAll;
+}
 
 const char* fbla_last_error(void) { return g_err; }
 

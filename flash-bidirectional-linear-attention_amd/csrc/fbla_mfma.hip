@@ -1956,7 +1956,7 @@ int rows_chunk(const Prob& p, int DR, int DC) {
   const int big = (tiled_dim(DR) == 128) + (tiled_dim(DC) == 128);
   const int rounds = p.cu ? packed_rounds : (big == 2 ? 1 : big == 1 ? (dense_rounds + 1) / 2 : dense_rounds);
   const int per_cu = big == 0 ? per_cu_knob : (big == 1 ? 2 : 1);
-  static const int min_chunk_knob = knob("FBLA_ROWS_MIN_CHUNK", 512);
+  static const int min_chunk_knob = knob("FBLA_ROWS_MIN_CHUNK", 256);
   // a problem too small to give every CU a workgroup: shorter chunks (the operand build of the
   // extra workgroups costs less than the idle CUs)
   int min_chunk = min_chunk_knob;

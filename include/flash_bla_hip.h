@@ -60,7 +60,8 @@ int fbla_version(void);
  * timed in isolation (bit 0 forward partial state, 1 forward state reduce,
  * 2 forward output, 3 backward pass A, 4 backward reduce, 5 backward pass B).
  * 0 restores the default (all kernels).  Skipped kernels leave their outputs
- * untouched, so results are only meaningful with the default mask. */
+ * untouched, so results are only meaningful with the default mask.  Ignored unless
+ * the process was started with FBLA_ALLOW_PHASE_MASK=1 in its environment. */
 void fbla_set_phase_mask(unsigned mask);
 
 /* Message of the last error raised on the calling thread ("" if none). */

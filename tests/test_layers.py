@@ -39,6 +39,36 @@ def test_linfusion_state_dict_names():
     assert "to_q.bias" not in names
 
 
+def test_state_dict_names_and_shapes_follow_the_reference_modules():
+    """A checkpoint of the reference's blocks must load: parameter / buffer names and shapes as the
+    reference's constructors create them (layers/mlla.py:29,54-57, rala.py:30-34,
+    focused_la.py:24-39, polaformer.py:22-40; qkv_bias defaults to False in the PVT-style blocks,
+    True in MLLA / RALA)."""
+    dim, heads, res = 64, 4, (4, 4)
+    want = {
+        "mlla": (MambaLikeLinearAttention(dim, res, heads), {
+            "qk.weight": (2 * dim, dim), "qk.bias": (2 * dim,), "lepe.weight": (dim, 1, 3, 3), "lepe.bias": (dim,),
+            "rope.rotations": (*res, dim // 2, 2)}),
+        "rala": (RALALinearAttention(dim, res, heads), {
+            "qkvo.weight": (4 * dim, dim), "qkvo.bias": (4 * dim,), "lepe.weight": (dim, 1, 5, 5),
+            "lepe.bias": (dim,), "rope.rotations": (*res, dim // heads // 2, 2), "proj.weight": (dim, dim),
+            "proj.bias": (dim,)}),
+        "focused": (FocusedLinearAttention(dim, 16, num_heads=heads, sr_ratio=2), {
+            "q.weight": (dim, dim), "kv.weight": (2 * dim, dim), "proj.weight": (dim, dim), "proj.bias": (dim,),
+            "sr.weight": (dim, dim, 2, 2), "sr.bias": (dim,), "norm.weight": (dim,), "norm.bias": (dim,),
+            "dwc.weight": (dim // heads, 1, 5, 5), "dwc.bias": (dim // heads,), "scale": (1, 1, dim),
+            "positional_encoding": (1, 16 // 4, dim)}),
+        "pola": (PolaLinearAttention(dim, 16, num_heads=heads, sr_ratio=2), {
+            "qg.weight": (2 * dim, dim), "kv.weight": (2 * dim, dim), "proj.weight": (dim, dim), "proj.bias": (dim,),
+            "sr.weight": (dim, dim, 2, 2), "sr.bias": (dim,), "norm.weight": (dim,), "norm.bias": (dim,),
+            "dwc.weight": (dim // heads, 1, 5, 5), "dwc.bias": (dim // heads,), "power": (1, heads, 1, dim // heads),
+            "scale": (1, 1, dim), "positional_encoding": (1, 16 // 4, dim)}),
+    }
+    for name, (module, shapes) in want.items():
+        got = {k: tuple(v.shape) for k, v in module.state_dict().items()}
+        assert got == shapes, name
+
+
 GPU_CASES = {
     # the shapes of the reference self-tests
     "linfusion": (lambda: GeneralizedLinearAttention(1024, heads=16, dim_head=64), (2, 4096, 1024), ()),
