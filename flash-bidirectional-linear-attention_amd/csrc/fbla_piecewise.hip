@@ -289,6 +289,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
   constexpr int MB = V / 32;                 // 32-row blocks of O^T
   constexpr int OLD = 64 * (V / 8) / kThreads;
   constexpr float kNegInf = -__builtin_huge_valf();
+  constexpr float kLazy = 8.f;
   // Two tile sets as two separate LDS objects: the compiler can then tell that a tile load
   // in flight towards one set does not touch the set being read, and does not make the reads
   // wait for it.  The selected-block bitmap is the dynamic part.
@@ -428,7 +429,12 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
       mx = fmaxf(mx, st[r]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m_i, mx);
+    // The reference point of the exponents follows the running maximum lazily: it moves only
+    // when the maximum has grown by more than kLazy binary orders, so p stays below 2^kLazy
+    // (exact in fp32 sums, in range for a 16-bit operand) and the accumulators are rescaled a
+    // few times per query block instead of on almost every tile (some row of the 32 sets a new
+    // maximum in most tiles).  m_i = -inf: the first finite score is taken at once.
+    const float m_new = ((mx - m_i) * c2 > kLazy) ? mx : m_i;
     const float m_safe = m_new == kNegInf ? 0.f : m_new;
     const float alpha = __builtin_amdgcn_exp2f((m_i - m_safe) * c2);
     const float mc = m_safe * c2;
