@@ -854,15 +854,21 @@ __device__ __forceinline__ void build_vec(uint32_t* pairs, float* f32, const flo
   }
 }
 
+// Denominator rows of the decoupled operator (DEN): with 64 x 64 tiles they are staged through LDS
+// like the numerator rows; with a 128-wide side there is no LDS for a second tile per wave, and
+// z_t = q_t . km is computed from the flat registers the rows were loaded into instead (the
+// lanes that hold the 16-byte pieces of one row add their partial dot products; kDenFlat).
+template <int DR, int DC, bool DEN> constexpr bool den_flat() { return DEN && !(DR == 64 && DC == 64); }
 template <int DR, int DC, bool DEN, int WAVES> struct RowsLayout {
   static constexpr int KS = DR / 16, NB = DC / 32;
   static constexpr int kStage = 32 * 2 * (DR > DC ? DR : DC);  // one 32-token tile of the wider side
   static constexpr int kOpnd = NB * KS * 2 * 1024;
   static constexpr int kStages = kOpnd;
-  static constexpr int kKm = kStages + WAVES * (DEN ? 2 : 1) * kStage;
+  static constexpr int kKm = kStages + WAVES * (DEN && !den_flat<DR, DC, DEN>() ? 2 : 1) * kStage;
   static constexpr int kAdd = kKm + DR * 4;
   static constexpr int kMax = kAdd + DC * 4;
-  static constexpr int kLpt = kMax + 64;
+  static constexpr int kZrow = kMax + 64;                                       // [WAVES][32] z of the wave's tile
+  static constexpr int kLpt = kZrow + (den_flat<DR, DC, DEN>() ? WAVES * 128 : 0);
   static constexpr int kTotal = kLpt + (kLptMax + 1) * 4;
 };
 
@@ -945,8 +951,10 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
   // 32-token sub-tiles, interleaved over the waves; the first one is requested
   // before the prologue so that its latency overlaps the operand build.
   const int ntok = lane & 31, kb = lane >> 5;  // MFMA view: token column, k half
-  unsigned char* stage = smem + LY::kStages + wave * (DEN ? 2 : 1) * kStage;
+  constexpr bool kDenFlat = den_flat<DR, DC, DEN>();
+  unsigned char* stage = smem + LY::kStages + wave * (DEN && !kDenFlat ? 2 : 1) * kStage;
   unsigned char* stage_den = stage + kStage;
+  float* zrow = reinterpret_cast<float*>(smem + LY::kZrow) + 32 * wave;  // kDenFlat only
   constexpr int XI = 32 * XCH / 64;  // flat 16-byte loads per lane per tile
   constexpr int OI = 32 * OCH / 64;
 
@@ -1036,7 +1044,25 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
   auto tile_step = [&](u32x4(&xcur)[XI], u32x4(&dcur)[XI]) {
     wave_sync();  // previous tile's staging reads are done
     stash_tile(xcur, stage);
-    if constexpr (DEN) stash_tile(dcur, stage_den);
+    if constexpr (DEN && !kDenFlat) stash_tile(dcur, stage_den);
+    if constexpr (kDenFlat) {
+      // piece i of this lane is chunk lane % XCH of row lane / XCH + (64 / XCH) i: its dot product
+      // with the km values of that chunk, then the sum over the XCH lanes of the row
+      const u32x4 khf = *reinterpret_cast<const u32x4*>(&lds_km[4 * (lane % XCH)]);
+      const u32x4 klf = *reinterpret_cast<const u32x4*>(&lds_km[DR / 2 + 4 * (lane % XCH)]);
+#pragma unroll
+      for (int i = 0; i < XI; ++i) {
+        float a = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          a = Ops<T>::dot2(dcur[i][w], khf[w], a);
+          a = Ops<T>::dot2(dcur[i][w], klf[w], a);
+        }
+#pragma unroll
+        for (int off = XCH / 2; off > 0; off >>= 1) a += __shfl_xor(a, off);
+        if (lane % XCH == 0) zrow[lane / XCH + (64 / XCH) * i] = a;
+      }
+    }
     const int tn = t0 + t_stride * PF;
     if ((FBLA_ROWS_FAST & 1) && !NORM && kFast && tn + 32 <= t_end) {
       load_tile_full(xcur, x, tn);
@@ -1065,7 +1091,7 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
         f.ah[b] = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * (b * KS + s) + 0) * 64 + lane) * 16);
         f.al[b] = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * (b * KS + s) + 1) * 64 + lane) * 16);
       }
-      if constexpr (NORM) {
+      if constexpr (NORM && !kDenFlat) {
         if constexpr (DEN) f.bd = *reinterpret_cast<const u32x4*>(stage_den + swz<XROWB>(ntok, KS * kb + s));
         f.kh = *reinterpret_cast<const u32x4*>(&lds_km[(DR / 4) * kb + 4 * s]);
         f.kl = *reinterpret_cast<const u32x4*>(&lds_km[DR / 2 + (DR / 4) * kb + 4 * s]);
@@ -1083,7 +1109,7 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
         acc[b] = Ops<T>::mma(f.ah[b], bq, acc[b]);
         acc[b] = Ops<T>::mma(f.al[b], bq, acc[b]);
       }
-      if constexpr (NORM) {
+      if constexpr (NORM && !kDenFlat) {
         u32x4 bd = bq;
         if constexpr (DEN) bd = f.bd;
         const u32x4 kh = f.kh, kl = f.kl;
@@ -1096,7 +1122,8 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
     }
     float rs = denorm;
     if constexpr (NORM) {
-      if constexpr (!PAIR) z += __shfl_xor(z, 32);  // pair mode: each half row has its own z
+      if constexpr (kDenFlat) z = zrow[ntok];  // written before the wave_sync above
+      else if constexpr (!PAIR) z += __shfl_xor(z, 32);  // pair mode: each half row has its own z
       rs = denorm / (z + p.eps);
     }
     wave_sync();  // all lanes have read their x chunks; staging is reused for out
@@ -1186,7 +1213,8 @@ template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struc
   static constexpr int KS = DV / 16, NB = DK / 32;
   static constexpr int kOpnd = NB * KS * 2 * 1024;
   static constexpr int kQ = 32 * DK * 2, kG = 32 * DV * 2;
-  static constexpr int kWave = kQ + kG + (NORM && FUSED && LO ? kG : 0) + (DEN ? kQ : 0) + 256;  // + dz[64]
+  // (DEN without FUSED: the denominator rows stay in the flat registers they were loaded into)
+  static constexpr int kWave = kQ + kG + (NORM && FUSED && LO ? kG : 0) + (DEN && FUSED ? kQ : 0) + 256;  // + dz[64]
   static constexpr int kKmPairs = kOpnd + kWaves * kWave;
   static constexpr int kKmF = kKmPairs + DK * 4;
   static constexpr int kMax = kKmF + DK * 4;
@@ -1263,8 +1291,12 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
   unsigned char* qt = smem + LY::kOpnd + wave * LY::kWave;
   unsigned char* gt = qt + LY::kQ;             // dO, later dO/z (hi part)
   unsigned char* gl = gt + LY::kG;             // dO/z (lo part), NORM && FUSED only
-  unsigned char* qdt = gl + (NORM && FUSED && LO ? LY::kG : 0);  // plain q, DEN only
-  float* dzs = reinterpret_cast<float*>(qdt + (DEN ? LY::kQ : 0));
+  // Token view alone (not FUSED) with the decoupled operator: z_t = q_t . km comes from the flat
+  // registers of the plain q rows (the lanes holding the pieces of a row add their partial dot
+  // products) and dq = dz_t km is stored from the same flat layout: no LDS tile for plain q.
+  constexpr bool kDenFlat = DEN && !FUSED;
+  unsigned char* qdt = gl + (NORM && FUSED && LO ? LY::kG : 0);  // plain q, DEN && FUSED only
+  float* dzs = reinterpret_cast<float*>(qdt + (DEN && FUSED ? LY::kQ : 0));  // [64]: dz (FUSED) or z | dz (kDenFlat)
   uint32_t* km_pairs = reinterpret_cast<uint32_t*>(smem + LY::kKmPairs);
   float* kmf = reinterpret_cast<float*>(smem + LY::kKmF);
   float* lds_max = reinterpret_cast<float*>(smem + LY::kMax);
@@ -1368,7 +1400,23 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
     wave_sync();  // the previous sub-tile's staged dq has been read out
     stash_q(rq, qt);
     stash_g(rg, gt);
-    if constexpr (DEN) stash_q(rd, qdt);
+    if constexpr (DEN && !kDenFlat) stash_q(rd, qdt);
+    if constexpr (kDenFlat) {
+      const u32x4 khf = *reinterpret_cast<const u32x4*>(&km_pairs[4 * (lane % QCH)]);
+      const u32x4 klf = *reinterpret_cast<const u32x4*>(&km_pairs[DK / 2 + 4 * (lane % QCH)]);
+#pragma unroll
+      for (int i = 0; i < QI; ++i) {
+        float a = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          a = Ops<T>::dot2(rd[i][w], khf[w], a);
+          a = Ops<T>::dot2(rd[i][w], klf[w], a);
+        }
+#pragma unroll
+        for (int off = QCH / 2; off > 0; off >>= 1) a += __shfl_xor(a, off);
+        if (lane % QCH == 0) dzs[lane / QCH + (64 / QCH) * i] = a;
+      }
+    }
     const int tn = t0 + t_stride;
     if (kFast && tn + 32 <= t_end) {
       load_q_full(rq, qn, tn);
@@ -1406,7 +1454,7 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
       for (int ch = 0; ch < QCH / 2; ++ch) {
         const u32x4 qw = *reinterpret_cast<const u32x4*>(qt + swz<QROWB>(ntok, (QCH / 2) * kb + ch));
         u32x4 qz = qw;
-        if constexpr (DEN) qz = *reinterpret_cast<const u32x4*>(qdt + swz<QROWB>(ntok, (QCH / 2) * kb + ch));
+        if constexpr (DEN && !kDenFlat) qz = *reinterpret_cast<const u32x4*>(qdt + swz<QROWB>(ntok, (QCH / 2) * kb + ch));
         const u32x4 kh = *reinterpret_cast<const u32x4*>(&km_pairs[(DK / 4) * kb + 4 * ch]);
         const u32x4 kl = *reinterpret_cast<const u32x4*>(&km_pairs[DK / 2 + (DK / 4) * kb + 4 * ch]);
 #pragma unroll
@@ -1414,14 +1462,17 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
           const int c0 = 8 * ch + 2 * i;
           P = fmaf(Ops<T>::lo(qw[i]), g[c0 >> 4][c0 & 15], P);
           P = fmaf(Ops<T>::hi(qw[i]), g[c0 >> 4][(c0 & 15) + 1], P);
-          z = Ops<T>::dot2(qz[i], kh[i], z);
-          z = Ops<T>::dot2(qz[i], kl[i], z);
+          if constexpr (!kDenFlat) {
+            z = Ops<T>::dot2(qz[i], kh[i], z);
+            z = Ops<T>::dot2(qz[i], kl[i], z);
+          }
         }
       }
       if constexpr (!PAIR) {  // pair mode: each half row is a token of its own
         P += __shfl_xor(P, 32);
         z += __shfl_xor(z, 32);
       }
+      if constexpr (kDenFlat) z = dzs[ntok];  // from the flat registers, before the wave_sync above
       if (PAIR ? (t0 + ntok < t_end && 2 * (t0 + ntok) + kb < len) : (t0 + ntok < t_end)) {
         rz = 1.f / (z + p.eps);
         dz = -(P * denorm) * rz * rz;
@@ -1436,10 +1487,13 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
           tokscal[row] = rz;
           tokscal[total_rows + row] = dz;
         }
+        if constexpr (kDenFlat) {
+          if (kb == 0) dzs[32 + ntok] = dz;
+        }
       }
     }
     // dq~ (and dq when decoupled), packed; staged after the feature view is done with qt
-    uint32_t dqp[DK / 4], dqdp[DEN ? DK / 4 : 1];
+    uint32_t dqp[DK / 4], dqdp[DEN && !kDenFlat ? DK / 4 : 1];
     {
       const float gs = denorm * rz;
 #pragma unroll
@@ -1448,9 +1502,9 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
         float v0 = g[c0 >> 4][c0 & 15] * gs, v1 = g[c0 >> 4][(c0 & 15) + 1] * gs;
         if constexpr (NORM) {
           const float d0 = dz * kmf[(DK / 2) * kb + c0], d1 = dz * kmf[(DK / 2) * kb + c0 + 1];
-          if constexpr (DEN) {
+          if constexpr (DEN && !kDenFlat) {
             dqdp[c2] = pack2<T>(d0, d1);
-          } else {
+          } else if constexpr (!DEN) {
             v0 += d0;
             v1 += d1;
           }
@@ -1523,17 +1577,30 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
     for (int ch = 0; ch < QCH / 2; ++ch) {
       const int off = swz<QROWB>(ntok, (QCH / 2) * kb + ch);
       *reinterpret_cast<u32x4*>(qt + off) = u32x4{dqp[4 * ch], dqp[4 * ch + 1], dqp[4 * ch + 2], dqp[4 * ch + 3]};
-      if constexpr (DEN)
+      if constexpr (DEN && !kDenFlat)
         *reinterpret_cast<u32x4*>(qdt + off) =
             u32x4{dqdp[4 * ch], dqdp[4 * ch + 1], dqdp[4 * ch + 2], dqdp[4 * ch + 3]};
     }
-    wave_sync();
+    wave_sync();  // (also orders the dz values written to dzs[32..] before the reads below)
     if (kFast && t0 + 32 <= t_end) {
       store_q_full(qt, dqn, t0);
-      if constexpr (DEN) store_q_full(qdt, dqd, t0);
+      if constexpr (DEN && !kDenFlat) store_q_full(qdt, dqd, t0);
     } else {
       store_q(qt, dqn, t0);
-      if constexpr (DEN) store_q(qdt, dqd, t0);
+      if constexpr (DEN && !kDenFlat) store_q(qdt, dqd, t0);
+    }
+    if constexpr (kDenFlat) {
+      // dq = dz_t km: piece i of this lane is chunk lane % QCH of row lane / QCH + (64 / QCH) i
+      const float* kmc = kmf + 8 * (lane % QCH);
+#pragma unroll
+      for (int i = 0; i < QI; ++i) {
+        const int row = lane / QCH + (64 / QCH) * i;
+        const float dzr = dzs[32 + row];
+        const u32x4 w{pack2<T>(dzr * kmc[0], dzr * kmc[1]), pack2<T>(dzr * kmc[2], dzr * kmc[3]),
+                      pack2<T>(dzr * kmc[4], dzr * kmc[5]), pack2<T>(dzr * kmc[6], dzr * kmc[7])};
+        const int64_t off = piece(t0 + row, lane % QCH, dk);
+        if (off >= 0) store_row16<kNtPassAStore>(dqd + off, w);
+      }
     }
     t0 = tn;
   }
@@ -1849,20 +1916,20 @@ bool pair_mode(const Prob& p, int dtype) {
   return (dtype == kF16 || dtype == kBF16) && !p.cu && p.DK == 32 && p.DV == 32;
 }
 
-// 16-bit inputs with head dims that are multiples of 8 (16-byte row pieces) up to 128; the
-// decoupled operator up to 64 x 64.
+// 16-bit inputs with head dims that are multiples of 8 (16-byte row pieces) up to 128.
 bool supported(const Prob& p, int dtype) {
   if (dtype == kF32) return mfma32::supported(p);
   if (dtype != kF16 && dtype != kBF16) return false;
   if (p.DK < 8 || p.DV < 8 || p.DK > 128 || p.DV > 128 || p.DK % 8 || p.DV % 8) return false;
-  if ((p.flags & kDecoupled) && !(p.DK <= 64 && p.DV <= 64)) return false;
   return true;
 }
 
 // The fused backward pass A exists for heads tiled as 64 x 64 and as 128 x 128 (the latter
-// not for the decoupled operator, which `supported` already limits to 64 x 64).
+// not for the decoupled operator).
 bool bwd_a_supported(const Prob& p, int dtype) {
-  return dtype != kF32 && supported(p, dtype) && tiled_dim(p.DK) == tiled_dim(p.DV);
+  if (dtype == kF32 || !supported(p, dtype) || tiled_dim(p.DK) != tiled_dim(p.DV)) return false;
+  // decoupled: fused for 64 x 64 tiles only (the 128 x 128 kernel has no room for the plain q tile)
+  return !(p.flags & kDecoupled) || tiled_dim(p.DK) == 64;
 }
 
 // Number of compute units of the current device (256 on MI355X; also the value
@@ -1989,7 +2056,9 @@ static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, fl
   if (bs.kc) {
     if constexpr (!PAD)
       state_kernel<T, DK, DV, false, 1, false, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
-  } else if (tokscal)
+  } else if (tokscal && (p.flags & kDecoupled))  // dkm = sum_t dz_t q_t over the plain q rows (kd)
+    state_kernel<T, DK, DV, true, 1, true, false, PAD><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fm, fv, chunk, nchunks, bs);
+  else if (tokscal)
     state_kernel<T, DK, DV, false, 1, true, false, PAD><<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, total_rows, fm, fv, chunk, nchunks, bs);
   else if (p.flags & kDecoupled)
     state_kernel<T, DK, DV, true, TL, false, false, PAD><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
@@ -2057,10 +2126,7 @@ static int launch_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, i
   const bool den = norm && job.xden != job.x;
   if (!norm) return launch_rows_k<T, DR, DC, false, false, WAVES, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
   if (!den) return launch_rows_k<T, DR, DC, true, false, WAVES, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
-  if constexpr (DR == 64 && DC == 64)
-    return launch_rows_k<T, DR, DC, true, true, WAVES, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
-  set_error("decoupled rows kernel exists only for heads up to 64 x 64");
-  return kErrUnsupported;
+  return launch_rows_k<T, DR, DC, true, true, WAVES, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
 }
 
 // two tokens per row: chunks are counted in row pairs
@@ -2159,9 +2225,9 @@ void scaled_state(const Prob& p, int dtype, const void* qn, const void* qd, cons
     return mfma32::state(p, (const float*)qn, (const float*)dout, (const float*)qd, partial, tokscal,
                          total_rows, chunk, nchunks, st, fin_mat, fin_vec);
   if (dtype == kF16)
-    run_state<_Float16>(p, qn, dout, qn, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, none, st);
+    run_state<_Float16>(p, qn, dout, qd, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, none, st);
   else
-    run_state<__bf16>(p, qn, dout, qn, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, none, st);
+    run_state<__bf16>(p, qn, dout, qd, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, none, st);
 }
 
 int rows(const Prob& p_, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {
@@ -2260,42 +2326,47 @@ int bwd_a(const Prob& p_, int dtype, const void* qn, const void* qd, const void*
 }
 
 template <typename T, int DK, int DV, bool PAD>
-static int launch_bwd_tokens(const Prob& p, const void* q, const void* dout, const float* S,
-                             const float* km, void* dq, float* tokscal, int64_t total_rows,
+static int launch_bwd_tokens(const Prob& p, const void* qn, const void* qd, const void* dout, const float* S,
+                             const float* km, void* dqn, void* dqd, float* tokscal, int64_t total_rows,
                              int chunk, int nchunks, hipStream_t st) {
-  const T *a = (const T*)q, *c = (const T*)dout;
+  const T *a = (const T*)qn, *b = (const T*)qd, *c = (const T*)dout;
+  if (p.flags & kDecoupled)  // z from the plain q rows, dq = dz km next to dq_rope
+    return launch_bwd_a<T, DK, DV, true, true, false, PAD>(p, a, b, c, S, km, (T*)dqn, (T*)dqd, nullptr, tokscal,
+                                                           total_rows, nullptr, nullptr, chunk, nchunks, st);
   if (p.flags & kNormalize)
-    return launch_bwd_a<T, DK, DV, true, false, false, PAD>(p, a, a, c, S, km, (T*)dq, nullptr, nullptr,
+    return launch_bwd_a<T, DK, DV, true, false, false, PAD>(p, a, a, c, S, km, (T*)dqn, nullptr, nullptr,
                                                             tokscal, total_rows, nullptr, nullptr, chunk,
                                                             nchunks, st);
-  return launch_bwd_a<T, DK, DV, false, false, false, PAD>(p, a, a, c, S, km, (T*)dq, nullptr, nullptr,
+  return launch_bwd_a<T, DK, DV, false, false, false, PAD>(p, a, a, c, S, km, (T*)dqn, nullptr, nullptr,
                                                            tokscal, total_rows, nullptr, nullptr, chunk,
                                                            nchunks, st);
 }
 
 template <typename T, bool PAD>
-static int run_bwd_tokens_dims(const Prob& p, const void* q, const void* dout, const float* S,
-                               const float* km, void* dq, float* tokscal, int64_t total_rows, int chunk,
-                               int nchunks, hipStream_t st) {
+static int run_bwd_tokens_dims(const Prob& p, const void* qn, const void* qd, const void* dout, const float* S,
+                               const float* km, void* dqn, void* dqd, float* tokscal, int64_t total_rows,
+                               int chunk, int nchunks, hipStream_t st) {
   const int DK = tiled_dim(p.DK), DV = tiled_dim(p.DV);
   if (DK == 64 && DV == 128)
-    return launch_bwd_tokens<T, 64, 128, PAD>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
+    return launch_bwd_tokens<T, 64, 128, PAD>(p, qn, qd, dout, S, km, dqn, dqd, tokscal, total_rows, chunk, nchunks, st);
   if (DK == 128 && DV == 64)
-    return launch_bwd_tokens<T, 128, 64, PAD>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
-  set_error("the token view alone exists for heads tiled 64 x 128 and 128 x 64");  // others: fused pass A
+    return launch_bwd_tokens<T, 128, 64, PAD>(p, qn, qd, dout, S, km, dqn, dqd, tokscal, total_rows, chunk, nchunks, st);
+  if (DK == 128 && DV == 128 && (p.flags & kDecoupled))  // the plain operator has the fused 128 x 128 pass A
+    return launch_bwd_tokens<T, 128, 128, PAD>(p, qn, qd, dout, S, km, dqn, dqd, tokscal, total_rows, chunk, nchunks, st);
+  set_error("the token view alone exists for heads tiled 64 x 128, 128 x 64 and (decoupled) 128 x 128");
   return kErrUnsupported;
 }
 
 template <typename T>
-static int run_bwd_tokens(const Prob& p, const void* q, const void* dout, const float* S,
-                          const float* km, void* dq, float* tokscal, int64_t total_rows,
+static int run_bwd_tokens(const Prob& p, const void* qn, const void* qd, const void* dout, const float* S,
+                          const float* km, void* dqn, void* dqd, float* tokscal, int64_t total_rows,
                           hipStream_t st) {
   const int big = (tiled_dim(p.DK) == 128) + (tiled_dim(p.DV) == 128);
   const int chunk = chunk_for(p, big == 2 ? 1 : 2, 1, 512, 128, false);
   const int nchunks = (int)cdiv64(p.L, chunk);
   if (padded(p))
-    return run_bwd_tokens_dims<T, true>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
-  return run_bwd_tokens_dims<T, false>(p, q, dout, S, km, dq, tokscal, total_rows, chunk, nchunks, st);
+    return run_bwd_tokens_dims<T, true>(p, qn, qd, dout, S, km, dqn, dqd, tokscal, total_rows, chunk, nchunks, st);
+  return run_bwd_tokens_dims<T, false>(p, qn, qd, dout, S, km, dqn, dqd, tokscal, total_rows, chunk, nchunks, st);
 }
 
 // token view of the backward alone: dq and the per-row scalars 1/z_t, dz_t
@@ -2304,8 +2375,8 @@ int bwd_tokens(const Prob& p, int dtype, const void* qn, const void* qd, const v
   if (dtype == kF32)
     return mfma32::bwd_tokens(p, (const float*)qn, (const float*)qd, (const float*)dout, S, km, (float*)dqn,
                               (float*)dqd, tokscal, total_rows, st);
-  if (dtype == kF16) return run_bwd_tokens<_Float16>(p, qn, dout, S, km, dqn, tokscal, total_rows, st);
-  return run_bwd_tokens<__bf16>(p, qn, dout, S, km, dqn, tokscal, total_rows, st);
+  if (dtype == kF16) return run_bwd_tokens<_Float16>(p, qn, qd, dout, S, km, dqn, dqd, tokscal, total_rows, st);
+  return run_bwd_tokens<__bf16>(p, qn, qd, dout, S, km, dqn, dqd, tokscal, total_rows, st);
 }
 
 }  // namespace mfma

@@ -66,6 +66,8 @@ def _check_dense(variant, B, H, L, DK, DV, dtype, scale=None, eps=1e-6, seed=42)
     (2, 3, 333, 128, 64),
     (1, 4, 4100, 128, 128),   # several chunks per head at the largest head dims
     (4, 16, 256, 32, 32),     # MLLA / RALA self-test shape (layers/mlla.py:102-127)
+    (1, 2, 777, 96, 80),      # both head dims padded to the 128-wide tiles, ragged length
+    (2, 2, 2050, 128, 72),    # several chunks, value dim padded to 128
 ])
 def test_dense_parity(variant, B, H, L, DK, DV, dtype):
     _check_dense(variant, B, H, L, DK, DV, dtype)
