@@ -267,8 +267,8 @@ static int check_cross(const char* what, int64_t Lk, int flags) {
     set_error("%s: the number of keys must be positive and fit 32-bit indexing, got %lld", what, (long long)Lk);
     return kErrBadArg;
   }
-  if (flags & (kDecoupled | kDefaultScale)) {
-    set_error("%s: not available for the decoupled operator or with a per-sequence default scale", what);
+  if (flags & kDefaultScale) {
+    set_error("%s: FBLA_DEFAULT_SCALE is only valid for the packed entry points", what);
     return kErrBadArg;
   }
   return kOk;
@@ -283,39 +283,82 @@ size_t fbla_la_cross_workspace_bytes(int pass, int64_t B, int64_t H, int64_t Lq,
   return workspace_bytes(p, dtype, pass);
 }
 
-int fbla_la_cross_fwd(const void* q, const void* k, const void* v, void* o, float* s, float* km,
-                      void* workspace, size_t workspace_bytes_, int64_t B, int64_t H, int64_t Lq, int64_t Lk,
-                      int DK, int DV, int dtype, int flags, float scale, float eps, void* stream) {
-  const char* what = "fbla_la_cross_fwd";
+static int cross_fwd(const char* what, const void* q, const void* k, const void* v, const void* q_rope,
+                     const void* k_rope, void* o, float* s, float* km, void* workspace, size_t workspace_bytes_,
+                     int64_t B, int64_t H, int64_t Lq, int64_t Lk, int DK, int DV, int dtype, int flags, float scale,
+                     float eps, void* stream) {
   int rc = check_dims(what, B, H, Lq, DK, DV, dtype, flags);
   if (rc == kOk) rc = check_cross(what, Lk, flags);
   if (rc != kOk) return rc;
-  if (B * H > 0 && Lq > 0 && (!q || !k || !v || !o || !s || ((flags & kNormalize) && !km))) {
+  if (B * H > 0 && Lq > 0 &&
+      (!q || !k || !v || !o || !s || ((flags & kNormalize) && !km) || ((flags & kDecoupled) && (!q_rope || !k_rope)))) {
     set_error("%s: null tensor pointer", what);
     return kErrBadArg;
   }
   Prob p = make_prob(nullptr, B, H, Lq, B * Lq, DK, DV, flags, scale, eps);
   p.Lk = (int)Lk;
-  FwdArgs a{q, k, v, nullptr, nullptr, o, s, km, workspace, workspace_bytes_};
+  FwdArgs a{q, k, v, q_rope, k_rope, o, s, km, workspace, workspace_bytes_};
   return run_fwd(what, p, dtype, a, (hipStream_t)stream);
+}
+
+int fbla_la_cross_fwd(const void* q, const void* k, const void* v, void* o, float* s, float* km,
+                      void* workspace, size_t workspace_bytes_, int64_t B, int64_t H, int64_t Lq, int64_t Lk,
+                      int DK, int DV, int dtype, int flags, float scale, float eps, void* stream) {
+  if (flags & kDecoupled) {
+    set_error("fbla_la_cross_fwd: the decoupled operator takes its rotary rows through fbla_decoupled_cross_fwd");
+    return kErrBadArg;
+  }
+  return cross_fwd("fbla_la_cross_fwd", q, k, v, nullptr, nullptr, o, s, km, workspace, workspace_bytes_, B, H, Lq, Lk,
+                   DK, DV, dtype, flags, scale, eps, stream);
+}
+
+int fbla_decoupled_cross_fwd(const void* q, const void* k, const void* q_rope, const void* k_rope, const void* v,
+                             void* o, float* s, float* km, void* workspace, size_t workspace_bytes_, int64_t B,
+                             int64_t H, int64_t Lq, int64_t Lk, int DK, int DV, int dtype, float scale, float eps,
+                             void* stream) {
+  return cross_fwd("fbla_decoupled_cross_fwd", q, k, v, q_rope, k_rope, o, s, km, workspace, workspace_bytes_, B, H, Lq,
+                   Lk, DK, DV, dtype, kNormalize | kDecoupled, scale, eps, stream);
+}
+
+static int cross_bwd(const char* what, const void* q, const void* k, const void* v, const void* q_rope,
+                     const void* k_rope, const void* dout, const float* s, const float* km, void* dq, void* dk,
+                     void* dv, void* dq_rope, void* dk_rope, void* workspace, size_t workspace_bytes_, int64_t B,
+                     int64_t H, int64_t Lq, int64_t Lk, int DK, int DV, int dtype, int flags, float scale, float eps,
+                     void* stream) {
+  int rc = check_dims(what, B, H, Lq, DK, DV, dtype, flags);
+  if (rc == kOk) rc = check_cross(what, Lk, flags);
+  if (rc != kOk) return rc;
+  const bool dec = flags & kDecoupled;
+  if (B * H > 0 && Lq > 0 &&
+      (!q || !v || !dout || !s || ((flags & kNormalize) && !km) || !dq || !dk || !dv || (!dec && !k) ||
+       (dec && (!q_rope || !k_rope || !dq_rope || !dk_rope)))) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  Prob p = make_prob(nullptr, B, H, Lq, B * Lq, DK, DV, flags, scale, eps);
+  p.Lk = (int)Lk;
+  BwdArgs a{q, k, v, q_rope, k_rope, dout, s, km, dq, dk, dv, dq_rope, dk_rope, workspace, workspace_bytes_};
+  return run_bwd(what, p, dtype, a, (hipStream_t)stream);
 }
 
 int fbla_la_cross_bwd(const void* q, const void* k, const void* v, const void* dout, const float* s,
                       const float* km, void* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes_,
                       int64_t B, int64_t H, int64_t Lq, int64_t Lk, int DK, int DV, int dtype, int flags,
                       float scale, float eps, void* stream) {
-  const char* what = "fbla_la_cross_bwd";
-  int rc = check_dims(what, B, H, Lq, DK, DV, dtype, flags);
-  if (rc == kOk) rc = check_cross(what, Lk, flags);
-  if (rc != kOk) return rc;
-  if (B * H > 0 && Lq > 0 && (!q || !k || !v || !dout || !s || ((flags & kNormalize) && !km) || !dq || !dk || !dv)) {
-    set_error("%s: null tensor pointer", what);
+  if (flags & kDecoupled) {
+    set_error("fbla_la_cross_bwd: the decoupled operator takes its rotary rows through fbla_decoupled_cross_bwd");
     return kErrBadArg;
   }
-  Prob p = make_prob(nullptr, B, H, Lq, B * Lq, DK, DV, flags, scale, eps);
-  p.Lk = (int)Lk;
-  BwdArgs a{q, k, v, nullptr, nullptr, dout, s, km, dq, dk, dv, nullptr, nullptr, workspace, workspace_bytes_};
-  return run_bwd(what, p, dtype, a, (hipStream_t)stream);
+  return cross_bwd("fbla_la_cross_bwd", q, k, v, nullptr, nullptr, dout, s, km, dq, dk, dv, nullptr, nullptr, workspace,
+                   workspace_bytes_, B, H, Lq, Lk, DK, DV, dtype, flags, scale, eps, stream);
+}
+
+int fbla_decoupled_cross_bwd(const void* q, const void* k, const void* q_rope, const void* k_rope, const void* v,
+                             const void* dout, const float* s, const float* km, void* dq, void* dk, void* dq_rope,
+                             void* dk_rope, void* dv, void* workspace, size_t workspace_bytes_, int64_t B, int64_t H,
+                             int64_t Lq, int64_t Lk, int DK, int DV, int dtype, float scale, float eps, void* stream) {
+  return cross_bwd("fbla_decoupled_cross_bwd", q, k, v, q_rope, k_rope, dout, s, km, dq, dk, dv, dq_rope, dk_rope,
+                   workspace, workspace_bytes_, B, H, Lq, Lk, DK, DV, dtype, kNormalize | kDecoupled, scale, eps, stream);
 }
 
 size_t fbla_varlen_workspace_bytes(int pass, int64_t total_tokens, int64_t N, int64_t H,

@@ -531,7 +531,7 @@ void bwd_b(const Prob& p, int dtype, const void* kn, const void* v, const float*
 
 template <typename T>
 __global__ __launch_bounds__(kThreads) void broadcast_rows_kernel(Prob p, const float* __restrict__ vec,
-                                                                  T* __restrict__ out, int ntiles) {
+                                                                  T* __restrict__ out, int ntiles, float factor) {
   const int nh = blockIdx.x / ntiles, tile = blockIdx.x - nh * ntiles;
   const int n = nh / p.H, h = nh - n * p.H;
   int64_t bos, row0, rstride;
@@ -544,17 +544,17 @@ __global__ __launch_bounds__(kThreads) void broadcast_rows_kernel(Prob p, const 
   const int DK = p.DK;
   for (int i = threadIdx.x; i < nvalid * DK; i += kThreads) {
     const int t = i / DK, d = i - t * DK;
-    out[(row0 + (int64_t)(t0 + t) * rstride) * DK + d] = from_f32<T>(vec[(int64_t)nh * DK + d]);
+    out[(row0 + (int64_t)(t0 + t) * rstride) * DK + d] = from_f32<T>(vec[(int64_t)nh * DK + d] * factor);
   }
 }
 
 // every row of out ([.., DK]) = vec of its (sequence, head): dk of the decoupled operator
-void broadcast_rows(const Prob& p, int dtype, const float* vec, void* out, hipStream_t st) {
+void broadcast_rows(const Prob& p, int dtype, const float* vec, void* out, hipStream_t st, float factor) {
   const int ntiles = (int)cdiv64(p.L, kTile);
   const dim3 grid((unsigned)((int64_t)p.N * p.H * ntiles)), block(kThreads);
-  if (dtype == kF16) broadcast_rows_kernel<_Float16><<<grid, block, 0, st>>>(p, vec, (_Float16*)out, ntiles);
-  else if (dtype == kBF16) broadcast_rows_kernel<__bf16><<<grid, block, 0, st>>>(p, vec, (__bf16*)out, ntiles);
-  else broadcast_rows_kernel<float><<<grid, block, 0, st>>>(p, vec, (float*)out, ntiles);
+  if (dtype == kF16) broadcast_rows_kernel<_Float16><<<grid, block, 0, st>>>(p, vec, (_Float16*)out, ntiles, factor);
+  else if (dtype == kBF16) broadcast_rows_kernel<__bf16><<<grid, block, 0, st>>>(p, vec, (__bf16*)out, ntiles, factor);
+  else broadcast_rows_kernel<float><<<grid, block, 0, st>>>(p, vec, (float*)out, ntiles, factor);
 }
 
 // One thread per sequence j counts the sequences that come before it in the order (longer,

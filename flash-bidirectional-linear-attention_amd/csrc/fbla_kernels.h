@@ -62,7 +62,7 @@ void bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void*
 void bwd_b(const Prob& p, int dtype, const void* kn, const void* v, const float* dS,
            const float* dSt, const float* dkm, void* dkn, void* dkd, void* dv, hipStream_t st,
            float dkm_scale = 1.f);
-void broadcast_rows(const Prob& p, int dtype, const float* vec, void* out, hipStream_t st);
+void broadcast_rows(const Prob& p, int dtype, const float* vec, void* out, hipStream_t st, float factor = 1.f);
 // perm[r] = index of the sequence with the r-th largest length (ties by index)
 void rank_sequences(const Prob& p, int32_t* perm, hipStream_t st);
 }  // namespace generic

@@ -107,14 +107,9 @@ size_t fwd_workspace_bytes(const Prob& pc, int dtype) { return fwd_used_bytes(pc
 // partials | S^T | s*dS | (s*dS)^T | dkm/L | per-row scalars | walking order
 size_t bwd_workspace_bytes(const Prob& pc, int dtype) { return bwd_used_bytes(pc, dtype) + perm_bytes(pc); }
 
-static int check_cross(const Prob& p, int dtype) {
-  if (!cross(p)) return kOk;
-  if (p.flags & kDecoupled) {
-    set_error("different numbers of queries and keys are not available for the decoupled operator");
-    return kErrUnsupported;
-  }
-  return kOk;
-}
+// Different numbers of queries and keys work for every operator family (the decoupled one too:
+// its rotary and plain rows come in pairs of equal length on either side).
+static int check_cross(const Prob&, int) { return kOk; }
 
 int forward(const Prob& pc_, int dtype, const FwdArgs& a, hipStream_t st) {
   int rc_cross = check_cross(pc_, dtype);
@@ -249,7 +244,8 @@ int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
         if (rc == kOk) rc = mfma::rows(pki, dtype, jv, p.DK, p.DV, st);
       }
       if (rc != kOk) return rc;
-      if (dec) generic::broadcast_rows(p, dtype, dkm, dkd, st);
+      // dk = dkm / (number of keys) in every key row; dkm arrives divided by the number of queries
+      if (dec) generic::broadcast_rows(pk, dtype, dkm, dkd, st, is_cross ? (float)p.L / (float)pk.L : 1.f);
     } else {
       generic::bwd_b(pk, dtype, kn, a.v, dS, dSt, dkm, dkn, dkd, a.dv, st,
                      is_cross ? (float)p.L / (float)pk.L : 1.f);

@@ -34,6 +34,8 @@ _SIGNATURES = {
     "fbla_la_cross_workspace_bytes": (_sz, [_i32, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32]),
     "fbla_la_cross_fwd": (_i32, [_vp] * 7 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_la_cross_bwd": (_i32, [_vp] * 10 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
+    "fbla_decoupled_cross_fwd": (_i32, [_vp] * 9 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _f32, _f32, _vp]),
+    "fbla_decoupled_cross_bwd": (_i32, [_vp] * 14 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_varlen_workspace_bytes": (_sz, [_i32, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32]),
     "fbla_varlen_fwd": (_i32, [_vp] * 8 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_varlen_bwd": (_i32, [_vp] * 11 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
@@ -152,6 +154,14 @@ def la_fwd(q, k, v, q_rope, k_rope, scale, eps, flags):
     o = torch.empty(B, H, T, DV, dtype=v.dtype, device=dev)
     s = torch.empty(B, H, DK, DV, dtype=torch.float32, device=dev)
     km = torch.empty(B, H, DK, dtype=torch.float32, device=dev)
+    if Tk != T and flags & DECOUPLED:
+        with _on(dev):
+            ws = _workspace(L.fbla_la_cross_workspace_bytes(0, B, H, T, Tk, DK, DV, code, flags), dev)
+            rc = L.fbla_decoupled_cross_fwd(_ptr(q), _ptr(k), _ptr(q_rope), _ptr(k_rope), _ptr(v), _ptr(o), _ptr(s),
+                                            _ptr(km), _ptr(ws), ws.numel(), B, H, T, Tk, DK, DV, code, float(scale),
+                                            float(eps), _stream(dev))
+        _check(rc, "fbla_decoupled_cross_fwd")
+        return o, s, km
     if Tk != T:
         with _on(dev):
             ws = _workspace(L.fbla_la_cross_workspace_bytes(0, B, H, T, Tk, DK, DV, code, flags), dev)
@@ -181,6 +191,15 @@ def la_bwd(q, k, v, q_rope, k_rope, do, s, km, scale, eps, flags):
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dqr = torch.empty_like(q_rope) if flags & DECOUPLED else None
     dkr = torch.empty_like(k_rope) if flags & DECOUPLED else None
+    if Tk != T and flags & DECOUPLED:
+        with _on(dev):
+            ws = _workspace(L.fbla_la_cross_workspace_bytes(1, B, H, T, Tk, DK, DV, code, flags), dev)
+            rc = L.fbla_decoupled_cross_bwd(_ptr(q), _ptr(k), _ptr(q_rope), _ptr(k_rope), _ptr(v), _ptr(do), _ptr(s),
+                                            _ptr(km), _ptr(dq), _ptr(dk), _ptr(dqr), _ptr(dkr), _ptr(dv), _ptr(ws),
+                                            ws.numel(), B, H, T, Tk, DK, DV, code, float(scale), float(eps),
+                                            _stream(dev))
+        _check(rc, "fbla_decoupled_cross_bwd")
+        return dq, dk, dv, dqr, dkr
     if Tk != T:
         with _on(dev):
             ws = _workspace(L.fbla_la_cross_workspace_bytes(1, B, H, T, Tk, DK, DV, code, flags), dev)

@@ -10,10 +10,13 @@ def check_dense(name, q, k, v, extra=()):
         if not isinstance(t, torch.Tensor) or t.ndim != 4:
             raise ValueError(f"{name}: tensors must have shape (B, H, L, D)")
     if extra:
-        if q.shape != k.shape or any(t.shape != q.shape for t in extra):
-            raise ValueError(f"{name}: q and k (and their rope versions) must have identical shapes, "
+        # decoupled operator: q_rope shaped like q, k_rope like k (which, like v, may have another
+        # number of tokens than q)
+        q_rope, k_rope = extra
+        if q_rope.shape != q.shape or k_rope.shape != k.shape:
+            raise ValueError(f"{name}: q_rope must be shaped like q and k_rope like k, "
                              f"got {[tuple(t.shape) for t in (q, k) + tuple(extra)]}")
-    elif q.shape[:2] != k.shape[:2] or q.shape[-1] != k.shape[-1]:
+    if q.shape[:2] != k.shape[:2] or q.shape[-1] != k.shape[-1]:
         # k and v may be shorter or longer than q (the PVT-style blocks reduce the keys spatially;
         # the reference reads one length from q, linear_attn/fused.py:355, and runs out of bounds)
         raise ValueError(f"{name}: q and k must agree in batch, head and feature dimensions, "

@@ -47,10 +47,11 @@ def decoupled_la(
 ) -> torch.Tensor:
     r"""
     Args:
-        q, k: plain queries / keys `(B, H, L, K)` (denominator)
-        q_rope, k_rope: rotary queries / keys `(B, H, L, K)` (numerator)
-        v: values `(B, H, L, V)`
-        scale: defaults to `1 / L` (decoupled.py:539-540)
+        q, q_rope: plain (denominator) and rotary (numerator) queries `(B, H, L, K)`
+        k, k_rope: plain and rotary keys `(B, H, Lk, K)`; `Lk` may differ from `L` (the reference
+            takes one length from q, decoupled.py:413-420)
+        v: values `(B, H, Lk, V)`
+        scale: defaults to `1 / Lk` (decoupled.py:539-540)
         eps: constant added to the denominator.
     """
     # RoPE modules hand back fp32 features next to 16-bit q, k (layers/mlla.py:32-36 of the

@@ -116,8 +116,9 @@ int fbla_la_fwd_static(const void* q, const void* k, const void* v, const void* 
  * over the Lk keys.  The reference has no counterpart: its dense kernels take one length from q
  * (linear_attn/fused.py:355) and read k, v out of bounds when the PVT-style blocks
  * (layers/focused_la.py:55,73-75, layers/polaformer.py) shorten the keys with sr_ratio > 1.
- * Flags as for fbla_la_fwd without FBLA_DECOUPLED (FBLA_ERR_UNSUPPORTED with it); every dtype
- * and head dim of fbla_la_fwd. */
+ * Flags as for fbla_la_fwd without FBLA_DECOUPLED (the decoupled operator has the pair of entry
+ * points below); every dtype and head dim of fbla_la_fwd.  fbla_la_cross_workspace_bytes takes
+ * FBLA_DECOUPLED in `flags` for the decoupled pair. */
 size_t fbla_la_cross_workspace_bytes(int pass, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int DK,
                                      int DV, int dtype, int flags);
 int fbla_la_cross_fwd(const void* q, const void* k, const void* v, void* o, float* s, float* km,
@@ -128,6 +129,20 @@ int fbla_la_cross_bwd(const void* q, const void* k, const void* v, const void* d
                       const float* km, void* dq, void* dk, void* dv, void* workspace,
                       size_t workspace_bytes, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int DK,
                       int DV, int dtype, int flags, float scale, float eps, void* stream);
+
+/* The decoupled operator with Lk != Lq: q, q_rope, dq, dq_rope: [B,H,Lq,DK]; k, k_rope, dk, dk_rope:
+ * [B,H,Lk,DK]; v, dv: [B,H,Lk,DV]; o, dout: [B,H,Lq,DV].  No counterpart in the reference
+ * (linear_attn/decoupled.py:413-509 takes one length from q).  Workspace: fbla_la_cross_workspace_bytes
+ * with flags = FBLA_NORMALIZE | FBLA_DECOUPLED. */
+int fbla_decoupled_cross_fwd(const void* q, const void* k, const void* q_rope, const void* k_rope,
+                             const void* v, void* o, float* s, float* km, void* workspace,
+                             size_t workspace_bytes, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int DK,
+                             int DV, int dtype, float scale, float eps, void* stream);
+int fbla_decoupled_cross_bwd(const void* q, const void* k, const void* q_rope, const void* k_rope,
+                             const void* v, const void* dout, const float* s, const float* km, void* dq,
+                             void* dk, void* dq_rope, void* dk_rope, void* dv, void* workspace,
+                             size_t workspace_bytes, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int DK,
+                             int DV, int dtype, float scale, float eps, void* stream);
 
 /* Workspace for the packed (variable-length) entry points. */
 size_t fbla_varlen_workspace_bytes(int pass, int64_t total_tokens, int64_t N, int64_t H,

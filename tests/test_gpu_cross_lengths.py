@@ -76,9 +76,37 @@ def test_shapes_of_the_generic_kernels():
         _check("simple", 1, 2, lq, lk, 6, 70, torch.float32, 350 + i)
 
 
-def test_the_decoupled_operator_is_refused():
+def _check_decoupled(B, H, lq, lk, DK, DV, dtype, seed):
+    from flash_bla.ops.linear_attn.decoupled import decoupled_la
+    q, _, _, do, qr = make_qkv((B, H, lq, DK), (B, H, lq, DV), dtype, seed, n_extra=1)
+    _, k, v, _, kr = make_qkv((B, H, lk, DK), (B, H, lk, DV), dtype, seed + 1, n_extra=1)
+    ref = cf.dense_backward(np64(q), np64(k), np64(v), np64(do), 1.0 / lk, 1e-6, True, q_rope=np64(qr), k_rope=np64(kr))
+    leaves = [t.cuda().requires_grad_() for t in (q, k, qr, kr, v)]
+    o = decoupled_la(*leaves)
+    assert o.shape == (B, H, lq, DV) and o.dtype == dtype
+    o.backward(do.cuda())
+    errs = {"o": parity_errors(o, ref["o"], dtype)}
+    for name, t in zip(("dq", "dk", "dq_rope", "dk_rope", "dv"), leaves):
+        assert t.grad.shape == t.shape
+        errs[name] = parity_errors(t.grad, ref[name], dtype, ref.get(name + "_mag"))
+    bad = {n: e for n, e in errs.items() if not e[2]}
+    assert not bad, f"decoupled {dtype} B{B} H{H} Lq{lq} Lk{lk} DK{DK} DV{DV}: {errs}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32], ids=str)
+@pytest.mark.parametrize("dims", [(32, 32), (64, 64), (128, 128), (64, 128), (20, 12)])
+def test_decoupled_operator(dims, dtype):
+    """Rotary and plain rows come in pairs of equal length on either side; the row-constant dk is
+    dkm over the number of keys."""
+    for i, (lq, lk) in enumerate(LENGTHS[:5]):
+        _check_decoupled(1, 2, lq, lk, dims[0], dims[1], dtype, 400 + 10 * i + dims[0])
+
+
+def test_decoupled_operator_shape_errors():
     from flash_bla.ops.linear_attn.decoupled import decoupled_la
     q64 = torch.rand(1, 2, 40, 64, device="cuda", dtype=torch.float16)
     k64 = torch.rand(1, 2, 10, 64, device="cuda", dtype=torch.float16)
-    with pytest.raises(ValueError, match="identical shapes"):
-        decoupled_la(q64, k64, q64, k64, k64)
+    with pytest.raises(ValueError, match="shaped like"):
+        decoupled_la(q64, k64, q64, q64, k64)     # k_rope with the queries' length
+    with pytest.raises(ValueError, match="matching batch"):
+        decoupled_la(q64, k64, q64, k64, q64)     # v with the queries' length

@@ -138,6 +138,26 @@ def test_fewer_or_more_keys_than_queries(normalize):
             np.testing.assert_allclose(g[name], np64(leaf.grad), rtol=1e-9, atol=1e-11)
 
 
+def test_decoupled_with_fewer_or_more_keys_than_queries():
+    """The decoupled closed form with Lq != Lk: output against the double sum written out
+    (numerator from the rotary rows, denominator from the plain ones, mean over the Lk keys), all
+    five gradients against autograd on the torch restatement."""
+    for lq, lk in ((23, 9), (5, 31)):
+        q, _, _, do, qr, _ = _dense_inputs(2, 2, lq, 8, 6, n_extra=2)
+        _, k, v, _, _, kr = _dense_inputs(2, 2, lk, 8, 6, n_extra=2)
+        scale, eps = 0.07, 1e-6
+        g = cf.dense_backward(np64(q), np64(k), np64(v), np64(do), scale, eps, True, q_rope=np64(qr), k_rope=np64(kr))
+        num = scale * np.einsum("bhij,bhjv->bhiv", np.einsum("bhik,bhjk->bhij", np64(qr), np64(kr)), np64(v))
+        den = np.einsum("bhik,bhjk->bhij", np64(q), np64(k)).mean(-1, keepdims=True) + eps
+        np.testing.assert_allclose(g["o"], num / den, rtol=1e-11, atol=1e-13)
+        leaves = [t.clone().requires_grad_() for t in (q, k, qr, kr, v)]
+        o = tr.naive_decoupled_la(*leaves, scale)
+        o.backward(do)
+        np.testing.assert_allclose(g["o"], np64(o), rtol=1e-11, atol=1e-13)
+        for name, leaf in zip(("dq", "dk", "dq_rope", "dk_rope", "dv"), leaves):
+            np.testing.assert_allclose(g[name], np64(leaf.grad), rtol=1e-9, atol=1e-11)
+
+
 def test_gradcheck_torch_ref():
     q, k, v, _ = _dense_inputs(1, 1, 7, 3, 2)
     args = [t.clone().requires_grad_() for t in (q, k, v)]
