@@ -1620,42 +1620,61 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
 // ===========================================================================
 // backward pass A, heads tiled 128 x 128
 // ===========================================================================
-// dS (128 x 128 fp32) does not fit one wave and the 64 KiB matrix operand leaves LDS for four
-// 32-token tiles only, so one workgroup of eight waves shares a step of 128 tokens:
-//   token view    wave w takes tile u = w % 4 and the output half hf = w / 4 of g = dO S^T (two
-//                 of the four 32-column blocks); the partial q~.g and q.km sums of the two
-//                 halves meet in LDS, then both waves know 1/z_t and dz_t and pack their half
-//                 of dq;
-//   feature view  wave w owns block w % 4 of dS (64 x 64) over the tiles 2*(w/4), 2*(w/4)+1;
-//                 dO rows are scaled by 1/z_t and split into hi + lo on the fly (no LDS left
-//                 for a staged copy); the two waves of a block are summed at the end;
-//   dq            goes back through the q tile so that whole rows are stored.
-// The steps are separated by workgroup barriers; all waves make the same number of steps (a
-// tile past the end of the chunk is all zeros).
+// dS (128 x 128 fp32) does not fit one wave, so a workgroup of four waves shares steps of 64
+// tokens (two 32-token tiles) and two workgroups share a CU, each filling the other's waits:
+//   prologue      the S^T operand (hi + lo, 64 KiB) is built in LDS once; wave w keeps the
+//                 fragments of output block w (32 of the 128 columns of g = dO S^T) in 64
+//                 registers, and the LDS they were built in becomes the tiles;
+//   token view    wave w multiplies both tiles by its block, adds its part of q~.g and q.km; the
+//                 four parts of a token meet in LDS, then every wave knows 1/z_t and dz_t, packs
+//                 its 32 columns of dq into a staging tile (whole rows leave from there) and
+//                 scales its quarter of the dO tile by 1/z_t into a hi and a lo tile, once for
+//                 all waves;
+//   feature view  wave w owns 64 x 64 block w of dS; q~^T and dO / z come straight out of the
+//                 row-major tiles in operand order through the transposing LDS read
+//                 (ds_read_b64_tr_b16: a lane receives four tokens of one feature), so there
+//                 is no in-register transposition and no rescaling here.
+// The contraction index of the feature view is a permutation of the tile's tokens (the same for
+// both operands): k-step ks, half-wave kb, element e = 4x + j is token 16ks + 4j + 2kb + x.  One
+// transposing read then touches four token rows that differ in bits 2..3, which the XOR swizzle
+// of the tiles spreads over all banks.
 struct BwdA128Layout {
   static constexpr int kOpnd = 4 * 8 * 2 * 1024;  // 4 blocks x 8 k-steps x (hi, lo) fragments
-  static constexpr int kTile = 2 * 32 * 256;      // q tile | dO tile
-  static constexpr int kTiles = kOpnd;
-  static constexpr int kPz = kTiles + 4 * kTile;  // [tile][half][32] partial (q~.g, q.km)
-  static constexpr int kScal = kPz + 4 * 2 * 32 * 8;  // [tile] dz[32], 1/z[32]
-  static constexpr int kKmPairs = kScal + 4 * 64 * 4;
+  static constexpr int kTile = 32 * 256;          // 32 tokens x 128 features x 2 bytes
+  static constexpr int kQ = 0;                    // q tiles [2]
+  static constexpr int kG = kQ + 2 * kTile;       // dO tiles [2], then the hi part of dO / z
+  static constexpr int kGl = kG + 2 * kTile;      // lo part of dO / z
+  static constexpr int kDq = kGl + 2 * kTile;     // dq staging [2]
+  static constexpr int kPz = kDq + 2 * kTile;     // [tile][block][32] partial (q~.g, q.km)
+  static constexpr int kDz = kPz + 2 * 4 * 32 * 8;  // [hi, lo][tile] dz in contraction order, 16-bit
+  static constexpr int kKmPairs = kDz + 2 * 32 * 4;
   static constexpr int kKmF = kKmPairs + 128 * 4;
   static constexpr int kMax = kKmF + 128 * 4;
   static constexpr int kLpt = kMax + 64;
   static constexpr int kTotal = kLpt + (kLptMax + 1) * 4;
-  // the final two-wave reduction reuses the tile area
-  static_assert(kKmPairs - kTiles >= 4 * 64 * 66 * 4, "reduction buffers of the four blocks");
-  static_assert(kTotal <= 160 * 1024, "LDS of one CU");
+  static_assert(kPz >= kOpnd, "the operand is built where the tiles will be");
+  static_assert(2 * kTotal <= 160 * 1024, "two workgroups per CU");
 };
 
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+// Eight tokens of one feature (an MFMA operand fragment of one k-step) out of a row-major tile:
+// two transposing reads, `off0` / `off1` are this lane's byte offsets for x = 0 / 1.
+__device__ __forceinline__ u32x4 tr_fragment(const unsigned char* tile, int off0, int off1) {
+  typedef i16x4 __attribute__((address_space(3))) * lds_ptr;
+  const i16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile + off0));
+  const i16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile + off1));
+  const u32x2 wa = __builtin_bit_cast(u32x2, a), wb = __builtin_bit_cast(u32x2, b);
+  return u32x4{wa[0], wa[1], wb[0], wb[1]};
+}
+
 template <typename T, bool NORM, bool PAD>
-__global__ __launch_bounds__(512, 1) void bwd_a128_kernel(
+__global__ __launch_bounds__(256, 2) void bwd_a128_kernel(
     Prob p, const T* __restrict__ qn, const T* __restrict__ dout, const float* __restrict__ S,
     const float* __restrict__ km, T* __restrict__ dqn, float* __restrict__ partial, float* fin_mat,
     float* fin_vec, int chunk, int nchunks) {
   using LY = BwdA128Layout;
   constexpr bool LO = !std::is_same<T, _Float16>::value;  // see launch_bwd_a
-  constexpr int KS = 8, ROWB = 256, NT = 512;
+  constexpr int KS = 8, ROWB = 256, NT = 256;
   const int dk = PAD ? p.DK : 128, dv = PAD ? p.DV : 128;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -1678,38 +1697,44 @@ __global__ __launch_bounds__(512, 1) void bwd_a128_kernel(
   }
   const int t_end = min(len, t_begin + chunk);
   row_base(p, n, h, bos, row0, rstride);
-  auto piece = [&](int tok, int ch, int rowlen) -> int64_t {
-    if (tok >= t_end || (PAD && ch * 8 >= rowlen)) return -1;
-    return (row0 + (int64_t)tok * rstride) * rowlen + ch * 8;
-  };
 
-  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int tid = threadIdx.x, blk = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int ntok = lane & 31, kb = lane >> 5;
-  const int u = wave & 3, hf = wave >> 2;  // token view: tile, output half; feature view: block, tile pair
-  unsigned char* lds_opnd = smem;
-  unsigned char* qt = smem + LY::kTiles + u * LY::kTile;
-  unsigned char* gt = qt + LY::kTile / 2;
+  const int bk = blk >> 1, bv = blk & 1;  // feature view: block (bk, bv) of dS
+  unsigned char* qtile = smem + LY::kQ;
+  unsigned char* gtile = smem + LY::kG;
+  unsigned char* gltile = smem + LY::kGl;
+  unsigned char* dqtile = smem + LY::kDq;
   float* pz = reinterpret_cast<float*>(smem + LY::kPz);
-  float* scal = reinterpret_cast<float*>(smem + LY::kScal) + 64 * u;
+  T* dzp = reinterpret_cast<T*>(smem + LY::kDz);  // [hi, lo][tile][32]
   uint32_t* km_pairs = reinterpret_cast<uint32_t*>(smem + LY::kKmPairs);
   float* kmf = reinterpret_cast<float*>(smem + LY::kKmF);
   float* lds_max = reinterpret_cast<float*>(smem + LY::kMax);
 
-  // a wave moves the half of its tile's 512 16-byte pieces given by hf (rows 16*hf .. 16*hf+15)
-  auto load_half = [&](u32x4(&dst)[4], const T* src, int tok0, int rowlen) {
+  // The workgroup moves the 1024 16-byte pieces of a step's 64 rows: thread t takes pieces
+  // t + 256 i, i.e. chunk t % 16 of rows t / 16 + 16 i.  A piece's address is the step's uniform
+  // address plus a uniform i-th distance plus the lane's one constant byte offset (32 bits: the
+  // host keeps packed tensors with more than 65536 heads away from this kernel).
+  const int prow = tid >> 4, pch = tid & 15;
+  const uint32_t qrow_b = (uint32_t)rstride * (uint32_t)dk * 2u, grow_b = (uint32_t)rstride * (uint32_t)dv * 2u;
+  const uint32_t qvoff = (uint32_t)prow * qrow_b + (uint32_t)pch * 16u;
+  const uint32_t gvoff = PAD ? (uint32_t)prow * grow_b + (uint32_t)pch * 16u : qvoff;
+  const bool q_piece = !PAD || pch * 8 < dk, g_piece = !PAD || pch * 8 < dv;  // the chunk exists in a row
+  auto step_ptr = [&](const void* src, int tok0, int rowlen) -> const char* {
+    return reinterpret_cast<const char*>(src) + ((row0 + (int64_t)tok0 * rstride) * rowlen) * (int64_t)sizeof(T);
+  };
+  auto load_step = [&](u32x4(&dst)[4], const T* src, int tok0, int rowlen, uint32_t row_b, uint32_t voff, bool has) {
+    const char* tp = step_ptr(src, tok0, rowlen);
+    const int rows = t_end - tok0;  // rows of this step that exist (may be <= 0)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int q = 256 * hf + lane + 64 * i;
-      const int64_t off = piece(tok0 + (q >> 4), q & 15, rowlen);
-      dst[i] = off >= 0 ? load_stream<u32x4, kNtPassALoad>(src + off) : u32x4{0u, 0u, 0u, 0u};
+      dst[i] = u32x4{0u, 0u, 0u, 0u};
+      if (has && prow + 16 * i < rows) dst[i] = load_stream<u32x4, kNtPassALoad>(tp + (size_t)(16 * i) * row_b + voff);
     }
   };
-  auto stash_half = [&](const u32x4(&src)[4], unsigned char* dstb) {
+  auto stash_step = [&](const u32x4(&src)[4], unsigned char* tiles) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int q = 256 * hf + lane + 64 * i;
-      *reinterpret_cast<u32x4*>(dstb + swz<ROWB>(q >> 4, q & 15)) = src[i];
-    }
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(tiles + swz<ROWB>(prow + 16 * i, pch)) = src[i];
   };
 
   f32x16 acc[2][2];
@@ -1719,186 +1744,218 @@ __global__ __launch_bounds__(512, 1) void bwd_a128_kernel(
     for (int b = 0; b < 2; ++b)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-  float dkm[2] = {0.f, 0.f};
+  float dkm = 0.f;  // row 64 bk + 32 bv + ntok, this half-wave's tokens
 
   u32x4 rq[4], rg[4];
-  load_half(rq, qn, t_begin + 32 * u, dk);
-  load_half(rg, dout, t_begin + 32 * u, dv);
+  load_step(rq, qn, t_begin, dk, qrow_b, qvoff, q_piece);
+  load_step(rg, dout, t_begin, dv, grow_b, gvoff, g_piece);
 
   // g_t = dO_t S^T: contraction over dv, M(r = dv, c = dk) = S[c][r]
-  const float denorm = build_operand<T, 128, 128, NT, PAD>(lds_opnd, lds_max, S + (int64_t)nh * dk * dv, 1, dv,
-                                                          1, 0, 1.f, nullptr, dv, dk);
+  const float denorm = build_operand<T, 128, 128, NT, PAD>(smem, lds_max, S + (int64_t)nh * dk * dv, 1, dv, 1, 0,
+                                                          1.f, nullptr, dv, dk);
   if constexpr (NORM) build_vec<T, NT>(km_pairs, kmf, km + (int64_t)nh * dk, dk, 1, 0, 1.f, nullptr, 128);
+  __syncthreads();
+  u32x4 sh[KS], sl[KS];  // output block blk: columns 64 kb' + 16 blk + 0..15 of lane (token, kb')
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    const int f = blk * KS + s;
+    sh[s] = *reinterpret_cast<const u32x4*>(smem + ((2 * f + 0) * 64 + lane) * 16);
+    sl[s] = *reinterpret_cast<const u32x4*>(smem + ((2 * f + 1) * 64 + lane) * 16);
+  }
+  __syncthreads();  // the operand has left LDS
 
-  for (int base = t_begin; base < t_end; base += 128) {
-    const int t0 = base + 32 * u;
-    __syncthreads();  // operand built / the previous step's dq has left the tiles
-    stash_half(rq, qt);
-    stash_half(rg, gt);
-    load_half(rq, qn, t0 + 128, dk);
-    load_half(rg, dout, t0 + 128, dv);
-    __syncthreads();
-
-    // ---- token view: output blocks 2*hf, 2*hf+1; this lane: columns 64*kb + 32*hf + 0..31
-    f32x16 g[2];
+  // transposing reads: this lane addresses, for element half x, token 4 (s >> 2) + 2 (g >> 1) + x
+  // (+ 16 ks) and the four features 16 (g & 1) + 4 (s & 3) .. + 3 of the fragment (g = lane / 16,
+  // s = lane % 16)
+  int qoff[2][2], goff[2][2];
+  {
+    const int g16 = lane >> 4, s16 = lane & 15;
 #pragma unroll
-    for (int bb = 0; bb < 2; ++bb)
+    for (int x = 0; x < 2; ++x) {
+      const int tok = 4 * (s16 >> 2) + 2 * (g16 >> 1) + x;
+      const int f0 = 16 * (g16 & 1) + 4 * (s16 & 3);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) g[bb][r] = 0.f;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const u32x4 bq = *reinterpret_cast<const u32x4*>(gt + swz<ROWB>(ntok, KS * kb + s));
-#pragma unroll
-      for (int bb = 0; bb < 2; ++bb) {
-        const int f = (2 * hf + bb) * KS + s;
-        const u32x4 ah = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * f + 0) * 64 + lane) * 16);
-        const u32x4 al = *reinterpret_cast<const u32x4*>(lds_opnd + ((2 * f + 1) * 64 + lane) * 16);
-        g[bb] = Ops<T>::mma(ah, bq, g[bb]);
-        g[bb] = Ops<T>::mma(al, bq, g[bb]);
+      for (int a = 0; a < 2; ++a) {
+        const int fq = 64 * bk + 32 * a + f0, fg = 64 * bv + 32 * a + f0;
+        qoff[a][x] = swz<ROWB>(tok, fq >> 3) + ((fq >> 2) & 1) * 8;
+        goff[a][x] = swz<ROWB>(tok, fg >> 3) + ((fg >> 2) & 1) * 8;
       }
     }
-    float rz = 1.f, dz = 0.f;
-    if constexpr (NORM) {
-      float P = 0.f, z = 0.f;
+  }
+  // position of token ntok in the contraction order of its tile
+  const int kpos = (ntok & 16) | ((ntok & 2) << 2) | ((ntok & 1) << 2) | ((ntok >> 2) & 3);
+
+  for (int base = t_begin; base < t_end; base += 64) {
+    stash_step(rq, qtile);
+    stash_step(rg, gtile);
+    load_step(rq, qn, base + 64, dk, qrow_b, qvoff, q_piece);
+    load_step(rg, dout, base + 64, dv, grow_b, gvoff, g_piece);
+    __syncthreads();
+
+    // ---- token view: this lane gets columns 64 kb + 16 blk + 0..15 of token ntok of both tiles
+    f32x16 g[2];
 #pragma unroll
-      for (int ch = 0; ch < 4; ++ch) {
-        const u32x4 qw = *reinterpret_cast<const u32x4*>(qt + swz<ROWB>(ntok, 8 * kb + 4 * hf + ch));
-        const u32x4 kh = *reinterpret_cast<const u32x4*>(&km_pairs[32 * kb + 16 * hf + 4 * ch]);
-        const u32x4 kl = *reinterpret_cast<const u32x4*>(&km_pairs[64 + 32 * kb + 16 * hf + 4 * ch]);
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) g[t][r] = 0.f;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const u32x4 bq = *reinterpret_cast<const u32x4*>(gtile + t * LY::kTile + swz<ROWB>(ntok, KS * kb + s));
+        g[t] = Ops<T>::mma(sh[s], bq, g[t]);
+        g[t] = Ops<T>::mma(sl[s], bq, g[t]);
+      }
+    }
+    float rz[2] = {1.f, 1.f}, dz[2] = {0.f, 0.f};
+    if constexpr (NORM) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        float P = 0.f, z = 0.f;
+#pragma unroll
+        for (int ch = 0; ch < 2; ++ch) {
+          const u32x4 qw =
+              *reinterpret_cast<const u32x4*>(qtile + t * LY::kTile + swz<ROWB>(ntok, 8 * kb + 2 * blk + ch));
+          const u32x4 kh = *reinterpret_cast<const u32x4*>(&km_pairs[32 * kb + 8 * blk + 4 * ch]);
+          const u32x4 kl = *reinterpret_cast<const u32x4*>(&km_pairs[64 + 32 * kb + 8 * blk + 4 * ch]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int c0 = 8 * ch + 2 * i;
+            P = fmaf(Ops<T>::lo(qw[i]), g[t][c0], P);
+            P = fmaf(Ops<T>::hi(qw[i]), g[t][c0 + 1], P);
+            z = Ops<T>::dot2(qw[i], kh[i], z);
+            z = Ops<T>::dot2(qw[i], kl[i], z);
+          }
+        }
+        P += __shfl_xor(P, 32);
+        z += __shfl_xor(z, 32);
+        if (kb == 0) *reinterpret_cast<float2*>(&pz[2 * ((4 * t + blk) * 32 + ntok)]) = float2{P, z};
+      }
+      __syncthreads();
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        float P = 0.f, z = 0.f;  // the four parts in block order: the same sum in every wave
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const float2 part = *reinterpret_cast<const float2*>(&pz[2 * ((4 * t + b) * 32 + ntok)]);
+          P += part.x;
+          z += part.y;
+        }
+        if (base + 32 * t + ntok < t_end) {
+          rz[t] = 1.f / (z + p.eps);
+          dz[t] = -(P * denorm) * rz[t] * rz[t];
+        } else {
+          rz[t] = 0.f;  // padding rows contribute nothing
+        }
+        if (blk == 0 && kb == 0) {  // dz as a 16-bit hi + lo pair, for the dot products of the feature view
+          const T dh = (T)dz[t], dl = (T)(dz[t] - (float)dh);
+          dzp[32 * t + kpos] = dh;
+          dzp[64 + 32 * t + kpos] = dl;
+        }
+      }
+    }
+    // dq: this wave's 32 columns of every row, into the staging tiles
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const float gs = denorm * rz[t];
+#pragma unroll
+      for (int ch = 0; ch < 2; ++ch) {
+        u32x4 w;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int c0 = 8 * ch + 2 * i;
-          P = fmaf(Ops<T>::lo(qw[i]), g[c0 >> 4][c0 & 15], P);
-          P = fmaf(Ops<T>::hi(qw[i]), g[c0 >> 4][(c0 & 15) + 1], P);
-          z = Ops<T>::dot2(qw[i], kh[i], z);
-          z = Ops<T>::dot2(qw[i], kl[i], z);
-        }
-      }
-      P += __shfl_xor(P, 32);
-      z += __shfl_xor(z, 32);
-      if (kb == 0) {
-        pz[2 * ((2 * u + hf) * 32 + ntok)] = P;
-        pz[2 * ((2 * u + hf) * 32 + ntok) + 1] = z;
-      }
-      __syncthreads();
-      P += pz[2 * ((2 * u + 1 - hf) * 32 + ntok)];
-      z += pz[2 * ((2 * u + 1 - hf) * 32 + ntok) + 1];
-      if (t0 + ntok < t_end) {
-        rz = 1.f / (z + p.eps);
-        dz = -(P * denorm) * rz * rz;
-      } else {
-        rz = 0.f;  // padding rows contribute nothing
-      }
-      if (hf == 0 && kb == 0) {
-        scal[ntok] = dz;
-        scal[32 + ntok] = rz;
-      }
-    }
-    uint32_t dqp[16];
-    {
-      const float gs = denorm * rz;
-#pragma unroll
-      for (int c2 = 0; c2 < 16; ++c2) {
-        const int c0 = 2 * c2;
-        float v0 = g[c0 >> 4][c0 & 15] * gs, v1 = g[c0 >> 4][(c0 & 15) + 1] * gs;
-        if constexpr (NORM) {
-          v0 = fmaf(dz, kmf[64 * kb + 32 * hf + c0], v0);
-          v1 = fmaf(dz, kmf[64 * kb + 32 * hf + c0 + 1], v1);
-        }
-        dqp[c2] = pack2<T>(v0, v1);
-      }
-    }
-    __syncthreads();  // all four tiles and their scalars are complete
-
-    // ---- feature view: block u = (bk, bv) of dS over the tiles 2*hf, 2*hf+1
-    {
-      const int bk = u >> 1, bv = u & 1;
-#pragma unroll 1
-      for (int uu = 0; uu < 2; ++uu) {
-        const unsigned char* qtu = smem + LY::kTiles + (2 * hf + uu) * LY::kTile;
-        const unsigned char* gtu = qtu + LY::kTile / 2;
-        const float* sc = reinterpret_cast<const float*>(smem + LY::kScal) + 64 * (2 * hf + uu);
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-          const int tok0 = 16 * ks + 8 * kb;
-          RowWords<2> qw, gw;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            qw.w[j][0] = *reinterpret_cast<const uint32_t*>(qtu + swz<ROWB>(tok0 + j, 8 * bk + (ntok >> 2)) +
-                                                            ((ntok & 3) << 2));
-            gw.w[j][0] = *reinterpret_cast<const uint32_t*>(gtu + swz<ROWB>(tok0 + j, 8 * bv + (ntok >> 2)) +
-                                                            ((ntok & 3) << 2));
-          }
-          u32x4 A[2], Bh[2];
-          transpose_rows<2>(qw, A);
+          float v0 = g[t][c0] * gs, v1 = g[t][c0 + 1] * gs;
           if constexpr (NORM) {
-            RowWords<2> vh, vl;
+            v0 = fmaf(dz[t], kmf[64 * kb + 16 * blk + c0], v0);
+            v1 = fmaf(dz[t], kmf[64 * kb + 16 * blk + c0 + 1], v1);
+          }
+          w[i] = pack2<T>(v0, v1);
+        }
+        *reinterpret_cast<u32x4*>(dqtile + t * LY::kTile + swz<ROWB>(ntok, 8 * kb + 2 * blk + ch)) = w;
+      }
+    }
+    // dO / z as hi + lo: this wave's quarter of every row (chunks 4 blk + 2 kb + 0..1)
+    if constexpr (NORM) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              const float rzj = sc[32 + tok0 + j];
-              const float x0 = Ops<T>::lo(gw.w[j][0]) * rzj, x1 = Ops<T>::hi(gw.w[j][0]) * rzj;
-              const T h0 = (T)x0, h1 = (T)x1;
-              vh.w[j][0] = pack2<T>((float)h0, (float)h1);
-              if constexpr (LO) vl.w[j][0] = pack2<T>(x0 - (float)h0, x1 - (float)h1);
-            }
-            transpose_rows<2>(vh, Bh);
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int ch = 0; ch < 2; ++ch) {
+          const int off = t * LY::kTile + swz<ROWB>(ntok, 4 * blk + 2 * kb + ch);
+          const u32x4 gw = *reinterpret_cast<const u32x4*>(gtile + off);
+          u32x4 wh, wl;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float a = Ops<T>::lo(gw[i]) * rz[t], b = Ops<T>::hi(gw[i]) * rz[t];
+            const T ah = (T)a, bh = (T)b;
+            wh[i] = pack2<T>((float)ah, (float)bh);
+            if constexpr (LO) wl[i] = pack2<T>(a - (float)ah, b - (float)bh);
+          }
+          *reinterpret_cast<u32x4*>(gtile + off) = wh;
+          if constexpr (LO) *reinterpret_cast<u32x4*>(gltile + off) = wl;
+        }
+    }
+    __syncthreads();  // dq rows, dO / z and dz are complete
+
+    {
+      char* tp = const_cast<char*>(step_ptr(dqn, base, dk));
+      const int rows = t_end - base;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (q_piece && prow + 16 * i < rows)
+          store_row16<kNtPassAStore>(tp + (size_t)(16 * i) * qrow_b + qvoff,
+                                     *reinterpret_cast<const u32x4*>(dqtile + swz<ROWB>(prow + 16 * i, pch)));
+    }
+
+    // ---- feature view: dS block (bk, bv) += q~^T (dO / z) over both tiles
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const int tb = t * LY::kTile + ks * 16 * ROWB;
+        u32x4 A[2], Bh[2];
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+          A[a] = tr_fragment(qtile + tb, qoff[a][0], qoff[a][1]);
+          Bh[a] = tr_fragment(gtile + tb, goff[a][0], goff[a][1]);
+        }
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+          for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bh[b], acc[a][b]);
+        if constexpr (NORM) {
+          if constexpr (LO) {
+            u32x4 Bl[2];
+#pragma unroll
+            for (int b = 0; b < 2; ++b) Bl[b] = tr_fragment(gltile + tb, goff[b][0], goff[b][1]);
 #pragma unroll
             for (int a = 0; a < 2; ++a)
 #pragma unroll
-              for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bh[b], acc[a][b]);
-            if constexpr (LO) {
-              u32x4 Bl[2];
-              transpose_rows<2>(vl, Bl);
+              for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bl[b], acc[a][b]);
+          }
+          // dkm of the rows of A[bv] (the two waves of a key half share its 64 rows)
+          const u32x4 Ad = bv ? A[1] : A[0];
+          const T* dzs = dzp + 32 * t + 16 * ks + 8 * kb;
+          const u32x4 dh = *reinterpret_cast<const u32x4*>(dzs), dl = *reinterpret_cast<const u32x4*>(dzs + 64);
 #pragma unroll
-              for (int a = 0; a < 2; ++a)
-#pragma unroll
-                for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bl[b], acc[a][b]);
-            }
-            if (bv == 0) {  // the waves of one value half of a key block sum dkm
-#pragma unroll
-              for (int j = 0; j < 8; ++j) {
-                const float dzj = sc[tok0 + j];
-                dkm[0] = fmaf(dzj, Ops<T>::lo(qw.w[j][0]), dkm[0]);
-                dkm[1] = fmaf(dzj, Ops<T>::hi(qw.w[j][0]), dkm[1]);
-              }
-            }
-          } else {
-            transpose_rows<2>(gw, Bh);
-#pragma unroll
-            for (int a = 0; a < 2; ++a)
-#pragma unroll
-              for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], Bh[b], acc[a][b]);
+          for (int i = 0; i < 4; ++i) {
+            dkm = Ops<T>::dot2(Ad[i], dh[i], dkm);
+            dkm = Ops<T>::dot2(Ad[i], dl[i], dkm);
           }
         }
       }
-    }
-    __syncthreads();  // every wave has read every tile: they can take the dq now
-#pragma unroll
-    for (int ch = 0; ch < 4; ++ch)
-      *reinterpret_cast<u32x4*>(qt + swz<ROWB>(ntok, 8 * kb + 4 * hf + ch)) =
-          u32x4{dqp[4 * ch], dqp[4 * ch + 1], dqp[4 * ch + 2], dqp[4 * ch + 3]};
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int q = 256 * hf + lane + 64 * i;
-      const int64_t off = piece(t0 + (q >> 4), q & 15, dk);
-      if (off >= 0)
-        store_row16<kNtPassAStore>(dqn + off, *reinterpret_cast<const u32x4*>(qt + swz<ROWB>(q >> 4, q & 15)));
-    }
+    __syncthreads();  // every wave has read the tiles: the next step may take their place
   }
 
-  __syncthreads();  // the tiles become the reduction buffers
   {
-    const int bk = u >> 1, bv = u & 1;
-    float* red = reinterpret_cast<float*>(smem + LY::kTiles) + u * 64 * 66;
     float* dst = fin_mat ? fin_mat + (int64_t)nh * dk * dv
                          : partial + ((int64_t)nh * nchunks + c) * (dk * dv + dk);
     float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : dst + dk * dv;
     const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
     const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
-    reduce_store_block<2>(acc, dkm, red, dst + (64 * bk) * dv + 64 * bv, dv,
-                          (dst_vec && bv == 0) ? dst_vec + 64 * bk : nullptr, mscale, vscale, hf, lane,
-                          dk - 64 * bk, dv - 64 * bv);
+    float none[2] = {0.f, 0.f};
+    reduce_store_block<1, false>(acc, none, nullptr, dst + (64 * bk) * dv + 64 * bv, dv, nullptr, mscale, vscale, 0,
+                                 lane, dk - 64 * bk, dv - 64 * bv);
+    const float tot = dkm + __shfl_xor(dkm, 32);
+    const int row = 64 * bk + 32 * bv + ntok;
+    if (dst_vec && kb == 0 && row < dk) dst_vec[row] = NORM ? tot * vscale : 0.f;
   }
 }
 
@@ -1928,6 +1985,8 @@ bool supported(const Prob& p, int dtype) {
 // not for the decoupled operator).
 bool bwd_a_supported(const Prob& p, int dtype) {
   if (dtype == kF32 || !supported(p, dtype) || tiled_dim(p.DK) != tiled_dim(p.DV)) return false;
+  // the 128 x 128 kernel addresses a step's rows with 32-bit lane offsets
+  if (tiled_dim(p.DK) == 128 && p.cu && p.H > 65536) return false;
   // decoupled: fused for 64 x 64 tiles only (the 128 x 128 kernel has no room for the plain q tile)
   return !(p.flags & kDecoupled) || tiled_dim(p.DK) == 64;
 }
@@ -2007,8 +2066,8 @@ int state_chunk(const Prob& p, bool block_stats) {
 
 int bwd_a_chunk(const Prob& p) {
   static const int per_cu = knob("FBLA_BWDA_WGS_PER_CU", 2);
-  // 128 x 128: one workgroup per CU, steps of 128 tokens
-  if (tiled_dim(p.DK) == 128) return chunk_for(p, 1, 1, 512, 128, true);
+  // 128 x 128: two workgroups of four waves per CU, steps of 64 tokens
+  if (tiled_dim(p.DK) == 128) return chunk_for(p, 2, 1, 512, 64, true);
   return chunk_for(p, per_cu, 1, 256, 128, true);
 }
 
@@ -2281,7 +2340,7 @@ static int launch_bwd_a128(const Prob& p, const T* q, const T* dout, const float
   int rc = reserve_lds(kernel, LY::kTotal, configured);
   if (rc != kOk) return rc;
   const unsigned grid = (unsigned)((int64_t)p.N * p.H * nchunks);
-  kernel<<<dim3(grid), dim3(512), LY::kTotal, st>>>(p, q, dout, S, km, dq, partial, fm, fv, chunk, nchunks);
+  kernel<<<dim3(grid), dim3(256), LY::kTotal, st>>>(p, q, dout, S, km, dq, partial, fm, fv, chunk, nchunks);
   return kOk;
 }
 
