@@ -382,6 +382,14 @@ def sweep(dtype, dev, flush):
                      "fwd_frac": round(4 * nbytes / f[0] / 1e6 / HBM_PEAK_GBPS, 4),
                      "fwd_bwd_ms": round(s[0], 5), "fwd_bwd_gbps": round(11 * nbytes / s[0] / 1e6, 1),
                      "fwd_bwd_frac": round(11 * nbytes / s[0] / 1e6 / HBM_PEAK_GBPS, 4)})
+        if T <= 4096:
+            # Short sequences: six short kernels per step, which a slow host issues more slowly than
+            # the GPU runs them.  The same step through autograd recorded into one HIP graph
+            # (flash_bla.utils.CapturedStep) is what such a caller would run.
+            from flash_bla.utils import CapturedStep
+            g = do_bench(CapturedStep(linear_attention, [q, k, v], do).replay, flush)
+            rows[-1].update({"fwd_bwd_graph_ms": round(g[0], 5),
+                             "fwd_bwd_graph_frac": round(11 * nbytes / g[0] / 1e6 / HBM_PEAK_GBPS, 4)})
         del q, k, v, do
     return rows
 

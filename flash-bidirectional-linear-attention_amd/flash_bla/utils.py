@@ -77,3 +77,44 @@ class CapturedForward:
             dst.copy_(src)
         self._graph.replay()
         return self._static_out
+
+
+class CapturedStep:
+    """Forward and backward of `fn` recorded once into one HIP graph and replayed per call.
+
+    For short sequences a training step of an operator is six short kernels whose launches,
+    together with the autograd bookkeeping around them, can take the host longer than the GPU
+    needs to run them; a replay is one launch.  `fn(*inputs)` must return one tensor.  Inputs
+    and the output gradient are copied into recorded tensors; the call returns the recorded
+    output and the recorded gradients of the inputs that require them (None for the others),
+    all overwritten by the next call.  Shapes and dtypes are fixed at construction."""
+
+    def __init__(self, fn, example_inputs, example_grad_output, warmup=3):
+        self._static_in = [t.detach().clone().requires_grad_(t.requires_grad) for t in example_inputs]
+        self._static_gout = example_grad_output.detach().clone()
+        self._leaves = [t for t in self._static_in if t.requires_grad]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(warmup):  # lazy initialisation (LDS attributes, caches) happens here
+                torch.autograd.grad(fn(*self._static_in), self._leaves, self._static_gout)
+        torch.cuda.current_stream().wait_stream(side)
+        self._graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self._graph):
+            self._static_out = fn(*self._static_in)
+            grads = torch.autograd.grad(self._static_out, self._leaves, self._static_gout)
+        grads = iter(grads)
+        self._static_grads = [next(grads) if t.requires_grad else None for t in self._static_in]
+
+    def __call__(self, inputs, grad_output):
+        with torch.no_grad():
+            for dst, src in zip(self._static_in, inputs):
+                dst.copy_(src)
+            self._static_gout.copy_(grad_output)
+        self._graph.replay()
+        return self._static_out, self._static_grads
+
+    def replay(self):
+        """Replays the step on the recorded tensors as they are (no copies)."""
+        self._graph.replay()
+        return self._static_out, self._static_grads
