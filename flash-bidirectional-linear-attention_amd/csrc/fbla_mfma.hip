@@ -125,6 +125,17 @@ template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{a, b}, tx2_t));
 }
 
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+// Eight tokens of one feature (an MFMA operand fragment of one k-step) out of a row-major tile:
+// two transposing reads, `off0` / `off1` are this lane's byte offsets for x = 0 / 1.
+__device__ __forceinline__ u32x4 tr_fragment(const unsigned char* tile, int off0, int off1) {
+  typedef i16x4 __attribute__((address_space(3))) * lds_ptr;
+  const i16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile + off0));
+  const i16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile + off1));
+  const u32x2 wa = __builtin_bit_cast(u32x2, a), wb = __builtin_bit_cast(u32x2, b);
+  return u32x4{wa[0], wa[1], wb[0], wb[1]};
+}
+
 // ===========================================================================
 // state kernel
 // ===========================================================================
@@ -510,29 +521,39 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
 // state kernel for heads tiled 128 x 128 (plain operator: no rotary keys, no row scaling,
 // no block statistics)
 // ===========================================================================
-// Every wave holds the whole 128 x 128 state (256 accumulator registers, which is why one
-// workgroup of four waves has a CU to itself) and the waves take interleaved steps of two
-// 16-token tiles.  Each row is therefore read by exactly one wave; in state_kernel's split by
-// 64 x 64 blocks every 128-byte half of a row is read by two waves, and with streaming loads
-// the second read is often served by HBM again.  A lane owns four adjacent features of k and
-// of v (one 8-byte load per row and tensor: 32 loads per step, so that "all but the newest
-// step" still fits the 6-bit counter of outstanding loads), which makes accumulator (a, b),
-// register r of lane (pp, kb) the element S[4 m + a][4 pp + b], m = 8 (r / 4) + 4 kb + r % 4.
+// A workgroup of four waves walks its chunk in steps of 64 tokens.  The rows of a step arrive
+// flat (16 bytes per lane, whole rows, each read from memory exactly once) and are staged in
+// LDS; wave w owns the 64 x 64 block w of the state and reads k^T and v for it straight out of
+// the row-major tiles in operand order with the transposing LDS read (ds_read_b64_tr_b16), so
+// nothing is transposed in registers and no wave's sum has to be added to another's at the
+// end.  Two LDS buffers alternate: the step after the current one sits in registers while the
+// current one is multiplied, and one barrier per step separates the writers of a buffer from
+// its readers.  The contraction index is the permutation of a tile's tokens that
+// bwd_a128_kernel uses (k-step ks, half-wave kb, element e = 4x + j is token 16ks + 4j + 2kb + x).
+struct State128Layout {
+  static constexpr int kTile = 32 * 256;     // 32 tokens x 128 features x 2 bytes
+  static constexpr int kStep = 2 * kTile;    // 64 tokens
+  static constexpr int kK = 0;               // k steps [2]
+  static constexpr int kV = 2 * kStep;       // v steps [2]
+  static constexpr int kLpt = 4 * kStep;
+  static constexpr int kTotal = kLpt + (kLptMax + 1) * 4;
+};
+
 template <typename T, bool PAD>
-__global__ __launch_bounds__(kThreads, 1) void state128_kernel(Prob p, const T* __restrict__ kn,
+__global__ __launch_bounds__(kThreads, 2) void state128_kernel(Prob p, const T* __restrict__ kn,
                                                                const T* __restrict__ v,
                                                                float* __restrict__ partial,
                                                                float* __restrict__ fin_mat,
                                                                float* __restrict__ fin_vec, int chunk,
                                                                int nchunks) {
+  using LY = State128Layout;
+  constexpr int ROWB = 256;
   const int dk = PAD ? p.DK : 128, dv = PAD ? p.DV : 128;  // row lengths in memory
-  constexpr int G = kWaves, TILES = 2, kStep = 16 * TILES;
-  __shared__ float red[64 * 65];  // one quarter of a wave's sums: [value][lane]
-  __shared__ int lpt_lens[kLptMax + 1];
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int wg_item = packed_item(p, blockIdx.x, p.H * nchunks);
   const int wg_nh = wg_item / nchunks, c = wg_item - wg_nh * nchunks;
   const int h = wg_nh % p.H;
-  const int n = lpt_sequence(p, wg_nh / p.H, lpt_lens);
+  const int n = lpt_sequence(p, wg_nh / p.H, reinterpret_cast<int*>(smem + LY::kLpt));
   const int nh = n * p.H + h;
   int64_t bos, row0, rstride;
   int len;
@@ -549,148 +570,112 @@ __global__ __launch_bounds__(kThreads, 1) void state128_kernel(Prob p, const T* 
   const int t_end = min(len, t_begin + chunk);
   row_base(p, n, h, bos, row0, rstride);
 
-  const int g = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const int pp = lane & 31, kb = lane >> 5;
-  // this lane's four features, and whether they exist (head dims are multiples of 8)
-  const bool k_ok = !PAD || 4 * pp < dk, v_ok = !PAD || 4 * pp < dv;
-  const int kcol0 = k_ok ? 4 * pp : 0, vcol0 = v_ok ? 4 * pp : 0;
-  const uint32_t k_keep = k_ok ? ~0u : 0u, v_keep = v_ok ? ~0u : 0u;
-  const uint32_t kstep = (uint32_t)(rstride * dk), vstep = (uint32_t)(rstride * dv);
-  const uint32_t kvoff = (uint32_t)(8 * kb) * kstep + (uint32_t)kcol0;
-  const uint32_t vvoff = (uint32_t)(8 * kb) * vstep + (uint32_t)vcol0;
+  const int tid = threadIdx.x, blk = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int ntok = lane & 31, kb = lane >> 5;
+  const int bk = blk >> 1, bv = blk & 1;  // block (bk, bv) of the state
+  unsigned char* ksteps = smem + LY::kK;
+  unsigned char* vsteps = smem + LY::kV;
 
-  f32x16 acc[4][4];
+  // The workgroup moves the 1024 16-byte pieces of a step's 64 rows: thread t takes pieces
+  // t + 256 i, i.e. chunk t % 16 of rows t / 16 + 16 i: the step's uniform address plus a uniform
+  // i-th distance plus the lane's one constant byte offset (32 bits: the host keeps packed
+  // tensors with more than 65536 heads away from this kernel).  Rows past the end of the chunk
+  // and chunks past the head dim are not read and count as zeros.
+  const int prow = tid >> 4, pch = tid & 15;
+  const uint32_t krow_b = (uint32_t)rstride * (uint32_t)dk * 2u, vrow_b = (uint32_t)rstride * (uint32_t)dv * 2u;
+  const uint32_t kvoff = (uint32_t)prow * krow_b + (uint32_t)pch * 16u;
+  const uint32_t vvoff = PAD ? (uint32_t)prow * vrow_b + (uint32_t)pch * 16u : kvoff;
+  const bool k_piece = !PAD || pch * 8 < dk, v_piece = !PAD || pch * 8 < dv;
+  auto load_step = [&](u32x4(&dst)[4], const T* src, int tok0, int rowlen, uint32_t row_b, uint32_t voff, bool has) {
+    const char* tp = reinterpret_cast<const char*>(src) + ((row0 + (int64_t)tok0 * rstride) * rowlen) * (int64_t)sizeof(T);
+    const int rows = t_end - tok0;  // rows of this step that exist (may be <= 0)
 #pragma unroll
-  for (int a = 0; a < 4; ++a)
+    for (int i = 0; i < 4; ++i) {
+      dst[i] = u32x4{0u, 0u, 0u, 0u};
+      if (has && prow + 16 * i < rows) dst[i] = load_stream<u32x4, kNtStateLoad>(tp + (size_t)(16 * i) * row_b + voff);
+    }
+  };
+  auto stash_step = [&](const u32x4(&src)[4], unsigned char* tiles) {
 #pragma unroll
-    for (int b = 0; b < 4; ++b)
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(tiles + swz<ROWB>(prow + 16 * i, pch)) = src[i];
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-  float ks[4] = {0.f, 0.f, 0.f, 0.f};
+  float ks = 0.f;  // row 64 bk + 32 bv + ntok of sum_t k_t, this half-wave's tokens
 
-  struct Buf {
-    RowWords<4> k[TILES], v[TILES];
-  };
-  // as in state_kernel: a tile that would cross the end of the chunk is moved back so that it
-  // ends there, and the rows it shares with the tile before it are zeroed before use
-  auto fetch = [&](Buf& b, int tok) {
+  // transposing reads: this lane addresses, for element half x, token 4 (s >> 2) + 2 (g >> 1) + x
+  // (+ 16 ks) and the four features 16 (g & 1) + 4 (s & 3) .. + 3 of the fragment (g = lane / 16,
+  // s = lane % 16)
+  int koff[2][2], voff2[2][2];
+  {
+    const int g16 = lane >> 4, s16 = lane & 15;
 #pragma unroll
-    for (int u = 0; u < TILES; ++u) {
-      const int tb = min(tok + 16 * u, t_end - 16);
-      const int64_t row = row0 + (int64_t)tb * rstride;
-      load_rows<T, 4>(b.k[u], kn + row * dk, kstep, kvoff);
-      load_rows<T, 4>(b.v[u], v + row * dv, vstep, vvoff);
-    }
-  };
-  auto fetch_checked = [&](Buf& b, int tok) {  // chunk shorter than a tile
+    for (int x = 0; x < 2; ++x) {
+      const int tok = 4 * (s16 >> 2) + 2 * (g16 >> 1) + x;
+      const int f0 = 16 * (g16 & 1) + 4 * (s16 & 3);
 #pragma unroll
-    for (int u = 0; u < TILES; ++u) {
-      const int rows = t_end - (tok + 16 * u);
-      const int64_t row = row0 + (int64_t)(tok + 16 * u) * rstride;
-      load_rows_checked<T, 4>(b.k[u], kn + row * dk, kstep, 8 * kb, kcol0, rows);
-      load_rows_checked<T, 4>(b.v[u], v + row * dv, vstep, 8 * kb, vcol0, rows);
-    }
-  };
-  auto compute = [&](Buf& b, int tok, bool checked) {
-#pragma unroll
-    for (int u = 0; u < TILES; ++u) {
-      if constexpr (PAD) {
-        keep_rows<4>(b.k[u], k_keep);
-        keep_rows<4>(b.v[u], v_keep);
+      for (int a = 0; a < 2; ++a) {
+        const int fk = 64 * bk + 32 * a + f0, fv = 64 * bv + 32 * a + f0;
+        koff[a][x] = swz<ROWB>(tok, fk >> 3) + ((fk >> 2) & 1) * 8;
+        voff2[a][x] = swz<ROWB>(tok, fv >> 3) + ((fv >> 2) & 1) * 8;
       }
-      if (!checked && tok + kStep > t_end) {  // last step of the chunk: some tiles were moved back
-        const int lo = min(16, tok + 16 * u - min(tok + 16 * u, t_end - 16));
-        mask_rows<4>(b.k[u], 8 * kb, lo);
-      }
-      u32x4 A[4], B[4];
-      transpose_rows<4>(b.k[u], A);
-      transpose_rows<4>(b.v[u], B);
-#pragma unroll
-      for (int a = 0; a < 4; ++a)
-#pragma unroll
-        for (int bb = 0; bb < 4; ++bb) acc[a][bb] = Ops<T>::mma(A[a], B[bb], acc[a][bb]);
-#pragma unroll
-      for (int a = 0; a < 4; ++a)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) ks[a] = Ops<T>::dot2(A[a][i], Ops<T>::kOnes, ks[a]);
-    }
-  };
-  int t0 = t_begin + kStep * g;
-  if (t_end - t_begin < 16) {
-    if (t0 < t_end) {
-      Buf b0;
-      fetch_checked(b0, t0);
-      compute(b0, t0, true);
-    }
-  } else if (t0 < t_end) {
-    Buf b0, b1;
-    fetch(b0, t0);
-    while (true) {
-      int tn = t0 + kStep * G;
-      fetch(b1, tn);
-      compute(b0, t0, false);
-      t0 = tn;
-      if (t0 >= t_end) break;
-      tn = t0 + kStep * G;
-      fetch(b0, tn);
-      compute(b1, t0, false);
-      t0 = tn;
-      if (t0 >= t_end) break;
     }
   }
 
-  // Fixed-order sum over the four waves, a quarter of the state (accumulator row a: 64
-  // registers) at a time through LDS: 2 -> 0, 3 -> 1, 1 -> 0 with the roles rotated by a, so
-  // that quarter a ends in wave a and the four quarters are stored by four waves.  One chunk
-  // per (sequence, head): the sum is final and is stored scaled where the reduce kernel would
-  // have put it; otherwise this chunk's partial is stored.
+  u32x4 rk[4], rv[4];
+  load_step(rk, kn, t_begin, dk, krow_b, kvoff, k_piece);
+  load_step(rv, v, t_begin, dv, vrow_b, vvoff, v_piece);
+  int buf = 0;
+  for (int base = t_begin; base < t_end; base += 64) {
+    unsigned char* kt = ksteps + buf * LY::kStep;
+    unsigned char* vt = vsteps + buf * LY::kStep;
+    stash_step(rk, kt);
+    stash_step(rv, vt);
+    load_step(rk, kn, base + 64, dk, krow_b, kvoff, k_piece);
+    load_step(rv, v, base + 64, dv, vrow_b, vvoff, v_piece);
+    __syncthreads();  // the step is in LDS; every wave is done with the other buffer's previous step
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const int tb = t * LY::kTile + s * 16 * ROWB;
+        u32x4 A[2], B[2];
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+          A[a] = tr_fragment(kt + tb, koff[a][0], koff[a][1]);
+          B[a] = tr_fragment(vt + tb, voff2[a][0], voff2[a][1]);
+        }
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+          for (int b = 0; b < 2; ++b) acc[a][b] = Ops<T>::mma(A[a], B[b], acc[a][b]);
+        // sum_t k_t for the rows of A[bv] (the two waves of a key half share its 64 rows)
+        const u32x4 Ak = bv ? A[1] : A[0];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ks = Ops<T>::dot2(Ak[i], Ops<T>::kOnes, ks);
+      }
+    buf ^= 1;
+  }
+
+  // one chunk per (sequence, head): the sum is final and is stored scaled where the reduce
+  // kernel would have put it; otherwise this chunk's partial is stored
   float* mat = fin_mat ? fin_mat + (int64_t)nh * dk * dv
                        : partial + ((int64_t)nh * nchunks + c) * (dk * dv + dk);
   float* vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : mat + dk * dv;
   const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
   const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
-  typedef float f32x4 __attribute__((ext_vector_type(4)));
-#pragma unroll
-  for (int a = 0; a < 4; ++a) {
-    const int role = (g + G - a) & (G - 1);
-    auto spill = [&]() {
-#pragma unroll
-      for (int b = 0; b < 4; ++b)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) red[(b * 16 + r) * 64 + lane] = acc[a][b][r];
-      red[64 * 64 + lane] = ks[a];
-    };
-    auto absorb = [&]() {
-#pragma unroll
-      for (int b = 0; b < 4; ++b)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][b][r] += red[(b * 16 + r) * 64 + lane];
-      ks[a] += red[64 * 64 + lane];
-    };
-    if (role == 2) spill();
-    __syncthreads();
-    if (role == 0) absorb();
-    __syncthreads();
-    if (role == 3) spill();
-    __syncthreads();
-    if (role == 1) absorb();
-    __syncthreads();
-    if (role == 1) spill();
-    __syncthreads();
-    if (role == 0) {
-      absorb();
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = 4 * (8 * (r >> 2) + 4 * kb + (r & 3)) + a;
-        if (row < dk && 4 * pp < dv)
-          *reinterpret_cast<f32x4*>(mat + row * dv + 4 * pp) =
-              f32x4{acc[a][0][r] * mscale, acc[a][1][r] * mscale, acc[a][2][r] * mscale, acc[a][3][r] * mscale};
-      }
-      const float tot = ks[a] + __shfl_xor(ks[a], 32);
-      if (vec && kb == 0 && 4 * pp + a < dk) vec[4 * pp + a] = tot * vscale;
-    }
-    __syncthreads();  // `red` is reused by the next quarter
-  }
+  float none[2] = {0.f, 0.f};
+  reduce_store_block<1, false>(acc, none, nullptr, mat + (64 * bk) * dv + 64 * bv, dv, nullptr, mscale, vscale, 0,
+                               lane, dk - 64 * bk, dv - 64 * bv);
+  const float tot = ks + __shfl_xor(ks, 32);
+  const int row = 64 * bk + 32 * bv + ntok;
+  if (vec && kb == 0 && row < dk) vec[row] = tot * vscale;
 }
 
 // ===========================================================================
@@ -1656,17 +1641,6 @@ struct BwdA128Layout {
   static_assert(2 * kTotal <= 160 * 1024, "two workgroups per CU");
 };
 
-typedef short i16x4 __attribute__((ext_vector_type(4)));
-// Eight tokens of one feature (an MFMA operand fragment of one k-step) out of a row-major tile:
-// two transposing reads, `off0` / `off1` are this lane's byte offsets for x = 0 / 1.
-__device__ __forceinline__ u32x4 tr_fragment(const unsigned char* tile, int off0, int off1) {
-  typedef i16x4 __attribute__((address_space(3))) * lds_ptr;
-  const i16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile + off0));
-  const i16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile + off1));
-  const u32x2 wa = __builtin_bit_cast(u32x2, a), wb = __builtin_bit_cast(u32x2, b);
-  return u32x4{wa[0], wa[1], wb[0], wb[1]};
-}
-
 template <typename T, bool NORM, bool PAD>
 __global__ __launch_bounds__(256, 2) void bwd_a128_kernel(
     Prob p, const T* __restrict__ qn, const T* __restrict__ dout, const float* __restrict__ S,
@@ -2047,15 +2021,12 @@ static int chunk_for(const Prob& p, int wgs_per_cu, int rounds, int min_chunk, i
 }
 
 // Reduction kernels (state, backward pass A): one round of resident workgroups.
-// 128 x 128 states of the plain operator: state128_kernel, one workgroup per CU, when that
-// leaves a workgroup at least 1024 tokens.  Its four waves each sum the whole state over a
-// quarter of the tokens and add the four sums at the end; with fewer tokens that addition
-// costs more than state_kernel's second read of every row.
+// 128 x 128 states of the plain operator: state128_kernel, two workgroups per CU.
 static int whole_state_chunk(const Prob& p) {
   static const int on = knob("FBLA_STATE128", 1);  // 2 = off (A/B comparisons)
   if (on != 1 || tiled_dim(p.DK) != 128 || tiled_dim(p.DV) != 128 || (p.flags & kDecoupled)) return 0;
-  const int chunk = chunk_for(p, 1, 1, 256, 64, true);
-  return chunk >= 1024 ? chunk : 0;
+  if (p.cu && p.H > 65536) return 0;  // 32-bit lane offsets
+  return chunk_for(p, 2, 1, 256, 64, true);
 }
 
 int state_chunk(const Prob& p, bool block_stats) {
@@ -2097,6 +2068,19 @@ int rows_chunk(const Prob& p, int DR, int DC) {
   return chunk;
 }
 
+// Reserves the kernel's dynamic LDS once per instantiation and thread.
+template <typename K> static int reserve_lds(K kernel, int bytes, bool& done) {
+  if (done) return kOk;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) {
+    set_error("cannot reserve %d bytes of LDS: %s", bytes, hipGetErrorString(e));
+    return kErrLaunch;
+  }
+  done = true;
+  return kOk;
+}
+
 template <typename T, int DK, int DV, bool PAD>
 static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, float* partial,
                          const float* tokscal, int64_t total_rows, float* fm, float* fv, int chunk,
@@ -2108,7 +2092,10 @@ static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, fl
   constexpr int TL = (DK == 128 && DV == 128) ? 2 : 1;
   if constexpr (DK == 128 && DV == 128) {
     if (!bs.kc && !tokscal && whole_state_chunk(p) == chunk) {
-      state128_kernel<T, PAD><<<grid, block, 0, st>>>(p, kn, v, partial, fm, fv, chunk, nchunks);
+      auto kernel = state128_kernel<T, PAD>;
+      static thread_local bool configured = false;  // per instantiation
+      if (reserve_lds(kernel, State128Layout::kTotal, configured) != kOk) return;
+      kernel<<<grid, block, State128Layout::kTotal, st>>>(p, kn, v, partial, fm, fv, chunk, nchunks);
       return;
     }
   }
@@ -2143,19 +2130,6 @@ static void run_state(const Prob& p, const void* kn, const void* v, const void* 
   const T *a = (const T*)kn, *b = (const T*)v, *c = (const T*)kd;
   if (padded(p)) run_state_dims<T, true>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
   else run_state_dims<T, false>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
-}
-
-// Reserves the kernel's dynamic LDS once per instantiation and thread.
-template <typename K> static int reserve_lds(K kernel, int bytes, bool& done) {
-  if (done) return kOk;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-  if (e != hipSuccess) {
-    set_error("cannot reserve %d bytes of LDS: %s", bytes, hipGetErrorString(e));
-    return kErrLaunch;
-  }
-  done = true;
-  return kOk;
 }
 
 template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD, bool PAIR = false>
