@@ -1168,6 +1168,216 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
 }
 
 // ===========================================================================
+// rows kernel for 128 x 128 matrices (not the decoupled operator's separate denominator rows)
+// ===========================================================================
+// The general kernel keeps the 64 KiB operand in LDS and lets every wave multiply its own tile
+// by all of it (64 operand reads per tile, one eight-wave workgroup per CU).  Here a workgroup of
+// four waves shares steps of 64 rows and two workgroups share a CU: the operand is built in LDS
+// once, wave w keeps the fragments of output block w (32 of the 128 output columns) in 64
+// registers, and the LDS becomes the row tiles.  Per step: the rows arrive flat and are staged
+// (z_t = x_t . km is added up from the flat pieces on the way), every wave multiplies both
+// tiles by its block, scales, adds, packs its 32 columns of every row into a staging step, and
+// whole rows leave from there.  Two barriers per step; the x steps alternate between two buffers.
+struct Rows128Layout {
+  static constexpr int kOpnd = 4 * 8 * 2 * 1024;  // 4 blocks x 8 k-steps x (hi, lo) fragments
+  static constexpr int kTile = 32 * 256;
+  static constexpr int kStep = 2 * kTile;
+  static constexpr int kX = 0;                  // x steps [2]
+  static constexpr int kOut = 2 * kStep;        // output staging
+  static constexpr int kKm = kOpnd;             // km as 16-bit pairs [2][64]
+  static constexpr int kAdd = kKm + 128 * 4;    // row added to every output row [128]
+  static constexpr int kZ = kAdd + 128 * 4;     // z of the step's rows [2][64]
+  static constexpr int kMax = kZ + 2 * 64 * 4;
+  static constexpr int kLpt = kMax + 64;
+  static constexpr int kTotal = kLpt + (kLptMax + 1) * 4;
+  static_assert(kOut + kStep <= kOpnd, "tiles live where the operand was built");
+  static_assert(2 * kTotal <= 160 * 1024, "two workgroups per CU");
+};
+
+template <typename T, bool NORM, bool PAD>
+__global__ __launch_bounds__(kThreads, 2) void rows128_kernel(Prob p, RowsJob job0, RowsJob job1, int wgs_per_job,
+                                                              int chunk, int nchunks, int dr_true, int dc_true) {
+  using LY = Rows128Layout;
+  constexpr int KS = 8, ROWB = 256, NT = kThreads;
+  const int dr = PAD ? dr_true : 128, dc = PAD ? dc_true : 128;
+  const int dpk = PAD ? (p.DK <= 64 ? 64 : 128) : p.DK;  // padded length of the km / dkm vector
+  const bool second = (int)blockIdx.x >= wgs_per_job;
+  const RowsJob& job = second ? job1 : job0;
+  const int wg = second ? blockIdx.x - wgs_per_job : blockIdx.x;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  uint32_t* lds_km = reinterpret_cast<uint32_t*>(smem + LY::kKm);
+  float* lds_add = reinterpret_cast<float*>(smem + LY::kAdd);
+  float* lds_z = reinterpret_cast<float*>(smem + LY::kZ);
+  float* lds_max = reinterpret_cast<float*>(smem + LY::kMax);
+
+  const int wg_item = packed_item(p, wg, p.H * nchunks);
+  const int wg_nh = wg_item / nchunks, c = wg_item - wg_nh * nchunks;
+  const int h = wg_nh % p.H;
+  const int n = lpt_sequence(p, wg_nh / p.H, reinterpret_cast<int*>(smem + LY::kLpt));
+  const int nh = n * p.H + h;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t_begin = c * chunk;
+  if (t_begin >= len) {
+    if (c == 0 && job.pnchunks > 0) {  // empty sequence: its state is zero
+      if (job.mat_out)
+        for (int e = threadIdx.x; e < dr * dc; e += NT) job.mat_out[(int64_t)nh * dr * dc + e] = 0.f;
+      if (job.vec_out)
+        for (int e = threadIdx.x; e < p.DK; e += NT) job.vec_out[(int64_t)nh * p.DK + e] = 0.f;
+    }
+    return;
+  }
+  const int t_end = min(len, t_begin + chunk);
+  row_base(p, n, h, bos, row0, rstride);
+
+  const int tid = threadIdx.x, blk = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int ntok = lane & 31, kb = lane >> 5;
+  const bool has_add = job.addvec != nullptr || job.vec_is_add;  // the same for all lanes
+  const T* x = (const T*)job.x;
+  T* out = (T*)job.out;
+
+  // The workgroup moves the 1024 16-byte pieces of a step's 64 rows: thread t takes pieces
+  // t + 256 i, i.e. chunk t % 16 of rows t / 16 + 16 i: the step's uniform address plus a uniform
+  // i-th distance plus the lane's one constant byte offset (32 bits: the host keeps packed
+  // tensors with more than 65536 heads away from this kernel).
+  const int prow = tid >> 4, pch = tid & 15;
+  const uint32_t xrow_b = (uint32_t)rstride * (uint32_t)dr * 2u, orow_b = (uint32_t)rstride * (uint32_t)dc * 2u;
+  const uint32_t xvoff = (uint32_t)prow * xrow_b + (uint32_t)pch * 16u;
+  const uint32_t ovoff = PAD ? (uint32_t)prow * orow_b + (uint32_t)pch * 16u : xvoff;
+  const bool x_piece = !PAD || pch * 8 < dr, o_piece = !PAD || pch * 8 < dc;
+  auto step_ptr = [&](const void* base, int tok0, int rowlen) -> const char* {
+    return reinterpret_cast<const char*>(base) + ((row0 + (int64_t)tok0 * rstride) * rowlen) * (int64_t)sizeof(T);
+  };
+  auto load_step = [&](u32x4(&dst)[4], int tok0) {
+    const char* tp = step_ptr(x, tok0, dr);
+    const int rows = t_end - tok0;  // rows of this step that exist (may be <= 0)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      dst[i] = u32x4{0u, 0u, 0u, 0u};
+      if (x_piece && prow + 16 * i < rows) dst[i] = load_stream<u32x4, kNtRowsLoad>(tp + (size_t)(16 * i) * xrow_b + xvoff);
+    }
+  };
+
+  u32x4 rx[4];
+  load_step(rx, t_begin);
+
+  // ---- prologue: matrix operand fragments, km pairs, addvec (as in rows_kernel) ----
+  float denorm;
+  if (job.pnchunks > 0) {
+    const int E = dr * dc;
+    const int64_t pstride = E + p.DK;
+    const int nsum = min(job.pnchunks, (len + job.pchunk - 1) / job.pchunk);
+    const float* part = job.mat + (int64_t)nh * job.pnchunks * pstride;
+    const bool writer = c == 0;
+    denorm = build_operand<T, 128, 128, NT, PAD>(smem, lds_max, part, job.ld_r, job.ld_c, nsum, pstride,
+                                                 seq_scale(p, len),
+                                                 writer && job.mat_out ? job.mat_out + (int64_t)nh * E : nullptr, dr,
+                                                 dc);
+    const float inv_len = 1.0f / (float)len;
+    float* vout = writer && job.vec_out ? job.vec_out + (int64_t)nh * p.DK : nullptr;
+    if (NORM || job.vec_is_add || vout)
+      build_vec<T, NT>(NORM ? lds_km : nullptr, job.vec_is_add ? lds_add : nullptr, part + E, p.DK, nsum, pstride,
+                       inv_len, vout, dpk);
+    if (!job.vec_is_add)
+      for (int e = tid; e < 128; e += NT) lds_add[e] = 0.f;
+  } else {
+    denorm = build_operand<T, 128, 128, NT, PAD>(smem, lds_max, job.mat + (int64_t)nh * dr * dc, job.ld_r, job.ld_c,
+                                                 1, 0, 1.f, nullptr, dr, dc);
+    if constexpr (NORM) build_vec<T, NT>(lds_km, nullptr, job.km + (int64_t)nh * dr, dr, 1, 0, 1.f, nullptr, 128);
+    for (int e = tid; e < 128; e += NT)
+      lds_add[e] = (job.addvec && e < dc) ? job.addvec[(int64_t)nh * dc + e] * job.add_scale : 0.f;
+  }
+  __syncthreads();
+  u32x4 sh[KS], sl[KS];  // output block blk: columns 64 kb' + 16 blk + 0..15 of lane (row, kb')
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    const int f = blk * KS + s;
+    sh[s] = *reinterpret_cast<const u32x4*>(smem + ((2 * f + 0) * 64 + lane) * 16);
+    sl[s] = *reinterpret_cast<const u32x4*>(smem + ((2 * f + 1) * 64 + lane) * 16);
+  }
+  // the row added to this lane's 16 columns, and the km pairs of this thread's chunk of a row
+  float addv[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) addv[r] = lds_add[64 * kb + 16 * blk + r];
+  u32x4 kmh = u32x4{0u, 0u, 0u, 0u}, kml = kmh;
+  if constexpr (NORM) {
+    kmh = *reinterpret_cast<const u32x4*>(&lds_km[4 * pch]);
+    kml = *reinterpret_cast<const u32x4*>(&lds_km[64 + 4 * pch]);
+  }
+  __syncthreads();  // the operand has left LDS
+
+  unsigned char* ostage = smem + LY::kOut;
+  int buf = 0;
+  for (int base = t_begin; base < t_end; base += 64) {
+    unsigned char* xt = smem + LY::kX + buf * LY::kStep;
+    float* zrow = lds_z + 64 * buf;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(xt + swz<ROWB>(prow + 16 * i, pch)) = rx[i];
+    if constexpr (NORM) {
+      // piece i of this thread is chunk pch of row prow + 16 i: its dot product with the km values
+      // of that chunk, then the sum over the 16 lanes of the row
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float a = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          a = Ops<T>::dot2(rx[i][w], kmh[w], a);
+          a = Ops<T>::dot2(rx[i][w], kml[w], a);
+        }
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) a += __shfl_xor(a, off);
+        if (pch == 0) zrow[prow + 16 * i] = a;
+      }
+    }
+    load_step(rx, base + 64);
+    __syncthreads();  // the step and its z are in LDS; the staging step has been read out
+
+    // this lane gets columns 64 kb + 16 blk + 0..15 of row ntok of both tiles
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      f32x16 acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const u32x4 bq = *reinterpret_cast<const u32x4*>(xt + t * LY::kTile + swz<ROWB>(ntok, KS * kb + s));
+        acc = Ops<T>::mma(sh[s], bq, acc);
+        acc = Ops<T>::mma(sl[s], bq, acc);
+      }
+      float rs = denorm;
+      if constexpr (NORM) rs = denorm / (zrow[32 * t + ntok] + p.eps);
+#pragma unroll
+      for (int ch = 0; ch < 2; ++ch) {
+        u32x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int c0 = 8 * ch + 2 * i;
+          float v0 = acc[c0] * rs, v1 = acc[c0 + 1] * rs;
+          if (has_add) {
+            v0 += addv[c0];
+            v1 += addv[c0 + 1];
+          }
+          w[i] = pack2<T>(v0, v1);
+        }
+        *reinterpret_cast<u32x4*>(ostage + t * LY::kTile + swz<ROWB>(ntok, 8 * kb + 2 * blk + ch)) = w;
+      }
+    }
+    __syncthreads();  // the output rows are complete
+    {
+      char* tp = const_cast<char*>(step_ptr(out, base, dc));
+      const int rows = t_end - base;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (o_piece && prow + 16 * i < rows)
+          store_row16<kNtRowsStore>(tp + (size_t)(16 * i) * orow_b + ovoff,
+                                    *reinterpret_cast<const u32x4*>(ostage + swz<ROWB>(prow + 16 * i, pch)));
+    }
+    buf ^= 1;
+  }
+}
+
+// ===========================================================================
 // backward pass A
 // ===========================================================================
 // Per 32-token sub-tile (one wave):
@@ -2042,6 +2252,7 @@ int bwd_a_chunk(const Prob& p) {
   return chunk_for(p, per_cu, 1, 256, 128, true);
 }
 
+static bool use_rows128(const Prob& p);
 // Row-parallel kernels: long enough chunks to amortise the operand prologue.
 int rows_chunk(const Prob& p, int DR, int DC) {
   static const int per_cu_knob = knob("FBLA_ROWS_WGS_PER_CU", 4);
@@ -2052,7 +2263,7 @@ int rows_chunk(const Prob& p, int DR, int DC) {
   // a 128 x 128 operand costs as much to build as 512 tokens cost to stream: one round there
   const int big = (tiled_dim(DR) == 128) + (tiled_dim(DC) == 128);
   const int rounds = p.cu ? packed_rounds : (big == 2 ? 1 : big == 1 ? (dense_rounds + 1) / 2 : dense_rounds);
-  const int per_cu = big == 0 ? per_cu_knob : (big == 1 ? 2 : 1);
+  const int per_cu = big == 0 ? per_cu_knob : (big == 1 || use_rows128(p) ? 2 : 1);
   static const int min_chunk_knob = knob("FBLA_ROWS_MIN_CHUNK", 256);
   // a problem too small to give every CU a workgroup: shorter chunks (the operand build of the
   // extra workgroups costs less than the idle CUs)
@@ -2147,6 +2358,26 @@ static int launch_rows_k(const Prob& p, const RowsJob& job, const RowsJob* job2,
   return kOk;
 }
 
+template <typename T, bool NORM, bool PAD>
+static int launch_rows128(const Prob& p, const RowsJob& job, const RowsJob* job2, int chunk, int nchunks, int dr,
+                          int dc, hipStream_t st) {
+  auto kernel = rows128_kernel<T, NORM, PAD>;
+  static thread_local bool configured = false;
+  int rc = reserve_lds(kernel, Rows128Layout::kTotal, configured);
+  if (rc != kOk) return rc;
+  const int wgs = (int)((int64_t)p.N * p.H * nchunks);
+  const dim3 grid((unsigned)(job2 ? 2 * wgs : wgs)), block(kThreads);
+  kernel<<<grid, block, Rows128Layout::kTotal, st>>>(p, job, job2 ? *job2 : job, wgs, chunk, nchunks, dr, dc);
+  return kOk;
+}
+
+// 128 x 128 matrices without separate denominator rows: rows128_kernel (FBLA_ROWS128=2 keeps the
+// general kernel, for comparisons)
+static bool use_rows128(const Prob& p) {
+  static const int on = knob("FBLA_ROWS128", 1);
+  return on == 1 && !(p.flags & kDecoupled) && !(p.cu && p.H > 65536);
+}
+
 template <typename T, int DR, int DC, bool PAD>
 static int launch_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, int dr, int dc,
                        hipStream_t st) {
@@ -2157,6 +2388,12 @@ static int launch_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, i
   const int nchunks = (int)cdiv64(p.L, chunk);
   const bool norm = job.xden != nullptr;
   const bool den = norm && job.xden != job.x;
+  if constexpr (DR == 128 && DC == 128) {
+    if (!den && use_rows128(p)) {
+      if (norm) return launch_rows128<T, true, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
+      return launch_rows128<T, false, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
+    }
+  }
   if (!norm) return launch_rows_k<T, DR, DC, false, false, WAVES, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
   if (!den) return launch_rows_k<T, DR, DC, true, false, WAVES, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
   return launch_rows_k<T, DR, DC, true, true, WAVES, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
