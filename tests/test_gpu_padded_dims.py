@@ -106,8 +106,9 @@ def test_heads_tiled_128_by_128():
 @pytest.mark.parametrize("dims,dtype,L", [((128, 128), torch.bfloat16, 1030), ((96, 120), torch.float16, 1100),
                                            ((128, 72), torch.bfloat16, 2049)])
 def test_whole_state_per_wave_dense(dims, dtype, L):
-    """256 heads of more than 1024 tokens with a state tiled 128 x 128: the state kernel in which
-    every wave keeps the whole state.  A few heads are checked against the oracle."""
+    """256 heads of more than 1024 tokens with a state tiled 128 x 128 (one workgroup per head in
+    the state kernel, the row kernel and backward pass A for 128-wide heads).  A few heads are
+    checked against the oracle."""
     from flash_bla.ops.linear_attn.fused import linear_attention
     DK, DV = dims
     B, H = 16, 16
@@ -128,8 +129,19 @@ def test_whole_state_per_wave_dense(dims, dtype, L):
             assert_parity(t.grad[sl], ref[name], dtype, f"{name} {tag}", ref.get(name + "_mag"))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dims", [(128, 128), (104, 96), (72, 128)])
+def test_heads_tiled_128_around_the_64_token_steps(dims, dtype):
+    """The kernels for heads tiled 128 x 128 walk steps of 64 tokens staged in LDS: lengths just
+    below, at and above one, two and three steps, one chunk and several chunks per head."""
+    for i, L in enumerate([63, 64, 65, 127, 128, 129, 191, 193, 640, 1153]):
+        _check_dense("linear", 1, 2, L, dims[0], dims[1], dtype, 90 * i + dims[0])
+    _check_dense("simple", 2, 1, 130, dims[0], dims[1], dtype, 7 + dims[1])
+    _check_dense("linear", 2, 70, 321, dims[0], dims[1], dtype, 11 + dims[1])  # one chunk per head
+
+
 def test_whole_state_per_wave_packed():
-    """The same kernel on a packed batch: 320 (sequence, head) pairs, the longest sequence above
+    """The same kernels on a packed batch: 320 (sequence, head) pairs, the longest sequence above
     1024 tokens, among them sequences shorter than one tile, of one token and empty ones."""
     from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
     H, DK, DV, dtype = 8, 128, 128, torch.bfloat16
