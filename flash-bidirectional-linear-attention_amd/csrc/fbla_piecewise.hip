@@ -210,9 +210,11 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
+// (written as a vector conversion so that the compiler can use the packed conversion instruction)
 template <typename T> __device__ __forceinline__ uint32_t pack_pair(float a, float b) {
-  return (uint32_t)__builtin_bit_cast(uint16_t, (T)a) |
-         ((uint32_t)__builtin_bit_cast(uint16_t, (T)b) << 16);
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef T tx2_t __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{a, b}, tx2_t));
 }
 template <typename T> __device__ __forceinline__ float unpack_lo(uint32_t w) {
   return (float)__builtin_bit_cast(T, (uint16_t)(w & 0xffffu));
@@ -276,25 +278,31 @@ struct Attn32Args {
 template <int K, int V> struct Attn32Layout {
   static constexpr int kKT = 64 * K * 2;   // K tile: 64 keys x K features
   static constexpr int kVT = V * 128;      // V^T tile: V value columns x 64 keys
-  static constexpr int kSet = kKT + kVT;
-  static constexpr int kTiles = 2 * kSet;  // double buffer; the selected-block bitmap follows
+  static constexpr int kSlot = kKT > kVT ? kKT : kVT;
+  static constexpr int kTiles = 3 * kSlot;  // ring of three tiles; the selected-block bitmap follows
 };
 
 typedef uint32_t u32x2p __attribute__((ext_vector_type(2)));
 
+// Tiles are consumed as one stream: K and V^T of selected block 0, K and V^T of block 1, ...,
+// then per group of 64 unselected-block statistics the mean keys (hi, lo) and the value sums
+// (hi, lo).  Stage s works on tile s in ring slot s % 3 while tile s+1 has landed or is landing
+// and tile s+2 is requested: three tiles of 16 KiB per workgroup instead of two K + V^T pairs,
+// so that three workgroups (three waves per SIMD, at most 168 registers) share a CU.
 template <typename T, int K, int V>
-__global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) {
+__global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) {
   using LY = Attn32Layout<K, V>;
   constexpr int KS = K / 16;                 // k-steps of the score product
   constexpr int MB = V / 32;                 // 32-row blocks of O^T
   constexpr int OLD = 64 * (V / 8) / kThreads;
   constexpr float kNegInf = -__builtin_huge_valf();
   constexpr float kLazy = 8.f;
-  // Two tile sets as two separate LDS objects: the compiler can then tell that a tile load
-  // in flight towards one set does not touch the set being read, and does not make the reads
-  // wait for it.  The selected-block bitmap is the dynamic part.
-  __shared__ __attribute__((aligned(1024))) unsigned char set_a[LY::kSet];
-  __shared__ __attribute__((aligned(1024))) unsigned char set_b[LY::kSet];
+  // Three separate LDS objects: the compiler can then tell that a tile load in flight towards
+  // one slot does not touch the slot being read, and does not make the reads wait for it.
+  // The selected-block bitmap is the dynamic part.
+  __shared__ __attribute__((aligned(1024))) unsigned char ring0[LY::kSlot];
+  __shared__ __attribute__((aligned(1024))) unsigned char ring1[LY::kSlot];
+  __shared__ __attribute__((aligned(1024))) unsigned char ring2[LY::kSlot];
   extern __shared__ __attribute__((aligned(16))) unsigned char sel[];
 
   const int tq = blockIdx.x % a.NT;
@@ -308,8 +316,13 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
   const int Tp = a.NT * 64;
 
   const T* qb = (const T*)a.q + bh * a.T * K;
+  // buffer descriptor: base, no stride, byte count (loads past it return zeros), raw 32-bit data
+  typedef int i32x4s __attribute__((ext_vector_type(4)));
   auto descriptor = [](const void* base, int64_t bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+    const uint64_t p = reinterpret_cast<uint64_t>(base);
+    return i32x4s{__builtin_amdgcn_readfirstlane((int)(uint32_t)p),
+                  __builtin_amdgcn_readfirstlane((int)((uint32_t)(p >> 32) & 0xffffu)),
+                  __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
   };
   const auto k_rs = descriptor((const T*)a.k + bh * a.T * K, (int64_t)a.T * K * 2);
   const auto vt_rs = descriptor((const T*)a.vt + bh * V * (int64_t)Tp, (int64_t)V * Tp * 2);
@@ -321,9 +334,14 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
   for (int i = tid; i < a.NTp; i += kThreads) sel[i] = 0;
   __syncthreads();
   const int32_t* idx = a.indices + (bh * a.NT + tq) * a.NS;
+  // first key row and row count of every selected block (0 rows: an index out of range), kept in
+  // LDS: the stages below read them with LDS loads, which the tile loads' counter does not see
+  int2* blk = reinterpret_cast<int2*>(sel + ((a.NTp + 15) & ~15));
   for (int i = tid; i < a.NS; i += kThreads) {
     const int b = idx[i];
-    if (b >= 0 && b < a.NT) sel[b] = 1;
+    const bool ok = b >= 0 && b < a.NT;
+    if (ok) sel[b] = 1;
+    blk[i] = ok ? int2{b * 64, min(64, a.T - b * 64)} : int2{0, 0};
   }
 
   // Q^T operand: k-step s covers features 16s + 8kg + i
@@ -349,37 +367,44 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
   // fills 1 KiB = 4 or 8 whole tile rows).  The swizzle is applied on the global side: the
   // lane that owns LDS slot s of row r fetches chunk s ^ swizzle(r).  Rows past the end of
   // the tensor arrive as zeros (the descriptor's byte count is the bounds check).
-  typedef __attribute__((address_space(3))) void* lds_ptr;
+  // The loads are written as assembly: the compiler's own wait insertion then neither counts
+  // them nor waits for all of them before the first read of a slot; the waits are the ones at
+  // the start of each stage below.
+  typedef __attribute__((address_space(3))) unsigned char* lds_ptr;
+  auto dma16 = [](i32x4s rs, unsigned char* dst, uint32_t lane_off, int wave_off) {
+    const uint32_t lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr)dst);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds), "v"(lane_off), "s"(rs), "s"(wave_off)
+                 : "memory", "m0");
+  };
   constexpr int KROWB = K * 2, KRW = 1024 / KROWB, KJ = 64 / (4 * KRW);
   const int krow_l = KRW * wave + lane / (KROWB / 16), kslot = lane % (KROWB / 16);
   const uint32_t k_lane_off =
       (uint32_t)(krow_l * KROWB + ((kslot ^ (K == 128 ? (krow_l & 15) : ((krow_l >> 1) & 7))) << 4));
-  auto dma_tile_k = [&](__amdgpu_buffer_rsrc_t rs, unsigned char* tile, int row0) {
+  auto dma_tile_k = [&](i32x4s rs, unsigned char* tile, int row0) {
 #pragma unroll
     for (int j = 0; j < KJ; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(tile + (4 * KRW * j + KRW * wave) * KROWB), 16,
-                                               k_lane_off, (row0 + 4 * KRW * j) * KROWB, 0, 0);
+      dma16(rs, tile + (4 * KRW * j + KRW * wave) * KROWB, k_lane_off, (row0 + 4 * KRW * j) * KROWB);
   };
   // V^T tile: V rows of 128 bytes (64 keys, permuted inside groups of 16 in global memory
   // already); source row stride `ld` elements
   constexpr int VJ = V / 32;
   const int vrow_l = 8 * wave + (lane >> 3), vslot = lane & 7;
   const uint32_t v_lane_chunk = (uint32_t)((vslot ^ ((vrow_l >> 1) & 7)) << 4);
-  auto dma_tile_v = [&](__amdgpu_buffer_rsrc_t rs, unsigned char* tile, int ld, int col0) {
+  auto dma_tile_v = [&](i32x4s rs, unsigned char* tile, int ld, int col0) {
     const uint32_t lane_off = (uint32_t)(vrow_l * ld * 2) + v_lane_chunk;
 #pragma unroll
-    for (int j = 0; j < VJ; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr)(tile + (32 * j + 8 * wave) * 128), 16, lane_off,
-                                               (col0 + 32 * j * ld) * 2, 0, 0);
+    for (int j = 0; j < VJ; ++j) dma16(rs, tile + (32 * j + 8 * wave) * 128, lane_off, (col0 + 32 * j * ld) * 2);
   };
 
   // per-lane LDS offsets of the operand reads
-  int koff[KS], voff[2];
-#pragma unroll
-  for (int s = 0; s < KS; ++s) koff[s] = kswz(32 * kh + n, 2 * s + kg);
+  // (k-step s of the key tile sits at koff0 ^ (s << 5): the swizzle is an XOR of the chunk index)
+  int koff0 = kswz(32 * kh + n, kg), voff[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) voff[t] = vswz(n, 2 * (2 * kh + t) + kg);
 
+  const int kbase = 32 * kh + 4 * kg;
   float m_i = kNegInf, l_p = 0.f, g_p = 0.f;  // running max (unscaled); per-lane partial sums
   f32x16 acc[MB];
 #pragma unroll
@@ -387,37 +412,19 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[mb][r] = 0.f;
 
-  // One 64-key block in three stages; this wave's keys are key(r) = 32kh + 8(r/4) + 4kg + r%4.
+  // This wave's keys of a 64-key block are key(r) = kbase + c(r), kbase = 32kh + 4kg (per lane),
+  // c(r) = 8(r/4) + r%4 (a constant per register): the predicates below compare kbase with a
+  // scalar, so that no register holds a key index.
   // The tags are compile-time (std::true_type / false_type): masked = some keys are invalid,
-  // weighted = the block statistics branch (hi + lo tiles, sums weighted by chunk length).
-  //   scores:   S^T = K Q^T, two accumulators (two independent MFMA chains)
+  // weighted = the block statistics branch (sums weighted by chunk length).
+  //   scores:   S^T += K Q^T
   //   softmax:  running maximum, p = exp2(...), partial sums, accumulator rescale; p packed
   //   values:   O^T += V^T P^T
-  auto scores = [&](const unsigned char* kt0, const unsigned char* kt1, auto weighted_tag) {
-    constexpr bool weighted = decltype(weighted_tag)::value;
-    f32x16 st, st2;
+  auto scores = [&](const unsigned char* kt, f32x16 st) {
+    asm volatile("" : "+v"(koff0));  // the eight offsets are derived here, not kept in registers
 #pragma unroll
-    for (int r = 0; r < 16; ++r) st[r] = st2[r] = 0.f;
-    // all operand reads are issued before the first MFMA: their latencies overlap
-    u32x4 ak[KS];
-#pragma unroll
-    for (int s = 0; s < KS; ++s) ak[s] = *reinterpret_cast<const u32x4*>(kt0 + koff[s]);
-#pragma unroll
-    for (int s = 0; s < KS; s += 2) {
-      st = Mma32<T>::run(ak[s], qop[s], st);
-      st2 = Mma32<T>::run(ak[s + 1], qop[s + 1], st2);
-    }
-    if constexpr (weighted) {
-#pragma unroll
-      for (int s = 0; s < KS; ++s) ak[s] = *reinterpret_cast<const u32x4*>(kt1 + koff[s]);
-#pragma unroll
-      for (int s = 0; s < KS; s += 2) {
-        st = Mma32<T>::run(ak[s], qop[s], st);
-        st2 = Mma32<T>::run(ak[s + 1], qop[s + 1], st2);
-      }
-    }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) st[r] += st2[r];
+    for (int s = 0; s < KS; ++s)
+      st = Mma32<T>::run(*reinterpret_cast<const u32x4*>(kt + (koff0 ^ (s << 5))), qop[s], st);
     return st;
   };
   auto softmax = [&](f32x16 st, u32x4(&pw)[2], auto valid, auto weight, auto masked_tag, auto weighted_tag) {
@@ -425,7 +432,7 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
     float mx = kNegInf;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      if constexpr (masked) st[r] = valid(32 * kh + 8 * (r >> 2) + 4 * kg + (r & 3)) ? st[r] : kNegInf;
+      if constexpr (masked) st[r] = valid(8 * (r >> 2) + (r & 3)) ? st[r] : kNegInf;
       mx = fmaxf(mx, st[r]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32));
@@ -449,8 +456,8 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
         const float p1 = __builtin_amdgcn_exp2f(fmaf(st[r + 1], c2, -mc));
         psum += p0 + p1;
         if constexpr (weighted) {
-          wsum = fmaf(p0, weight(32 * kh + 8 * (r >> 2) + 4 * kg + (r & 3)), wsum);
-          wsum = fmaf(p1, weight(32 * kh + 8 * ((r + 1) >> 2) + 4 * kg + ((r + 1) & 3)), wsum);
+          wsum = fmaf(p0, weight(8 * (r >> 2) + (r & 3)), wsum);
+          wsum = fmaf(p1, weight(8 * ((r + 1) >> 2) + ((r + 1) & 3)), wsum);
         }
         pw[t][i] = pack_pair<T>(p0, p1);
       }
@@ -468,103 +475,168 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
         for (int r = 0; r < 16; ++r) acc[mb][r] *= alpha;
     }
   };
-  auto values = [&](const unsigned char* vt0, const unsigned char* vt1, const u32x4(&pw)[2],
-                    auto weighted_tag) {
-    constexpr bool weighted = decltype(weighted_tag)::value;
-    u32x4 av[2][MB];
+  auto values = [&](const unsigned char* vt, const u32x4(&pw)[2]) {
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
-        av[t][mb] = *reinterpret_cast<const u32x4*>(vt0 + voff[t] + mb * (32 * 128));
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) acc[mb] = Mma32<T>::run(av[t][mb], pw[t], acc[mb]);
-    if constexpr (weighted) {
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          av[t][mb] = *reinterpret_cast<const u32x4*>(vt1 + voff[t] + mb * (32 * 128));
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) acc[mb] = Mma32<T>::run(av[t][mb], pw[t], acc[mb]);
-    }
+        acc[mb] = Mma32<T>::run(*reinterpret_cast<const u32x4*>(vt + voff[t] + mb * (32 * 128)), pw[t], acc[mb]);
   };
   const std::true_type yes{};
   const std::false_type no{};
 
-  // ---- phase 1: selected blocks.  The tile of block i+1 is in flight towards the other LDS
-  // set while block i is computed (the loop is unrolled by two: constant addresses).
-  auto block_rows = [&](int b) { return b >= 0 && b < a.NT ? min(64, a.T - b * 64) : 0; };
-  auto fetch_block = [&](int i, unsigned char* set) {
-    if (i < a.NS) {
-      const int bn = idx[i], nn = block_rows(bn);
-      dma_tile_k(k_rs, set, nn ? bn * 64 : 0);
-      dma_tile_v(vt_rs, set + LY::kKT, Tp, nn ? bn * 64 : 0);
+  // ---- the tile stream ----
+  // Phase 1 is padded to a multiple of three blocks (six stages) and phase 2 to a multiple of
+  // three groups (twelve stages), so that the ring slot of every stage is a compile-time
+  // constant in loops unrolled by that much; padding stages request and compute nothing.
+  const int NS3 = (a.NS + 2) / 3 * 3, S1 = 2 * NS3;
+  const int NG = (a.NT + 63) / 64;
+  auto block_rows = [&](int i) { return __builtin_amdgcn_readfirstlane(blk[i].y); };
+  // number of load instructions a wave issues for tile s (0: no such tile)
+  auto tile_loads = [&](int s) {
+    if (s < S1) return (s >> 1) < a.NS ? ((s & 1) ? VJ : KJ) : 0;
+    const int s2 = s - S1;
+    return (s2 >> 2) < NG ? ((s2 & 2) ? VJ : KJ) : 0;
+  };
+  auto fetch = [&](int s, unsigned char* slot) {
+    if (s < S1) {
+      const int i = s >> 1;
+      if (i < a.NS) {
+        const int row0 = __builtin_amdgcn_readfirstlane(blk[i].x);
+        if (s & 1) dma_tile_v(vt_rs, slot, Tp, row0);
+        else dma_tile_k(k_rs, slot, row0);
+      }
+    } else {
+      const int s2 = s - S1, g = s2 >> 2;
+      if (g < NG) {
+        switch (s2 & 3) {
+          case 0: dma_tile_k(kch_rs, slot, g * 64); break;
+          case 1: dma_tile_k(kcl_rs, slot, g * 64); break;
+          case 2: dma_tile_v(vch_rs, slot, a.NTp, g * 64); break;
+          default: dma_tile_v(vcl_rs, slot, a.NTp, g * 64); break;
+        }
+      }
     }
   };
-  fetch_block(0, set_a);
-  __syncthreads();
+  // Start of stage s: this wave's loads of tile s have landed (the loads of tile s+1, issued
+  // later, may still be in flight: the counter retires in order), every wave has said so and
+  // has finished reading tile s-1, whose slot then receives tile s+2.
+  auto begin_stage = [&](int s, unsigned char* slot_s2) {
+    const int pending = tile_loads(s + 1);
+    if (pending >= 4) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else if (pending >= 2) asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    fetch(s + 2, slot_s2);
+  };
+  static_assert(KJ == 2 || KJ == 4, "tile load counts are waited for as 2 or 4");
+  static_assert(VJ == 2 || VJ == 4, "tile load counts are waited for as 2 or 4");
+
   u32x4 pw[2];
-  auto step = [&](int i, unsigned char* cur, unsigned char* nxt) {
-    fetch_block(i + 1, nxt);
-    const int nrows = block_rows(idx[i]);
-    const auto none = [](int) { return 0.f; };
-    if (nrows == 64) {
-      const f32x16 st = scores(cur, cur, no);
-      softmax(st, pw, [](int) { return true; }, none, no, no);
-      values(cur + LY::kKT, cur, pw, no);
-    } else if (nrows > 0) {
-      const f32x16 st = scores(cur, cur, no);
-      softmax(st, pw, [&](int key) { return key < nrows; }, none, yes, no);
-      values(cur + LY::kKT, cur, pw, no);
+  f32x16 zero16;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) zero16[r] = 0.f;
+  const auto none = [](int) { return 0.f; };
+
+  // ---- phase 1: selected blocks ----
+  auto key_stage = [&](int s, unsigned char* cur, unsigned char* slot_s2) {
+    begin_stage(s, slot_s2);
+    const int i = s >> 1;
+    if (i < a.NS) {
+      const int nrows = block_rows(i);
+      if (nrows == 64) {
+        const f32x16 st = scores(cur, zero16);
+        softmax(st, pw, [](int) { return true; }, none, no, no);
+      } else if (nrows > 0) {
+        const f32x16 st = scores(cur, zero16);
+        int kb = kbase;
+        asm volatile("" : "+v"(kb));  // (keeps the sixteen sums kb + c out of registers across the loop)
+        softmax(st, pw, [&](int c) { return kb < nrows - c; }, none, yes, no);
+      }
     }
-    __syncthreads();
   };
-  for (int i = 0; i < a.NS; i += 2) {
-    step(i, set_a, set_b);
-    if (i + 1 < a.NS) step(i + 1, set_b, set_a);
+  auto value_stage = [&](int s, unsigned char* cur, unsigned char* slot_s2) {
+    begin_stage(s, slot_s2);
+    const int i = s >> 1;
+    if (i < a.NS && block_rows(i) > 0) values(cur, pw);
+  };
+  // the query operand has arrived before the first tile is requested: a later wait for it would
+  // also wait for every tile load issued in between (the counter retires in order)
+#pragma unroll
+  for (int s = 0; s < KS; ++s) asm volatile("" ::"v"(qop[s]));
+  __syncthreads();  // the selected blocks' rows are in LDS
+  fetch(0, ring0);
+  fetch(1, ring1);
+  for (int s = 0; s < S1; s += 6) {
+    key_stage(s + 0, ring0, ring2);
+    value_stage(s + 1, ring1, ring0);
+    key_stage(s + 2, ring2, ring1);
+    value_stage(s + 3, ring0, ring2);
+    key_stage(s + 4, ring1, ring0);
+    value_stage(s + 5, ring2, ring1);
   }
 
-  // ---- phase 2: unselected blocks through their means / sums ----
+  // ---- phase 2: unselected blocks through their means / sums (hi + lo 16-bit pairs) ----
   const int last_len = a.T - (a.NT - 1) * 64;
-  for (int grp = 0; grp * 64 < a.NT; ++grp) {
-    dma_tile_k(kch_rs, set_a, grp * 64);
-    dma_tile_k(kcl_rs, set_b, grp * 64);
-    dma_tile_v(vch_rs, set_a + LY::kKT, a.NTp, grp * 64);
-    dma_tile_v(vcl_rs, set_b + LY::kKT, a.NTp, grp * 64);
-    __syncthreads();
-    const int c0 = grp * 64;
-    const f32x16 st = scores(set_a, set_b, yes);
-    softmax(st, pw, [&](int key) { return c0 + key < a.NT && !sel[c0 + key]; },
-            [&](int key) { return c0 + key == a.NT - 1 ? (float)last_len : 64.f; }, yes, yes);
-    values(set_a + LY::kKT, set_b + LY::kKT, pw, yes);
-    __syncthreads();
+  f32x16 stw;
+  auto mean_hi_stage = [&](int s, unsigned char* cur, unsigned char* slot_s2) {
+    begin_stage(s, slot_s2);
+    if (((s - S1) >> 2) < NG) stw = scores(cur, zero16);
+  };
+  auto mean_lo_stage = [&](int s, unsigned char* cur, unsigned char* slot_s2) {
+    begin_stage(s, slot_s2);
+    const int g = (s - S1) >> 2;
+    if (g < NG) {
+      const int c0 = g * 64;
+      const f32x16 st = scores(cur, stw);
+      int kb = kbase;
+      asm volatile("" : "+v"(kb));
+      const unsigned char* selk = sel + c0 + kb;
+      const int left = a.NT - c0;  // blocks from c0 on
+      softmax(st, pw, [&](int c) { return kb < left - c && !selk[c]; },
+              [&](int c) { return kb == left - 1 - c ? (float)last_len : 64.f; }, yes, yes);
+    }
+  };
+  auto sum_stage = [&](int s, unsigned char* cur, unsigned char* slot_s2) {
+    begin_stage(s, slot_s2);
+    if (((s - S1) >> 2) < NG) values(cur, pw);
+  };
+  for (int s = S1; s < S1 + 4 * NG; s += 12) {
+    mean_hi_stage(s + 0, ring0, ring2);
+    mean_lo_stage(s + 1, ring1, ring0);
+    sum_stage(s + 2, ring2, ring1);
+    sum_stage(s + 3, ring0, ring2);
+    mean_hi_stage(s + 4, ring1, ring0);
+    mean_lo_stage(s + 5, ring2, ring1);
+    sum_stage(s + 6, ring0, ring2);
+    sum_stage(s + 7, ring1, ring0);
+    mean_hi_stage(s + 8, ring2, ring1);
+    mean_lo_stage(s + 9, ring0, ring2);
+    sum_stage(s + 10, ring1, ring0);
+    sum_stage(s + 11, ring2, ring1);
   }
+  __syncthreads();  // nothing is in flight any more (the stream has ended); the slots are free
 
   // ---- merge the two key halves: waves kh = 1 hand their state to waves kh = 0 ----
   float L = l_p + __shfl_xor(l_p, 32), G = g_p + __shfl_xor(g_p, 32);
-  float* mrg = reinterpret_cast<float*>(qh ? set_b : set_a);  // [value][lane], 64 * (16 MB + 3) floats
+  float* mrg = reinterpret_cast<float*>(qh ? ring1 : ring0);           // [value][lane]: 64 * 16 MB floats
+  float* mrg3 = reinterpret_cast<float*>(ring2) + qh * 3 * 64;         // m, L, G per lane
   if (kh == 1) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) mrg[(mb * 16 + r) * 64 + lane] = acc[mb][r];
-    mrg[(MB * 16 + 0) * 64 + lane] = m_i;
-    mrg[(MB * 16 + 1) * 64 + lane] = L;
-    mrg[(MB * 16 + 2) * 64 + lane] = G;
+    mrg3[0 * 64 + lane] = m_i;
+    mrg3[1 * 64 + lane] = L;
+    mrg3[2 * 64 + lane] = G;
   }
   __syncthreads();
   if (kh == 0) {
-    const float m1 = mrg[(MB * 16 + 0) * 64 + lane];
+    const float m1 = mrg3[0 * 64 + lane];
     const float m = fmaxf(m_i, m1);
     const float ms = m == kNegInf ? 0.f : m;
     const float a0 = __builtin_amdgcn_exp2f((m_i - ms) * c2), a1 = __builtin_amdgcn_exp2f((m1 - ms) * c2);
-    L = L * a0 + mrg[(MB * 16 + 1) * 64 + lane] * a1;
-    G = G * a0 + mrg[(MB * 16 + 2) * 64 + lane] * a1;
+    L = L * a0 + mrg3[1 * 64 + lane] * a1;
+    G = G * a0 + mrg3[2 * 64 + lane] * a1;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -573,8 +645,8 @@ __global__ __launch_bounds__(kThreads, 2) void attention32_kernel(Attn32Args a) 
   __syncthreads();
 
   // ---- phase 3 and output (waves kh = 0): acc += (q H) * (G/T) * scale, o = acc / (L + G) ----
-  unsigned char* rt = set_a;  // q H tile [64][V]
-  unsigned char* ot = set_b;  // output tile [64][V]
+  unsigned char* rt = ring2;  // q H tile [64][V]
+  unsigned char* ot = ring0;  // output tile [64][V]
   {
     const T* rsrc = (const T*)a.r + (bh * a.T + (int64_t)tq * 64) * V;
     const int nrows = a.T - tq * 64;
@@ -949,11 +1021,12 @@ size_t attention_workspace_bytes(int64_t BH, int64_t T, int K, int V) {
 template <typename T, int K, int V>
 static int launch_attention(const Attn32Args& a, const void* v, int64_t BH, hipStream_t st) {
   using LY = Attn32Layout<K, V>;
-  if (LY::kTiles + a.NTp > 80 * 1024) {
+  // the tile ring is static; dynamic: the selected-block bitmap and the selected blocks' rows
+  const int lds = ((a.NTp + 15) & ~15) + a.NS * 8;
+  if (LY::kTiles + lds > 64 * 1024) {
     set_error("piecewise attention: %d key blocks need more LDS than a workgroup has", a.NT);
     return kErrUnsupported;
   }
-  const int lds = a.NTp;  // the tile sets are static
   auto kernel = attention32_kernel<T, K, V>;
   transpose_values_kernel<T, V><<<dim3((unsigned)(BH * a.NT)), dim3(kThreads), 0, st>>>(
       (const T*)v, (T*)const_cast<void*>(a.vt), a.T, a.NT);
