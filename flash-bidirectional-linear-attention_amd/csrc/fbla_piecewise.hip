@@ -336,9 +336,10 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   const int32_t* idx = a.indices + (bh * a.NT + tq) * a.NS;
   // first key row and row count of every selected block (0 rows: an index out of range), kept in
   // LDS: the stages below read them with LDS loads, which the tile loads' counter does not see
+  // (the list is padded with empty blocks to a multiple of three, and one more group of three)
   int2* blk = reinterpret_cast<int2*>(sel + ((a.NTp + 15) & ~15));
-  for (int i = tid; i < a.NS; i += kThreads) {
-    const int b = idx[i];
+  for (int i = tid; i < (a.NS + 2) / 3 * 3 + 3; i += kThreads) {
+    const int b = i < a.NS ? idx[i] : -1;
     const bool ok = b >= 0 && b < a.NT;
     if (ok) sel[b] = 1;
     blk[i] = ok ? int2{b * 64, min(64, a.T - b * 64)} : int2{0, 0};
@@ -491,42 +492,31 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   // constant in loops unrolled by that much; padding stages request and compute nothing.
   const int NS3 = (a.NS + 2) / 3 * 3, S1 = 2 * NS3;
   const int NG = (a.NT + 63) / 64;
-  auto block_rows = [&](int i) { return __builtin_amdgcn_readfirstlane(blk[i].y); };
-  // number of load instructions a wave issues for tile s (0: no such tile)
+  // phase 2 by stream position (s >= S1): number of load instructions a wave issues for tile s
+  // (0: no such tile), and the request itself
   auto tile_loads = [&](int s) {
-    if (s < S1) return (s >> 1) < a.NS ? ((s & 1) ? VJ : KJ) : 0;
     const int s2 = s - S1;
     return (s2 >> 2) < NG ? ((s2 & 2) ? VJ : KJ) : 0;
   };
   auto fetch = [&](int s, unsigned char* slot) {
-    if (s < S1) {
-      const int i = s >> 1;
-      if (i < a.NS) {
-        const int row0 = __builtin_amdgcn_readfirstlane(blk[i].x);
-        if (s & 1) dma_tile_v(vt_rs, slot, Tp, row0);
-        else dma_tile_k(k_rs, slot, row0);
-      }
-    } else {
-      const int s2 = s - S1, g = s2 >> 2;
-      if (g < NG) {
-        switch (s2 & 3) {
-          case 0: dma_tile_k(kch_rs, slot, g * 64); break;
-          case 1: dma_tile_k(kcl_rs, slot, g * 64); break;
-          case 2: dma_tile_v(vch_rs, slot, a.NTp, g * 64); break;
-          default: dma_tile_v(vcl_rs, slot, a.NTp, g * 64); break;
-        }
+    const int s2 = s - S1, g = s2 >> 2;
+    if (g < NG) {
+      switch (s2 & 3) {
+        case 0: dma_tile_k(kch_rs, slot, g * 64); break;
+        case 1: dma_tile_k(kcl_rs, slot, g * 64); break;
+        case 2: dma_tile_v(vch_rs, slot, a.NTp, g * 64); break;
+        default: dma_tile_v(vcl_rs, slot, a.NTp, g * 64); break;
       }
     }
   };
-  // Start of stage s: this wave's loads of tile s have landed (the loads of tile s+1, issued
-  // later, may still be in flight: the counter retires in order), every wave has said so and
-  // has finished reading tile s-1, whose slot then receives tile s+2.
-  auto begin_stage = [&](int s, unsigned char* slot_s2) {
-    const int pending = tile_loads(s + 1);
+  // Start of a stage: this wave's loads of the stage's tile have landed (the `pending` loads of
+  // the next tile, issued later, may still be in flight: the counter retires in order), every
+  // wave has said so and has finished reading the previous tile, whose slot is then free for
+  // the tile after the next.
+  auto begin_stage = [&](int pending) {
     if (pending >= 4) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     else if (pending >= 2) asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    fetch(s + 2, slot_s2);
   };
   static_assert(KJ == 2 || KJ == 4, "tile load counts are waited for as 2 or 4");
   static_assert(VJ == 2 || VJ == 4, "tile load counts are waited for as 2 or 4");
@@ -537,53 +527,81 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   for (int r = 0; r < 16; ++r) zero16[r] = 0.f;
   const auto none = [](int) { return 0.f; };
 
-  // ---- phase 1: selected blocks ----
-  auto key_stage = [&](int s, unsigned char* cur, unsigned char* slot_s2) {
-    begin_stage(s, slot_s2);
-    const int i = s >> 1;
-    if (i < a.NS) {
-      const int nrows = block_rows(i);
-      if (nrows == 64) {
-        const f32x16 st = scores(cur, zero16);
-        softmax(st, pw, [](int) { return true; }, none, no, no);
-      } else if (nrows > 0) {
-        const f32x16 st = scores(cur, zero16);
-        int kb = kbase;
-        asm volatile("" : "+v"(kb));  // (keeps the sixteen sums kb + c out of registers across the loop)
-        softmax(st, pw, [&](int c) { return kb < nrows - c; }, none, yes, no);
-      }
-    }
+  // ---- phase 1: selected blocks, three per iteration (first key row x, row count y of each;
+  // y = 0: no such block, nothing is requested or computed) ----
+  auto block_info = [&](int i) {
+    const int2 v = blk[i];
+    return int2{__builtin_amdgcn_readfirstlane(v.x), __builtin_amdgcn_readfirstlane(v.y)};
   };
-  auto value_stage = [&](int s, unsigned char* cur, unsigned char* slot_s2) {
-    begin_stage(s, slot_s2);
-    const int i = s >> 1;
-    if (i < a.NS && block_rows(i) > 0) values(cur, pw);
+  auto key_compute = [&](const unsigned char* cur, int nrows) {
+    if (nrows == 64) {
+      const f32x16 st = scores(cur, zero16);
+      softmax(st, pw, [](int) { return true; }, none, no, no);
+    } else if (nrows > 0) {
+      const f32x16 st = scores(cur, zero16);
+      int kb = kbase;
+      asm volatile("" : "+v"(kb));  // (keeps the sixteen sums kb + c out of registers across the loop)
+      softmax(st, pw, [&](int c) { return kb < nrows - c; }, none, yes, no);
+    }
   };
   // the query operand has arrived before the first tile is requested: a later wait for it would
   // also wait for every tile load issued in between (the counter retires in order)
 #pragma unroll
   for (int s = 0; s < KS; ++s) asm volatile("" ::"v"(qop[s]));
   __syncthreads();  // the selected blocks' rows are in LDS
-  fetch(0, ring0);
-  fetch(1, ring1);
-  for (int s = 0; s < S1; s += 6) {
-    key_stage(s + 0, ring0, ring2);
-    value_stage(s + 1, ring1, ring0);
-    key_stage(s + 2, ring2, ring1);
-    value_stage(s + 3, ring0, ring2);
-    key_stage(s + 4, ring1, ring0);
-    value_stage(s + 5, ring2, ring1);
+  if (NS3 > 0) {
+    const int2 b0 = block_info(0);
+    if (b0.y) {
+      dma_tile_k(k_rs, ring0, b0.x);
+      dma_tile_v(vt_rs, ring1, Tp, b0.x);
+    }
+  } else {
+    fetch(S1, ring0);
+    fetch(S1 + 1, ring1);
+  }
+  for (int i0 = 0; i0 < NS3; i0 += 3) {
+    const bool last = i0 + 3 == NS3;  // the tiles after this iteration's are phase 2's first two
+    const int2 b0 = block_info(i0), b1 = block_info(i0 + 1), b2 = block_info(i0 + 2), b3 = block_info(i0 + 3);
+    const int k3 = last ? tile_loads(S1) : (b3.y ? KJ : 0);
+    // K of b0 in slot 0
+    begin_stage(b0.y ? VJ : 0);
+    if (b1.y) dma_tile_k(k_rs, ring2, b1.x);
+    key_compute(ring0, b0.y);
+    // V of b0 in slot 1
+    begin_stage(b1.y ? KJ : 0);
+    if (b1.y) dma_tile_v(vt_rs, ring0, Tp, b1.x);
+    if (b0.y) values(ring1, pw);
+    // K of b1 in slot 2
+    begin_stage(b1.y ? VJ : 0);
+    if (b2.y) dma_tile_k(k_rs, ring1, b2.x);
+    key_compute(ring2, b1.y);
+    // V of b1 in slot 0
+    begin_stage(b2.y ? KJ : 0);
+    if (b2.y) dma_tile_v(vt_rs, ring2, Tp, b2.x);
+    if (b1.y) values(ring0, pw);
+    // K of b2 in slot 1
+    begin_stage(b2.y ? VJ : 0);
+    if (last) fetch(S1, ring0);
+    else if (b3.y) dma_tile_k(k_rs, ring0, b3.x);
+    key_compute(ring1, b2.y);
+    // V of b2 in slot 2
+    begin_stage(k3);
+    if (last) fetch(S1 + 1, ring1);
+    else if (b3.y) dma_tile_v(vt_rs, ring1, Tp, b3.x);
+    if (b2.y) values(ring2, pw);
   }
 
   // ---- phase 2: unselected blocks through their means / sums (hi + lo 16-bit pairs) ----
   const int last_len = a.T - (a.NT - 1) * 64;
   f32x16 stw;
   auto mean_hi_stage = [&](int s, unsigned char* cur, unsigned char* slot_s2) {
-    begin_stage(s, slot_s2);
+    begin_stage(tile_loads(s + 1));
+    fetch(s + 2, slot_s2);
     if (((s - S1) >> 2) < NG) stw = scores(cur, zero16);
   };
   auto mean_lo_stage = [&](int s, unsigned char* cur, unsigned char* slot_s2) {
-    begin_stage(s, slot_s2);
+    begin_stage(tile_loads(s + 1));
+    fetch(s + 2, slot_s2);
     const int g = (s - S1) >> 2;
     if (g < NG) {
       const int c0 = g * 64;
@@ -597,7 +615,8 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
     }
   };
   auto sum_stage = [&](int s, unsigned char* cur, unsigned char* slot_s2) {
-    begin_stage(s, slot_s2);
+    begin_stage(tile_loads(s + 1));
+    fetch(s + 2, slot_s2);
     if (((s - S1) >> 2) < NG) values(cur, pw);
   };
   for (int s = S1; s < S1 + 4 * NG; s += 12) {
@@ -1022,7 +1041,7 @@ template <typename T, int K, int V>
 static int launch_attention(const Attn32Args& a, const void* v, int64_t BH, hipStream_t st) {
   using LY = Attn32Layout<K, V>;
   // the tile ring is static; dynamic: the selected-block bitmap and the selected blocks' rows
-  const int lds = ((a.NTp + 15) & ~15) + a.NS * 8;
+  const int lds = ((a.NTp + 15) & ~15) + ((a.NS + 2) / 3 * 3 + 3) * 8;
   if (LY::kTiles + lds > 64 * 1024) {
     set_error("piecewise attention: %d key blocks need more LDS than a workgroup has", a.NT);
     return kErrUnsupported;
