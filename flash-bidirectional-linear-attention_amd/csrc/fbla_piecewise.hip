@@ -233,8 +233,9 @@ template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t w) {
 // k = 8*(l/32)+i; B lane l: n = l%32, same k; C lane l: column l%32, register r is row
 // 8*(r/4) + 4*(l/32) + r%4).
 //   S^T[key][query] = K Q^T      A = K tile row (16 B of one key), B = Q^T in registers
-//   O^T[vcol][query] += V^T P^T  A = V^T tile row (16 B = 8 keys of one value column),
-//                                B = exp2(S^T) packed to 16 bits, straight from the
+//   O^T[vcol][query] += V^T P^T  A = eight keys of one value column, taken out of the
+//                                row-major V tile by the transposing LDS read (two reads of
+//                                four keys), B = exp2(S^T) packed to 16 bits, straight from the
 //                                accumulator registers: k-slot i of k-step t is register
 //                                8t+i, i.e. key 16t + 8*(i/4) + 4*(l/32) + i%4
 //   phase 1  exact softmax attention over the NS selected 64-key blocks
@@ -244,10 +245,21 @@ template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t w) {
 //   o = acc / (l + G)
 // Unlike the Triton kernel (kernel.py:263-276) the running G is rescaled together with
 // acc and l whenever the running maximum grows.
-// Values arrive transposed ([BH, V, Tp], Tp = 64*NT, zero padded) so that a V^T tile row
-// is 128 contiguous bytes; inside every group of 16 keys the LDS copy is stored in the
-// order (4b+j, 8+4b+j) so that the eight keys of a k-slot group are one 16-byte read.
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2t __attribute__((ext_vector_type(2)));
+// Eight keys of one value column (an MFMA operand fragment of one k-step) out of a row-major
+// tile: two transposing reads of gfx950 (in a block of 16 lanes, lane i receives element i%4 of
+// the 8 bytes addressed by lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4); `off0` / `off1` are this lane's
+// byte offsets for the first / second four keys.
+__device__ __forceinline__ u32x4 tr_fragment(const unsigned char* tile, int off0, int off1) {
+  typedef i16x4 __attribute__((address_space(3))) * lds_i16x4;
+  const i16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4)(tile + off0));
+  const i16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4)(tile + off1));
+  const u32x2t wa = __builtin_bit_cast(u32x2t, a), wb = __builtin_bit_cast(u32x2t, b);
+  return u32x4{wa[0], wa[1], wb[0], wb[1]};
+}
 
 template <typename T> struct Mma32;
 template <> struct Mma32<_Float16> {
@@ -265,9 +277,9 @@ template <> struct Mma32<__bf16> {
 
 struct Attn32Args {
   const void *q, *k;             // [BH, T, K]
-  const void* vt;                // [BH, V, Tp] transposed values, zero padded
+  const void* v;                 // [BH, T, V]
   const void *kc_hi, *kc_lo;     // [BH, NTp, K] chunk mean keys, hi + lo
-  const void *vct_hi, *vct_lo;   // [BH, V, NTp] transposed chunk value sums, hi + lo
+  const void *vc_hi, *vc_lo;     // [BH, NTp, V] chunk value sums, hi + lo
   const void* r;                 // [BH, T, V] q H per token
   const int32_t* indices;        // [BH, NT, NS]
   void* o;                       // [BH, T, V]
@@ -277,7 +289,7 @@ struct Attn32Args {
 
 template <int K, int V> struct Attn32Layout {
   static constexpr int kKT = 64 * K * 2;   // K tile: 64 keys x K features
-  static constexpr int kVT = V * 128;      // V^T tile: V value columns x 64 keys
+  static constexpr int kVT = 64 * V * 2;   // V tile: 64 keys x V value columns
   static constexpr int kSlot = kKT > kVT ? kKT : kVT;
   static constexpr int kTiles = 3 * kSlot;  // ring of three tiles; the selected-block bitmap follows
 };
@@ -313,7 +325,6 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   const int n = lane & 31, kg = lane >> 5;
   const int qtok = tq * 64 + 32 * qh + n;  // this lane's query
   const float c2 = a.scale * 1.44269504f;  // scores are kept unscaled; p = exp2(s*c2 - m*c2)
-  const int Tp = a.NT * 64;
 
   const T* qb = (const T*)a.q + bh * a.T * K;
   // buffer descriptor: base, no stride, byte count (loads past it return zeros), raw 32-bit data
@@ -325,11 +336,11 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
                   __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
   };
   const auto k_rs = descriptor((const T*)a.k + bh * a.T * K, (int64_t)a.T * K * 2);
-  const auto vt_rs = descriptor((const T*)a.vt + bh * V * (int64_t)Tp, (int64_t)V * Tp * 2);
+  const auto v_rs = descriptor((const T*)a.v + bh * a.T * V, (int64_t)a.T * V * 2);
   const auto kch_rs = descriptor((const T*)a.kc_hi + bh * a.NTp * K, (int64_t)a.NTp * K * 2);
   const auto kcl_rs = descriptor((const T*)a.kc_lo + bh * a.NTp * K, (int64_t)a.NTp * K * 2);
-  const auto vch_rs = descriptor((const T*)a.vct_hi + bh * V * (int64_t)a.NTp, (int64_t)V * a.NTp * 2);
-  const auto vcl_rs = descriptor((const T*)a.vct_lo + bh * V * (int64_t)a.NTp, (int64_t)V * a.NTp * 2);
+  const auto vch_rs = descriptor((const T*)a.vc_hi + bh * a.NTp * V, (int64_t)a.NTp * V * 2);
+  const auto vcl_rs = descriptor((const T*)a.vc_lo + bh * a.NTp * V, (int64_t)a.NTp * V * 2);
 
   for (int i = tid; i < a.NTp; i += kThreads) sel[i] = 0;
   __syncthreads();
@@ -360,7 +371,12 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   auto swz256 = [](int row, int ch) { return row * 256 + ((ch ^ (row & 15)) << 4); };
   auto swz128 = [](int row, int ch) { return row * 128 + ((ch ^ ((row >> 1) & 7)) << 4); };
   auto kswz = [&](int row, int ch) { return K == 128 ? swz256(row, ch) : swz128(row, ch); };
-  auto vswz = [&](int row, int ch) { return swz128(row, ch); };
+  // V tiles are read four consecutive keys x 64 bytes at a time (transposing reads): the 64-byte
+  // group of a row moves with the two low key bits (256-byte rows) / with key bit 1 (128-byte
+  // rows, whose neighbours already differ in the upper half of the banks)
+  auto vswz = [&](int row, int ch) {
+    return V == 128 ? row * 256 + ((ch ^ ((row & 3) << 2)) << 4) : row * 128 + ((ch ^ (((row >> 1) & 1) << 2)) << 4);
+  };
   auto oswz = [&](int row, int ch) { return V == 128 ? swz256(row, ch) : swz128(row, ch); };
 
   // Tiles go from global memory straight into LDS (buffer load with the LDS destination:
@@ -388,22 +404,30 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
     for (int j = 0; j < KJ; ++j)
       dma16(rs, tile + (4 * KRW * j + KRW * wave) * KROWB, k_lane_off, (row0 + 4 * KRW * j) * KROWB);
   };
-  // V^T tile: V rows of 128 bytes (64 keys, permuted inside groups of 16 in global memory
-  // already); source row stride `ld` elements
-  constexpr int VJ = V / 32;
-  const int vrow_l = 8 * wave + (lane >> 3), vslot = lane & 7;
-  const uint32_t v_lane_chunk = (uint32_t)((vslot ^ ((vrow_l >> 1) & 7)) << 4);
-  auto dma_tile_v = [&](i32x4s rs, unsigned char* tile, int ld, int col0) {
-    const uint32_t lane_off = (uint32_t)(vrow_l * ld * 2) + v_lane_chunk;
+  // V tile: the same with its own row size and swizzle
+  constexpr int VROWB = V * 2, VRW = 1024 / VROWB, VJ = 64 / (4 * VRW);
+  const int vrow_l = VRW * wave + lane / (VROWB / 16), vslot = lane % (VROWB / 16);
+  const uint32_t v_lane_off =
+      (uint32_t)(vrow_l * VROWB + ((vslot ^ (V == 128 ? ((vrow_l & 3) << 2) : (((vrow_l >> 1) & 1) << 2))) << 4));
+  auto dma_tile_v = [&](i32x4s rs, unsigned char* tile, int row0) {
 #pragma unroll
-    for (int j = 0; j < VJ; ++j) dma16(rs, tile + (32 * j + 8 * wave) * 128, lane_off, (col0 + 32 * j * ld) * 2);
+    for (int j = 0; j < VJ; ++j)
+      dma16(rs, tile + (4 * VRW * j + VRW * wave) * VROWB, v_lane_off, (row0 + 4 * VRW * j) * VROWB);
   };
 
   // per-lane LDS offsets of the operand reads
   // (k-step s of the key tile sits at koff0 ^ (s << 5): the swizzle is an XOR of the chunk index)
-  int koff0 = kswz(32 * kh + n, kg), voff[2];
-#pragma unroll
-  for (int t = 0; t < 2; ++t) voff[t] = vswz(n, 2 * (2 * kh + t) + kg);
+  int koff0 = kswz(32 * kh + n, kg);
+  // transposing reads of the V tile: in a block of 16 lanes, lane s addresses key
+  // 32kh + 4kg + s/4 (+ 16t + 8x for k-step t, half x: immediate offsets) and the four value
+  // columns 16(g&1) + 4(s%4) .. +3 of the 32-column block (g = lane/16); block mb of the 32-column
+  // blocks sits at voff0 ^ (mb << 6)
+  int voff0;
+  {
+    const int g16 = lane >> 4, s16 = lane & 15;
+    const int f0 = 16 * (g16 & 1) + 4 * (s16 & 3);
+    voff0 = vswz(32 * kh + 4 * kg + (s16 >> 2), f0 >> 3) + ((f0 >> 2) & 1) * 8;
+  }
 
   const int kbase = 32 * kh + 4 * kg;
   float m_i = kNegInf, l_p = 0.f, g_p = 0.f;  // running max (unscaled); per-lane partial sums
@@ -477,11 +501,14 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
     }
   };
   auto values = [&](const unsigned char* vt, const u32x4(&pw)[2]) {
+    asm volatile("" : "+v"(voff0));  // the offsets of the column blocks are derived here
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int mb = 0; mb < MB; ++mb) {
+      const int off = voff0 ^ (mb << 6);
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-        acc[mb] = Mma32<T>::run(*reinterpret_cast<const u32x4*>(vt + voff[t] + mb * (32 * 128)), pw[t], acc[mb]);
+      for (int t = 0; t < 2; ++t)
+        acc[mb] = Mma32<T>::run(tr_fragment(vt + 16 * t * VROWB, off, off + 8 * VROWB), pw[t], acc[mb]);
+    }
   };
   const std::true_type yes{};
   const std::false_type no{};
@@ -504,8 +531,8 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
       switch (s2 & 3) {
         case 0: dma_tile_k(kch_rs, slot, g * 64); break;
         case 1: dma_tile_k(kcl_rs, slot, g * 64); break;
-        case 2: dma_tile_v(vch_rs, slot, a.NTp, g * 64); break;
-        default: dma_tile_v(vcl_rs, slot, a.NTp, g * 64); break;
+        case 2: dma_tile_v(vch_rs, slot, g * 64); break;
+        default: dma_tile_v(vcl_rs, slot, g * 64); break;
       }
     }
   };
@@ -553,7 +580,7 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
     const int2 b0 = block_info(0);
     if (b0.y) {
       dma_tile_k(k_rs, ring0, b0.x);
-      dma_tile_v(vt_rs, ring1, Tp, b0.x);
+      dma_tile_v(v_rs, ring1, b0.x);
     }
   } else {
     fetch(S1, ring0);
@@ -569,7 +596,7 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
     key_compute(ring0, b0.y);
     // V of b0 in slot 1
     begin_stage(b1.y ? KJ : 0);
-    if (b1.y) dma_tile_v(vt_rs, ring0, Tp, b1.x);
+    if (b1.y) dma_tile_v(v_rs, ring0, b1.x);
     if (b0.y) values(ring1, pw);
     // K of b1 in slot 2
     begin_stage(b1.y ? VJ : 0);
@@ -577,7 +604,7 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
     key_compute(ring2, b1.y);
     // V of b1 in slot 0
     begin_stage(b2.y ? KJ : 0);
-    if (b2.y) dma_tile_v(vt_rs, ring2, Tp, b2.x);
+    if (b2.y) dma_tile_v(v_rs, ring2, b2.x);
     if (b1.y) values(ring0, pw);
     // K of b2 in slot 1
     begin_stage(b2.y ? VJ : 0);
@@ -587,7 +614,7 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
     // V of b2 in slot 2
     begin_stage(k3);
     if (last) fetch(S1 + 1, ring1);
-    else if (b3.y) dma_tile_v(vt_rs, ring1, Tp, b3.x);
+    else if (b3.y) dma_tile_v(v_rs, ring1, b3.x);
     if (b2.y) values(ring2, pw);
   }
 
@@ -707,42 +734,6 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   }
 }
 
-// values [BH, T, V] -> [BH, V, Tp] (Tp = 64 * NT, zero padded): one workgroup per (head,
-// 64-token block), through a padded LDS tile
-template <typename T, int V>
-__global__ __launch_bounds__(kThreads) void transpose_values_kernel(const T* __restrict__ v,
-                                                                   T* __restrict__ vt, int Tn, int NT) {
-  constexpr int LDW = V + 2;  // row stride in elements: odd number of dwords
-  __shared__ T tile[64 * LDW];
-  const int tb = blockIdx.x % NT;
-  const int64_t bh = blockIdx.x / NT;
-  const int nrows = min(64, Tn - tb * 64);
-  const T* src = v + (bh * Tn + (int64_t)tb * 64) * V;
-  for (int qq = threadIdx.x; qq < 64 * (V / 2); qq += kThreads) {
-    const int row = qq / (V / 2), dw = qq % (V / 2);
-    const uint32_t x = row < nrows ? *reinterpret_cast<const uint32_t*>(src + (int64_t)row * V + 2 * dw) : 0u;
-    *reinterpret_cast<uint32_t*>(&tile[row * LDW + 2 * dw]) = x;
-  }
-  __syncthreads();
-  T* dst = vt + bh * V * (int64_t)NT * 64 + (int64_t)tb * 64;
-  for (int qq = threadIdx.x; qq < V * 8; qq += kThreads) {
-    const int col = qq >> 3, ch = qq & 7;
-    // positions 8ch .. 8ch+7 of the row hold keys 16g + 4b + (0..3), 16g + 8 + 4b + (0..3)
-    // (g = ch/2, b = ch%2): the order in which the attention kernel's accumulator registers
-    // hold the keys of a group of 16
-    const int kb0 = 16 * (ch >> 1) + 4 * (ch & 1);
-    uint32_t w[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int key = kb0 + 8 * (i >> 1) + 2 * (i & 1);
-      const uint16_t lo = __builtin_bit_cast(uint16_t, tile[key * LDW + col]);
-      const uint16_t hi = __builtin_bit_cast(uint16_t, tile[(key + 1) * LDW + col]);
-      w[i] = (uint32_t)lo | ((uint32_t)hi << 16);
-    }
-    *reinterpret_cast<u32x4*>(dst + (int64_t)col * NT * 64 + ch * 8) = u32x4{w[0], w[1], w[2], w[3]};
-  }
-}
-
 // kc (fp32 mean) / vc (fp32 sum) -> zero-padded 16-bit hi + lo arrays [BH, NTp, D]
 template <typename T>
 __global__ __launch_bounds__(kThreads) void split_hi_lo_kernel(const float* __restrict__ src,
@@ -755,29 +746,6 @@ __global__ __launch_bounds__(kThreads) void split_hi_lo_kernel(const float* __re
     const int64_t bc = e / D;
     const int c = (int)(bc % NTp);
     const int64_t bh = bc / NTp;
-    float x = 0.f;
-    if (c < NT) x = src[(bh * NT + c) * D + d];
-    const T h = (T)x;
-    hi[e] = h;
-    lo[e] = (T)(x - (float)h);
-  }
-}
-
-// The same, transposed: [BH, NT, D] -> [BH, D, NTp], with the order inside groups of 16 chunks
-// that the attention kernel expects of a V^T tile row
-template <typename T>
-__global__ __launch_bounds__(kThreads) void split_hi_lo_t_kernel(const float* __restrict__ src,
-                                                                 T* __restrict__ hi, T* __restrict__ lo,
-                                                                 int64_t BH, int NT, int NTp, int D) {
-  const int64_t total = BH * D * NTp;
-  for (int64_t e = (int64_t)blockIdx.x * kThreads + threadIdx.x; e < total;
-       e += (int64_t)gridDim.x * kThreads) {
-    const int cpos = (int)(e % NTp);  // position; chunks are permuted inside groups of 16 like keys
-    const int pos = cpos & 15;
-    const int c = (cpos & ~15) + 8 * ((pos >> 2) & 1) + 4 * (pos >> 3) + (pos & 3);
-    const int64_t bd = e / NTp;
-    const int d = (int)(bd % D);
-    const int64_t bh = bd / D;
     float x = 0.f;
     if (c < NT) x = src[(bh * NT + c) * D + d];
     const T h = (T)x;
@@ -1030,15 +998,15 @@ bool attention_supported(int K, int V, int block, int dtype) {
 
 static int64_t padded_chunks(int64_t T) { return cdiv64(cdiv64(T, 64), 64) * 64; }
 
-// kc_hi | kc_lo | vc_hi | vc_lo (transposed) | r | v transposed
+// kc_hi | kc_lo | vc_hi | vc_lo | r
 size_t attention_workspace_bytes(int64_t BH, int64_t T, int K, int V) {
-  const int64_t NTp = padded_chunks(T), Tp = cdiv64(T, 64) * 64;
+  const int64_t NTp = padded_chunks(T);
   return 2 * align_up((size_t)BH * NTp * K * 2, 256) + 2 * align_up((size_t)BH * NTp * V * 2, 256) +
-         align_up((size_t)BH * T * V * 2, 256) + align_up((size_t)BH * V * Tp * 2, 256);
+         align_up((size_t)BH * T * V * 2, 256);
 }
 
 template <typename T, int K, int V>
-static int launch_attention(const Attn32Args& a, const void* v, int64_t BH, hipStream_t st) {
+static int launch_attention(const Attn32Args& a, int64_t BH, hipStream_t st) {
   using LY = Attn32Layout<K, V>;
   // the tile ring is static; dynamic: the selected-block bitmap and the selected blocks' rows
   const int lds = ((a.NTp + 15) & ~15) + ((a.NS + 2) / 3 * 3 + 3) * 8;
@@ -1047,8 +1015,6 @@ static int launch_attention(const Attn32Args& a, const void* v, int64_t BH, hipS
     return kErrUnsupported;
   }
   auto kernel = attention32_kernel<T, K, V>;
-  transpose_values_kernel<T, V><<<dim3((unsigned)(BH * a.NT)), dim3(kThreads), 0, st>>>(
-      (const T*)v, (T*)const_cast<void*>(a.vt), a.T, a.NT);
   kernel<<<dim3((unsigned)(BH * a.NT)), dim3(kThreads), lds, st>>>(a);
   return kOk;
 }
@@ -1058,34 +1024,31 @@ static int attention_t(const void* q, const void* k, const void* v, const float*
                        const float* h, const int32_t* indices, void* o, void* workspace, int64_t BH,
                        int64_t Tn, int K, int V, int NS, float scale, int dtype, hipStream_t st) {
   const int NT = (int)cdiv64(Tn, 64);
-  const int64_t NTp = padded_chunks(Tn), Tp = (int64_t)NT * 64;
+  const int64_t NTp = padded_chunks(Tn);
   char* ws = (char*)workspace;
   T* kc_hi = (T*)ws;
   ws += align_up((size_t)BH * NTp * K * 2, 256);
   T* kc_lo = (T*)ws;
   ws += align_up((size_t)BH * NTp * K * 2, 256);
-  T* vct_hi = (T*)ws;
+  T* vc_hi = (T*)ws;
   ws += align_up((size_t)BH * NTp * V * 2, 256);
-  T* vct_lo = (T*)ws;
+  T* vc_lo = (T*)ws;
   ws += align_up((size_t)BH * NTp * V * 2, 256);
   T* r = (T*)ws;
-  ws += align_up((size_t)BH * Tn * V * 2, 256);
-  T* vt = (T*)ws;
-  (void)Tp;
   const unsigned gk = (unsigned)std::min<int64_t>(cdiv64(BH * NTp * K, kThreads), 4096);
   const unsigned gv = (unsigned)std::min<int64_t>(cdiv64(BH * NTp * V, kThreads), 4096);
   split_hi_lo_kernel<T><<<dim3(gk), dim3(kThreads), 0, st>>>(kc, kc_hi, kc_lo, BH, NT, (int)NTp, K);
-  split_hi_lo_t_kernel<T><<<dim3(gv), dim3(kThreads), 0, st>>>(vc, vct_hi, vct_lo, BH, NT, (int)NTp, V);
+  split_hi_lo_kernel<T><<<dim3(gv), dim3(kThreads), 0, st>>>(vc, vc_hi, vc_lo, BH, NT, (int)NTp, V);
   // r_t = q_t H: the row-parallel kernel with M = H
   const Prob p = dense_prob(BH, Tn, K, V);
   mfma::RowsJob job{q, nullptr, h, V, 1, nullptr, nullptr, r};
   int rc = mfma::rows(p, dtype, job, K, V, st);
   if (rc != kOk) return rc;
-  Attn32Args a{q, k, vt, kc_hi, kc_lo, vct_hi, vct_lo, r, indices, o, (int)Tn, NT, (int)NTp, NS, scale};
-  if (K == 64 && V == 64) return launch_attention<T, 64, 64>(a, v, BH, st);
-  if (K == 64) return launch_attention<T, 64, 128>(a, v, BH, st);
-  if (V == 64) return launch_attention<T, 128, 64>(a, v, BH, st);
-  return launch_attention<T, 128, 128>(a, v, BH, st);
+  Attn32Args a{q, k, v, kc_hi, kc_lo, vc_hi, vc_lo, r, indices, o, (int)Tn, NT, (int)NTp, NS, scale};
+  if (K == 64 && V == 64) return launch_attention<T, 64, 64>(a, BH, st);
+  if (K == 64) return launch_attention<T, 64, 128>(a, BH, st);
+  if (V == 64) return launch_attention<T, 128, 64>(a, BH, st);
+  return launch_attention<T, 128, 128>(a, BH, st);
 }
 
 // ===========================================================================
