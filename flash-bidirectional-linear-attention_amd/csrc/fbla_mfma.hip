@@ -539,13 +539,16 @@ struct State128Layout {
   static constexpr int kTotal = kLpt + (kLptMax + 1) * 4;
 };
 
-template <typename T, bool PAD>
+// STATS = true additionally writes the mean key and the value sum of every 64-token block (a
+// step of this kernel), like state_kernel's STATS.
+template <typename T, bool PAD, bool STATS = false>
 __global__ __launch_bounds__(kThreads, 2) void state128_kernel(Prob p, const T* __restrict__ kn,
                                                                const T* __restrict__ v,
                                                                float* __restrict__ partial,
                                                                float* __restrict__ fin_mat,
                                                                float* __restrict__ fin_vec, int chunk,
-                                                               int nchunks) {
+                                                               int nchunks, BlockStats stats) {
+  static_assert(!STATS || !PAD, "block statistics: full head dims only");
   using LY = State128Layout;
   constexpr int ROWB = 256;
   const int dk = PAD ? p.DK : 128, dv = PAD ? p.DV : 128;  // row lengths in memory
@@ -640,6 +643,7 @@ __global__ __launch_bounds__(kThreads, 2) void state128_kernel(Prob p, const T* 
     load_step(rk, kn, base + 64, dk, krow_b, kvoff, k_piece);
     load_step(rv, v, base + 64, dv, vrow_b, vvoff, v_piece);
     __syncthreads();  // the step is in LDS; every wave is done with the other buffer's previous step
+    float kstep = 0.f, vstep = 0.f;  // this step's sums (STATS: the step is a block of the statistics)
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -658,8 +662,24 @@ __global__ __launch_bounds__(kThreads, 2) void state128_kernel(Prob p, const T* 
         // sum_t k_t for the rows of A[bv] (the two waves of a key half share its 64 rows)
         const u32x4 Ak = bv ? A[1] : A[0];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ks = Ops<T>::dot2(Ak[i], Ops<T>::kOnes, ks);
+        for (int i = 0; i < 4; ++i) kstep = Ops<T>::dot2(Ak[i], Ops<T>::kOnes, kstep);
+        if constexpr (STATS) {  // likewise sum_t v_t for the columns of B[bk]
+          const u32x4 Bv = bk ? B[1] : B[0];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) vstep = Ops<T>::dot2(Bv[i], Ops<T>::kOnes, vstep);
+        }
       }
+    ks += kstep;
+    if constexpr (STATS) {
+      const int cb = base >> 6;
+      const float inv_n = 1.0f / (float)min(64, len - 64 * cb);
+      const int64_t slot = ((int64_t)nh * stats.NT + cb) * 128;
+      const float totk = kstep + __shfl_xor(kstep, 32), totv = vstep + __shfl_xor(vstep, 32);
+      if (kb == 0) {
+        stats.kc[slot + 64 * bk + 32 * bv + ntok] = totk * inv_n;
+        stats.vc[slot + 64 * bv + 32 * bk + ntok] = totv;
+      }
+    }
     buf ^= 1;
   }
 
@@ -2241,7 +2261,7 @@ static int whole_state_chunk(const Prob& p) {
 
 int state_chunk(const Prob& p, bool block_stats) {
   static const int per_cu = knob("FBLA_STATE_WGS_PER_CU", 2);
-  const int whole = block_stats ? 0 : whole_state_chunk(p);
+  const int whole = block_stats && padded(p) ? 0 : whole_state_chunk(p);
   return whole ? whole : chunk_for(p, per_cu, 1, 256, 64, true);
 }
 
@@ -2302,11 +2322,19 @@ static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, fl
   // few long sequences finish 9 % sooner)
   constexpr int TL = (DK == 128 && DV == 128) ? 2 : 1;
   if constexpr (DK == 128 && DV == 128) {
-    if (!bs.kc && !tokscal && whole_state_chunk(p) == chunk) {
-      auto kernel = state128_kernel<T, PAD>;
-      static thread_local bool configured = false;  // per instantiation
-      if (reserve_lds(kernel, State128Layout::kTotal, configured) != kOk) return;
-      kernel<<<grid, block, State128Layout::kTotal, st>>>(p, kn, v, partial, fm, fv, chunk, nchunks);
+    if (!tokscal && whole_state_chunk(p) == chunk && !(bs.kc && PAD)) {
+      static thread_local bool configured[2] = {false, false};  // per instantiation
+      if (bs.kc) {
+        if constexpr (!PAD) {
+          auto kernel = state128_kernel<T, false, true>;
+          if (reserve_lds(kernel, State128Layout::kTotal, configured[1]) != kOk) return;
+          kernel<<<grid, block, State128Layout::kTotal, st>>>(p, kn, v, partial, fm, fv, chunk, nchunks, bs);
+        }
+      } else {
+        auto kernel = state128_kernel<T, PAD>;
+        if (reserve_lds(kernel, State128Layout::kTotal, configured[0]) != kOk) return;
+        kernel<<<grid, block, State128Layout::kTotal, st>>>(p, kn, v, partial, fm, fv, chunk, nchunks, bs);
+      }
       return;
     }
   }

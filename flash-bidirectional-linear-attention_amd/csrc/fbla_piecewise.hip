@@ -75,16 +75,19 @@ __global__ __launch_bounds__(kThreads) void chunk_sums16_kernel(
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-  for (int base = 0; base < n; base += 4 * RPI) {
-    u32x4s w[4];
+  // 64 rows per trip (a whole chunk of the usual size): every load of the chunk is in flight
+  // before the first sum, the wave waits for memory once
+  constexpr int NLD = 64 / RPI;
+  for (int base = 0; base < n; base += 64) {
+    u32x4s w[NLD];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < NLD; ++u) {
       const int row = base + u * RPI + r0;
       w[u] = row < n ? *reinterpret_cast<const u32x4s*>(src + (int64_t)row * D + ch * 8)
                      : u32x4s{0u, 0u, 0u, 0u};
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+    for (int u = 0; u < NLD; ++u)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         acc[2 * i] += (float)__builtin_bit_cast(T, (uint16_t)(w[u][i] & 0xffffu));
