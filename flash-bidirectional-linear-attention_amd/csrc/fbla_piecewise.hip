@@ -463,7 +463,12 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
       if constexpr (masked) st[r] = valid(8 * (r >> 2) + (r & 3)) ? st[r] : kNegInf;
       mx = fmaxf(mx, st[r]);
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    {  // maximum with the other half-wave's lane of the same query: one swap of the 32-lane halves
+      typedef unsigned u32x2v __attribute__((ext_vector_type(2)));
+      const unsigned bits = __builtin_bit_cast(unsigned, mx);
+      const u32x2v sw = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+      mx = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+    }
     // The reference point of the exponents follows the running maximum lazily: it moves only
     // when the maximum has grown by more than kLazy binary orders, so p stays below 2^kLazy
     // (exact in fp32 sums, in range for a 16-bit operand) and the accumulators are rescaled a
