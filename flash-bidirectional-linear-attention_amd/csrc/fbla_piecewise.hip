@@ -510,13 +510,29 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   };
   auto values = [&](const unsigned char* vt, const u32x4(&pw)[2]) {
     asm volatile("" : "+v"(voff0));  // the offsets of the column blocks are derived here
+    // every fragment is requested before the first product (the score accumulators are dead
+    // here, so the registers are there): one LDS latency per stage instead of one per column block
+    u32x4 av[MB][2];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       const int off = voff0 ^ (mb << 6);
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
-        acc[mb] = Mma32<T>::run(tr_fragment(vt + 16 * t * VROWB, off, off + 8 * VROWB), pw[t], acc[mb]);
+      for (int t = 0; t < 2; ++t) av[mb][t] = tr_fragment(vt + 16 * t * VROWB, off, off + 8 * VROWB);
     }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) acc[mb] = Mma32<T>::run(av[mb][t], pw[t], acc[mb]);
+    // (scheduling groups: the reads of two column blocks, then products and the reads of the next
+    // column block in turn, so that eight reads are in flight ahead of the matrix instructions;
+    // the scheduler would otherwise read one column block, wait, multiply, read the next)
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+    for (int mb = 2; mb < MB; ++mb) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
   };
   const std::true_type yes{};
   const std::false_type no{};
