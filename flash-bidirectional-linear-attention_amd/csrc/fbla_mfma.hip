@@ -125,6 +125,17 @@ template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{a, b}, tx2_t));
 }
 
+// x of this lane + x of the lane 32 away (the other half-wave): one swap of the 32-lane halves in
+// the vector unit instead of a permute through LDS and a wait for it
+// (written as assembly: the second result of the compiler's builtin for this instruction comes
+// back equal to the first in this toolchain; the two wait states cover a vector write of the
+// operands just before)
+__device__ __forceinline__ float sum_halves(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return a + b;  // lanes 0-31: a own, b the partner's; lanes 32-63 the other way round
+}
+
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 // Eight tokens of one feature (an MFMA operand fragment of one k-step) out of a row-major tile:
 // two transposing reads, `off0` / `off1` are this lane's byte offsets for x = 0 / 1.
@@ -1128,7 +1139,7 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
     float rs = denorm;
     if constexpr (NORM) {
       if constexpr (kDenFlat) z = zrow[ntok];  // written before the wave_sync above
-      else if constexpr (!PAIR) z += __shfl_xor(z, 32);  // pair mode: each half row has its own z
+      else if constexpr (!PAIR) z = sum_halves(z);  // pair mode: each half row has its own z
       rs = denorm / (z + p.eps);
     }
     wave_sync();  // all lanes have read their x chunks; staging is reused for out
@@ -1684,8 +1695,8 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
         }
       }
       if constexpr (!PAIR) {  // pair mode: each half row is a token of its own
-        P += __shfl_xor(P, 32);
-        z += __shfl_xor(z, 32);
+        P = sum_halves(P);
+        z = sum_halves(z);
       }
       if constexpr (kDenFlat) z = dzs[ntok];  // from the flat registers, before the wave_sync above
       if (PAIR ? (t0 + ntok < t_end && 2 * (t0 + ntok) + kb < len) : (t0 + ntok < t_end)) {
@@ -2029,8 +2040,8 @@ __global__ __launch_bounds__(256, 2) void bwd_a128_kernel(
             z = Ops<T>::dot2(qw[i], kl[i], z);
           }
         }
-        P += __shfl_xor(P, 32);
-        z += __shfl_xor(z, 32);
+        P = sum_halves(P);
+        z = sum_halves(z);
         if (kb == 0) *reinterpret_cast<float2*>(&pz[2 * ((4 * t + blk) * 32 + ntok)]) = float2{P, z};
       }
       __syncthreads();

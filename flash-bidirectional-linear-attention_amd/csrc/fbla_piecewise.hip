@@ -464,10 +464,11 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
       mx = fmaxf(mx, st[r]);
     }
     {  // maximum with the other half-wave's lane of the same query: one swap of the 32-lane halves
-      typedef unsigned u32x2v __attribute__((ext_vector_type(2)));
-      const unsigned bits = __builtin_bit_cast(unsigned, mx);
-      const u32x2v sw = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
-      mx = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+       // (assembly: the second result of the compiler's builtin for this instruction comes back
+       // equal to the first in this toolchain; two wait states after the vector write of mx)
+      float own = mx, other = mx;
+      asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(own), "+v"(other));
+      mx = fmaxf(own, other);
     }
     // The reference point of the exponents follows the running maximum lazily: it moves only
     // when the maximum has grown by more than kLazy binary orders, so p stays below 2^kLazy

@@ -122,6 +122,31 @@ def test_piecewise_attention_matches_oracle(dtype, T, K, V, density):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("high", [(0, 1, 2, 3), (4, 5, 6, 7), (12, 13, 14, 15, 28), (33,)])
+def test_row_maximum_sees_every_key_of_a_block(dtype, high):
+    """Scores that differ by more than the exponent range of fp32 between groups of keys: keys
+    whose index inside their block of 64 is in `high` score +112 (natural units), all others
+    -112.  A running maximum that missed a group of keys of a block (one half-wave's keys, one
+    register's key) would overflow exp2 and return inf / nan; with the true maximum the
+    output is softmax attention over the high keys only."""
+    from flash_bla.ops.piecewise_attn.kernel import piecewise_sparse_attention
+    T, K, V = 192, 64, 64
+    g = torch.Generator().manual_seed(11)
+    q = torch.zeros(1, 1, T, K)
+    q[..., 0] = 30.0
+    k = 0.01 * torch.randn(1, 1, T, K, generator=g)
+    k[..., 0] = -30.0
+    for j in high:
+        k[0, 0, j::64, 0] = 30.0
+    v = torch.randn(1, 1, T, V, generator=g)
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    o = piecewise_sparse_attention(q.cuda(), k.cuda(), v.cuda(), density=1.0)
+    assert torch.isfinite(o).all()
+    ref = torch.nn.functional.scaled_dot_product_attention(q.double(), k.double(), v.double())
+    assert_parity(o, ref, dtype, f"high keys {high}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
 def test_all_blocks_selected_is_softmax_attention(dtype):
     from flash_bla.ops.piecewise_attn.kernel import piecewise_sparse_attention
     q, k, v = _inputs(2, 2, 300, 64, 64, dtype, seed=3)
