@@ -453,6 +453,20 @@ def other_configs(dev, flush):
         else:
             f, s = run(simple_la, (q, k, v), do)
             _report(f"simple_la B8-H16-T16384-D64 {tag}", 4 * nb, 11 * nb, f, s, flush)
+    # the blocks' feature map with the attention (inference forward): applied by the kernels as they
+    # load q and k, against one elementwise launch for q and k followed by the operator
+    from flash_bla.ops.feature_map import elu_plus_one
+    g = torch.Generator(device=dev).manual_seed(3)
+    q, k, v = (torch.randn((8, 16, 16384, 64), generator=g, device=dev).half() for _ in range(3))
+    nb = q.numel() * 2
+    with torch.no_grad():
+        t_load = do_bench(lambda: linear_attention(q, k, v, feature_map="elu+1"), flush)
+        t_first = do_bench(lambda: linear_attention(*elu_plus_one(q, k), v), flush)
+    print(json.dumps({"config": "elu+1 feature map + linear_attn fwd B8-H16-T16384-D64 fp16 (inference)",
+                      "mapped_on_load_ms": round(t_load[0], 5), "mapped_on_load_gbps": round(4 * nb / t_load[0] / 1e6, 1),
+                      "mapped_on_load_frac": round(4 * nb / t_load[0] / 1e6 / HBM_PEAK_GBPS, 4),
+                      "mapped_first_ms": round(t_first[0], 5)}), file=sys.stderr, flush=True)
+    del q, k, v
     q, k, v, do = make_inputs(2, 16, 16384, 64, torch.bfloat16, dev)
     qr, kr, _, _ = make_inputs(2, 16, 16384, 64, torch.bfloat16, dev, seed=7)
     leaves(q, k, qr, kr, v)

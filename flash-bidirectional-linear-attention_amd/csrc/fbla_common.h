@@ -16,6 +16,7 @@ enum Flags : int {
   kNormalize = 1,     // divide by z = q.km + eps (linear_attn); off = simple_la
   kDecoupled = 2,     // numerator uses q_rope/k_rope, denominator q/k
   kDefaultScale = 4,  // varlen only: scale = 1/len_i per sequence
+  kElu1 = 8,          // forward only: q and k arrive before the feature map, the kernels apply elu(x) + 1 on load
   kXcdOrder = 256,    // internal (set per launch): packed batches keep a sequence's heads on one XCD
   kInterleave = 512,  // internal (set per launch): the workgroups of a head take interleaved token steps
 };

@@ -136,6 +136,16 @@ __device__ __forceinline__ float sum_halves(float x) {
   return a + b;  // lanes 0-31: a own, b the partner's; lanes 32-63 the other way round
 }
 
+// The callers' feature map phi(x) = elu(x) + 1 on a pair of 16-bit values, with the rounding steps
+// of the torch expression `F.elu(x) + 1.0` on a 16-bit tensor (elu rounded to the type, then the sum
+// rounded again), so that a forward that applies it on load agrees with one fed the mapped tensors.
+template <typename T> __device__ __forceinline__ uint32_t phi_pair(uint32_t w) {
+  const float x0 = Ops<T>::lo(w), x1 = Ops<T>::hi(w);
+  const float e0 = x0 > 0.f ? x0 : __expf(x0) - 1.f, e1 = x1 > 0.f ? x1 : __expf(x1) - 1.f;
+  const uint32_t e = pack2<T>(e0, e1);
+  return pack2<T>(Ops<T>::lo(e) + 1.f, Ops<T>::hi(e) + 1.f);
+}
+
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 // Eight tokens of one feature (an MFMA operand fragment of one k-step) out of a row-major tile:
 // two transposing reads, `off0` / `off1` are this lane's byte offsets for x = 0 / 1.
@@ -247,7 +257,9 @@ struct BlockStats {
   int NT;
 };
 
-template <typename T, int DK, int DV, bool SPLIT_KD, int TILES, bool SCALED, bool STATS = false, bool PAD = false>
+// FMAP = true: the key rows arrive before the feature map and are mapped (phi_pair) as they are used.
+template <typename T, int DK, int DV, bool SPLIT_KD, int TILES, bool SCALED, bool STATS = false, bool PAD = false,
+          bool FMAP = false>
 __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2) void state_kernel(Prob p, const T* __restrict__ kn,
                                                          const T* __restrict__ v,
                                                          const T* __restrict__ kd,
@@ -257,6 +269,7 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
                                                          float* fin_vec, int chunk, int nchunks,
                                                          BlockStats stats) {
   static_assert(!STATS || (TILES == 1 && !SCALED && !SPLIT_KD && !PAD), "block statistics: plain variant only");
+  static_assert(!FMAP || (!SCALED && !SPLIT_KD && !PAD && !STATS), "feature map on load: plain variant only");
   const int dk = PAD ? p.DK : DK, dv = PAD ? p.DV : DV;  // row lengths in memory
   // The state is tiled into 64 x 64 blocks (64 accumulator registers per lane); a block is
   // owned by G waves that take interleaved token tiles.  For a 128 x 128 state the four
@@ -372,6 +385,17 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
     }
   };
   auto compute = [&](Buf& b, int tok, bool checked) {
+    if constexpr (FMAP) {  // before any masking: phi(0) = 1, and rows that do not exist must stay zero
+#pragma unroll
+      for (int u = 0; u < TILES; ++u) {
+        const int rows = checked ? t_end - (tok + 16 * u) : 16;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+          for (int c2 = 0; c2 < CK / 2; ++c2)
+            b.k[u].w[j][c2] = 8 * kb + j < rows ? phi_pair<T>(b.k[u].w[j][c2]) : 0u;
+      }
+    }
     if constexpr (PAD) {
 #pragma unroll
       for (int u = 0; u < TILES; ++u) {
@@ -897,12 +921,14 @@ template <int DR, int DC, bool DEN, int WAVES> struct RowsLayout {
 // its output features both belong to one half of the row, the halves never mix: the kernel
 // streams full 128-byte rows at the cost of multiplying zeros.  `chunk` counts row pairs; an
 // odd length leaves the second half of the last pair out.  No partial sums in the prologue.
+// FMAP = true: the rows of x arrive before the feature map and are mapped (phi_pair) on their way into LDS.
 template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD = false,
-          int PF = (DR == 128 && DC == 128) ? FBLA_ROWS_PF128 : FBLA_ROWS_PF, bool PAIR = false>
+          int PF = (DR == 128 && DC == 128) ? FBLA_ROWS_PF128 : FBLA_ROWS_PF, bool PAIR = false, bool FMAP = false>
 __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64 && !DEN) ? 4 : 1) void rows_kernel(Prob p, RowsJob job0, RowsJob job1,
                                                           int wgs_per_job, int chunk, int nchunks,
                                                           int dr_true, int dc_true) {
   static_assert(!PAIR || (DR == 64 && DC == 64 && !PAD), "pair mode: two 32-wide rows per 64-wide row");
+  static_assert(!FMAP || (!DEN && !PAD && !PAIR), "feature map on load: plain rows only");
   const int dr = PAD ? dr_true : (PAIR ? 32 : DR), dc = PAD ? dc_true : (PAIR ? 32 : DC);
   const int dpk = PAD ? (p.DK <= 64 ? 64 : 128) : p.DK;  // padded length of the km / dkm vector
   using LY = RowsLayout<DR, DC, DEN, WAVES>;
@@ -1059,6 +1085,12 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
   // with the tile PF steps ahead, then the tile is multiplied and stored
   auto tile_step = [&](u32x4(&xcur)[XI], u32x4(&dcur)[XI]) {
     wave_sync();  // previous tile's staging reads are done
+    if constexpr (FMAP) {  // (rows past the end become phi(0) = 1: their outputs are not stored)
+#pragma unroll
+      for (int i = 0; i < XI; ++i)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) xcur[i][w] = phi_pair<T>(xcur[i][w]);
+    }
     stash_tile(xcur, stage);
     if constexpr (DEN && !kDenFlat) stash_tile(dcur, stage_den);
     if constexpr (kDenFlat) {
@@ -2349,7 +2381,10 @@ static void launch_state(const Prob& p, const T* kn, const T* v, const T* kd, fl
       return;
     }
   }
-  if (bs.kc) {
+  if (p.flags & kElu1) {  // (the plan has checked: 64 x 64, plain operator)
+    if constexpr (DK == 64 && DV == 64 && !PAD)
+      state_kernel<T, 64, 64, false, 1, false, false, false, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
+  } else if (bs.kc) {
     if constexpr (!PAD)
       state_kernel<T, DK, DV, false, 1, false, true><<<grid, block, 0, st>>>(p, kn, v, kd, partial, nullptr, 0, fm, fv, chunk, nchunks, bs);
   } else if (tokscal && (p.flags & kDecoupled))  // dkm = sum_t dz_t q_t over the plain q rows (kd)
@@ -2382,12 +2417,12 @@ static void run_state(const Prob& p, const void* kn, const void* v, const void* 
   else run_state_dims<T, false>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
 }
 
-template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD, bool PAIR = false>
+template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD, bool PAIR = false, bool FMAP = false>
 static int launch_rows_k(const Prob& p, const RowsJob& job, const RowsJob* job2, int chunk,
                          int nchunks, int dr, int dc, hipStream_t st) {
   using LY = RowsLayout<DR, DC, DEN, WAVES>;
   constexpr int PF = (DR == 128 && DC == 128) ? FBLA_ROWS_PF128 : FBLA_ROWS_PF;
-  auto kernel = rows_kernel<T, DR, DC, NORM, DEN, WAVES, PAD, PF, PAIR>;
+  auto kernel = rows_kernel<T, DR, DC, NORM, DEN, WAVES, PAD, PF, PAIR, FMAP>;
   static thread_local bool configured = false;
   int rc = reserve_lds(kernel, LY::kTotal, configured);
   if (rc != kOk) return rc;
@@ -2431,6 +2466,12 @@ static int launch_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, i
     if (!den && use_rows128(p)) {
       if (norm) return launch_rows128<T, true, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
       return launch_rows128<T, false, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);
+    }
+  }
+  if constexpr (DR == 64 && DC == 64 && !PAD) {
+    if (p.flags & kElu1) {  // (the plan has checked: plain operator, forward output)
+      if (norm) return launch_rows_k<T, 64, 64, true, false, WAVES, false, false, true>(p, job, job2, chunk, nchunks, dr, dc, st);
+      return launch_rows_k<T, 64, 64, false, false, WAVES, false, false, true>(p, job, job2, chunk, nchunks, dr, dc, st);
     }
   }
   if (!norm) return launch_rows_k<T, DR, DC, false, false, WAVES, PAD>(p, job, job2, chunk, nchunks, dr, dc, st);

@@ -123,6 +123,10 @@ int forward(const Prob& pc_, int dtype, const FwdArgs& a, hipStream_t st) {
   const void* qn = dec ? a.q_rope : a.q;
   const void* kn = dec ? a.k_rope : a.k;
   const bool fast = mfma::supported(p, dtype);
+  if ((p.flags & kElu1) && !(fast && dtype != kF32 && p.DK == 64 && p.DV == 64 && !dec)) {
+    set_error("the feature map on load (FBLA_ELU1_QK) covers fp16 / bf16 heads of 64 x 64, not the decoupled operator");
+    return kErrUnsupported;
+  }
   const int chunk = fwd_chunk(p, dtype);
   const int nchunks = (int)cdiv64(p.L, chunk);
   float* partial = (float*)a.workspace;
@@ -164,6 +168,10 @@ int forward(const Prob& pc_, int dtype, const FwdArgs& a, hipStream_t st) {
 int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
   int rc_cross = check_cross(pc_, dtype);
   if (rc_cross != kOk) return rc_cross;
+  if (pc_.flags & kElu1) {
+    set_error("the feature map on load (FBLA_ELU1_QK) is forward only: map q and k first, then differentiate");
+    return kErrUnsupported;
+  }
   const Prob pc = with_order(pc_, a.workspace, bwd_used_bytes(pc_, dtype), st);
   const bool is_cross = cross(pc);
   const Prob p = query_side(pc);  // pass A, reduce

@@ -15,7 +15,7 @@ _LIB_PATH = os.environ.get("FBLA_LIB_PATH") or os.path.join(
 _lib = None
 
 F16, BF16, F32 = 0, 1, 2
-NORMALIZE, DECOUPLED, DEFAULT_SCALE = 1, 2, 4
+NORMALIZE, DECOUPLED, DEFAULT_SCALE, ELU1_QK = 1, 2, 4, 8
 
 _DTYPES = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
 
@@ -218,7 +218,7 @@ def la_bwd(q, k, v, q_rope, k_rope, do, s, km, scale, eps, flags):
     return dq, dk, dv, dqr, dkr
 
 
-def varlen_fwd(q, k, v, cu_seqlens, max_seqlen, scale, eps):
+def varlen_fwd(q, k, v, cu_seqlens, max_seqlen, scale, eps, extra_flags=0):
     """Packed forward: returns (o, s, km).  Tensors contiguous [T,H,D]."""
     _require_gpu(q, k, v, cu_seqlens)
     q, k, v, cu_seqlens = _aligned(q, k, v, cu_seqlens)
@@ -228,7 +228,7 @@ def varlen_fwd(q, k, v, cu_seqlens, max_seqlen, scale, eps):
     N = cu_seqlens.numel() - 1
     code = dtype_code(q)
     dev = q.device
-    flags = NORMALIZE | (DEFAULT_SCALE if scale is None else 0)
+    flags = NORMALIZE | (DEFAULT_SCALE if scale is None else 0) | extra_flags
     o = torch.empty_like(v)
     s = torch.empty(N, H, DK, DV, dtype=torch.float32, device=dev)
     km = torch.empty(N, H, DK, dtype=torch.float32, device=dev)

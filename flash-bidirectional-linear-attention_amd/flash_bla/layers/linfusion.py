@@ -11,7 +11,6 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from flash_bla.layers._common import check_mode, torch_linear_attention
-from flash_bla.ops.feature_map import elu_plus_one
 from flash_bla.ops.linear_attn.fused import linear_attention
 from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
 
@@ -74,18 +73,20 @@ class GeneralizedLinearAttention(nn.Module):
             # The projections come out token-major, (batch, tokens, heads * dim): that is the
             # packed layout of the variable-length operator with equal lengths, so the head
             # split / merge copies of the reference (linfusion.py:98,102) are not needed at all.
+            # The feature map is the operator's: an inference forward of 64-wide heads applies it
+            # while loading q and k, anything else maps them first (one launch for both).
             b, n, _ = q.shape
-            q, k = elu_plus_one(q, k)
             packed = [t.reshape(b * n, self.heads, -1) for t in (q, k, v)]
-            out = varlen_linear_attention(*packed, _equal_cu_seqlens(b, n, q.device), n, eps=1e-4)
+            out = varlen_linear_attention(*packed, _equal_cu_seqlens(b, n, q.device), n, eps=1e-4,
+                                          feature_map="elu+1")
             return self.to_out[1](self.to_out[0](out.reshape(b, n, -1)))
         q, k, v = (self.head_to_batch_dim(t) for t in (q, k, v))
-        q, k = elu_plus_one(q, k) if fast else (F.elu(q) + 1.0, F.elu(k) + 1.0)
         if fast:
             b = hidden_states.shape[0]
             q4, k4, v4 = (t.view(b, self.heads, *t.shape[1:]) for t in (q, k, v))
-            out = linear_attention(q4, k4, v4, eps=1e-4).flatten(0, 1)
+            out = linear_attention(q4, k4, v4, eps=1e-4, feature_map="elu+1").flatten(0, 1)
         else:
+            q, k = F.elu(q) + 1.0, F.elu(k) + 1.0
             out = torch_linear_attention(q, k, v, eps=1e-4)
         out = self.batch_to_head_dim(out)
         return self.to_out[1](self.to_out[0](out))

@@ -39,3 +39,22 @@ def elu_plus_one(x, y=None):
         raise TypeError(f"elu_plus_one: unsupported dtype {x.dtype}")
     out = EluPlusOneFunction.apply(x, y)
     return out[0] if y is None else out
+
+
+ELU_PLUS_ONE = "elu+1"
+
+
+def check_feature_map(feature_map):
+    """The operators' `feature_map` argument: None or "elu+1"."""
+    if feature_map is not None and feature_map != ELU_PLUS_ONE:
+        raise ValueError(f'feature_map must be None or "{ELU_PLUS_ONE}", got {feature_map!r}')
+    return feature_map is not None
+
+
+def applied_on_load(q, k, v):
+    """True when the forward kernels can apply elu(x) + 1 to q and k as they load them: 16-bit
+    heads of 64 x 64 and nothing to differentiate (the backward needs the mapped tensors, so a
+    call that records a graph maps them first with `elu_plus_one`)."""
+    if q.dtype not in (torch.float16, torch.bfloat16) or q.shape[-1] != 64 or v.shape[-1] != 64:
+        return False
+    return not (torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)))

@@ -13,6 +13,7 @@ import torch
 
 from flash_bla import _hip
 from flash_bla.ops._check import check_dense
+from flash_bla.ops.feature_map import applied_on_load, check_feature_map, elu_plus_one
 from flash_bla.utils import contiguous
 
 
@@ -42,7 +43,8 @@ def linear_attention(
     k: torch.Tensor,
     v: torch.Tensor,
     scale: Optional[float] = None,
-    eps: float = 1e-6
+    eps: float = 1e-6,
+    feature_map: Optional[str] = None,
 ) -> torch.Tensor:
     r"""
     Args:
@@ -52,9 +54,19 @@ def linear_attention(
         scale: factor applied to the key-value state; defaults to `1 / L`
             (linear_attn/fused.py:477-478).
         eps: constant added to the denominator.
+        feature_map: None (the reference's signature: q and k are features already) or "elu+1":
+            q and k are given before the blocks' feature map `elu(x) + 1`
+            (layers/linfusion.py:88-89).  An inference forward of 16-bit heads of 64 x 64 applies
+            it inside the kernels as they load q and k (no mapped copies are written); every
+            other call maps them first with one launch and proceeds as usual.
     Returns the output of shape `(B, H, L, V)` with `v`'s dtype.
     """
     check_dense("linear_attention", q, k, v)
     if scale is None:
         scale = k.shape[-2] ** -1.0
+    if check_feature_map(feature_map):
+        if applied_on_load(q, k, v):
+            return _hip.la_fwd(q.contiguous(), k.contiguous(), v.contiguous(), None, None, scale, eps,
+                               _hip.NORMALIZE | _hip.ELU1_QK)[0]
+        q, k = elu_plus_one(q, k)
     return LinearAttnFunction.apply(q, k, v, scale, eps)

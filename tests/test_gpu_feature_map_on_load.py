@@ -1,0 +1,119 @@
+"""The operators' `feature_map="elu+1"` argument: q and k are given before the blocks' feature map
+(layers/linfusion.py:88-89) and an inference forward of 16-bit heads of 64 x 64 applies it inside
+the kernels as they load them.  Checked against the float64 oracle evaluated on the mapped tensors
+(mapped the way the reference's layers map them: `F.elu(x) + 1.0` in the tensor's type), against
+the path that maps first, through autograd (which must map first), on shapes the kernels do not
+cover (which must map first too), and at the C ABI's edges."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import assert_parity, max_rel_err, np64
+from oracle import closed_form as cf
+
+pytestmark = pytest.mark.gpu
+
+
+def _raw(shape_qk, shape_v, dtype, seed, spread=1.5):
+    g = torch.Generator().manual_seed(seed)
+    q = (spread * torch.randn(shape_qk, generator=g)).to(dtype)
+    k = (spread * torch.randn(shape_qk, generator=g)).to(dtype)
+    v = torch.randn(shape_v, generator=g).to(dtype)
+    return q, k, v
+
+
+def _mapped(x):
+    """The reference layers' expression on a tensor of the inputs' type (computed on the GPU, where
+    torch rounds the elu to the type and then the sum)."""
+    return (F.elu(x.cuda()) + 1.0).cpu()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("B,H,L", [(2, 3, 300), (1, 2, 1000), (1, 5, 10), (2, 2, 17), (1, 1, 64), (1, 16, 4099),
+                                   (8, 16, 2048)])
+def test_dense_forward_maps_on_load(B, H, L, dtype):
+    from flash_bla.ops.feature_map import elu_plus_one
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    q, k, v = _raw((B, H, L, 64), (B, H, L, 64), dtype, seed=L)
+    with torch.no_grad():
+        o = linear_attention(q.cuda(), k.cuda(), v.cuda(), feature_map="elu+1")
+        o_two_steps = linear_attention(*elu_plus_one(q.cuda(), k.cuda()), v.cuda())
+    assert o.dtype == dtype and o.shape == v.shape
+    ref = cf.dense_forward(np64(_mapped(q)), np64(_mapped(k)), np64(v), 1.0 / L)[0]
+    assert_parity(o, ref, dtype, f"mapped on load B{B} H{H} L{L}")
+    # the two paths differ only in the last place of their exp routines
+    assert max_rel_err(o, np64(o_two_steps)) < 2e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_unnormalised_forward_maps_on_load(dtype):
+    """The C ABI's flag without FBLA_NORMALIZE (the simple_la family)."""
+    from flash_bla import _hip
+    B, H, L = 2, 3, 777
+    q, k, v = _raw((B, H, L, 64), (B, H, L, 64), dtype, seed=5)
+    scale = 64 ** -0.5
+    o = _hip.la_fwd(q.cuda(), k.cuda(), v.cuda(), None, None, scale, 1e-6, _hip.ELU1_QK)[0]
+    ref = cf.dense_forward(np64(_mapped(q)), np64(_mapped(k)), np64(v), scale, normalize=False)[0]
+    assert_parity(o, ref, dtype, "simple_la mapped on load")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_packed_forward_maps_on_load(dtype):
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    lens = [5, 300, 1, 64, 1000, 17, 16, 2049]
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32)
+    T, H = int(cu[-1]), 4
+    q, k, v = _raw((T, H, 64), (T, H, 64), dtype, seed=9)
+    with torch.no_grad():
+        o = varlen_linear_attention(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), max(lens), feature_map="elu+1")
+    ref = cf.varlen_forward(np64(_mapped(q)), np64(_mapped(k)), np64(v), cu.numpy())
+    assert_parity(o, ref, dtype, "packed, mapped on load")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_gradients_flow_through_the_feature_map(dtype):
+    """With something to differentiate the operator maps q and k first (one launch) and autograd sees
+    the map: the gradients are those of the composed function."""
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    B, H, L = 1, 2, 500
+    q, k, v = _raw((B, H, L, 64), (B, H, L, 64), dtype, seed=3)
+    g = torch.Generator().manual_seed(4)
+    do = torch.randn(B, H, L, 64, generator=g).to(dtype)
+    leaves = [t.cuda().requires_grad_() for t in (q, k, v)]
+    o = linear_attention(*leaves, feature_map="elu+1")
+    o.backward(do.cuda())
+    fq, fk = np64(_mapped(q)), np64(_mapped(k))
+    ref = cf.dense_backward(fq, fk, np64(v), np64(do), 1.0 / L)
+    assert_parity(o, ref["o"], dtype, "o")
+    # d phi(x)/dx = 1 for x > 0, exp(x) otherwise
+    dphi = lambda x: np.where(np64(x) > 0, 1.0, np.exp(np.minimum(np64(x), 0.0)))
+    assert_parity(leaves[0].grad, ref["dq"] * dphi(q), dtype, "dq")
+    assert_parity(leaves[1].grad, ref["dk"] * dphi(k), dtype, "dk")
+    assert_parity(leaves[2].grad, ref["dv"], dtype, "dv")
+
+
+@pytest.mark.parametrize("D,dtype", [(32, torch.float16), (128, torch.bfloat16), (64, torch.float32), (48, torch.float16)])
+def test_other_shapes_map_first(D, dtype):
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    B, H, L = 2, 2, 333
+    q, k, v = _raw((B, H, L, D), (B, H, L, D), dtype, seed=D)
+    with torch.no_grad():
+        o = linear_attention(q.cuda(), k.cuda(), v.cuda(), feature_map="elu+1")
+    ref = cf.dense_forward(np64(_mapped(q)), np64(_mapped(k)), np64(v), 1.0 / L)[0]
+    assert_parity(o, ref, dtype, f"D{D}")
+
+
+def test_argument_and_flag_errors():
+    from flash_bla import _hip
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    q, k, v = (t.cuda() for t in _raw((1, 1, 64, 64), (1, 1, 64, 64), torch.float16, seed=1))
+    with pytest.raises(ValueError):
+        linear_attention(q, k, v, feature_map="relu")
+    # the C ABI refuses the flag where the kernels do not implement it
+    q32, k32, v32 = (t.cuda() for t in _raw((1, 1, 64, 32), (1, 1, 64, 32), torch.float16, seed=2))
+    with pytest.raises(ValueError, match="feature map on load"):
+        _hip.la_fwd(q32, k32, v32, None, None, 1.0, 1e-6, _hip.NORMALIZE | _hip.ELU1_QK)
+    o, s, km = _hip.la_fwd(q, k, v, None, None, 1.0, 1e-6, _hip.NORMALIZE)
+    with pytest.raises(ValueError, match="forward only"):
+        _hip.la_bwd(q, k, v, None, None, torch.ones_like(v), s, km, 1.0, 1e-6, _hip.NORMALIZE | _hip.ELU1_QK)
