@@ -47,6 +47,18 @@ def test_dense_forward_maps_on_load(B, H, L, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("lq,lk", [(300, 75), (64, 1000)])
+def test_fewer_or_more_keys_than_queries(lq, lk, dtype):
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    q, _, _ = _raw((2, 3, lq, 64), (2, 3, lq, 64), dtype, seed=lq)
+    _, k, v = _raw((2, 3, lk, 64), (2, 3, lk, 64), dtype, seed=lk)
+    with torch.no_grad():
+        o = linear_attention(q.cuda(), k.cuda(), v.cuda(), feature_map="elu+1")
+    ref = cf.dense_forward(np64(_mapped(q)), np64(_mapped(k)), np64(v), 1.0 / lk)[0]
+    assert_parity(o, ref, dtype, f"Lq{lq} Lk{lk}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
 def test_unnormalised_forward_maps_on_load(dtype):
     """The C ABI's flag without FBLA_NORMALIZE (the simple_la family)."""
     from flash_bla import _hip
