@@ -75,10 +75,10 @@ __global__ __launch_bounds__(kThreads) void chunk_sums16_kernel(
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-  // 64 rows per trip (a whole chunk of the usual size): every load of the chunk is in flight
-  // before the first sum, the wave waits for memory once
-  constexpr int NLD = 64 / RPI;
-  for (int base = 0; base < n; base += 64) {
+  // 32 rows per trip: half a chunk of the usual size is in flight before the first sum (a whole
+  // one costs so many registers that the waves of config 5 no longer fit the GPU at once)
+  constexpr int NLD = 32 / RPI;
+  for (int base = 0; base < n; base += 32) {
     u32x4s w[NLD];
 #pragma unroll
     for (int u = 0; u < NLD; ++u) {
