@@ -219,6 +219,31 @@ def test_block_selection_ties_go_to_lower_index():
     assert (idx.cpu() == torch.tensor([0, 1, 2, 3, 10], dtype=torch.int32)).all()
 
 
+@pytest.mark.parametrize("K,V", [(128, 128), (64, 64), (64, 128)])
+def test_selection_lengths_around_the_unrolled_stream(K, V):
+    """The kernel walks the selected blocks three at a time: every list length from 1 to 8, with the
+    ragged last block inside or outside the list, and lists padded with -1 (no block) in the middle
+    and at the end give the result of the unpadded list."""
+    from flash_bla.ops.piecewise_attn.kernel import piecewise_sparse_attention
+    T, dtype = 9 * 64 + 20, torch.bfloat16
+    NT = (T + 63) // 64
+    q, k, v = _inputs(1, 1, T, K, V, dtype, seed=77)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    rng = np.random.default_rng(5)
+    for ns in range(1, 9):
+        lists = [rng.permutation(NT)[:ns] for _ in range(NT)]
+        first = np.concatenate([[NT - 1], [b for b in rng.permutation(NT - 1)][:ns - 1]])
+        lists[0] = first.astype(lists[1].dtype)  # the ragged block first in one list (no duplicates)
+        indices = torch.tensor(np.stack(lists), dtype=torch.int32)[None, None].cuda()
+        o = piecewise_sparse_attention(qd, kd, vd, indices=indices)
+        assert_parity(o, _oracle(q, k, v, indices), dtype, f"{ns} blocks", _oracle(q, k, v.abs(), indices))
+        padded = torch.full((1, 1, NT, min(ns + 3, NT)), -1, dtype=torch.int32)  # (at most NT entries)
+        padded[..., 0] = indices[..., 0].cpu()
+        padded[..., 2:ns + 1] = indices[..., 1:].cpu()  # a hole at position 1, the rest at the end
+        o_padded = piecewise_sparse_attention(qd, kd, vd, indices=padded.cuda())
+        assert torch.equal(o, o_padded), f"{ns} blocks, padded list"
+
+
 @pytest.mark.parametrize("seed", range(3))
 def test_random_piecewise_cases(seed):
     """Seeded random lengths (ragged last blocks, one block, many blocks), head dims, densities
