@@ -75,6 +75,7 @@ static Prob make_prob(const int32_t* cu, int64_t N, int64_t H, int64_t L, int64_
   Prob p;
   p.cu = cu;
   p.perm = nullptr;
+  p.chunk_base = nullptr;
   p.N = (int)N;
   p.H = (int)H;
   p.L = (int)L;

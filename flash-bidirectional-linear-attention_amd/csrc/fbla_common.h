@@ -34,6 +34,9 @@ constexpr int kRankMax = 1 << 16;
 struct Prob {
   const int32_t* cu;
   const int32_t* perm;  // packed: perm[r] = index of the sequence with the r-th largest length, or null
+  const int32_t* chunk_base;  // packed, skewed batches: chunk_base[n] = number of reduction chunks of the
+                              // sequences before n (one partial per chunk that exists), or null: every
+                              // (sequence, head) has room for the chunks of the longest sequence
   int N, H, L;  // L: dense length, or max_seqlen upper bound when packed
   int Lk;       // dense only: number of key / value tokens when it differs from L (the number of
                 // queries), else 0.  Only the plan looks at it: kernels get a problem whose L is
@@ -44,6 +47,15 @@ struct Prob {
   float eps;
   int flags;
 };
+
+// The reduction kernels (forward state, backward pass A) write one partial per chunk of a
+// (sequence, head); their consumers add them up in chunk order.  Slot of the partial of chunk c
+// (of nchunks provided for) of (sequence n, head h), and the distance in slots between the
+// partials of consecutive chunks.
+__device__ __forceinline__ int64_t partial_slot(const Prob& p, int n, int h, int c, int nchunks) {
+  return p.chunk_base ? ((int64_t)p.chunk_base[n] + c) * p.H + h : ((int64_t)n * p.H + h) * nchunks + c;
+}
+__device__ __forceinline__ int64_t partial_step(const Prob& p) { return p.chunk_base ? p.H : 1; }
 
 // Token range of sequence n.
 __device__ __forceinline__ void seq_range(const Prob& p, int n, int64_t& bos, int& len) {

@@ -151,16 +151,17 @@ __global__ __launch_bounds__(kThreads) void state_reduce_kernel(
   const int e = blk * kThreads + threadIdx.x;
   if (e >= stride) return;
   const int nvalid = len > 0 ? min(nchunks, (len + chunk - 1) / chunk) : 0;
-  const float* src = partial + (int64_t)nh * nchunks * stride + e;
+  const float* src = partial + partial_slot(p, n, nh - n * p.H, 0, nchunks) * stride + e;
+  const int64_t cstride = (int64_t)stride * partial_step(p);  // between consecutive chunks
   // fixed order: chunk 0, 1, 2, ... (four independent loads in flight at a time)
   float a = 0.f;
   int c = 0;
   for (; c + 4 <= nvalid; c += 4) {
-    const float x0 = src[(int64_t)c * stride], x1 = src[(int64_t)(c + 1) * stride];
-    const float x2 = src[(int64_t)(c + 2) * stride], x3 = src[(int64_t)(c + 3) * stride];
+    const float x0 = src[c * cstride], x1 = src[(c + 1) * cstride];
+    const float x2 = src[(c + 2) * cstride], x3 = src[(c + 3) * cstride];
     a = (((a + x0) + x1) + x2) + x3;
   }
-  for (; c < nvalid; ++c) a += src[(int64_t)c * stride];
+  for (; c < nvalid; ++c) a += src[c * cstride];
   if (e < E) {
     a *= seq_scale(p, len);
     mat[(int64_t)nh * E + e] = a;
@@ -577,6 +578,35 @@ __global__ __launch_bounds__(256) void rank_sequences_kernel(const int32_t* __re
     __syncthreads();
   }
   if (j < N) perm[r] = j;
+}
+
+// base[n] = number of chunks of `chunk` tokens of the sequences before n, base[N] = all of them.
+// One workgroup walks the sequences 256 at a time with a running total.
+__global__ __launch_bounds__(256) void chunk_bases_kernel(const int32_t* __restrict__ cu, int N, int chunk,
+                                                         int32_t* __restrict__ base) {
+  __shared__ int scan[256];
+  int total = 0;
+  for (int first = 0; first < N; first += 256) {
+    const int j = first + threadIdx.x;
+    const int len = j < N ? cu[j + 1] - cu[j] : 0;
+    const int cnt = len > 0 ? (len + chunk - 1) / chunk : 0;
+    scan[threadIdx.x] = cnt;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {  // inclusive scan
+      const int add = threadIdx.x >= off ? scan[threadIdx.x - off] : 0;
+      __syncthreads();
+      scan[threadIdx.x] += add;
+      __syncthreads();
+    }
+    if (j < N) base[j] = total + scan[threadIdx.x] - cnt;
+    total += scan[255];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) base[N] = total;
+}
+
+void chunk_bases(const Prob& p, int chunk, int32_t* base, hipStream_t st) {
+  chunk_bases_kernel<<<dim3(1), dim3(256), 0, st>>>(p.cu, p.N, chunk, base);
 }
 
 void rank_sequences(const Prob& p, int32_t* perm, hipStream_t st) {

@@ -65,6 +65,8 @@ void bwd_b(const Prob& p, int dtype, const void* kn, const void* v, const float*
 void broadcast_rows(const Prob& p, int dtype, const float* vec, void* out, hipStream_t st, float factor = 1.f);
 // perm[r] = index of the sequence with the r-th largest length (ties by index)
 void rank_sequences(const Prob& p, int32_t* perm, hipStream_t st);
+// base[0..N]: exclusive prefix sums of the sequences' numbers of chunks of `chunk` tokens
+void chunk_bases(const Prob& p, int chunk, int32_t* base, hipStream_t st);
 }  // namespace generic
 
 // MFMA kernels for 16-bit inputs (fbla_mfma.hip).

@@ -543,7 +543,7 @@ __global__ __launch_bounds__(kThreads, (DK == 64 && DV == 64 && !SCALED) ? 3 : 2
   // one chunk per (sequence, head): the sum is final, store it scaled where the reduce
   // kernel would have put it; otherwise store this chunk's partial
   float* mat = fin_mat ? fin_mat + (int64_t)nh * dk * dv
-                       : partial + ((int64_t)nh * nchunks + c) * (dk * dv + dk);
+                       : partial + partial_slot(p, n, h, c, nchunks) * (dk * dv + dk);
   float* vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : mat + dk * dv;
   const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
   const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
@@ -721,7 +721,7 @@ __global__ __launch_bounds__(kThreads, 2) void state128_kernel(Prob p, const T* 
   // one chunk per (sequence, head): the sum is final and is stored scaled where the reduce
   // kernel would have put it; otherwise this chunk's partial is stored
   float* mat = fin_mat ? fin_mat + (int64_t)nh * dk * dv
-                       : partial + ((int64_t)nh * nchunks + c) * (dk * dv + dk);
+                       : partial + partial_slot(p, n, h, c, nchunks) * (dk * dv + dk);
   float* vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : mat + dk * dv;
   const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
   const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
@@ -1055,9 +1055,10 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
     const int E = dr * dc;
     const int64_t pstride = E + p.DK;
     const int nsum = min(job.pnchunks, (len + job.pchunk - 1) / job.pchunk);
-    const float* part = job.mat + (int64_t)nh * job.pnchunks * pstride;
+    const float* part = job.mat + partial_slot(p, n, h, 0, job.pnchunks) * pstride;
+    const int64_t sstride = pstride * partial_step(p);  // between the partials of consecutive chunks
     const bool writer = c == 0;
-    denorm = build_operand<T, DR, DC, NT, PAD>(lds_opnd, lds_max, part, job.ld_r, job.ld_c, nsum, pstride,
+    denorm = build_operand<T, DR, DC, NT, PAD>(lds_opnd, lds_max, part, job.ld_r, job.ld_c, nsum, sstride,
                                                seq_scale(p, len),
                                                writer && job.mat_out ? job.mat_out + (int64_t)nh * E : nullptr,
                                                dr, dc);
@@ -1065,7 +1066,7 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
     float* vout = writer && job.vec_out ? job.vec_out + (int64_t)nh * p.DK : nullptr;
     if (NORM || job.vec_is_add || vout)
       build_vec<T, NT>(NORM ? lds_km : nullptr, job.vec_is_add ? lds_add : nullptr, part + E, p.DK,
-                       nsum, pstride, inv_len, vout, dpk);
+                       nsum, sstride, inv_len, vout, dpk);
     if (!job.vec_is_add)
       for (int e = tid; e < DC; e += NT) lds_add[e] = 0.f;
   } else {
@@ -1331,16 +1332,17 @@ __global__ __launch_bounds__(kThreads, 2) void rows128_kernel(Prob p, RowsJob jo
     const int E = dr * dc;
     const int64_t pstride = E + p.DK;
     const int nsum = min(job.pnchunks, (len + job.pchunk - 1) / job.pchunk);
-    const float* part = job.mat + (int64_t)nh * job.pnchunks * pstride;
+    const float* part = job.mat + partial_slot(p, n, h, 0, job.pnchunks) * pstride;
+    const int64_t sstride = pstride * partial_step(p);  // between the partials of consecutive chunks
     const bool writer = c == 0;
-    denorm = build_operand<T, 128, 128, NT, PAD>(smem, lds_max, part, job.ld_r, job.ld_c, nsum, pstride,
+    denorm = build_operand<T, 128, 128, NT, PAD>(smem, lds_max, part, job.ld_r, job.ld_c, nsum, sstride,
                                                  seq_scale(p, len),
                                                  writer && job.mat_out ? job.mat_out + (int64_t)nh * E : nullptr, dr,
                                                  dc);
     const float inv_len = 1.0f / (float)len;
     float* vout = writer && job.vec_out ? job.vec_out + (int64_t)nh * p.DK : nullptr;
     if (NORM || job.vec_is_add || vout)
-      build_vec<T, NT>(NORM ? lds_km : nullptr, job.vec_is_add ? lds_add : nullptr, part + E, p.DK, nsum, pstride,
+      build_vec<T, NT>(NORM ? lds_km : nullptr, job.vec_is_add ? lds_add : nullptr, part + E, p.DK, nsum, sstride,
                        inv_len, vout, dpk);
     if (!job.vec_is_add)
       for (int e = tid; e < 128; e += NT) lds_add[e] = 0.f;
@@ -1867,7 +1869,7 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
     __syncthreads();  // every wave is done with its tiles: reuse them for the reduction
     float* red = reinterpret_cast<float*>(smem + LY::kOpnd);
     float* dst = fin_mat ? fin_mat + (int64_t)nh * dk * dv
-                         : partial + ((int64_t)nh * nchunks + c) * (dk * dv + dk);
+                         : partial + partial_slot(p, n, h, c, nchunks) * (dk * dv + dk);
     float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : dst + dk * dv;
     const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
     const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
@@ -2193,7 +2195,7 @@ __global__ __launch_bounds__(256, 2) void bwd_a128_kernel(
 
   {
     float* dst = fin_mat ? fin_mat + (int64_t)nh * dk * dv
-                         : partial + ((int64_t)nh * nchunks + c) * (dk * dv + dk);
+                         : partial + partial_slot(p, n, h, c, nchunks) * (dk * dv + dk);
     float* dst_vec = fin_mat ? (fin_vec ? fin_vec + (int64_t)nh * dk : nullptr) : dst + dk * dv;
     const float mscale = fin_mat ? seq_scale(p, len) : 1.f;
     const float vscale = fin_mat ? 1.0f / (float)len : 1.f;
@@ -2580,8 +2582,15 @@ void scaled_state(const Prob& p, int dtype, const void* qn, const void* qd, cons
     run_state<__bf16>(p, qn, dout, qd, partial, tokscal, total_rows, fin_mat, fin_vec, chunk, nchunks, none, st);
 }
 
+// (not for batches whose longest sequence is split into many chunks: all of them on one XCD would
+// leave the other seven to the short sequences - one sequence of 65536 tokens among 63 of 256,
+// H16-D64: forward output 286 -> 70 us, pass B 552 -> 120 us)
+static bool xcd_order_rows(const Prob& p, int DR, int DC) {
+  return small_tiles(DR, DC) && cdiv64(p.L, rows_chunk(p, DR, DC)) <= 4;
+}
+
 int rows(const Prob& p_, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st) {
-  const Prob p = small_tiles(DR, DC) ? xcd_ordered(p_, 2) : p_;
+  const Prob p = xcd_order_rows(p_, DR, DC) ? xcd_ordered(p_, 2) : p_;
   if (dtype == kF32) return mfma32::rows(p, job, nullptr, DR, DC, st);
   if (dtype == kF16) return run_rows<_Float16>(p, job, nullptr, DR, DC, st);
   return run_rows<__bf16>(p, job, nullptr, DR, DC, st);
@@ -2590,7 +2599,7 @@ int rows(const Prob& p_, int dtype, const RowsJob& job, int DR, int DC, hipStrea
 // two jobs of the same shape and normalisation mode in one launch
 int rows2(const Prob& p_, int dtype, const RowsJob& job0, const RowsJob& job1, int DR, int DC,
           hipStream_t st) {
-  const Prob p = small_tiles(DR, DC) ? xcd_ordered(p_, 2) : p_;
+  const Prob p = xcd_order_rows(p_, DR, DC) ? xcd_ordered(p_, 2) : p_;
   if (dtype == kF32) return mfma32::rows(p, job0, &job1, DR, DC, st);
   if (dtype == kF16) return run_rows<_Float16>(p, job0, &job1, DR, DC, st);
   return run_rows<__bf16>(p, job0, &job1, DR, DC, st);

@@ -942,6 +942,7 @@ static Prob dense_prob(int64_t BH, int64_t T, int K, int V) {
   Prob p;
   p.cu = nullptr;
   p.perm = nullptr;
+  p.chunk_base = nullptr;
   p.N = (int)BH;
   p.H = 1;
   p.L = (int)T;

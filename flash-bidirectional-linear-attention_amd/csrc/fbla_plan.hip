@@ -43,9 +43,35 @@ static size_t state_bytes(const Prob& p) {
 static size_t vec_bytes(const Prob& p) {
   return align_up((size_t)p.N * p.H * p.DK * sizeof(float), 256);
 }
-static size_t partial_bytes(const Prob& p, int chunk) {
+// Packed batches whose longest sequence has many more chunks than the others (one long sequence
+// among short ones): the partials get one slot per chunk that exists instead of the longest
+// sequence's number of chunks for every (sequence, head).  The sequences have at most
+// T / chunk + N chunks together whatever their lengths are, which bounds the storage on the host;
+// a one-workgroup kernel writes each sequence's first slot (Prob::chunk_base) once per call.
+// Only where every kernel that touches the partials knows that layout: the 16-bit matrix-core path.
+static bool compact_partials(const Prob& p, int dtype, int chunk) {
+  if (!p.cu || dtype == kF32 || !mfma::supported(p, dtype)) return false;
   const int64_t nchunks = cdiv64(p.L, chunk);
-  return align_up((size_t)p.N * p.H * nchunks * ((size_t)p.DK * p.DV + p.DK) * sizeof(float), 256);
+  return nchunks >= 4 && (int64_t)p.N * nchunks > 2 * (cdiv64(p.T, chunk) + p.N);
+}
+static size_t chunk_base_bytes(const Prob& p) { return align_up((size_t)(p.N + 1) * sizeof(int32_t), 256); }
+// partials (| first slot of every sequence)
+static size_t partial_bytes(const Prob& p, int dtype, int chunk) {
+  const size_t slot = ((size_t)p.DK * p.DV + p.DK) * sizeof(float);
+  if (compact_partials(p, dtype, chunk))
+    return align_up((size_t)(cdiv64(p.T, chunk) + p.N) * p.H * slot, 256) + chunk_base_bytes(p);
+  const int64_t nchunks = cdiv64(p.L, chunk);
+  return align_up((size_t)p.N * p.H * nchunks * slot, 256);
+}
+// The problem with its chunk bases, written behind the partials at the start of `workspace`.
+static Prob with_chunk_bases(const Prob& p, int dtype, int chunk, void* workspace, hipStream_t st) {
+  Prob r = p;
+  if (compact_partials(p, dtype, chunk)) {
+    int32_t* base = reinterpret_cast<int32_t*>((char*)workspace + partial_bytes(p, dtype, chunk) - chunk_base_bytes(p));
+    generic::chunk_bases(p, chunk, base, st);
+    r.chunk_base = base;
+  }
+  return r;
 }
 static int fwd_chunk(const Prob& p, int dtype) {
   return mfma::supported(p, dtype) ? mfma::state_chunk(p) : generic::state_chunk(p);
@@ -93,11 +119,11 @@ static Prob with_order(const Prob& p, void* workspace, size_t used, hipStream_t 
 
 static size_t fwd_used_bytes(const Prob& pc, int dtype) {
   const Prob p = key_side(pc);
-  return partial_bytes(p, fwd_chunk(p, dtype));
+  return partial_bytes(p, dtype, fwd_chunk(p, dtype));
 }
 static size_t bwd_used_bytes(const Prob& pc, int dtype) {
   const Prob p = query_side(pc);
-  return partial_bytes(p, bwd_chunk(p, dtype)) + 3 * state_bytes(p) + vec_bytes(p) +
+  return partial_bytes(p, dtype, bwd_chunk(p, dtype)) + 3 * state_bytes(p) + vec_bytes(p) +
          tokscal_bytes(p, dtype);
 }
 
@@ -116,20 +142,24 @@ int forward(const Prob& pc_, int dtype, const FwdArgs& a, hipStream_t st) {
   if (rc_cross != kOk) return rc_cross;
   const Prob pc = with_order(pc_, a.workspace, fwd_used_bytes(pc_, dtype), st);
   const bool is_cross = cross(pc);
-  const Prob p = key_side(pc);    // state kernel, reduce
-  const Prob pq = query_side(pc);  // output kernel
-  const bool dec = p.flags & kDecoupled;
-  const bool normalize = p.flags & kNormalize;
+  const Prob p_ = key_side(pc);    // state kernel, reduce
+  const Prob pq_ = query_side(pc);  // output kernel
+  const bool dec = p_.flags & kDecoupled;
+  const bool normalize = p_.flags & kNormalize;
   const void* qn = dec ? a.q_rope : a.q;
   const void* kn = dec ? a.k_rope : a.k;
-  const bool fast = mfma::supported(p, dtype);
-  if ((p.flags & kElu1) && !(fast && dtype != kF32 && p.DK == 64 && p.DV == 64 && !dec)) {
+  const bool fast = mfma::supported(p_, dtype);
+  if ((p_.flags & kElu1) && !(fast && dtype != kF32 && p_.DK == 64 && p_.DV == 64 && !dec)) {
     set_error("the feature map on load (FBLA_ELU1_QK) covers fp16 / bf16 heads of 64 x 64, not the decoupled operator");
     return kErrUnsupported;
   }
-  const int chunk = fwd_chunk(p, dtype);
-  const int nchunks = (int)cdiv64(p.L, chunk);
+  const int chunk = fwd_chunk(p_, dtype);
+  const int nchunks = (int)cdiv64(p_.L, chunk);
   float* partial = (float*)a.workspace;
+  // (skewed packed batches: one partial per chunk that exists)
+  const Prob p = with_chunk_bases(p_, dtype, chunk, a.workspace, st);
+  Prob pq = pq_;
+  pq.chunk_base = p.chunk_base;
   const unsigned phases = phase_mask();
   // one chunk per (sequence, head): the state kernel stores the finished S and km itself
   const bool direct = fast && nchunks == 1;
@@ -174,8 +204,12 @@ int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
   }
   const Prob pc = with_order(pc_, a.workspace, bwd_used_bytes(pc_, dtype), st);
   const bool is_cross = cross(pc);
-  const Prob p = query_side(pc);  // pass A, reduce
-  const Prob pk = key_side(pc);   // pass B
+  const Prob p_ = query_side(pc);  // pass A, reduce
+  const Prob pk_ = key_side(pc);   // pass B
+  // (skewed packed batches: one partial per chunk that exists)
+  const Prob p = with_chunk_bases(p_, dtype, bwd_chunk(p_, dtype), a.workspace, st);
+  Prob pk = pk_;
+  pk.chunk_base = p.chunk_base;
   const bool dec = p.flags & kDecoupled;
   const bool normalize = p.flags & kNormalize;
   const void* qn = dec ? a.q_rope : a.q;
@@ -189,7 +223,7 @@ int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
   const int nchunks = (int)cdiv64(p.L, chunk);
   char* ws = (char*)a.workspace;
   float* partial = (float*)ws;
-  ws += partial_bytes(p, chunk);
+  ws += partial_bytes(p, dtype, chunk);
   float* St = (float*)ws;
   ws += state_bytes(p);
   float* dS = (float*)ws;

@@ -47,6 +47,20 @@ def test_host_only_entry_points():
     assert L.fbla_varlen_workspace_bytes(0, 73000, 64, 16, 2048, 64, 64, _hip.BF16, 5) > 0
 
 
+def test_skewed_packed_batches_reserve_partials_for_the_chunks_that_exist():
+    """One sequence of 65536 tokens among 63 of 256 (H16, D128, bf16): the longest sequence is split
+    into many chunks; the partial sums of the reductions get a slot per chunk that exists (at most
+    T / chunk + N per head), not the long sequence's number of chunks for each of the 64 sequences."""
+    L = _hip.lib()
+    T, N, H = 65536 + 63 * 256, 64, 16
+    slot = (128 * 128 + 128) * 4
+    for which in (0, 1):
+        need = L.fbla_varlen_workspace_bytes(which, T, N, H, 65536, 128, 128, _hip.BF16, 5)
+        assert 0 < need < 160 * N * H * slot // 10   # well under 16 slots per (sequence, head)
+    # an even batch keeps the plain layout and a small workspace
+    assert L.fbla_varlen_workspace_bytes(0, 64 * 1200, 64, 16, 1200, 128, 128, _hip.BF16, 5) <= 2 * N * H * slot + 4096
+
+
 def test_bad_arguments_return_error_codes_without_touching_the_gpu():
     L = _hip.lib()
     args = [None] * 9 + [0, 1, 1, 16, 0, 64, _hip.F16, _hip.NORMALIZE, 1.0, 1e-6, None]
