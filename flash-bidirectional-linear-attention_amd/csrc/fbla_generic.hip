@@ -465,8 +465,57 @@ void state_partial(const Prob& p, int dtype, const void* kn, const void* v, cons
   else state_partial_t<float>(p, kn, v, kd, partial, chunk, nchunks, st);
 }
 
+// The same with four consecutive elements per thread (16-byte loads and stores): head dims that
+// are multiples of four.  A quarter of the workgroups: with thousands of (sequence, head) pairs the
+// kernel's time is the time to start its workgroups.
+__global__ __launch_bounds__(kThreads) void state_reduce4_kernel(
+    Prob p, const float* __restrict__ partial, int chunk, int nchunks, float* __restrict__ mat,
+    float* __restrict__ mat_t, float* __restrict__ vec, int blocks_per_head) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  const int nh = blockIdx.x / blocks_per_head, blk = blockIdx.x - nh * blocks_per_head;
+  const int n = nh / p.H;
+  int64_t bos;
+  int len;
+  seq_range(p, n, bos, len);
+  const int DK = p.DK, DV = p.DV, E = DK * DV, stride = E + DK;
+  const int e = 4 * (blk * kThreads + threadIdx.x);
+  if (e >= stride) return;
+  const int nvalid = len > 0 ? min(nchunks, (len + chunk - 1) / chunk) : 0;
+  const float* src = partial + partial_slot(p, n, nh - n * p.H, 0, nchunks) * stride + e;
+  const int64_t cstride = (int64_t)stride * partial_step(p);
+  f32x4 a = {0.f, 0.f, 0.f, 0.f};
+  int c = 0;
+  for (; c + 4 <= nvalid; c += 4) {  // fixed order: chunk 0, 1, 2, ...
+    const f32x4 x0 = *reinterpret_cast<const f32x4*>(src + c * cstride);
+    const f32x4 x1 = *reinterpret_cast<const f32x4*>(src + (c + 1) * cstride);
+    const f32x4 x2 = *reinterpret_cast<const f32x4*>(src + (c + 2) * cstride);
+    const f32x4 x3 = *reinterpret_cast<const f32x4*>(src + (c + 3) * cstride);
+    a = (((a + x0) + x1) + x2) + x3;
+  }
+  for (; c < nvalid; ++c) a += *reinterpret_cast<const f32x4*>(src + c * cstride);
+  if (e < E) {
+    a *= seq_scale(p, len);
+    *reinterpret_cast<f32x4*>(mat + (int64_t)nh * E + e) = a;
+    if (mat_t) {
+      const int dk = e / DV, dv = e - dk * DV;  // four consecutive dv of one dk
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mat_t[(int64_t)nh * E + (dv + i) * DK + dk] = a[i];
+    }
+  } else if (vec) {
+    const f32x4 r = {len > 0 ? a[0] / (float)len : 0.f, len > 0 ? a[1] / (float)len : 0.f,
+                     len > 0 ? a[2] / (float)len : 0.f, len > 0 ? a[3] / (float)len : 0.f};
+    *reinterpret_cast<f32x4*>(vec + (int64_t)nh * DK + (e - E)) = r;
+  }
+}
+
 void state_reduce(const Prob& p, const float* partial, int chunk, int nchunks, float* mat,
                   float* mat_t, float* vec, hipStream_t st) {
+  if (p.DK % 4 == 0 && p.DV % 4 == 0) {
+    const int blocks_per_head = (p.DK * p.DV + p.DK + 4 * kThreads - 1) / (4 * kThreads);
+    state_reduce4_kernel<<<dim3((unsigned)((int64_t)p.N * p.H * blocks_per_head)), dim3(kThreads), 0, st>>>(
+        p, partial, chunk, nchunks, mat, mat_t, vec, blocks_per_head);
+    return;
+  }
   const int blocks_per_head = (p.DK * p.DV + p.DK + kThreads - 1) / kThreads;
   state_reduce_kernel<<<dim3((unsigned)((int64_t)p.N * p.H * blocks_per_head)), dim3(kThreads), 0, st>>>(
       p, partial, chunk, nchunks, mat, mat_t, vec, blocks_per_head);
