@@ -462,11 +462,30 @@ def other_configs(dev, flush):
     with torch.no_grad():
         t_load = do_bench(lambda: linear_attention(q, k, v, feature_map="elu+1"), flush)
         t_first = do_bench(lambda: linear_attention(*elu_plus_one(q, k), v), flush)
-    print(json.dumps({"config": "elu+1 feature map + linear_attn fwd B8-H16-T16384-D64 fp16 (inference)",
-                      "mapped_on_load_ms": round(t_load[0], 5), "mapped_on_load_gbps": round(4 * nb / t_load[0] / 1e6, 1),
-                      "mapped_on_load_frac": round(4 * nb / t_load[0] / 1e6 / HBM_PEAK_GBPS, 4),
-                      "mapped_first_ms": round(t_first[0], 5)}), file=sys.stderr, flush=True)
-    del q, k, v
+    # training step through the map: dq, dk with respect to the raw tensors from the backward kernels,
+    # against the map differentiated by autograd (two more elementwise launches)
+    from flash_bla.ops.linear_attn.fused import LinearAttnFunction
+    do = torch.randn(q.shape, generator=g, device=dev).half()
+    leaves(q, k, v)
+
+    def step_kernels():
+        linear_attention(q, k, v, feature_map="elu+1").backward(do)
+        q.grad = k.grad = v.grad = None
+
+    def step_autograd():
+        LinearAttnFunction.apply(*elu_plus_one(q, k), v, 1.0 / q.shape[2], 1e-6).backward(do)
+        q.grad = k.grad = v.grad = None
+
+    t_step = do_bench(step_kernels, flush)
+    t_step_auto = do_bench(step_autograd, flush)
+    print(json.dumps({"config": "elu+1 feature map + linear_attn B8-H16-T16384-D64 fp16",
+                      "fwd_mapped_on_load_ms": round(t_load[0], 5),
+                      "fwd_mapped_on_load_gbps": round(4 * nb / t_load[0] / 1e6, 1),
+                      "fwd_mapped_on_load_frac": round(4 * nb / t_load[0] / 1e6 / HBM_PEAK_GBPS, 4),
+                      "fwd_mapped_first_ms": round(t_first[0], 5),
+                      "fwd_bwd_gradients_from_kernels_ms": round(t_step[0], 5),
+                      "fwd_bwd_map_by_autograd_ms": round(t_step_auto[0], 5)}), file=sys.stderr, flush=True)
+    del q, k, v, do
     q, k, v, do = make_inputs(2, 16, 16384, 64, torch.bfloat16, dev)
     qr, kr, _, _ = make_inputs(2, 16, 16384, 64, torch.bfloat16, dev, seed=7)
     leaves(q, k, qr, kr, v)

@@ -17,6 +17,8 @@ enum Flags : int {
   kDecoupled = 2,     // numerator uses q_rope/k_rope, denominator q/k
   kDefaultScale = 4,  // varlen only: scale = 1/len_i per sequence
   kElu1 = 8,          // forward only: q and k arrive before the feature map, the kernels apply elu(x) + 1 on load
+  kElu1Grad = 16,     // backward only: q and k are the mapped tensors phi(x) = elu(x) + 1 and dq, dk are wanted
+                      // with respect to x: the kernels multiply them by phi'(x) = min(phi(x), 1)
   kXcdOrder = 256,    // internal (set per launch): packed batches keep a sequence's heads on one XCD
   kInterleave = 512,  // internal (set per launch): the workgroups of a head take interleaved token steps
 };

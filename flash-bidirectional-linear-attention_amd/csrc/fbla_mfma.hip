@@ -146,6 +146,12 @@ template <typename T> __device__ __forceinline__ uint32_t phi_pair(uint32_t w) {
   return pack2<T>(Ops<T>::lo(e) + 1.f, Ops<T>::hi(e) + 1.f);
 }
 
+// A pair of gradients with respect to phi(x) times phi'(x) = min(phi(x), 1) (phi = elu + 1: 1 for
+// x > 0, exp(x) = phi(x) otherwise), from the pair of mapped values.
+template <typename T> __device__ __forceinline__ uint32_t gate_pair(uint32_t grad, uint32_t mapped) {
+  return pack2<T>(Ops<T>::lo(grad) * fminf(Ops<T>::lo(mapped), 1.f), Ops<T>::hi(grad) * fminf(Ops<T>::hi(mapped), 1.f));
+}
+
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 // Eight tokens of one feature (an MFMA operand fragment of one k-step) out of a row-major tile:
 // two transposing reads, `off0` / `off1` are this lane's byte offsets for x = 0 / 1.
@@ -923,12 +929,14 @@ template <int DR, int DC, bool DEN, int WAVES> struct RowsLayout {
 // odd length leaves the second half of the last pair out.  No partial sums in the prologue.
 // FMAP = true: the rows of x arrive before the feature map and are mapped (phi_pair) on their way into LDS.
 template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD = false,
-          int PF = (DR == 128 && DC == 128) ? FBLA_ROWS_PF128 : FBLA_ROWS_PF, bool PAIR = false, bool FMAP = false>
-__global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64 && !DEN) ? 4 : 1) void rows_kernel(Prob p, RowsJob job0, RowsJob job1,
+          int PF = (DR == 128 && DC == 128) ? FBLA_ROWS_PF128 : FBLA_ROWS_PF, bool PAIR = false, bool FMAP = false,
+          bool GATE = false>
+__global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64 && !DEN && !GATE) ? 4 : 1) void rows_kernel(Prob p, RowsJob job0, RowsJob job1,
                                                           int wgs_per_job, int chunk, int nchunks,
                                                           int dr_true, int dc_true) {
   static_assert(!PAIR || (DR == 64 && DC == 64 && !PAD), "pair mode: two 32-wide rows per 64-wide row");
   static_assert(!FMAP || (!DEN && !PAD && !PAIR), "feature map on load: plain rows only");
+  static_assert(!GATE || (!DEN && !PAD && !PAIR && !FMAP && DR == DC), "gated output: plain square tiles only");
   const int dr = PAD ? dr_true : (PAIR ? 32 : DR), dc = PAD ? dc_true : (PAIR ? 32 : DC);
   const int dpk = PAD ? (p.DK <= 64 ? 64 : 128) : p.DK;  // padded length of the km / dkm vector
   using LY = RowsLayout<DR, DC, DEN, WAVES>;
@@ -1039,11 +1047,16 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
   // PF register sets hold the tiles in flight: a tile is requested PF tiles ahead of its use
   int t0 = t_begin + 32 * wave;
   u32x4 xr[PF][XI], xd[DEN ? PF : 1][XI];
+  // GATE: the mapped rows that scale this job's output (same pieces as the output's), or none
+  const T* gate = GATE ? (const T*)job.gate : nullptr;
+  u32x4 xg[GATE ? PF : 1][XI];
 #pragma unroll
   for (int f = 0; f < PF; ++f)
     if (t0 + t_stride * f < t_end) {
       load_tile(xr[f], x, t0 + t_stride * f);
       if constexpr (DEN) load_tile(xd[f], xden, t0 + t_stride * f);
+      if constexpr (GATE)
+        if (gate) load_tile(xg[f], gate, t0 + t_stride * f);
     }
 
   // ---- prologue: matrix operand fragments, km pairs, addvec ----
@@ -1084,7 +1097,7 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
   // ---- main loop ----
   // one tile: its rows move from the register set to the staging area, the set is refilled
   // with the tile PF steps ahead, then the tile is multiplied and stored
-  auto tile_step = [&](u32x4(&xcur)[XI], u32x4(&dcur)[XI]) {
+  auto tile_step = [&](u32x4(&xcur)[XI], u32x4(&dcur)[XI], u32x4(&gcur)[XI]) {
     wave_sync();  // previous tile's staging reads are done
     if constexpr (FMAP) {  // (rows past the end become phi(0) = 1: their outputs are not stored)
 #pragma unroll
@@ -1210,6 +1223,16 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
       const int q = lane + 64 * i;
       wout[i] = *reinterpret_cast<const u32x4*>(stage + swz<OROWB>(q / OCH, q % OCH));
     }
+    if constexpr (GATE) {
+      if (gate) {  // the same for all lanes
+#pragma unroll
+        for (int i = 0; i < OI; ++i)
+#pragma unroll
+          for (int w = 0; w < 4; ++w) wout[i][w] = gate_pair<T>(wout[i][w], gcur[i][w]);
+        // this set is free now: the mapped rows of the tile PF steps ahead
+        if (t0 + t_stride * PF < t_end) load_tile(gcur, gate, t0 + t_stride * PF);
+      }
+    }
     if ((FBLA_ROWS_FAST & 2) && !NORM && kFast && t0 + 32 <= t_end) {
       char* tp = const_cast<char*>(tile_ptr(out, t0, DC));
 #pragma unroll
@@ -1227,7 +1250,7 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
   while (t0 < t_end) {
 #pragma unroll
     for (int f = 0; f < PF; ++f)
-      if (t0 < t_end) tile_step(xr[f], xd[DEN ? f : 0]);
+      if (t0 < t_end) tile_step(xr[f], xd[DEN ? f : 0], xg[GATE ? f : 0]);
   }
 }
 
@@ -1491,8 +1514,9 @@ template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struc
 // 64-wide row as in the rows kernel; the token view never mixes the halves of a row, the
 // feature view accumulates blockdiag-shaped sums whose two diagonal 32 x 32 blocks are added
 // before the store.  `chunk` counts row pairs.
+// GATE = true: q are the mapped rows phi(x) and dq is wanted with respect to x: times min(q, 1).
 template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true, bool PAD = false,
-          bool PAIR = false>
+          bool PAIR = false, bool GATE = false>
 __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) ? 3 : 2) void bwd_a_kernel(
     Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const T* __restrict__ dout,
     const float* __restrict__ S, const float* __restrict__ km, T* __restrict__ dqn,
@@ -1756,6 +1780,13 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
     uint32_t dqp[DK / 4], dqdp[DEN && !kDenFlat ? DK / 4 : 1];
     {
       const float gs = denorm * rz;
+      static_assert(!GATE || (FUSED && !DEN && !PAD && !PAIR), "gated dq: the plain fused kernel only");
+      u32x4 qmapped[GATE ? QCH / 2 : 1];  // this lane's half of its token's (mapped) q row, still in the tile
+      if constexpr (GATE) {
+#pragma unroll
+        for (int ch = 0; ch < QCH / 2; ++ch)
+          qmapped[ch] = *reinterpret_cast<const u32x4*>(qt + swz<QROWB>(ntok, (QCH / 2) * kb + ch));
+      }
 #pragma unroll
       for (int c2 = 0; c2 < DK / 4; ++c2) {
         const int c0 = 2 * c2;
@@ -1768,6 +1799,11 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
             v0 += d0;
             v1 += d1;
           }
+        }
+        if constexpr (GATE) {  // phi'(x) = min(phi(x), 1)
+          const uint32_t w = qmapped[c2 >> 2][c2 & 3];
+          v0 *= fminf(Ops<T>::lo(w), 1.f);
+          v1 *= fminf(Ops<T>::hi(w), 1.f);
         }
         dqp[c2] = pack2<T>(v0, v1);
       }
@@ -2419,12 +2455,13 @@ static void run_state(const Prob& p, const void* kn, const void* v, const void* 
   else run_state_dims<T, false>(p, a, b, c, partial, ts, rows, fm, fv, chunk, nchunks, bs, st);
 }
 
-template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD, bool PAIR = false, bool FMAP = false>
+template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD, bool PAIR = false, bool FMAP = false,
+          bool GATE = false>
 static int launch_rows_k(const Prob& p, const RowsJob& job, const RowsJob* job2, int chunk,
                          int nchunks, int dr, int dc, hipStream_t st) {
   using LY = RowsLayout<DR, DC, DEN, WAVES>;
   constexpr int PF = (DR == 128 && DC == 128) ? FBLA_ROWS_PF128 : FBLA_ROWS_PF;
-  auto kernel = rows_kernel<T, DR, DC, NORM, DEN, WAVES, PAD, PF, PAIR, FMAP>;
+  auto kernel = rows_kernel<T, DR, DC, NORM, DEN, WAVES, PAD, PF, PAIR, FMAP, GATE>;
   static thread_local bool configured = false;
   int rc = reserve_lds(kernel, LY::kTotal, configured);
   if (rc != kOk) return rc;
@@ -2471,6 +2508,8 @@ static int launch_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, i
     }
   }
   if constexpr (DR == 64 && DC == 64 && !PAD) {
+    if (job.gate || (job2 && job2->gate))  // (the plan has checked: pass B of the plain operator)
+      return launch_rows_k<T, 64, 64, false, false, WAVES, false, false, false, true>(p, job, job2, chunk, nchunks, dr, dc, st);
     if (p.flags & kElu1) {  // (the plan has checked: plain operator, forward output)
       if (norm) return launch_rows_k<T, 64, 64, true, false, WAVES, false, false, true>(p, job, job2, chunk, nchunks, dr, dc, st);
       return launch_rows_k<T, 64, 64, false, false, WAVES, false, false, true>(p, job, job2, chunk, nchunks, dr, dc, st);
@@ -2605,7 +2644,7 @@ int rows2(const Prob& p_, int dtype, const RowsJob& job0, const RowsJob& job1, i
   return run_rows<__bf16>(p, job0, &job1, DR, DC, st);
 }
 
-template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool PAD, bool PAIR = false>
+template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool PAD, bool PAIR = false, bool GATE = false>
 static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, const float* S,
                         const float* km, T* dqn, T* dqd, float* partial, float* tokscal,
                         int64_t total_rows, float* fm, float* fv, int chunk, int nchunks,
@@ -2621,7 +2660,7 @@ static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, 
                               (int)sizeof(float) * 64 * ((DK / 32) * (DV / 32) * 16 + DK / 32),
                 "reduction buffer must fit in the tile area");
   static_assert(LY::kTotal <= 160 * 1024, "LDS budget of one workgroup");
-  auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN, FUSED, LO, PAD, PAIR>;
+  auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN, FUSED, LO, PAD, PAIR, GATE>;
   static thread_local bool configured = false;  // per instantiation
   int rc = reserve_lds(kernel, LY::kTotal, configured);
   if (rc != kOk) return rc;
@@ -2655,6 +2694,13 @@ static int run_bwd_a_pad(const Prob& p, const void* qn, const void* qd, const vo
       if (!(p.flags & kNormalize))
         return launch_bwd_a128<T, false, PAD>(p, a, c, S, km, x, partial, fm, fv, chunk, nchunks, st);
       return launch_bwd_a128<T, true, PAD>(p, a, c, S, km, x, partial, fm, fv, chunk, nchunks, st);
+    }
+  }
+  if constexpr (!PAD && !PAIR) {
+    if (p.flags & kElu1Grad) {  // (the plan has checked: plain operator, 64 x 64)
+      if (!(p.flags & kNormalize))
+        return launch_bwd_a<T, 64, 64, false, false, true, false, false, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+      return launch_bwd_a<T, 64, 64, true, false, true, false, false, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
     }
   }
   if (!(p.flags & kNormalize))

@@ -149,6 +149,10 @@ int forward(const Prob& pc_, int dtype, const FwdArgs& a, hipStream_t st) {
   const void* qn = dec ? a.q_rope : a.q;
   const void* kn = dec ? a.k_rope : a.k;
   const bool fast = mfma::supported(p_, dtype);
+  if (p_.flags & kElu1Grad) {
+    set_error("FBLA_ELU1_GRAD is a flag of the backward entry points");
+    return kErrBadArg;
+  }
   if ((p_.flags & kElu1) && !(fast && dtype != kF32 && p_.DK == 64 && p_.DV == 64 && !dec)) {
     set_error("the feature map on load (FBLA_ELU1_QK) covers fp16 / bf16 heads of 64 x 64, not the decoupled operator");
     return kErrUnsupported;
@@ -200,6 +204,11 @@ int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
   if (rc_cross != kOk) return rc_cross;
   if (pc_.flags & kElu1) {
     set_error("the feature map on load (FBLA_ELU1_QK) is forward only: map q and k first, then differentiate");
+    return kErrUnsupported;
+  }
+  if ((pc_.flags & kElu1Grad) && !(dtype != kF32 && pc_.DK == 64 && pc_.DV == 64 && !(pc_.flags & kDecoupled) &&
+                                   mfma::bwd_a_supported(pc_, dtype))) {
+    set_error("gradients through the feature map (FBLA_ELU1_GRAD) cover fp16 / bf16 heads of 64 x 64, not the decoupled operator");
     return kErrUnsupported;
   }
   const Prob pc = with_order(pc_, a.workspace, bwd_used_bytes(pc_, dtype), st);
@@ -265,6 +274,7 @@ int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
     if (fast) {
       // dk~_t = v_t (s dS)^T (+ dkm/L): contraction over dv, M(r=dv, c=dk) = dS[c][r]
       mfma::RowsJob jk{a.v, nullptr, dS, 1, p.DV, nullptr, (!dec && normalize) ? dkm : nullptr, dkn};
+      if (p.flags & kElu1Grad) jk.gate = a.k;  // dk with respect to the keys before the feature map
       // dv_t = k~_t (s dS): contraction over dk
       mfma::RowsJob jv{kn, nullptr, dS, p.DV, 1, nullptr, nullptr, a.dv};
       if (fold) {  // both kernels sum the pass-A partials themselves (s dS, dkm/L)

@@ -15,7 +15,7 @@ _LIB_PATH = os.environ.get("FBLA_LIB_PATH") or os.path.join(
 _lib = None
 
 F16, BF16, F32 = 0, 1, 2
-NORMALIZE, DECOUPLED, DEFAULT_SCALE, ELU1_QK = 1, 2, 4, 8
+NORMALIZE, DECOUPLED, DEFAULT_SCALE, ELU1_QK, ELU1_GRAD = 1, 2, 4, 8, 16
 
 _DTYPES = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
 
@@ -242,7 +242,7 @@ def varlen_fwd(q, k, v, cu_seqlens, max_seqlen, scale, eps, extra_flags=0):
     return o, s, km
 
 
-def varlen_bwd(q, k, v, cu_seqlens, max_seqlen, do, s, km, scale, eps):
+def varlen_bwd(q, k, v, cu_seqlens, max_seqlen, do, s, km, scale, eps, extra_flags=0):
     """Packed backward: returns (dq, dk, dv)."""
     _require_gpu(q, k, v, do, cu_seqlens)
     q, k, v, do, cu_seqlens, s, km = _aligned(q, k, v, do, cu_seqlens, s, km)
@@ -252,7 +252,7 @@ def varlen_bwd(q, k, v, cu_seqlens, max_seqlen, do, s, km, scale, eps):
     N = cu_seqlens.numel() - 1
     code = dtype_code(q)
     dev = q.device
-    flags = NORMALIZE | (DEFAULT_SCALE if scale is None else 0)
+    flags = NORMALIZE | (DEFAULT_SCALE if scale is None else 0) | extra_flags
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     with _on(dev):
         ws = _workspace(L.fbla_varlen_workspace_bytes(1, T, N, H, max_seqlen, DK, DV, code, flags), dev)

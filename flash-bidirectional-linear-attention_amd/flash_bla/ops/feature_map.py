@@ -51,10 +51,16 @@ def check_feature_map(feature_map):
     return feature_map is not None
 
 
+def mapped_in_kernels(q, v):
+    """16-bit heads of 64 x 64: the shapes for which the attention kernels take part in the feature
+    map (on load in an inference forward, on the gradients in a backward)."""
+    return q.dtype in (torch.float16, torch.bfloat16) and q.shape[-1] == 64 and v.shape[-1] == 64
+
+
 def applied_on_load(q, k, v):
     """True when the forward kernels can apply elu(x) + 1 to q and k as they load them: 16-bit
     heads of 64 x 64 and nothing to differentiate (the backward needs the mapped tensors, so a
     call that records a graph maps them first with `elu_plus_one`)."""
-    if q.dtype not in (torch.float16, torch.bfloat16) or q.shape[-1] != 64 or v.shape[-1] != 64:
+    if not mapped_in_kernels(q, v):
         return False
     return not (torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)))

@@ -13,7 +13,7 @@ import torch
 
 from flash_bla import _hip
 from flash_bla.ops._check import check_dense
-from flash_bla.ops.feature_map import applied_on_load, check_feature_map, elu_plus_one
+from flash_bla.ops.feature_map import applied_on_load, check_feature_map, elu_plus_one, mapped_in_kernels
 from flash_bla.utils import contiguous
 
 
@@ -38,6 +38,32 @@ class LinearAttnFunction(torch.autograd.Function):
         return dq, dk, dv, None, None
 
 
+class MappedLinearAttnFunction(torch.autograd.Function):
+    """linear_attention(elu(q) + 1, elu(k) + 1, v) as one autograd node (16-bit heads of 64 x 64):
+    the forward maps q and k with one launch and keeps the mapped tensors (the backward needs
+    them, not the raw ones); the backward kernels return dq and dk with respect to the raw
+    tensors themselves (times min(mapped, 1), the map's derivative), so that the two elementwise
+    launches of the map's autograd disappear."""
+
+    @staticmethod
+    @contiguous
+    def forward(ctx, q, k, v, scale, eps):
+        qm, km_ = _hip.elu1_fwd(q, k)
+        o, s, km = _hip.la_fwd(qm, km_, v, None, None, scale, eps, _hip.NORMALIZE)
+        ctx.save_for_backward(qm, km_, v, s, km)
+        ctx.scale = scale
+        ctx.eps = eps
+        return o
+
+    @staticmethod
+    @contiguous
+    def backward(ctx, do):
+        qm, km_, v, s, km = ctx.saved_tensors
+        dq, dk, dv, _, _ = _hip.la_bwd(qm, km_, v, None, None, do, s, km, ctx.scale, ctx.eps,
+                                       _hip.NORMALIZE | _hip.ELU1_GRAD)
+        return dq, dk, dv, None, None
+
+
 def linear_attention(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -57,8 +83,10 @@ def linear_attention(
         feature_map: None (the reference's signature: q and k are features already) or "elu+1":
             q and k are given before the blocks' feature map `elu(x) + 1`
             (layers/linfusion.py:88-89).  An inference forward of 16-bit heads of 64 x 64 applies
-            it inside the kernels as they load q and k (no mapped copies are written); every
-            other call maps them first with one launch and proceeds as usual.
+            it inside the kernels as they load q and k (no mapped copies are written); with
+            gradients, the same heads map q and k with one launch and get dq, dk with respect to
+            the raw tensors from the backward kernels; every other call maps them first and lets
+            autograd differentiate the map.
     Returns the output of shape `(B, H, L, V)` with `v`'s dtype.
     """
     check_dense("linear_attention", q, k, v)
@@ -68,5 +96,7 @@ def linear_attention(
         if applied_on_load(q, k, v):
             return _hip.la_fwd(q.contiguous(), k.contiguous(), v.contiguous(), None, None, scale, eps,
                                _hip.NORMALIZE | _hip.ELU1_QK)[0]
+        if mapped_in_kernels(q, v):
+            return MappedLinearAttnFunction.apply(q, k, v, scale, eps)
         q, k = elu_plus_one(q, k)
     return LinearAttnFunction.apply(q, k, v, scale, eps)

@@ -48,6 +48,11 @@ extern "C" {
                               * phi(x) = elu(x) + 1 (layers/linfusion.py:88-89, layers/mlla.py:74-75) and the
                               * kernels apply it as they load them; fp16 / bf16, DK = DV = 64, not decoupled
                               * (FBLA_ERR_UNSUPPORTED otherwise, and from the backward entry points) */
+#define FBLA_ELU1_GRAD 16    /* backward entry points only: q and k are the MAPPED tensors phi(x) = elu(x) + 1 (what
+                              * the forward consumed and saved) and dq, dk are wanted with respect to x: the
+                              * kernels multiply them by phi'(x) = min(phi(x), 1) as they write them, which
+                              * replaces the autograd of `F.elu(x) + 1.0` (two elementwise launches per call);
+                              * fp16 / bf16, DK = DV = 64, not decoupled (FBLA_ERR_UNSUPPORTED otherwise) */
 
 /* error codes */
 #define FBLA_OK 0

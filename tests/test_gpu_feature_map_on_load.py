@@ -105,6 +105,56 @@ def test_gradients_flow_through_the_feature_map(dtype):
     assert_parity(leaves[2].grad, ref["dv"], dtype, "dv")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("B,H,L", [(2, 3, 300), (1, 2, 77), (8, 16, 2048)])
+def test_gradients_with_respect_to_the_raw_tensors_from_the_kernels(B, H, L, dtype):
+    """64-wide 16-bit heads: the backward kernels multiply dq and dk by the map's derivative
+    themselves; the result agrees with the map differentiated by autograd (the path other shapes
+    take), and the simple_la family does the same through the C ABI's flag."""
+    from flash_bla import _hip
+    from flash_bla.ops.feature_map import elu_plus_one
+    from flash_bla.ops.linear_attn.fused import LinearAttnFunction, linear_attention
+    q, k, v = _raw((B, H, L, 64), (B, H, L, 64), dtype, seed=L + 1)
+    do = torch.randn(B, H, L, 64, generator=torch.Generator().manual_seed(L)).to(dtype).cuda()
+    a = [t.cuda().requires_grad_() for t in (q, k, v)]
+    linear_attention(*a, feature_map="elu+1").backward(do)
+    b = [t.cuda().requires_grad_() for t in (q, k, v)]
+    LinearAttnFunction.apply(*elu_plus_one(b[0], b[1]), b[2], 1.0 / L, 1e-6).backward(do)
+    # (the kernels round dq, dk once, the other path twice: a couple of last places of the type)
+    close = 1e-2 if dtype == torch.bfloat16 else 2e-3
+    for name, x, y in zip(("dq", "dk", "dv"), a, b):
+        assert max_rel_err(x.grad, np64(y.grad)) < close, name
+    # without the denominator: dq, dk of simple_la on mapped tensors, gated by the kernels
+    qm, km_ = elu_plus_one(q.cuda(), k.cuda())
+    scale = 0.125
+    _, s, km = _hip.la_fwd(qm, km_, v.cuda(), None, None, scale, 1e-6, 0)
+    dq, dk, dv, _, _ = _hip.la_bwd(qm, km_, v.cuda(), None, None, do, s, km, scale, 1e-6, _hip.ELU1_GRAD)
+    ref = cf.dense_backward(np64(qm), np64(km_), np64(v), np64(do), scale, 1e-6, False)
+    gate = lambda m: np.minimum(np64(m), 1.0)
+    assert_parity(dq, ref["dq"] * gate(qm), dtype, "simple dq", ref["dq_mag"] if "dq_mag" in ref else None)
+    assert_parity(dk, ref["dk"] * gate(km_), dtype, "simple dk", ref["dk_mag"] if "dk_mag" in ref else None)
+    assert_parity(dv, ref["dv"], dtype, "simple dv", ref["dv_mag"] if "dv_mag" in ref else None)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_packed_gradients_through_the_feature_map(dtype):
+    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
+    lens = [5, 300, 1, 64, 1000, 17, 0, 2049]
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32)
+    T, H = int(cu[-1]), 3
+    q, k, v = _raw((T, H, 64), (T, H, 64), dtype, seed=19)
+    do = torch.randn(T, H, 64, generator=torch.Generator().manual_seed(2)).to(dtype)
+    leaves = [t.cuda().requires_grad_() for t in (q, k, v)]
+    o = varlen_linear_attention(*leaves, cu.cuda(), max(lens), feature_map="elu+1")
+    o.backward(do.cuda())
+    ref = cf.varlen_backward(np64(_mapped(q)), np64(_mapped(k)), np64(v), np64(do), cu.numpy())
+    dphi = lambda x: np.where(np64(x) > 0, 1.0, np.exp(np.minimum(np64(x), 0.0)))
+    assert_parity(o, ref["o"], dtype, "o")
+    assert_parity(leaves[0].grad, ref["dq"] * dphi(q), dtype, "dq", ref.get("dq_mag"))
+    assert_parity(leaves[1].grad, ref["dk"] * dphi(k), dtype, "dk", ref.get("dk_mag"))
+    assert_parity(leaves[2].grad, ref["dv"], dtype, "dv", ref.get("dv_mag"))
+
+
 @pytest.mark.parametrize("D,dtype", [(32, torch.float16), (128, torch.bfloat16), (64, torch.float32), (48, torch.float16)])
 def test_other_shapes_map_first(D, dtype):
     from flash_bla.ops.linear_attn.fused import linear_attention
@@ -129,3 +179,9 @@ def test_argument_and_flag_errors():
     o, s, km = _hip.la_fwd(q, k, v, None, None, 1.0, 1e-6, _hip.NORMALIZE)
     with pytest.raises(ValueError, match="forward only"):
         _hip.la_bwd(q, k, v, None, None, torch.ones_like(v), s, km, 1.0, 1e-6, _hip.NORMALIZE | _hip.ELU1_QK)
+    with pytest.raises(ValueError, match="backward entry points"):
+        _hip.la_fwd(q, k, v, None, None, 1.0, 1e-6, _hip.NORMALIZE | _hip.ELU1_GRAD)
+    o32, s32, km32 = _hip.la_fwd(q32, k32, v32, None, None, 1.0, 1e-6, _hip.NORMALIZE)
+    with pytest.raises(ValueError, match="gradients through the feature map"):
+        _hip.la_bwd(q32, k32, v32, None, None, torch.ones_like(v32), s32, km32, 1.0, 1e-6,
+                    _hip.NORMALIZE | _hip.ELU1_GRAD)
