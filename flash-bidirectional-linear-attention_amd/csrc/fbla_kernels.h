@@ -89,8 +89,10 @@ struct RowsJob {
   float* mat_out = nullptr;
   float* vec_out = nullptr;
   float add_scale = 1.f;  // factor on addvec (queries / keys when their numbers differ)
+  bool map_x = false;          // kElu1 together with kElu1Grad: this job's x rows arrive before the map
   const void* gate = nullptr;  // [rows][DC] mapped rows phi(x): the output is multiplied by min(gate, 1), the
-                               // derivative of phi (kElu1Grad; the dk job of the backward), or null
+                               // derivative of phi (kElu1Grad; the dk job of the backward; rows before the map
+                               // when kElu1 is set as well), or null
 };
 bool supported(const Prob& p, int dtype);
 bool bwd_a_supported(const Prob& p, int dtype);

@@ -936,12 +936,16 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
                                                           int dr_true, int dc_true) {
   static_assert(!PAIR || (DR == 64 && DC == 64 && !PAD), "pair mode: two 32-wide rows per 64-wide row");
   static_assert(!FMAP || (!DEN && !PAD && !PAIR), "feature map on load: plain rows only");
-  static_assert(!GATE || (!DEN && !PAD && !PAIR && !FMAP && DR == DC), "gated output: plain square tiles only");
+  static_assert(!GATE || (!DEN && !PAD && !PAIR && DR == DC), "gated output: plain square tiles only");
+
   const int dr = PAD ? dr_true : (PAIR ? 32 : DR), dc = PAD ? dc_true : (PAIR ? 32 : DC);
   const int dpk = PAD ? (p.DK <= 64 ? 64 : 128) : p.DK;  // padded length of the km / dkm vector
   using LY = RowsLayout<DR, DC, DEN, WAVES>;
   const bool second = (int)blockIdx.x >= wgs_per_job;
   const RowsJob& job = second ? job1 : job0;
+  // FMAP and GATE together (pass B of a backward given the rows before the map): a job maps its x rows
+  // when job.map_x is set, and its gate rows arrive before the map too
+  const bool map_x = FMAP && (!GATE || job.map_x);
   const int wg = second ? blockIdx.x - wgs_per_job : blockIdx.x;
   constexpr int NT = WAVES * 64;
   constexpr int KS = DR / 16;  // k-steps
@@ -1100,10 +1104,12 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
   auto tile_step = [&](u32x4(&xcur)[XI], u32x4(&dcur)[XI], u32x4(&gcur)[XI]) {
     wave_sync();  // previous tile's staging reads are done
     if constexpr (FMAP) {  // (rows past the end become phi(0) = 1: their outputs are not stored)
+      if (map_x) {  // the same for all lanes
 #pragma unroll
-      for (int i = 0; i < XI; ++i)
+        for (int i = 0; i < XI; ++i)
 #pragma unroll
-        for (int w = 0; w < 4; ++w) xcur[i][w] = phi_pair<T>(xcur[i][w]);
+          for (int w = 0; w < 4; ++w) xcur[i][w] = phi_pair<T>(xcur[i][w]);
+      }
     }
     stash_tile(xcur, stage);
     if constexpr (DEN && !kDenFlat) stash_tile(dcur, stage_den);
@@ -1228,7 +1234,7 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
 #pragma unroll
         for (int i = 0; i < OI; ++i)
 #pragma unroll
-          for (int w = 0; w < 4; ++w) wout[i][w] = gate_pair<T>(wout[i][w], gcur[i][w]);
+          for (int w = 0; w < 4; ++w) wout[i][w] = gate_pair<T>(wout[i][w], FMAP ? phi_pair<T>(gcur[i][w]) : gcur[i][w]);
         // this set is free now: the mapped rows of the tile PF steps ahead
         if (t0 + t_stride * PF < t_end) load_tile(gcur, gate, t0 + t_stride * PF);
       }
@@ -1515,8 +1521,9 @@ template <int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true> struc
 // feature view accumulates blockdiag-shaped sums whose two diagonal 32 x 32 blocks are added
 // before the store.  `chunk` counts row pairs.
 // GATE = true: q are the mapped rows phi(x) and dq is wanted with respect to x: times min(q, 1).
+// FMAP = true (with GATE): q are the rows x themselves and are mapped on their way into LDS.
 template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool LO = true, bool PAD = false,
-          bool PAIR = false, bool GATE = false>
+          bool PAIR = false, bool GATE = false, bool FMAP = false>
 __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) ? 3 : 2) void bwd_a_kernel(
     Prob p, const T* __restrict__ qn, const T* __restrict__ qd, const T* __restrict__ dout,
     const float* __restrict__ S, const float* __restrict__ km, T* __restrict__ dqn,
@@ -1680,8 +1687,15 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
   }
   __syncthreads();
 
+  static_assert(!FMAP || GATE, "q mapped on load: together with the gated dq");
   while (t0 < t_end) {
     wave_sync();  // the previous sub-tile's staged dq has been read out
+    if constexpr (FMAP) {  // (rows past the end become phi(0) = 1: they are masked by rz = 0 and not stored)
+#pragma unroll
+      for (int i = 0; i < QI; ++i)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) rq[i][w] = phi_pair<T>(rq[i][w]);
+    }
     stash_q(rq, qt);
     stash_g(rg, gt);
     if constexpr (DEN && !kDenFlat) stash_q(rd, qdt);
@@ -2508,8 +2522,11 @@ static int launch_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, i
     }
   }
   if constexpr (DR == 64 && DC == 64 && !PAD) {
-    if (job.gate || (job2 && job2->gate))  // (the plan has checked: pass B of the plain operator)
+    if (job.gate || (job2 && job2->gate)) {  // (the plan has checked: pass B of the plain operator)
+      if (p.flags & kElu1)  // keys before the map
+        return launch_rows_k<T, 64, 64, false, false, WAVES, false, false, true, true>(p, job, job2, chunk, nchunks, dr, dc, st);
       return launch_rows_k<T, 64, 64, false, false, WAVES, false, false, false, true>(p, job, job2, chunk, nchunks, dr, dc, st);
+    }
     if (p.flags & kElu1) {  // (the plan has checked: plain operator, forward output)
       if (norm) return launch_rows_k<T, 64, 64, true, false, WAVES, false, false, true>(p, job, job2, chunk, nchunks, dr, dc, st);
       return launch_rows_k<T, 64, 64, false, false, WAVES, false, false, true>(p, job, job2, chunk, nchunks, dr, dc, st);
@@ -2644,7 +2661,8 @@ int rows2(const Prob& p_, int dtype, const RowsJob& job0, const RowsJob& job1, i
   return run_rows<__bf16>(p, job0, &job1, DR, DC, st);
 }
 
-template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool PAD, bool PAIR = false, bool GATE = false>
+template <typename T, int DK, int DV, bool NORM, bool DEN, bool FUSED, bool PAD, bool PAIR = false, bool GATE = false,
+          bool FMAP = false>
 static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, const float* S,
                         const float* km, T* dqn, T* dqd, float* partial, float* tokscal,
                         int64_t total_rows, float* fm, float* fv, int chunk, int nchunks,
@@ -2660,7 +2678,7 @@ static int launch_bwd_a(const Prob& p, const T* qn, const T* qd, const T* dout, 
                               (int)sizeof(float) * 64 * ((DK / 32) * (DV / 32) * 16 + DK / 32),
                 "reduction buffer must fit in the tile area");
   static_assert(LY::kTotal <= 160 * 1024, "LDS budget of one workgroup");
-  auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN, FUSED, LO, PAD, PAIR, GATE>;
+  auto kernel = bwd_a_kernel<T, DK, DV, NORM, DEN, FUSED, LO, PAD, PAIR, GATE, FMAP>;
   static thread_local bool configured = false;  // per instantiation
   int rc = reserve_lds(kernel, LY::kTotal, configured);
   if (rc != kOk) return rc;
@@ -2698,6 +2716,11 @@ static int run_bwd_a_pad(const Prob& p, const void* qn, const void* qd, const vo
   }
   if constexpr (!PAD && !PAIR) {
     if (p.flags & kElu1Grad) {  // (the plan has checked: plain operator, 64 x 64)
+      if (p.flags & kElu1) {  // q before the map
+        if (!(p.flags & kNormalize))
+          return launch_bwd_a<T, 64, 64, false, false, true, false, false, true, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+        return launch_bwd_a<T, 64, 64, true, false, true, false, false, true, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
+      }
       if (!(p.flags & kNormalize))
         return launch_bwd_a<T, 64, 64, false, false, true, false, false, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);
       return launch_bwd_a<T, 64, 64, true, false, true, false, false, true>(p, a, b, c, S, km, x, y, partial, nullptr, 0, fm, fv, chunk, nchunks, st);

@@ -202,8 +202,9 @@ int forward(const Prob& pc_, int dtype, const FwdArgs& a, hipStream_t st) {
 int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
   int rc_cross = check_cross(pc_, dtype);
   if (rc_cross != kOk) return rc_cross;
-  if (pc_.flags & kElu1) {
-    set_error("the feature map on load (FBLA_ELU1_QK) is forward only: map q and k first, then differentiate");
+  if ((pc_.flags & kElu1) && !(pc_.flags & kElu1Grad)) {
+    set_error("the feature map on load (FBLA_ELU1_QK) in a backward needs FBLA_ELU1_GRAD as well: dq, dk are then "
+              "gradients with respect to the q, k given");
     return kErrUnsupported;
   }
   if ((pc_.flags & kElu1Grad) && !(dtype != kF32 && pc_.DK == 64 && pc_.DV == 64 && !(pc_.flags & kDecoupled) &&
@@ -277,6 +278,7 @@ int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
       if (p.flags & kElu1Grad) jk.gate = a.k;  // dk with respect to the keys before the feature map
       // dv_t = k~_t (s dS): contraction over dk
       mfma::RowsJob jv{kn, nullptr, dS, p.DV, 1, nullptr, nullptr, a.dv};
+      jv.map_x = (p.flags & kElu1) != 0;  // (with kElu1: k itself is given before the map)
       if (fold) {  // both kernels sum the pass-A partials themselves (s dS, dkm/L)
         jk.mat = jv.mat = partial;
         jk.pchunk = jv.pchunk = pchunk;

@@ -58,9 +58,9 @@ def mapped_in_kernels(q, v):
 
 
 def applied_on_load(q, k, v):
-    """True when the forward kernels can apply elu(x) + 1 to q and k as they load them: 16-bit
-    heads of 64 x 64 and nothing to differentiate (the backward needs the mapped tensors, so a
-    call that records a graph maps them first with `elu_plus_one`)."""
+    """True when a plain forward call suffices: the kernels apply elu(x) + 1 to q and k as they
+    load them (16-bit heads of 64 x 64) and nothing is to be differentiated (a call that records a
+    graph goes through the autograd nodes, whose backward kernels map on load as well)."""
     if not mapped_in_kernels(q, v):
         return False
     return not (torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)))

@@ -39,18 +39,17 @@ class LinearAttnFunction(torch.autograd.Function):
 
 
 class MappedLinearAttnFunction(torch.autograd.Function):
-    """linear_attention(elu(q) + 1, elu(k) + 1, v) as one autograd node (16-bit heads of 64 x 64):
-    the forward maps q and k with one launch and keeps the mapped tensors (the backward needs
-    them, not the raw ones); the backward kernels return dq and dk with respect to the raw
-    tensors themselves (times min(mapped, 1), the map's derivative), so that the two elementwise
-    launches of the map's autograd disappear."""
+    """linear_attention(elu(q) + 1, elu(k) + 1, v) as one autograd node (16-bit heads of 64 x 64).
+    No mapped copy of q or k is ever written: the forward kernels map q and k as they load them,
+    the backward kernels do the same and return dq and dk with respect to the raw tensors (times
+    min(mapped, 1), the map's derivative), so the map costs no launch and no tensor pass of its
+    own in either direction."""
 
     @staticmethod
     @contiguous
     def forward(ctx, q, k, v, scale, eps):
-        qm, km_ = _hip.elu1_fwd(q, k)
-        o, s, km = _hip.la_fwd(qm, km_, v, None, None, scale, eps, _hip.NORMALIZE)
-        ctx.save_for_backward(qm, km_, v, s, km)
+        o, s, km = _hip.la_fwd(q, k, v, None, None, scale, eps, _hip.NORMALIZE | _hip.ELU1_QK)
+        ctx.save_for_backward(q, k, v, s, km)
         ctx.scale = scale
         ctx.eps = eps
         return o
@@ -58,9 +57,9 @@ class MappedLinearAttnFunction(torch.autograd.Function):
     @staticmethod
     @contiguous
     def backward(ctx, do):
-        qm, km_, v, s, km = ctx.saved_tensors
-        dq, dk, dv, _, _ = _hip.la_bwd(qm, km_, v, None, None, do, s, km, ctx.scale, ctx.eps,
-                                       _hip.NORMALIZE | _hip.ELU1_GRAD)
+        q, k, v, s, km = ctx.saved_tensors
+        dq, dk, dv, _, _ = _hip.la_bwd(q, k, v, None, None, do, s, km, ctx.scale, ctx.eps,
+                                       _hip.NORMALIZE | _hip.ELU1_QK | _hip.ELU1_GRAD)
         return dq, dk, dv, None, None
 
 
@@ -84,9 +83,9 @@ def linear_attention(
             q and k are given before the blocks' feature map `elu(x) + 1`
             (layers/linfusion.py:88-89).  An inference forward of 16-bit heads of 64 x 64 applies
             it inside the kernels as they load q and k (no mapped copies are written); with
-            gradients, the same heads map q and k with one launch and get dq, dk with respect to
-            the raw tensors from the backward kernels; every other call maps them first and lets
-            autograd differentiate the map.
+            gradients, the backward kernels of the same heads map q and k on load as well and
+            return dq, dk with respect to the raw tensors; every other call maps them first and
+            lets autograd differentiate the map.
     Returns the output of shape `(B, H, L, V)` with `v`'s dtype.
     """
     check_dense("linear_attention", q, k, v)

@@ -47,11 +47,14 @@ extern "C" {
 #define FBLA_ELU1_QK 8       /* forward entry points only: q and k are given BEFORE the callers' feature map
                               * phi(x) = elu(x) + 1 (layers/linfusion.py:88-89, layers/mlla.py:74-75) and the
                               * kernels apply it as they load them; fp16 / bf16, DK = DV = 64, not decoupled
-                              * (FBLA_ERR_UNSUPPORTED otherwise, and from the backward entry points) */
+                              * (FBLA_ERR_UNSUPPORTED otherwise, and from the backward entry points without
+                              * FBLA_ELU1_GRAD) */
 #define FBLA_ELU1_GRAD 16    /* backward entry points only: q and k are the MAPPED tensors phi(x) = elu(x) + 1 (what
                               * the forward consumed and saved) and dq, dk are wanted with respect to x: the
                               * kernels multiply them by phi'(x) = min(phi(x), 1) as they write them, which
-                              * replaces the autograd of `F.elu(x) + 1.0` (two elementwise launches per call);
+                              * replaces the autograd of `F.elu(x) + 1.0` (two elementwise launches per call).
+                              * Together with FBLA_ELU1_QK, q and k are given before the map here as well and the
+                              * backward kernels map them on load (no mapped copies exist anywhere).
                               * fp16 / bf16, DK = DV = 64, not decoupled (FBLA_ERR_UNSUPPORTED otherwise) */
 
 /* error codes */

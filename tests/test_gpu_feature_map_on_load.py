@@ -124,16 +124,24 @@ def test_gradients_with_respect_to_the_raw_tensors_from_the_kernels(B, H, L, dty
     close = 1e-2 if dtype == torch.bfloat16 else 2e-3
     for name, x, y in zip(("dq", "dk", "dv"), a, b):
         assert max_rel_err(x.grad, np64(y.grad)) < close, name
-    # without the denominator: dq, dk of simple_la on mapped tensors, gated by the kernels
+    # the C ABI's other form: q, k are the mapped tensors (a binding that kept them), gradients gated
     qm, km_ = elu_plus_one(q.cuda(), k.cuda())
+    _, s, km = _hip.la_fwd(qm, km_, v.cuda(), None, None, 1.0 / L, 1e-6, _hip.NORMALIZE)
+    dq, dk, dv, _, _ = _hip.la_bwd(qm, km_, v.cuda(), None, None, do, s, km, 1.0 / L, 1e-6,
+                                   _hip.NORMALIZE | _hip.ELU1_GRAD)
+    for name, x, y in zip(("dq", "dk", "dv"), (dq, dk, dv), b):
+        assert max_rel_err(x, np64(y.grad)) < close, name + " from mapped tensors"
+    # without the denominator (the simple_la family), from mapped and from raw tensors
     scale = 0.125
     _, s, km = _hip.la_fwd(qm, km_, v.cuda(), None, None, scale, 1e-6, 0)
-    dq, dk, dv, _, _ = _hip.la_bwd(qm, km_, v.cuda(), None, None, do, s, km, scale, 1e-6, _hip.ELU1_GRAD)
     ref = cf.dense_backward(np64(qm), np64(km_), np64(v), np64(do), scale, 1e-6, False)
     gate = lambda m: np.minimum(np64(m), 1.0)
-    assert_parity(dq, ref["dq"] * gate(qm), dtype, "simple dq", ref["dq_mag"] if "dq_mag" in ref else None)
-    assert_parity(dk, ref["dk"] * gate(km_), dtype, "simple dk", ref["dk_mag"] if "dk_mag" in ref else None)
-    assert_parity(dv, ref["dv"], dtype, "simple dv", ref["dv_mag"] if "dv_mag" in ref else None)
+    for what, args, flags in (("mapped", (qm, km_), _hip.ELU1_GRAD),
+                              ("raw", (q.cuda(), k.cuda()), _hip.ELU1_QK | _hip.ELU1_GRAD)):
+        dq, dk, dv, _, _ = _hip.la_bwd(*args, v.cuda(), None, None, do, s, km, scale, 1e-6, flags)
+        assert_parity(dq, ref["dq"] * gate(qm), dtype, f"simple dq from {what}", ref.get("dq_mag"))
+        assert_parity(dk, ref["dk"] * gate(km_), dtype, f"simple dk from {what}", ref.get("dk_mag"))
+        assert_parity(dv, ref["dv"], dtype, f"simple dv from {what}", ref.get("dv_mag"))
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
@@ -177,7 +185,7 @@ def test_argument_and_flag_errors():
     with pytest.raises(ValueError, match="feature map on load"):
         _hip.la_fwd(q32, k32, v32, None, None, 1.0, 1e-6, _hip.NORMALIZE | _hip.ELU1_QK)
     o, s, km = _hip.la_fwd(q, k, v, None, None, 1.0, 1e-6, _hip.NORMALIZE)
-    with pytest.raises(ValueError, match="forward only"):
+    with pytest.raises(ValueError, match="needs FBLA_ELU1_GRAD"):
         _hip.la_bwd(q, k, v, None, None, torch.ones_like(v), s, km, 1.0, 1e-6, _hip.NORMALIZE | _hip.ELU1_QK)
     with pytest.raises(ValueError, match="backward entry points"):
         _hip.la_fwd(q, k, v, None, None, 1.0, 1e-6, _hip.NORMALIZE | _hip.ELU1_GRAD)
