@@ -44,11 +44,11 @@ extern "C" {
 #define FBLA_NORMALIZE 1     /* o = (q S)/(q.km + eps); clear = simple_la (no denominator) */
 #define FBLA_DECOUPLED 2     /* numerator from q_rope/k_rope, denominator from q/k */
 #define FBLA_DEFAULT_SCALE 4 /* packed layout only: scale = 1/len_i per sequence */
-#define FBLA_ELU1_QK 8       /* forward entry points only: q and k are given BEFORE the callers' feature map
+#define FBLA_ELU1_QK 8       /* q and k are given BEFORE the callers' feature map
                               * phi(x) = elu(x) + 1 (layers/linfusion.py:88-89, layers/mlla.py:74-75) and the
                               * kernels apply it as they load them; fp16 / bf16, DK = DV = 64, not decoupled
-                              * (FBLA_ERR_UNSUPPORTED otherwise, and from the backward entry points without
-                              * FBLA_ELU1_GRAD) */
+                              * (FBLA_ERR_UNSUPPORTED otherwise); the backward entry points take it together
+                              * with FBLA_ELU1_GRAD only */
 #define FBLA_ELU1_GRAD 16    /* backward entry points only: q and k are the MAPPED tensors phi(x) = elu(x) + 1 (what
                               * the forward consumed and saved) and dq, dk are wanted with respect to x: the
                               * kernels multiply them by phi'(x) = min(phi(x), 1) as they write them, which
