@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kThreads) void chunk_sums16_kernel(
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
   // 32 rows per trip: half a chunk of the usual size is in flight before the first sum (a whole
-  // one costs so many registers that the waves of config 5 no longer fit the GPU at once)
+  // one costs so many registers that the 6144 waves of a B1-H24-T16384 problem no longer fit the GPU at once)
   constexpr int NLD = 32 / RPI;
   for (int base = 0; base < n; base += 32) {
     u32x4s w[NLD];
