@@ -146,12 +146,6 @@ template <typename T> __device__ __forceinline__ uint32_t phi_pair(uint32_t w) {
   return pack2<T>(Ops<T>::lo(e) + 1.f, Ops<T>::hi(e) + 1.f);
 }
 
-// A pair of gradients with respect to phi(x) times phi'(x) = min(phi(x), 1) (phi = elu + 1: 1 for
-// x > 0, exp(x) = phi(x) otherwise), from the pair of mapped values.
-template <typename T> __device__ __forceinline__ uint32_t gate_pair(uint32_t grad, uint32_t mapped) {
-  return pack2<T>(Ops<T>::lo(grad) * fminf(Ops<T>::lo(mapped), 1.f), Ops<T>::hi(grad) * fminf(Ops<T>::hi(mapped), 1.f));
-}
-
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 // Eight tokens of one feature (an MFMA operand fragment of one k-step) out of a row-major tile:
 // two transposing reads, `off0` / `off1` are this lane's byte offsets for x = 0 / 1.
@@ -905,12 +899,12 @@ __device__ __forceinline__ void build_vec(uint32_t* pairs, float* f32, const flo
 // z_t = q_t . km is computed from the flat registers the rows were loaded into instead (the
 // lanes that hold the 16-byte pieces of one row add their partial dot products; kDenFlat).
 template <int DR, int DC, bool DEN> constexpr bool den_flat() { return DEN && !(DR == 64 && DC == 64); }
-template <int DR, int DC, bool DEN, int WAVES> struct RowsLayout {
+template <int DR, int DC, bool DEN, int WAVES, bool GATE = false> struct RowsLayout {
   static constexpr int KS = DR / 16, NB = DC / 32;
   static constexpr int kStage = 32 * 2 * (DR > DC ? DR : DC);  // one 32-token tile of the wider side
   static constexpr int kOpnd = NB * KS * 2 * 1024;
   static constexpr int kStages = kOpnd;
-  static constexpr int kKm = kStages + WAVES * (DEN && !den_flat<DR, DC, DEN>() ? 2 : 1) * kStage;
+  static constexpr int kKm = kStages + WAVES * ((DEN && !den_flat<DR, DC, DEN>()) || GATE ? 2 : 1) * kStage;
   static constexpr int kAdd = kKm + DR * 4;
   static constexpr int kMax = kAdd + DC * 4;
   static constexpr int kZrow = kMax + 64;                                       // [WAVES][32] z of the wave's tile
@@ -940,7 +934,7 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
 
   const int dr = PAD ? dr_true : (PAIR ? 32 : DR), dc = PAD ? dc_true : (PAIR ? 32 : DC);
   const int dpk = PAD ? (p.DK <= 64 ? 64 : 128) : p.DK;  // padded length of the km / dkm vector
-  using LY = RowsLayout<DR, DC, DEN, WAVES>;
+  using LY = RowsLayout<DR, DC, DEN, WAVES, GATE>;
   const bool second = (int)blockIdx.x >= wgs_per_job;
   const RowsJob& job = second ? job1 : job0;
   // FMAP and GATE together (pass B of a backward given the rows before the map): a job maps its x rows
@@ -1006,7 +1000,7 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
   // before the prologue so that its latency overlaps the operand build.
   const int ntok = lane & 31, kb = lane >> 5;  // MFMA view: token column, k half
   constexpr bool kDenFlat = den_flat<DR, DC, DEN>();
-  unsigned char* stage = smem + LY::kStages + wave * (DEN && !kDenFlat ? 2 : 1) * kStage;
+  unsigned char* stage = smem + LY::kStages + wave * ((DEN && !kDenFlat) || GATE ? 2 : 1) * kStage;
   unsigned char* stage_den = stage + kStage;
   float* zrow = reinterpret_cast<float*>(smem + LY::kZrow) + 32 * wave;  // kDenFlat only
   constexpr int XI = 32 * XCH / 64;  // flat 16-byte loads per lane per tile
@@ -1113,6 +1107,17 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
     }
     stash_tile(xcur, stage);
     if constexpr (DEN && !kDenFlat) stash_tile(dcur, stage_den);
+    if constexpr (GATE) {
+      if (gate) {  // the same for all lanes: the mapped rows go to the second stage, to be read per token
+        if constexpr (FMAP) {
+#pragma unroll
+          for (int i = 0; i < XI; ++i)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) gcur[i][w] = phi_pair<T>(gcur[i][w]);
+        }
+        stash_tile(gcur, stage_den);
+      }
+    }
     if constexpr (kDenFlat) {
       // piece i of this lane is chunk lane % XCH of row lane / XCH + (64 / XCH) i: its dot product
       // with the km values of that chunk, then the sum over the XCH lanes of the row
@@ -1138,6 +1143,9 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
     } else if (tn < t_end) {
       load_tile(xcur, x, tn);
       if constexpr (DEN) load_tile(dcur, xden, tn);
+    }
+    if constexpr (GATE) {
+      if (gate && tn < t_end) load_tile(gcur, gate, tn);
     }
     wave_sync();
 
@@ -1195,7 +1203,24 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
       rs = denorm / (z + p.eps);
     }
     wave_sync();  // all lanes have read their x chunks; staging is reused for out
-    if (has_add) {  // only the dk job of the backward adds a row (dkm / L)
+    if (GATE && gate) {  // out = (acc * rs + add) * min(mapped, 1): everything before the one rounding
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        u32x4 w0, w1;
+        const float* av = &lds_add[(DC / 2) * kb + 16 * b];
+        const u32x4 g0 = *reinterpret_cast<const u32x4*>(stage_den + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b));
+        const u32x4 g1 = *reinterpret_cast<const u32x4*>(stage_den + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b + 1));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          w0[i] = pack2<T>(fmaf(acc[b][2 * i], rs, av[2 * i]) * fminf(Ops<T>::lo(g0[i]), 1.f),
+                           fmaf(acc[b][2 * i + 1], rs, av[2 * i + 1]) * fminf(Ops<T>::hi(g0[i]), 1.f));
+          w1[i] = pack2<T>(fmaf(acc[b][8 + 2 * i], rs, av[8 + 2 * i]) * fminf(Ops<T>::lo(g1[i]), 1.f),
+                           fmaf(acc[b][8 + 2 * i + 1], rs, av[8 + 2 * i + 1]) * fminf(Ops<T>::hi(g1[i]), 1.f));
+        }
+        *reinterpret_cast<u32x4*>(stage + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b)) = w0;
+        *reinterpret_cast<u32x4*>(stage + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b + 1)) = w1;
+      }
+    } else if (has_add) {  // only the dk job of the backward adds a row (dkm / L)
 #pragma unroll
       for (int b = 0; b < NB; ++b) {
         u32x4 w0, w1;
@@ -1228,16 +1253,6 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
     for (int i = 0; i < OI; ++i) {
       const int q = lane + 64 * i;
       wout[i] = *reinterpret_cast<const u32x4*>(stage + swz<OROWB>(q / OCH, q % OCH));
-    }
-    if constexpr (GATE) {
-      if (gate) {  // the same for all lanes
-#pragma unroll
-        for (int i = 0; i < OI; ++i)
-#pragma unroll
-          for (int w = 0; w < 4; ++w) wout[i][w] = gate_pair<T>(wout[i][w], FMAP ? phi_pair<T>(gcur[i][w]) : gcur[i][w]);
-        // this set is free now: the mapped rows of the tile PF steps ahead
-        if (t0 + t_stride * PF < t_end) load_tile(gcur, gate, t0 + t_stride * PF);
-      }
     }
     if ((FBLA_ROWS_FAST & 2) && !NORM && kFast && t0 + 32 <= t_end) {
       char* tp = const_cast<char*>(tile_ptr(out, t0, DC));
@@ -2473,7 +2488,7 @@ template <typename T, int DR, int DC, bool NORM, bool DEN, int WAVES, bool PAD, 
           bool GATE = false>
 static int launch_rows_k(const Prob& p, const RowsJob& job, const RowsJob* job2, int chunk,
                          int nchunks, int dr, int dc, hipStream_t st) {
-  using LY = RowsLayout<DR, DC, DEN, WAVES>;
+  using LY = RowsLayout<DR, DC, DEN, WAVES, GATE>;
   constexpr int PF = (DR == 128 && DC == 128) ? FBLA_ROWS_PF128 : FBLA_ROWS_PF;
   auto kernel = rows_kernel<T, DR, DC, NORM, DEN, WAVES, PAD, PF, PAIR, FMAP, GATE>;
   static thread_local bool configured = false;

@@ -145,6 +145,29 @@ def test_gradients_with_respect_to_the_raw_tensors_from_the_kernels(B, H, L, dty
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("D", [64, 32])
+def test_simple_la_with_the_feature_map(D, dtype):
+    """simple_la(..., feature_map="elu+1"): forward and gradients against the oracle on the mapped
+    tensors, for the head size the kernels map themselves and for one that is mapped first."""
+    from flash_bla.ops.simple_la.fused import simple_la
+    B, H, L = 2, 2, 700
+    q, k, v = _raw((B, H, L, D), (B, H, L, D), dtype, seed=D, spread=1.0)
+    do = torch.randn(B, H, L, D, generator=torch.Generator().manual_seed(8)).to(dtype)
+    with torch.no_grad():
+        o_inference = simple_la(q.cuda(), k.cuda(), v.cuda(), feature_map="elu+1")
+    leaves = [t.cuda().requires_grad_() for t in (q, k, v)]
+    o = simple_la(*leaves, feature_map="elu+1")
+    o.backward(do.cuda())
+    ref = cf.dense_backward(np64(_mapped(q)), np64(_mapped(k)), np64(v), np64(do), D ** -0.5, 1e-6, False)
+    dphi = lambda x: np.where(np64(x) > 0, 1.0, np.exp(np.minimum(np64(x), 0.0)))
+    assert_parity(o_inference, ref["o"], dtype, "o (inference)")
+    assert_parity(o, ref["o"], dtype, "o")
+    assert_parity(leaves[0].grad, ref["dq"] * dphi(q), dtype, "dq", ref.get("dq_mag"))
+    assert_parity(leaves[1].grad, ref["dk"] * dphi(k), dtype, "dk", ref.get("dk_mag"))
+    assert_parity(leaves[2].grad, ref["dv"], dtype, "dv", ref.get("dv_mag"))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
 def test_packed_gradients_through_the_feature_map(dtype):
     from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
     lens = [5, 300, 1, 64, 1000, 17, 0, 2049]
