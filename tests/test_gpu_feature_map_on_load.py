@@ -59,6 +59,24 @@ def test_fewer_or_more_keys_than_queries(lq, lk, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("lq,lk", [(300, 75), (64, 1000)])
+def test_gradients_with_fewer_or_more_keys_than_queries(lq, lk, dtype):
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    q, _, _ = _raw((2, 3, lq, 64), (2, 3, lq, 64), dtype, seed=lq + 3)
+    _, k, v = _raw((2, 3, lk, 64), (2, 3, lk, 64), dtype, seed=lk + 3)
+    do = torch.randn(2, 3, lq, 64, generator=torch.Generator().manual_seed(lq)).to(dtype)
+    leaves = [t.cuda().requires_grad_() for t in (q, k, v)]
+    o = linear_attention(*leaves, feature_map="elu+1")
+    o.backward(do.cuda())
+    ref = cf.dense_backward(np64(_mapped(q)), np64(_mapped(k)), np64(v), np64(do), 1.0 / lk)
+    dphi = lambda x: np.where(np64(x) > 0, 1.0, np.exp(np.minimum(np64(x), 0.0)))
+    assert_parity(o, ref["o"], dtype, "o")
+    assert_parity(leaves[0].grad, ref["dq"] * dphi(q), dtype, "dq", ref.get("dq_mag"))
+    assert_parity(leaves[1].grad, ref["dk"] * dphi(k), dtype, "dk", ref.get("dk_mag"))
+    assert_parity(leaves[2].grad, ref["dv"], dtype, "dv", ref.get("dv_mag"))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
 def test_unnormalised_forward_maps_on_load(dtype):
     """The C ABI's flag without FBLA_NORMALIZE (the simple_la family)."""
     from flash_bla import _hip
