@@ -232,9 +232,10 @@ def main():
                          "followed by a 256 MiB device copy of known traffic, then exit")
     ap.add_argument("--tables", action="store_true",
                     help="also print the reference's benchmark tables (torch formula, this library, SDPA) on stderr")
-    ap.add_argument("--only", choices=["c3", "c5"], default=None,
+    ap.add_argument("--only", choices=["c3", "c5", "fm"], default=None,
                     help="profiling aid: time just BASELINE config 3 (packed variable-length, D=64 and "
-                         "D=128) or config 5 (piecewise attention), table on stderr, no headline line")
+                         "D=128), config 5 (piecewise attention) or the feature map together with the "
+                         "attention (fm), table on stderr, no headline line")
     ap.add_argument("--configs", action="store_true",
                     help="also time the other operator families / BASELINE configs (table on stderr)")
     args = ap.parse_args()
@@ -254,6 +255,8 @@ def main():
         flush = torch.empty(256 << 20, dtype=torch.int8, device=dev)
         if args.only == "c3":
             varlen_config(dev, flush)
+        elif args.only == "fm":
+            feature_map_config(dev, flush)
         else:
             piecewise_config(dev, flush)
         return
@@ -411,6 +414,50 @@ def _report(name, nbytes_fwd, nbytes_step, fwd_fn, step_fn, flush, extra=None):
     print(json.dumps(row), file=sys.stderr, flush=True)
 
 
+def feature_map_config(dev, flush):
+    """The blocks' feature map elu(x) + 1 together with linear_attn at the headline shape: applied by
+    the kernels as they load q and k (forward; forward + backward with dq, dk from the kernels)
+    against the map as launches of its own."""
+    from flash_bla.ops.linear_attn.fused import linear_attention
+
+    def leaves(*ts):
+        return [t.requires_grad_() for t in ts]
+
+    # the blocks' feature map with the attention (inference forward): applied by the kernels as they
+    # load q and k, against one elementwise launch for q and k followed by the operator
+    from flash_bla.ops.feature_map import elu_plus_one
+    g = torch.Generator(device=dev).manual_seed(3)
+    q, k, v = (torch.randn((8, 16, 16384, 64), generator=g, device=dev).half() for _ in range(3))
+    nb = q.numel() * 2
+    with torch.no_grad():
+        t_load = do_bench(lambda: linear_attention(q, k, v, feature_map="elu+1"), flush)
+        t_first = do_bench(lambda: linear_attention(*elu_plus_one(q, k), v), flush)
+    # training step through the map: dq, dk with respect to the raw tensors from the backward kernels,
+    # against the map differentiated by autograd (two more elementwise launches)
+    from flash_bla.ops.linear_attn.fused import LinearAttnFunction
+    do = torch.randn(q.shape, generator=g, device=dev).half()
+    leaves(q, k, v)
+
+    def step_kernels():
+        linear_attention(q, k, v, feature_map="elu+1").backward(do)
+        q.grad = k.grad = v.grad = None
+
+    def step_autograd():
+        LinearAttnFunction.apply(*elu_plus_one(q, k), v, 1.0 / q.shape[2], 1e-6).backward(do)
+        q.grad = k.grad = v.grad = None
+
+    t_step = do_bench(step_kernels, flush)
+    t_step_auto = do_bench(step_autograd, flush)
+    print(json.dumps({"config": "elu+1 feature map + linear_attn B8-H16-T16384-D64 fp16",
+                      "fwd_mapped_on_load_ms": round(t_load[0], 5),
+                      "fwd_mapped_on_load_gbps": round(4 * nb / t_load[0] / 1e6, 1),
+                      "fwd_mapped_on_load_frac": round(4 * nb / t_load[0] / 1e6 / HBM_PEAK_GBPS, 4),
+                      "fwd_mapped_first_ms": round(t_first[0], 5),
+                      "fwd_bwd_gradients_from_kernels_ms": round(t_step[0], 5),
+                      "fwd_bwd_map_by_autograd_ms": round(t_step_auto[0], 5)}), file=sys.stderr, flush=True)
+    del q, k, v, do
+
+
 def other_configs(dev, flush):
     """Flushed-median timings of the remaining BASELINE configs and operator families."""
     from flash_bla.ops.linear_attn.decoupled import decoupled_la
@@ -453,39 +500,7 @@ def other_configs(dev, flush):
         else:
             f, s = run(simple_la, (q, k, v), do)
             _report(f"simple_la B8-H16-T16384-D64 {tag}", 4 * nb, 11 * nb, f, s, flush)
-    # the blocks' feature map with the attention (inference forward): applied by the kernels as they
-    # load q and k, against one elementwise launch for q and k followed by the operator
-    from flash_bla.ops.feature_map import elu_plus_one
-    g = torch.Generator(device=dev).manual_seed(3)
-    q, k, v = (torch.randn((8, 16, 16384, 64), generator=g, device=dev).half() for _ in range(3))
-    nb = q.numel() * 2
-    with torch.no_grad():
-        t_load = do_bench(lambda: linear_attention(q, k, v, feature_map="elu+1"), flush)
-        t_first = do_bench(lambda: linear_attention(*elu_plus_one(q, k), v), flush)
-    # training step through the map: dq, dk with respect to the raw tensors from the backward kernels,
-    # against the map differentiated by autograd (two more elementwise launches)
-    from flash_bla.ops.linear_attn.fused import LinearAttnFunction
-    do = torch.randn(q.shape, generator=g, device=dev).half()
-    leaves(q, k, v)
-
-    def step_kernels():
-        linear_attention(q, k, v, feature_map="elu+1").backward(do)
-        q.grad = k.grad = v.grad = None
-
-    def step_autograd():
-        LinearAttnFunction.apply(*elu_plus_one(q, k), v, 1.0 / q.shape[2], 1e-6).backward(do)
-        q.grad = k.grad = v.grad = None
-
-    t_step = do_bench(step_kernels, flush)
-    t_step_auto = do_bench(step_autograd, flush)
-    print(json.dumps({"config": "elu+1 feature map + linear_attn B8-H16-T16384-D64 fp16",
-                      "fwd_mapped_on_load_ms": round(t_load[0], 5),
-                      "fwd_mapped_on_load_gbps": round(4 * nb / t_load[0] / 1e6, 1),
-                      "fwd_mapped_on_load_frac": round(4 * nb / t_load[0] / 1e6 / HBM_PEAK_GBPS, 4),
-                      "fwd_mapped_first_ms": round(t_first[0], 5),
-                      "fwd_bwd_gradients_from_kernels_ms": round(t_step[0], 5),
-                      "fwd_bwd_map_by_autograd_ms": round(t_step_auto[0], 5)}), file=sys.stderr, flush=True)
-    del q, k, v, do
+    feature_map_config(dev, flush)
     q, k, v, do = make_inputs(2, 16, 16384, 64, torch.bfloat16, dev)
     qr, kr, _, _ = make_inputs(2, 16, 16384, 64, torch.bfloat16, dev, seed=7)
     leaves(q, k, qr, kr, v)
