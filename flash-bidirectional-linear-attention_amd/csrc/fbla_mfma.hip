@@ -1108,15 +1108,7 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
     stash_tile(xcur, stage);
     if constexpr (DEN && !kDenFlat) stash_tile(dcur, stage_den);
     if constexpr (GATE) {
-      if (gate) {  // the same for all lanes: the mapped rows go to the second stage, to be read per token
-        if constexpr (FMAP) {
-#pragma unroll
-          for (int i = 0; i < XI; ++i)
-#pragma unroll
-            for (int w = 0; w < 4; ++w) gcur[i][w] = phi_pair<T>(gcur[i][w]);
-        }
-        stash_tile(gcur, stage_den);
-      }
+      if (gate) stash_tile(gcur, stage_den);  // (the same for all lanes) to be read per token below
     }
     if constexpr (kDenFlat) {
       // piece i of this lane is chunk lane % XCH of row lane / XCH + (64 / XCH) i: its dot product
@@ -1203,7 +1195,9 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
       rs = denorm / (z + p.eps);
     }
     wave_sync();  // all lanes have read their x chunks; staging is reused for out
-    if (GATE && gate) {  // out = (acc * rs + add) * min(mapped, 1): everything before the one rounding
+    if (GATE && gate) {  // out = (acc * rs + add) * phi'(x): everything before the one rounding
+      // phi'(x) = 1 for x > 0, exp(x) otherwise: from x itself (FMAP), or as min(phi(x), 1) from the mapped value
+      auto dphi = [](float g) { return FMAP ? (g > 0.f ? 1.f : __expf(g)) : fminf(g, 1.f); };
 #pragma unroll
       for (int b = 0; b < NB; ++b) {
         u32x4 w0, w1;
@@ -1212,10 +1206,10 @@ __global__ __launch_bounds__(WAVES * 64, (FBLA_ROWS_OCC4 && DR == 64 && DC == 64
         const u32x4 g1 = *reinterpret_cast<const u32x4*>(stage_den + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b + 1));
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          w0[i] = pack2<T>(fmaf(acc[b][2 * i], rs, av[2 * i]) * fminf(Ops<T>::lo(g0[i]), 1.f),
-                           fmaf(acc[b][2 * i + 1], rs, av[2 * i + 1]) * fminf(Ops<T>::hi(g0[i]), 1.f));
-          w1[i] = pack2<T>(fmaf(acc[b][8 + 2 * i], rs, av[8 + 2 * i]) * fminf(Ops<T>::lo(g1[i]), 1.f),
-                           fmaf(acc[b][8 + 2 * i + 1], rs, av[8 + 2 * i + 1]) * fminf(Ops<T>::hi(g1[i]), 1.f));
+          w0[i] = pack2<T>(fmaf(acc[b][2 * i], rs, av[2 * i]) * dphi(Ops<T>::lo(g0[i])),
+                           fmaf(acc[b][2 * i + 1], rs, av[2 * i + 1]) * dphi(Ops<T>::hi(g0[i])));
+          w1[i] = pack2<T>(fmaf(acc[b][8 + 2 * i], rs, av[8 + 2 * i]) * dphi(Ops<T>::lo(g1[i])),
+                           fmaf(acc[b][8 + 2 * i + 1], rs, av[8 + 2 * i + 1]) * dphi(Ops<T>::hi(g1[i])));
         }
         *reinterpret_cast<u32x4*>(stage + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b)) = w0;
         *reinterpret_cast<u32x4*>(stage + swz<OROWB>(ntok, (OCH / 2) * kb + 2 * b + 1)) = w1;
