@@ -2386,8 +2386,17 @@ int rows_chunk(const Prob& p, int DR, int DC) {
   static const int packed_rounds = knob("FBLA_ROWS_ROUNDS_PACKED", 1);
   // a 128 x 128 operand costs as much to build as 512 tokens cost to stream: one round there
   const int big = (tiled_dim(DR) == 128) + (tiled_dim(DC) == 128);
-  const int rounds = p.cu ? packed_rounds : (big == 2 ? 1 : big == 1 ? (dense_rounds + 1) / 2 : dense_rounds);
   const int per_cu = big == 0 ? per_cu_knob : (big == 1 || use_rows128(p) ? 2 : 1);
+  int rounds = p.cu ? packed_rounds : (big == 2 ? 1 : big == 1 ? (dense_rounds + 1) / 2 : dense_rounds);
+  // packed batches of 64-wide tiles whose lengths are of one order (not the one-long-among-short
+  // case that chunk_for treats by itself): up to three chunks per sequence, so that the longest
+  // sequences, which start first, do not each keep one workgroup busy to the end (64 sequences of
+  // 256..2048 tokens, H16-D64: forward output 84 -> 75 us, forward + backward 0.427 -> 0.404 ms)
+  static const int even_rounds = knob("FBLA_ROWS_ROUNDS_PACKED_EVEN", 3);
+  if (p.cu && big == 0 && rounds < even_rounds) {
+    const int64_t fair = cdiv64(p.T * p.H, (int64_t)cu_count() * per_cu * rounds);
+    if (p.L <= 4 * fair) rounds = even_rounds;
+  }
   static const int min_chunk_knob = knob("FBLA_ROWS_MIN_CHUNK", 256);
   // a problem too small to give every CU a workgroup: shorter chunks (the operand build of the
   // extra workgroups costs less than the idle CUs)
