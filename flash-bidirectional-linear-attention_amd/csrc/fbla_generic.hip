@@ -598,8 +598,51 @@ __global__ __launch_bounds__(kThreads) void broadcast_rows_kernel(Prob p, const 
   }
 }
 
+// The same for rows made of a power-of-two number of 16-byte pieces: a thread builds its piece of the
+// row once and stores it (streaming) to that piece of every row it owns.
+constexpr int kBroadcastRows = 256;
+template <typename T>
+__global__ __launch_bounds__(kThreads) void broadcast_rows16_kernel(Prob p, const float* __restrict__ vec,
+                                                                    T* __restrict__ out, int nchunks,
+                                                                    float factor, int piece_shift) {
+  typedef uint32_t words4 __attribute__((ext_vector_type(4)));
+  constexpr int E = 16 / (int)sizeof(T);
+  const int nh = blockIdx.x / nchunks, chunk = blockIdx.x - nh * nchunks;
+  const int n = nh / p.H, h = nh - n * p.H;
+  int64_t bos, row0, rstride;
+  int len;
+  seq_range(p, n, bos, len);
+  const int t0 = chunk * kBroadcastRows;
+  if (t0 >= len) return;
+  const int nvalid = min(kBroadcastRows, len - t0);
+  row_base(p, n, h, bos, row0, rstride);
+  const int piece = threadIdx.x & ((1 << piece_shift) - 1), first = threadIdx.x >> piece_shift;
+  const int step = kThreads >> piece_shift;
+  union { T e[E]; words4 w; } val;
+  for (int i = 0; i < E; ++i) val.e[i] = from_f32<T>(vec[(int64_t)nh * p.DK + piece * E + i] * factor);
+  T* dst = out + (row0 + (int64_t)(t0 + first) * rstride) * p.DK + piece * E;
+  const int64_t stride = (int64_t)step * rstride * p.DK;
+  for (int t = first; t < nvalid; t += step, dst += stride) __builtin_nontemporal_store(val.w, (words4*)dst);
+}
+
+template <typename T>
+static bool broadcast_rows16(const Prob& p, const float* vec, T* out, hipStream_t st, float factor) {
+  const int row_bytes = p.DK * (int)sizeof(T), pieces = row_bytes / 16;
+  if (row_bytes % 16 || (pieces & (pieces - 1)) || pieces > kThreads || ((uintptr_t)out & 15)) return false;
+  int shift = 0;
+  while ((1 << shift) < pieces) ++shift;
+  const int nchunks = (int)cdiv64(p.L, kBroadcastRows);
+  broadcast_rows16_kernel<T><<<dim3((unsigned)((int64_t)p.N * p.H * nchunks)), dim3(kThreads), 0, st>>>(
+      p, vec, out, nchunks, factor, shift);
+  return true;
+}
+
 // every row of out ([.., DK]) = vec of its (sequence, head): dk of the decoupled operator
 void broadcast_rows(const Prob& p, int dtype, const float* vec, void* out, hipStream_t st, float factor) {
+  if (dtype == kF16 ? broadcast_rows16(p, vec, (_Float16*)out, st, factor)
+      : dtype == kBF16 ? broadcast_rows16(p, vec, (__bf16*)out, st, factor)
+                       : broadcast_rows16(p, vec, (float*)out, st, factor))
+    return;
   const int ntiles = (int)cdiv64(p.L, kTile);
   const dim3 grid((unsigned)((int64_t)p.N * p.H * ntiles)), block(kThreads);
   if (dtype == kF16) broadcast_rows_kernel<_Float16><<<grid, block, 0, st>>>(p, vec, (_Float16*)out, ntiles, factor);
