@@ -2291,12 +2291,18 @@ bool supported(const Prob& p, int dtype) {
 
 // The fused backward pass A exists for heads tiled as 64 x 64 and as 128 x 128 (the latter
 // not for the decoupled operator).
+static int knob(const char* name, int dflt);
 bool bwd_a_supported(const Prob& p, int dtype) {
-  if (dtype == kF32 || !supported(p, dtype) || tiled_dim(p.DK) != tiled_dim(p.DV)) return false;
+  if (dtype == kF32 || !supported(p, dtype)) return false;
+  const bool wide = tiled_dim(p.DK) == 128 || tiled_dim(p.DV) == 128;
+  // heads with one 128-wide side run as padded 128 x 128 heads of the plain operator (one pass over
+  // q and dO instead of two)
+  static const bool mixed = knob("FBLA_BWDA_MIXED", 1) == 1;
+  if (tiled_dim(p.DK) != tiled_dim(p.DV) && ((p.flags & kDecoupled) || !mixed)) return false;
   // the 128 x 128 kernel addresses a step's rows with 32-bit lane offsets
-  if (tiled_dim(p.DK) == 128 && p.cu && p.H > 65536) return false;
+  if (wide && p.cu && p.H > 65536) return false;
   // decoupled: fused for 64 x 64 tiles only (the 128 x 128 kernel has no room for the plain q tile)
-  return !(p.flags & kDecoupled) || tiled_dim(p.DK) == 64;
+  return !(p.flags & kDecoupled) || !wide;
 }
 
 // Number of compute units of the current device (256 on MI355X; also the value
@@ -2372,7 +2378,7 @@ int state_chunk(const Prob& p, bool block_stats) {
 int bwd_a_chunk(const Prob& p) {
   static const int per_cu = knob("FBLA_BWDA_WGS_PER_CU", 2);
   // 128 x 128: two workgroups of four waves per CU, steps of 64 tokens
-  if (tiled_dim(p.DK) == 128) return chunk_for(p, 2, 1, 512, 64, true);
+  if (tiled_dim(p.DK) == 128 || tiled_dim(p.DV) == 128) return chunk_for(p, 2, 1, 512, 64, true);
   return chunk_for(p, per_cu, 1, 256, 128, true);
 }
 
@@ -2726,7 +2732,7 @@ static int run_bwd_a_pad(const Prob& p, const void* qn, const void* qd, const vo
   const T *a = (const T*)qn, *b = (const T*)qd, *c = (const T*)dout;
   T *x = (T*)dqn, *y = (T*)dqd;
   if constexpr (!PAIR) {
-    if (tiled_dim(p.DK) == 128) {
+    if (tiled_dim(p.DK) == 128 || tiled_dim(p.DV) == 128) {
       if (!(p.flags & kNormalize))
         return launch_bwd_a128<T, false, PAD>(p, a, c, S, km, x, partial, fm, fv, chunk, nchunks, st);
       return launch_bwd_a128<T, true, PAD>(p, a, c, S, km, x, partial, fm, fv, chunk, nchunks, st);
@@ -2758,7 +2764,7 @@ static int run_bwd_a(const Prob& p, const void* qn, const void* qd, const void* 
   // pair mode: the chunk (a multiple of 128 tokens) becomes a count of row pairs
   if (pair_mode(p, kF16))
     return run_bwd_a_pad<T, false, true>(p, qn, qd, dout, S, km, dqn, dqd, partial, fm, fv, chunk / 2, nchunks, st);
-  if (padded(p)) return run_bwd_a_pad<T, true>(p, qn, qd, dout, S, km, dqn, dqd, partial, fm, fv, chunk, nchunks, st);
+  if (padded(p) || tiled_dim(p.DK) != tiled_dim(p.DV)) return run_bwd_a_pad<T, true>(p, qn, qd, dout, S, km, dqn, dqd, partial, fm, fv, chunk, nchunks, st);
   return run_bwd_a_pad<T, false>(p, qn, qd, dout, S, km, dqn, dqd, partial, fm, fv, chunk, nchunks, st);
 }
 
