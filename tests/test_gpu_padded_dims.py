@@ -130,10 +130,11 @@ def test_whole_state_per_wave_dense(dims, dtype, L):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("dims", [(128, 128), (104, 96), (72, 128)])
+@pytest.mark.parametrize("dims", [(128, 128), (104, 96), (72, 128), (128, 32), (64, 128), (96, 48), (16, 120)])
 def test_heads_tiled_128_around_the_64_token_steps(dims, dtype):
     """The kernels for heads tiled 128 x 128 walk steps of 64 tokens staged in LDS: lengths just
-    below, at and above one, two and three steps, one chunk and several chunks per head."""
+    below, at and above one, two and three steps, one chunk and several chunks per head.  Heads
+    with one side of at most 64 take the same backward pass A (as padded 128 x 128 heads)."""
     for i, L in enumerate([63, 64, 65, 127, 128, 129, 191, 193, 640, 1153]):
         _check_dense("linear", 1, 2, L, dims[0], dims[1], dtype, 90 * i + dims[0])
     _check_dense("simple", 2, 1, 130, dims[0], dims[1], dtype, 7 + dims[1])
