@@ -125,8 +125,8 @@ void state_with_block_stats(const Prob& p, int dtype, const void* k, const void*
 int rows(const Prob& p, int dtype, const RowsJob& job, int DR, int DC, hipStream_t st);
 int rows2(const Prob& p, int dtype, const RowsJob& job0, const RowsJob& job1, int DR, int DC,
           hipStream_t st);
-// two-kernel form of backward pass A (16-bit heads tiled 64 x 128 / 128 x 64, the decoupled operator
-// with a 128-wide side, fp32 inputs): qn / dqn are the rows of the numerator and their gradient
+// two-kernel form of backward pass A (the 16-bit decoupled operator with a 128-wide side, packed
+// batches of more than 65536 heads with one, fp32 inputs): qn / dqn are the rows of the numerator and their gradient
 // (q_rope, dq_rope when decoupled; then qd = q, dqd = dq), otherwise qn == qd and dqd is unused.
 // bwd_tokens writes dq and tokscal = [1/z_t | dz_t] per (token, head) row, scaled_state
 // accumulates the partials of dS = sum_t q_t^T (dO_t / z_t) and dkm = sum_t dz_t q_t

@@ -16,8 +16,8 @@
 //  rows32_kernel    out_t = (x_t M) * rowscale_t + addvec: forward output and both
 //                   products of backward pass B.  TOKENS: the token view of backward
 //                   pass A (x = dO, M = S^T; then q.g, z, dz, dq and the per-row scalars).
-// The backward pass A is therefore two kernels (5 tensor passes), as for 16-bit heads
-// above 64.
+// The backward pass A is therefore two kernels (5 tensor passes), as for the 16-bit decoupled
+// operator with a 128-wide side.
 #include <stdlib.h>
 
 #include "fbla_kernels.h"

@@ -253,7 +253,7 @@ int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
                            partial, chunk, nchunks, st, fm, fv);
       if (rc != kOk) return rc;
     } else if (fast) {
-      // head dims above 64: token view and feature view as two kernels
+      // no fused kernel for this shape: token view and feature view as two kernels
       const int64_t rows = p.T * p.H;
       int rc = mfma::bwd_tokens(p, dtype, qn, a.q, a.dout, a.s, a.km, dqn, dqd, tokscal, rows, st);
       if (rc != kOk) return rc;
