@@ -2393,7 +2393,10 @@ int rows_chunk(const Prob& p, int DR, int DC) {
   // a 128 x 128 operand costs as much to build as 512 tokens cost to stream: one round there
   const int big = (tiled_dim(DR) == 128) + (tiled_dim(DC) == 128);
   const int per_cu = big == 0 ? per_cu_knob : (big == 1 || use_rows128(p) ? 2 : 1);
-  int rounds = p.cu ? packed_rounds : (big == 2 ? 1 : big == 1 ? (dense_rounds + 1) / 2 : dense_rounds);
+  // (one 128-wide side: half the operand, still one round - B8-H16-T4096 fp16 fwd+bwd with two rounds
+  // DK128-DV64 0.304 against 0.298 ms, DK96-DV48 0.277 against 0.265 ms)
+  static const int rect_rounds = knob("FBLA_ROWS_ROUNDS_RECT", 1);
+  int rounds = p.cu ? packed_rounds : (big == 2 ? 1 : big == 1 ? rect_rounds : dense_rounds);
   // packed batches of 64-wide tiles whose lengths are of one order (not the one-long-among-short
   // case that chunk_for treats by itself): up to three chunks per sequence, so that the longest
   // sequences, which start first, do not each keep one workgroup busy to the end (64 sequences of
