@@ -232,10 +232,11 @@ def main():
                          "followed by a 256 MiB device copy of known traffic, then exit")
     ap.add_argument("--tables", action="store_true",
                     help="also print the reference's benchmark tables (torch formula, this library, SDPA) on stderr")
-    ap.add_argument("--only", choices=["c3", "c5", "fm"], default=None,
+    ap.add_argument("--only", choices=["c3", "c5", "fm", "callers"], default=None,
                     help="profiling aid: time just BASELINE config 3 (packed variable-length, D=64 and "
-                         "D=128), config 5 (piecewise attention) or the feature map together with the "
-                         "attention (fm), table on stderr, no headline line")
+                         "D=128), config 5 (piecewise attention), the feature map together with the "
+                         "attention (fm) or the decoupled operator and the layer callers' head dims "
+                         "(callers), table on stderr, no headline line")
     ap.add_argument("--configs", action="store_true",
                     help="also time the other operator families / BASELINE configs (table on stderr)")
     args = ap.parse_args()
@@ -257,6 +258,8 @@ def main():
             varlen_config(dev, flush)
         elif args.only == "fm":
             feature_map_config(dev, flush)
+        elif args.only == "callers":
+            caller_configs(dev, flush)
         else:
             piecewise_config(dev, flush)
         return
@@ -458,6 +461,19 @@ def feature_map_config(dev, flush):
     del q, k, v, do
 
 
+def _fwd_and_step(op, args, do_):
+    """(forward under no_grad, forward + backward with the gradients reset) of one operator call."""
+    def step():
+        for t in args:
+            t.grad = None
+        op(*args).backward(do_)
+
+    def fwd():
+        with torch.no_grad():
+            return op(*args)
+    return fwd, step
+
+
 def other_configs(dev, flush):
     """Flushed-median timings of the remaining BASELINE configs and operator families."""
     from flash_bla.ops.linear_attn.decoupled import decoupled_la
@@ -473,16 +489,7 @@ def other_configs(dev, flush):
     leaves(q, k, v)
     nb = q.numel() * 4
 
-    def run(op, args, do_):
-        def step():
-            for t in args:
-                t.grad = None
-            op(*args).backward(do_)
-
-        def fwd():
-            with torch.no_grad():
-                return op(*args)
-        return fwd, step
+    run = _fwd_and_step
 
     f, s = run(linear_attention, (q, k, v), do)
     _report("C1 linear_attn B2-H4-T1024-D64 fp32", 4 * nb, 11 * nb, f, s, flush)
@@ -501,6 +508,19 @@ def other_configs(dev, flush):
             f, s = run(simple_la, (q, k, v), do)
             _report(f"simple_la B8-H16-T16384-D64 {tag}", 4 * nb, 11 * nb, f, s, flush)
     feature_map_config(dev, flush)
+    caller_configs(dev, flush)
+    varlen_config(dev, flush)
+
+
+def caller_configs(dev, flush):
+    """The decoupled operator at the shape of benchmark_decoupled_la.py and the head dims of the layer callers."""
+    from flash_bla.ops.linear_attn.decoupled import decoupled_la
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    run = _fwd_and_step
+
+    def leaves(*ts):
+        return [t.requires_grad_() for t in ts]
+
     q, k, v, do = make_inputs(2, 16, 16384, 64, torch.bfloat16, dev)
     qr, kr, _, _ = make_inputs(2, 16, 16384, 64, torch.bfloat16, dev, seed=7)
     leaves(q, k, qr, kr, v)
@@ -530,8 +550,6 @@ def other_configs(dev, flush):
         else:
             f, s = run(linear_attention, (q, k, v), do)
             _report(name, 2 * nqk + 2 * nv, 6 * nqk + 5 * nv, f, s, flush)
-
-    varlen_config(dev, flush)
 
 
 def varlen_config(dev, flush):
