@@ -782,15 +782,15 @@ __global__ __launch_bounds__(kThreads) void split_hi_lo_kernel(const float* __re
 // ===========================================================================
 // block selection (replaces score = qc (kc*scale)^T; torch.topk, kernel.py:304-318)
 // ===========================================================================
-// One workgroup per (head, 16 query blocks).  Scores of its 16 rows against all NT key
+// One workgroup per (head, kSelRows query blocks).  Scores of its rows against all NT key
 // blocks are computed with fp32 FMAs out of LDS tiles (64 key blocks at a time) and kept in
-// LDS; then every wave selects, for four of the rows, the NS largest scores: the threshold
+// LDS; then every wave selects, for its kSelRowsPerWave rows, the NS largest scores: the threshold
 // (the NS-th largest value) comes from a bitwise descent over the order-preserving integer
 // image of the floats with wave-wide counts, and the selected block indices are written in
 // ascending index order (ties at the threshold: lower index first).  With a bias (the
 // per-block norms), log(bias + 1e-5) is added to the score: the softmax of the reference
 // (kernel.py:314-315) is monotonic per row and does not change the selection.
-constexpr int kSelRows = 16, kSelKeys = 64;
+constexpr int kSelRowsPerWave = 2, kSelRows = 4 * kSelRowsPerWave, kSelKeys = 64;
 
 __device__ __forceinline__ uint32_t order_bits(float x) {
   const uint32_t b = __builtin_bit_cast(uint32_t, x);
@@ -802,12 +802,13 @@ template <int KT>
 __global__ __launch_bounds__(kThreads) void select_blocks_kernel(
     const float* __restrict__ qc, const float* __restrict__ kc, const float* __restrict__ bias,
     int32_t* __restrict__ indices, int NT, int NS, float scale, int Kr) {
+  constexpr int RW = kSelRowsPerWave;
   const int K = KT ? KT : ((Kr + 3) & ~3);  // row length in LDS
   const int KLD = K + 4;  // padded key rows: 16-byte reads of 16 lanes hit 16 bank groups
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  float* qs = reinterpret_cast<float*>(smem);          // [16][K]
+  float* qs = reinterpret_cast<float*>(smem);          // [kSelRows][K]
   float* kt = qs + kSelRows * K;                       // [64][K + 4]
-  float* sc = kt + kSelKeys * KLD;                     // [16][NTs]
+  float* sc = kt + kSelKeys * KLD;                     // [kSelRows][NTs]
   const int NTs = (NT + 63) & ~63;
   const int nrt = (NT + kSelRows - 1) / kSelRows;
   const int r0 = (blockIdx.x % nrt) * kSelRows;
@@ -845,48 +846,48 @@ __global__ __launch_bounds__(kThreads) void select_blocks_kernel(
       *reinterpret_cast<f4*>(kt + row * KLD + 4 * c4) = x;
     }
     __syncthreads();
-    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;  // rows 4*wave .. +3 against key j0 + lane
+    float acc[RW];  // rows RW*wave .. +RW-1 against key j0 + lane
+#pragma unroll
+    for (int rr = 0; rr < RW; ++rr) acc[rr] = 0.f;
     const float* kr = kt + lane * KLD;
-    const float* q0 = qs + (4 * wave) * K;
+    const float* q0 = qs + (RW * wave) * K;
 #pragma unroll 4
     for (int d = 0; d < K; d += 4) {
       const f4 kv = *reinterpret_cast<const f4*>(kr + d);
-      const f4 x0 = *reinterpret_cast<const f4*>(q0 + d);
-      const f4 x1 = *reinterpret_cast<const f4*>(q0 + K + d);
-      const f4 x2 = *reinterpret_cast<const f4*>(q0 + 2 * K + d);
-      const f4 x3 = *reinterpret_cast<const f4*>(q0 + 3 * K + d);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        a0 = fmaf(x0[i], kv[i], a0);
-        a1 = fmaf(x1[i], kv[i], a1);
-        a2 = fmaf(x2[i], kv[i], a2);
-        a3 = fmaf(x3[i], kv[i], a3);
+      for (int rr = 0; rr < RW; ++rr) {
+        const f4 x = *reinterpret_cast<const f4*>(q0 + rr * K + d);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[rr] = fmaf(x[i], kv[i], acc[rr]);
       }
     }
     const int key = j0 + lane;
     const float off = key < NT ? (bias ? logf(bias[bh * NT + key] + 1e-5f) : 0.f) : -__builtin_huge_valf();
-    sc[(4 * wave + 0) * NTs + key] = key < NT ? a0 * scale + off : off;
-    sc[(4 * wave + 1) * NTs + key] = key < NT ? a1 * scale + off : off;
-    sc[(4 * wave + 2) * NTs + key] = key < NT ? a2 * scale + off : off;
-    sc[(4 * wave + 3) * NTs + key] = key < NT ? a3 * scale + off : off;
+#pragma unroll
+    for (int rr = 0; rr < RW; ++rr) sc[(RW * wave + rr) * NTs + key] = key < NT ? acc[rr] * scale + off : off;
   }
   __syncthreads();
 
-  // the wave's four rows advance through the bitwise descent together: four independent
+  // the wave's rows advance through the bitwise descent together: independent
   // chains of LDS reads and wave-wide counts instead of one
-  uint32_t thr[4] = {0u, 0u, 0u, 0u};
+  uint32_t thr[RW];
+#pragma unroll
+  for (int rr = 0; rr < RW; ++rr) thr[rr] = 0u;
   for (int bit = 31; bit >= 0; --bit) {
-    int cnt[4] = {0, 0, 0, 0};
+    int cnt[RW];
+#pragma unroll
+    for (int rr = 0; rr < RW; ++rr) cnt[rr] = 0;
     for (int j = lane; j < NTs; j += 64)
 #pragma unroll
-      for (int rr = 0; rr < 4; ++rr)
-        cnt[rr] += __popcll(__ballot(order_bits(sc[(4 * wave + rr) * NTs + j]) >= (thr[rr] | (1u << bit))));
+      for (int rr = 0; rr < RW; ++rr)
+        cnt[rr] += __popcll(__ballot(order_bits(sc[(RW * wave + rr) * NTs + j]) >= (thr[rr] | (1u << bit))));
 #pragma unroll
-    for (int rr = 0; rr < 4; ++rr)
+    for (int rr = 0; rr < RW; ++rr)
       if (cnt[rr] >= NS) thr[rr] |= 1u << bit;
   }
-  for (int rr = 0; rr < 4; ++rr) {
-    const int row = 4 * wave + rr;
+#pragma unroll
+  for (int rr = 0; rr < RW; ++rr) {
+    const int row = RW * wave + rr;
     if (r0 + row >= NT) break;  // uniform over the wave
     const float* srow = sc + row * NTs;
     const uint32_t t = thr[rr];
