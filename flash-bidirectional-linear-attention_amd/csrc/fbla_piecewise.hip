@@ -108,9 +108,9 @@ __global__ __launch_bounds__(kThreads) void chunk_sums16_kernel(
 // H[bh][dk][dv] = sum_p partial_p[dk][dv] - sum_c kc_c[dk] * vc_c[dv]   (kc the MEAN and vc
 // the SUM of chunk c, so their product is the whole correction of that chunk).
 // One workgroup per (head, 32x32 tile of H); a thread owns a 2x2 patch.  The chunk
-// statistics go through LDS in slabs of 64 chunks (coalesced loads, every value is
+// statistics go through LDS in slabs of 128 chunks (coalesced loads, every value is
 // then used 16 times from LDS); the chunk order of the sum is fixed.
-constexpr int kHTile = 32, kHSlab = 64;
+constexpr int kHTile = 32, kHSlab = 128;
 __global__ __launch_bounds__(kThreads) void finish_h_kernel(
     const float* __restrict__ partial, int nparts, const float* __restrict__ kc,
     const float* __restrict__ vc, float* __restrict__ h, int NT, int K, int V) {
@@ -127,10 +127,24 @@ __global__ __launch_bounds__(kThreads) void finish_h_kernel(
   for (int cb = 0; cb < NT; cb += kHSlab) {
     const int nc = min(kHSlab, NT - cb);
     __syncthreads();
-    for (int i = threadIdx.x; i < kHSlab * kHTile; i += kThreads) {
-      const int c = i / kHTile, d = i % kHTile;
-      ks[c][d] = (c < nc && dk0 + d < K) ? kch[(int64_t)(cb + c) * K + dk0 + d] : 0.f;
-      vs[c][d] = (c < nc && dv0 + d < V) ? vch[(int64_t)(cb + c) * V + dv0 + d] : 0.f;
+    // all of a thread's loads are issued before the first is used (clamped addresses instead of
+    // branches: a loop of guarded loads waits for every single one)
+    constexpr int NF = kHSlab * kHTile / kThreads;
+    float kr[NF], vr[NF];
+#pragma unroll
+    for (int u = 0; u < NF; ++u) {
+      const int i = threadIdx.x + u * kThreads, c = i / kHTile, d = i % kHTile;
+      const bool kin = c < nc && dk0 + d < K, vin = c < nc && dv0 + d < V;
+      kr[u] = kch[kin ? (int64_t)(cb + c) * K + dk0 + d : 0];
+      vr[u] = vch[vin ? (int64_t)(cb + c) * V + dv0 + d : 0];
+      kr[u] = kin ? kr[u] : 0.f;
+      vr[u] = vin ? vr[u] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < NF; ++u) {
+      const int i = threadIdx.x + u * kThreads, c = i / kHTile, d = i % kHTile;
+      ks[c][d] = kr[u];
+      vs[c][d] = vr[u];
     }
     __syncthreads();
 #pragma unroll 8
@@ -826,7 +840,11 @@ __global__ __launch_bounds__(kThreads) void select_blocks_kernel(
     } else {
       f4 x;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) x[i] = 4 * c4 + i < Km ? rowp[4 * c4 + i] : 0.f;
+      for (int i = 0; i < 4; ++i) {
+        const bool in = 4 * c4 + i < Km;
+        x[i] = rowp[in ? 4 * c4 + i : 0];
+        x[i] = in ? x[i] : 0.f;
+      }
       return x;
     }
   };
@@ -838,12 +856,22 @@ __global__ __launch_bounds__(kThreads) void select_blocks_kernel(
     *reinterpret_cast<f4*>(qs + row * K + 4 * c4) = x;
   }
   for (int j0 = 0; j0 < NT; j0 += kSelKeys) {
+    // the tile's pieces of this thread are all requested before the first is stored (clamped
+    // addresses instead of branches: a loop of guarded loads waits for every single one)
+    constexpr int NPRE = KT ? kSelKeys * (KT / 4) / kThreads : kSelKeys * 32 / kThreads;
+    f4 pre[NPRE];
+#pragma unroll
+    for (int u = 0; u < NPRE; ++u) {
+      const int e = tid + u * kThreads, row = e / (K / 4), c4 = e % (K / 4);
+      const bool in = e < kSelKeys * (K / 4) && j0 + row < NT;
+      pre[u] = load4(kh + (int64_t)(in ? j0 + row : 0) * Km, in ? c4 : 0);
+      if (!in) pre[u] = f4{0.f, 0.f, 0.f, 0.f};
+    }
     __syncthreads();  // previous tile consumed (first trip: nothing to wait for but cheap)
-    for (int e = tid; e < kSelKeys * (K / 4); e += kThreads) {
-      const int row = e / (K / 4), c4 = e % (K / 4);
-      f4 x = f4{0.f, 0.f, 0.f, 0.f};
-      if (j0 + row < NT) x = load4(kh + (int64_t)(j0 + row) * Km, c4);
-      *reinterpret_cast<f4*>(kt + row * KLD + 4 * c4) = x;
+#pragma unroll
+    for (int u = 0; u < NPRE; ++u) {
+      const int e = tid + u * kThreads, row = e / (K / 4), c4 = e % (K / 4);
+      if (e < kSelKeys * (K / 4)) *reinterpret_cast<f4*>(kt + row * KLD + 4 * c4) = pre[u];
     }
     __syncthreads();
     float acc[RW];  // rows RW*wave .. +RW-1 against key j0 + lane
