@@ -786,19 +786,31 @@ __device__ __forceinline__ float build_operand(unsigned char* lds_opnd, float* l
   const int rstep = c_fast ? (PAIR ? 32 : dc) : 1;  // memory distance of consecutive rows
   for (int c = 0; c < nsum; ++c) {
     const float* src = mat + (int64_t)c * sum_stride;
+    // A unit without memory behind it reads the matrix's first unit and drops it, and the choice
+    // of the memory order is made outside the loops over the units: no branch between the units,
+    // so the loads of all of them are in flight together.
+    if (c_fast) {
 #pragma unroll
-    for (int i = 0; i < kUnits; ++i) {
-      if (kHoles && first[i] < 0) continue;
-      if (c_fast) {
+      for (int i = 0; i < kUnits; ++i) {
+        const bool hole = kHoles && first[i] < 0;
+        const int f0 = hole ? 0 : first[i];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) vals[i][j] += src[first[i] + j * rstep];
-      } else {
-        const f32x4 a = *reinterpret_cast<const f32x4*>(src + first[i]);
-        const f32x4 b = *reinterpret_cast<const f32x4*>(src + first[i] + 4);
+        for (int j = 0; j < 8; ++j) {
+          const float x = src[f0 + j * rstep];
+          vals[i][j] += hole ? 0.f : x;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kUnits; ++i) {
+        const bool hole = kHoles && first[i] < 0;
+        const int f0 = hole ? 0 : first[i];
+        const f32x4 a = *reinterpret_cast<const f32x4*>(src + f0);
+        const f32x4 b = *reinterpret_cast<const f32x4*>(src + f0 + 4);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          vals[i][j] += a[j];
-          vals[i][4 + j] += b[j];
+          vals[i][j] += hole ? 0.f : a[j];
+          vals[i][4 + j] += hole ? 0.f : b[j];
         }
       }
     }
