@@ -235,14 +235,27 @@ __global__ __launch_bounds__(kThreads, 2) void state32_kernel(
 // The matrix in memory is dr x dc; rows and columns past that are zero in the operand.
 __device__ __forceinline__ void build_operand32(float* frag, const float* __restrict__ mat, int ld_r,
                                                 int ld_c, float mscale, int dr, int dc) {
-  for (int e = threadIdx.x; e < D * D; e += blockDim.x) {
-    // walk the matrix along its contiguous direction
-    const int r = ld_c == 1 ? e / D : e % D, cc = ld_c == 1 ? e % D : e / D;
+  // a thread's elements are all requested before the first is stored (clamped addresses instead
+  // of branches: a loop of guarded loads waits for every single one)
+  constexpr int kPer = D * D / kThreads;
+  float val[kPer];
+  const bool c_fast = ld_c == 1;  // walk the matrix along its contiguous direction
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int e = threadIdx.x + i * kThreads;
+    const int r = c_fast ? e / D : e % D, cc = c_fast ? e % D : e / D;
+    const bool in = r < dr && cc < dc;
+    val[i] = mat[in ? (int64_t)r * ld_r + (int64_t)cc * ld_c : 0];
+    val[i] = in ? val[i] * mscale : 0.f;
+  }
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int e = threadIdx.x + i * kThreads;
+    const int r = c_fast ? e / D : e % D, cc = c_fast ? e % D : e / D;
     const int s = 2 * (r >> 2) + (r & 1), kb = (r >> 1) & 1;
     const int kbp = cc >> 5, b = (cc >> 4) & 1, gq = (cc >> 2) & 3, j = cc & 3;
     const int m = 8 * gq + 4 * kbp + j;
-    const float val = (r < dr && cc < dc) ? mat[(int64_t)r * ld_r + (int64_t)cc * ld_c] * mscale : 0.f;
-    frag[((b * 8 + (s >> 2)) * 64 + m + 32 * kb) * 4 + (s & 3)] = val;
+    frag[((b * 8 + (s >> 2)) * 64 + m + 32 * kb) * 4 + (s & 3)] = val[i];
   }
 }
 
@@ -323,9 +336,12 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
 
   build_operand32(frag, job.mat + (int64_t)nh * dr * dc, job.ld_r, job.ld_c, 1.f, dr, dc);
   const int dkm = NORM ? dr : dc;  // length of km: the contracted side (output) or q's (token view)
-  for (int e = tid; e < D; e += kThreads) {
-    kmv[e] = (NORM || TOKENS) && job.km && e < dkm ? job.km[(int64_t)nh * dkm + e] : 0.f;
-    addv[e] = job.addvec && e < dc ? job.addvec[(int64_t)nh * dc + e] * job.add_scale : 0.f;
+  if (tid < D) {  // (both loads before either is used)
+    const bool has_km = (NORM || TOKENS) && job.km && tid < dkm, has_add = job.addvec && tid < dc;
+    const float kmx = has_km ? job.km[(int64_t)nh * dkm + tid] : 0.f;
+    const float addx = has_add ? job.addvec[(int64_t)nh * dc + tid] * job.add_scale : 0.f;
+    kmv[tid] = kmx;
+    addv[tid] = addx;
   }
   __syncthreads();
   const bool with_den = (NORM || TOKENS) && job.km != nullptr;
