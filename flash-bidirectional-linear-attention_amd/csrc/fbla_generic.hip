@@ -21,14 +21,36 @@ constexpr int kLd = 129;    // LDS row pitch in floats (128 + 1: conflict-free c
 
 // Copy rows [t0, t0+nvalid) x [0,D) of X into dst[kTile][kLd] as fp32, zero-filling
 // the rest of the [kTile][Dpad] rectangle.
-template <typename T>
+// BATCH = false: one element at a time (backward pass A, whose accumulators leave no registers
+// for sixteen loads in flight per tensor: batched, it runs at half the occupancy and half the speed).
+template <typename T, bool BATCH = true>
 __device__ __forceinline__ void load_tile(float* dst, const T* __restrict__ X, int64_t row0,
                                           int64_t rstride, int D, int Dpad, int t0, int nvalid) {
-  for (int i = threadIdx.x; i < kTile * Dpad; i += kThreads) {
-    int t = i / Dpad, d = i - t * Dpad;
-    float x = 0.f;
-    if (t < nvalid && d < D) x = to_f32(X[(row0 + (int64_t)(t0 + t) * rstride) * D + d]);
-    dst[t * kLd + d] = x;
+  if constexpr (!BATCH) {
+    for (int i = threadIdx.x; i < kTile * Dpad; i += kThreads) {
+      const int t = i / Dpad, d = i - t * Dpad;
+      float x = 0.f;
+      if (t < nvalid && d < D) x = to_f32(X[(row0 + (int64_t)(t0 + t) * rstride) * D + d]);
+      dst[t * kLd + d] = x;
+    }
+    return;
+  }
+  // A thread's elements are all requested before the first is stored (clamped addresses instead
+  // of branches: a loop of guarded loads waits for every single one).  Dpad <= 128.
+  constexpr int kPer = kTile * 128 / kThreads;
+  const int n = kTile * Dpad;
+  float x[kPer];
+#pragma unroll
+  for (int u = 0; u < kPer; ++u) {
+    const int i = threadIdx.x + u * kThreads, t = i / Dpad, d = i - t * Dpad;
+    const bool in = i < n && t < nvalid && d < D;
+    x[u] = to_f32(X[in ? (row0 + (int64_t)(t0 + t) * rstride) * D + d : 0]);
+    x[u] = in ? x[u] : 0.f;
+  }
+#pragma unroll
+  for (int u = 0; u < kPer; ++u) {
+    const int i = threadIdx.x + u * kThreads, t = i / Dpad, d = i - t * Dpad;
+    if (i < n) dst[t * kLd + d] = x[u];
   }
 }
 
@@ -51,6 +73,7 @@ __device__ __forceinline__ void outer_accumulate(float (&acc)[M][M], const float
 }
 
 // acc[i][j] = sum_r Xs[tg+8i][r] * Mat[r][lane+32j]   (token rows times a small matrix)
+template <int UNROLL = 4>
 __device__ __forceinline__ void rows_times_matrix(float (&acc)[4][4], const float* Xs,
                                                   const float* __restrict__ Mat, int R, int C,
                                                   int tg, int lane) {
@@ -58,12 +81,16 @@ __device__ __forceinline__ void rows_times_matrix(float (&acc)[4][4], const floa
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  // (clamped column instead of a branch, UNROLL rows per trip: their loads of the matrix are in
+  // flight together - guarded loads in a rolled loop wait for every single one)
+#pragma unroll UNROLL
   for (int r = 0; r < R; ++r) {
     float m[4], x[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      int c = lane + 32 * j;
-      m[j] = c < C ? Mat[(int64_t)r * C + c] : 0.f;
+      const int c = lane + 32 * j;
+      m[j] = Mat[(int64_t)r * C + (c < C ? c : 0)];
+      m[j] = c < C ? m[j] : 0.f;
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) x[i] = Xs[(tg + 8 * i) * kLd + r];
@@ -284,9 +311,9 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
 
   for (int t0 = t_begin; t0 < t_end; t0 += kTile) {
     const int nvalid = min(kTile, t_end - t0);
-    load_tile(Qn, qn, row0, rstride, DK, Dpad, t0, nvalid);
-    load_tile(Gs, dout, row0, rstride, DV, Dpad, t0, nvalid);
-    if (split) load_tile(Qd, qd, row0, rstride, DK, Dpad, t0, nvalid);
+    load_tile<T, false>(Qn, qn, row0, rstride, DK, Dpad, t0, nvalid);
+    load_tile<T, false>(Gs, dout, row0, rstride, DV, Dpad, t0, nvalid);
+    if (split) load_tile<T, false>(Qd, qd, row0, rstride, DK, Dpad, t0, nvalid);
     __syncthreads();
     const float* Qden = split ? Qd : Qn;
     float u[4][4];
@@ -297,7 +324,7 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
         zs[threadIdx.x] = (int)threadIdx.x < nvalid ? z + p.eps : 1.0f;  // padding rows: dz = 0
       }
       // P_t = (q~_t S) . dO_t
-      rows_times_matrix(u, Qn, Sh, DK, DV, tg, lane);
+      rows_times_matrix<2>(u, Qn, Sh, DK, DV, tg, lane);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int t = tg + 8 * i;
@@ -319,7 +346,7 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
       __syncthreads();
     }
     // dq~_t = dO_t S^T / z_t (+ dz_t km when q~ == q)
-    rows_times_matrix(u, Gs, Sth, DV, DK, tg, lane);
+    rows_times_matrix<2>(u, Gs, Sth, DV, DK, tg, lane);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int t = tg + 8 * i;
