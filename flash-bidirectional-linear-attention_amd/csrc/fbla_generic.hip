@@ -21,36 +21,33 @@ constexpr int kLd = 129;    // LDS row pitch in floats (128 + 1: conflict-free c
 
 // Copy rows [t0, t0+nvalid) x [0,D) of X into dst[kTile][kLd] as fp32, zero-filling
 // the rest of the [kTile][Dpad] rectangle.
-// BATCH = false: one element at a time (backward pass A, whose accumulators leave no registers
-// for sixteen loads in flight per tensor: batched, it runs at half the occupancy and half the speed).
-template <typename T, bool BATCH = true>
+// BATCH: loads in flight per thread and tensor (16 = the whole tile at once).  Backward pass A,
+// whose accumulators leave fewer registers, takes 8: with 16 it runs at half the occupancy and half
+// the speed.
+template <typename T, int BATCH = 16>
 __device__ __forceinline__ void load_tile(float* dst, const T* __restrict__ X, int64_t row0,
                                           int64_t rstride, int D, int Dpad, int t0, int nvalid) {
-  if constexpr (!BATCH) {
-    for (int i = threadIdx.x; i < kTile * Dpad; i += kThreads) {
-      const int t = i / Dpad, d = i - t * Dpad;
-      float x = 0.f;
-      if (t < nvalid && d < D) x = to_f32(X[(row0 + (int64_t)(t0 + t) * rstride) * D + d]);
-      dst[t * kLd + d] = x;
-    }
-    return;
-  }
-  // A thread's elements are all requested before the first is stored (clamped addresses instead
+  // A batch's elements are all requested before the first is stored (clamped addresses instead
   // of branches: a loop of guarded loads waits for every single one).  Dpad <= 128.
   constexpr int kPer = kTile * 128 / kThreads;
+  static_assert(kPer % BATCH == 0, "whole batches");
   const int n = kTile * Dpad;
-  float x[kPer];
 #pragma unroll
-  for (int u = 0; u < kPer; ++u) {
-    const int i = threadIdx.x + u * kThreads, t = i / Dpad, d = i - t * Dpad;
-    const bool in = i < n && t < nvalid && d < D;
-    x[u] = to_f32(X[in ? (row0 + (int64_t)(t0 + t) * rstride) * D + d : 0]);
-    x[u] = in ? x[u] : 0.f;
-  }
+  for (int b0 = 0; b0 < kPer; b0 += BATCH) {
+    if (b0 * kThreads >= n) break;  // uniform: narrower tiles need fewer batches
+    float x[BATCH];
 #pragma unroll
-  for (int u = 0; u < kPer; ++u) {
-    const int i = threadIdx.x + u * kThreads, t = i / Dpad, d = i - t * Dpad;
-    if (i < n) dst[t * kLd + d] = x[u];
+    for (int u = 0; u < BATCH; ++u) {
+      const int i = threadIdx.x + (b0 + u) * kThreads, t = i / Dpad, d = i - t * Dpad;
+      const bool in = i < n && t < nvalid && d < D;
+      x[u] = to_f32(X[in ? (row0 + (int64_t)(t0 + t) * rstride) * D + d : 0]);
+      x[u] = in ? x[u] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      const int i = threadIdx.x + (b0 + u) * kThreads, t = i / Dpad, d = i - t * Dpad;
+      if (i < n) dst[t * kLd + d] = x[u];
+    }
   }
 }
 
@@ -311,9 +308,9 @@ __global__ __launch_bounds__(kThreads) void bwd_a_kernel(
 
   for (int t0 = t_begin; t0 < t_end; t0 += kTile) {
     const int nvalid = min(kTile, t_end - t0);
-    load_tile<T, false>(Qn, qn, row0, rstride, DK, Dpad, t0, nvalid);
-    load_tile<T, false>(Gs, dout, row0, rstride, DV, Dpad, t0, nvalid);
-    if (split) load_tile<T, false>(Qd, qd, row0, rstride, DK, Dpad, t0, nvalid);
+    load_tile<T, 8>(Qn, qn, row0, rstride, DK, Dpad, t0, nvalid);
+    load_tile<T, 8>(Gs, dout, row0, rstride, DV, Dpad, t0, nvalid);
+    if (split) load_tile<T, 8>(Qd, qd, row0, rstride, DK, Dpad, t0, nvalid);
     __syncthreads();
     const float* Qden = split ? Qd : Qn;
     float u[4][4];
