@@ -2108,8 +2108,6 @@ __global__ __launch_bounds__(256, 2) void bwd_a128_kernel(
   for (int base = t_begin; base < t_end; base += 64) {
     stash_step(rq, qtile);
     stash_step(rg, gtile);
-    load_step(rq, qn, base + 64, dk, qrow_b, qvoff, q_piece);
-    load_step(rg, dout, base + 64, dv, grow_b, gvoff, g_piece);
     __syncthreads();
 
     // ---- token view: this lane gets columns 64 kb + 16 blk + 0..15 of token ntok of both tiles
@@ -2125,6 +2123,10 @@ __global__ __launch_bounds__(256, 2) void bwd_a128_kernel(
         g[t] = Ops<T>::mma(sl[s], bq, g[t]);
       }
     }
+    // the next step's rows are requested here, not at the top of the step: their 32 registers are
+    // then free during the token view, whose LDS reads need buffers to be in flight ahead of the products
+    load_step(rq, qn, base + 64, dk, qrow_b, qvoff, q_piece);
+    load_step(rg, dout, base + 64, dv, grow_b, gvoff, g_piece);
     float rz[2] = {1.f, 1.f}, dz[2] = {0.f, 0.f};
     if constexpr (NORM) {
 #pragma unroll
