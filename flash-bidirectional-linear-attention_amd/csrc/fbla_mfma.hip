@@ -71,6 +71,9 @@ constexpr int kWaves = 4;
 #ifndef FBLA_ROWS_FAST
 #define FBLA_ROWS_FAST 3
 #endif
+#ifndef FBLA_BWDA_NEXT_AT
+#define FBLA_BWDA_NEXT_AT 1
+#endif
 #ifndef FBLA_BWDA_OCC3
 #define FBLA_BWDA_OCC3 0
 #endif
@@ -1737,15 +1740,18 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
       }
     }
     const int tn = t0 + t_stride;
-    if (kFast && tn + 32 <= t_end) {
-      load_q_full(rq, qn, tn);
-      load_g_full(rg, dout, tn);
-      if constexpr (DEN) load_q_full(rd, qd, tn);
-    } else if (tn < t_end) {
-      load_q(rq, qn, tn);
-      load_g(rg, dout, tn);
-      if constexpr (DEN) load_q(rd, qd, tn);
-    }
+    auto request_next = [&]() {
+      if (kFast && tn + 32 <= t_end) {
+        load_q_full(rq, qn, tn);
+        load_g_full(rg, dout, tn);
+        if constexpr (DEN) load_q_full(rd, qd, tn);
+      } else if (tn < t_end) {
+        load_q(rq, qn, tn);
+        load_g(rg, dout, tn);
+        if constexpr (DEN) load_q(rd, qd, tn);
+      }
+    };
+    if constexpr (FBLA_BWDA_NEXT_AT == 0) request_next();
     wave_sync();
 
     // ---- token view ----
@@ -1765,6 +1771,7 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
         g[b] = Ops<T>::mma(al, bq, g[b]);
       }
     }
+    if constexpr (FBLA_BWDA_NEXT_AT == 1) request_next();
     // this lane: g[token][c], c = (DK/2)*kb + 16b + r
     float rz = 1.f, dz = 0.f;
     if constexpr (NORM) {
@@ -1862,6 +1869,7 @@ __global__ __launch_bounds__(kThreads, (FBLA_BWDA_OCC3 && FUSED && !DEN && !LO) 
       }
     }
     wave_sync();
+    if constexpr (FBLA_BWDA_NEXT_AT == 2) request_next();
 
     // ---- feature view: two k-steps of 16 tokens ----
     if constexpr (FUSED) {
