@@ -32,6 +32,7 @@ import torch  # noqa: E402
 import torch.nn.functional as F  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16 matrix peak
 
 CLOCK_RAMP_S = 0.1  # untimed work before the warm-up steps
 
@@ -231,14 +232,19 @@ def main():
                     help="counter-collection mode for rocprofv3 --pmc: run N steps of the workload, each "
                          "followed by a 256 MiB device copy of known traffic, then exit")
     ap.add_argument("--tables", action="store_true",
-                    help="also print the reference's benchmark tables (torch formula, this library, SDPA) on stderr")
-    ap.add_argument("--only", choices=["c3", "c5", "fm", "callers"], default=None,
+                    help="the reference's benchmark tables (torch formula, this library, SDPA; `tables` of the "
+                         "JSON line) are on by default; this adds the linear_attn table at the README's B8 fp16")
+    ap.add_argument("--no-tables", action="store_true", help="skip the reference's benchmark tables")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the other BASELINE configs (the `configs` list of the JSON line)")
+    ap.add_argument("--only", choices=["c3", "c5", "fm", "callers", "tables"], default=None,
                     help="profiling aid: time just BASELINE config 3 (packed variable-length, D=64 and "
                          "D=128), config 5 (piecewise attention), the feature map together with the "
                          "attention (fm) or the decoupled operator and the layer callers' head dims "
                          "(callers), table on stderr, no headline line")
     ap.add_argument("--configs", action="store_true",
-                    help="also time the other operator families / BASELINE configs (table on stderr)")
+                    help="add the other operator families (simple_la, bf16, the feature map, the layer callers' "
+                         "head dims) to the `configs` list")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path needs no collective: heads "
@@ -256,10 +262,12 @@ def main():
         flush = torch.empty(256 << 20, dtype=torch.int8, device=dev)
         if args.only == "c3":
             varlen_config(dev, flush)
+        elif args.only == "tables":
+            print(json.dumps(reference_tables(dev, flush, args.tables_md, readme_table=args.tables)), flush=True)
         elif args.only == "fm":
             feature_map_config(dev, flush)
         elif args.only == "callers":
-            caller_configs(dev, flush)
+            caller_configs(dev, flush, head_dims=True)
         else:
             piecewise_config(dev, flush)
         return
@@ -286,13 +294,16 @@ def main():
         print(json.dumps({"probe_steps": args.probe, "copy_bytes_each_way": a.numel()}))
         return
 
-    # the GPU reaches its steady clocks only after tens of milliseconds of work: bring it there
-    # first, whatever W is (untimed, like the W warm-up steps that follow)
-    t_ramp = time.perf_counter()
-    while time.perf_counter() - t_ramp < CLOCK_RAMP_S:
-        for _ in range(20):
-            step()
-        torch.cuda.synchronize()
+    def clock_ramp():
+        """The GPU reaches its steady clocks only after tens of milliseconds of work, and leaves them
+        again while the host computes (the parity check below): untimed steps bring it there."""
+        t_ramp = time.perf_counter()
+        while time.perf_counter() - t_ramp < CLOCK_RAMP_S:
+            for _ in range(20):
+                step()
+            torch.cuda.synchronize()
+
+    clock_ramp()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -306,6 +317,7 @@ def main():
     parity = parity_spot_check(q.detach(), k.detach(), v.detach(), do, o, (q.grad, k.grad, v.grad))
 
     flush = torch.empty(256 << 20, dtype=torch.int8, device=dev)
+    clock_ramp()  # the GPU idled during the host-side parity check
     for _ in range(args.warmup):
         fwd_only()
     # back-to-back, no cache-flush write in between; an auxiliary figure (the headline `value` times
@@ -357,15 +369,20 @@ def main():
         "device_copy_gbps": copy_gbps,
         "parity": parity,
     }
+    del q, k, v, do, o
     if not args.no_sweep:
-        del q, k, v, do, o
         line["sweep"] = sweep(dtype, dev, flush)
-    if args.configs:
-        other_configs(dev, flush)
-        layer_config(dev, flush)
-        piecewise_config(dev, flush)
-    if args.tables:
-        reference_tables(dev, flush, args.tables_md)
+    if not args.no_configs:
+        # every other BASELINE config under the same clock: ms, algorithmic bytes (or FLOPs) per
+        # second, fraction of the 8 TB/s (2.5 PFLOP/s) peak, parity of one head against the oracle
+        rows = config1_on_gpu(dev, flush) + varlen_config(dev, flush) + layer_config(dev, flush)
+        rows.append(piecewise_config(dev, flush))
+        rows += caller_configs(dev, flush)
+        if args.configs:
+            rows += other_configs(dev, flush)
+        line["configs"] = rows
+    if not args.no_tables:
+        line["tables"] = reference_tables(dev, flush, args.tables_md, readme_table=args.tables)
     print(json.dumps(line), flush=True)
 
 
@@ -415,6 +432,7 @@ def _report(name, nbytes_fwd, nbytes_step, fwd_fn, step_fn, flush, extra=None):
     if extra:
         row.update(extra)
     print(json.dumps(row), file=sys.stderr, flush=True)
+    return row
 
 
 def feature_map_config(dev, flush):
@@ -451,14 +469,16 @@ def feature_map_config(dev, flush):
 
     t_step = do_bench(step_kernels, flush)
     t_step_auto = do_bench(step_autograd, flush)
-    print(json.dumps({"config": "elu+1 feature map + linear_attn B8-H16-T16384-D64 fp16",
-                      "fwd_mapped_on_load_ms": round(t_load[0], 5),
-                      "fwd_mapped_on_load_gbps": round(4 * nb / t_load[0] / 1e6, 1),
-                      "fwd_mapped_on_load_frac": round(4 * nb / t_load[0] / 1e6 / HBM_PEAK_GBPS, 4),
-                      "fwd_mapped_first_ms": round(t_first[0], 5),
-                      "fwd_bwd_gradients_from_kernels_ms": round(t_step[0], 5),
-                      "fwd_bwd_map_by_autograd_ms": round(t_step_auto[0], 5)}), file=sys.stderr, flush=True)
+    row = {"config": "elu+1 feature map + linear_attn B8-H16-T16384-D64 fp16",
+           "fwd_mapped_on_load_ms": round(t_load[0], 5),
+           "fwd_mapped_on_load_gbps": round(4 * nb / t_load[0] / 1e6, 1),
+           "fwd_mapped_on_load_frac": round(4 * nb / t_load[0] / 1e6 / HBM_PEAK_GBPS, 4),
+           "fwd_mapped_first_ms": round(t_first[0], 5),
+           "fwd_bwd_gradients_from_kernels_ms": round(t_step[0], 5),
+           "fwd_bwd_map_by_autograd_ms": round(t_step_auto[0], 5)}
+    print(json.dumps(row), file=sys.stderr, flush=True)
     del q, k, v, do
+    return row
 
 
 def _fwd_and_step(op, args, do_):
@@ -474,60 +494,98 @@ def _fwd_and_step(op, args, do_):
     return fwd, step
 
 
-def other_configs(dev, flush):
-    """Flushed-median timings of the remaining BASELINE configs and operator families."""
-    from flash_bla.ops.linear_attn.decoupled import decoupled_la
+def _one_head_parity(tensors, refs, dtype):
+    """{name: plain max-rel error} of GPU results against float64 oracle arrays, plus `ok` (both the
+    plain and the rounding-removed gate of tests/helpers.py)."""
+    from helpers import parity_errors
+    out, ok = {}, True
+    for name, (x, ref, floor) in zip(refs, tensors):
+        plain, excess, good = parity_errors(x, ref, dtype, floor)
+        out[name] = float(f"{plain:.2e}")
+        out[name + "_excess"] = float(f"{excess:.2e}")
+        ok = ok and good
+    out["ok"] = ok
+    return out
+
+
+def config1_on_gpu(dev, flush):
+    """BASELINE config 1 (the reference's CPU-runnable case: B2-H4-T1024-D64 fp32, simple_la and
+    linear_attn) through the HIP path, every head against the float64 oracle."""
+    from helpers import np64
+    from oracle import closed_form as cf
     from flash_bla.ops.linear_attn.fused import linear_attention
-    from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
     from flash_bla.ops.simple_la.fused import simple_la
-
-    def leaves(*ts):
-        return [t.requires_grad_() for t in ts]
-
-    # config 1 shape on the GPU (the CPU-runnable reference case): fp32, tiny
     q, k, v, do = make_inputs(2, 4, 1024, 64, torch.float32, dev)
-    leaves(q, k, v)
+    for t in (q, k, v):
+        t.requires_grad_()
     nb = q.numel() * 4
+    rows = []
+    for name, op, scale, norm in (("linear_attn", linear_attention, 1.0 / 1024, True),
+                                  ("simple_la", simple_la, 64 ** -0.5, False)):
+        f, s = _fwd_and_step(op, (q, k, v), do)
+        s()
+        ref = cf.dense_backward(np64(q), np64(k), np64(v), np64(do), scale, normalize=norm)
+        par = _one_head_parity([(f(), ref["o"], None), (q.grad, ref["dq"], ref.get("dq_mag")),
+                                (k.grad, ref["dk"], ref.get("dk_mag")), (v.grad, ref["dv"], None)],
+                               ("o", "dq", "dk", "dv"), torch.float32)
+        rows.append(_report(f"C1 {name} B2-H4-T1024-D64 fp32", 4 * nb, 11 * nb, f, s, flush, {"parity": par}))
+    return rows
 
+
+def other_configs(dev, flush):
+    """Flushed-median timings of the remaining operator families at the headline shape."""
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    from flash_bla.ops.simple_la.fused import simple_la
     run = _fwd_and_step
-
-    f, s = run(linear_attention, (q, k, v), do)
-    _report("C1 linear_attn B2-H4-T1024-D64 fp32", 4 * nb, 11 * nb, f, s, flush)
-    f, s = run(simple_la, (q, k, v), do)
-    _report("C1 simple_la B2-H4-T1024-D64 fp32", 4 * nb, 11 * nb, f, s, flush)
-
-    # simple_la / decoupled at the headline shape, and bf16 linear_attn
+    rows = []
+    # simple_la at the headline shape, and bf16 linear_attn
     for dtype, tag in ((torch.float16, "fp16"), (torch.bfloat16, "bf16")):
         q, k, v, do = make_inputs(8, 16, 16384, 64, dtype, dev)
-        leaves(q, k, v)
+        for t in (q, k, v):
+            t.requires_grad_()
         nb = q.numel() * 2
         if dtype == torch.bfloat16:
             f, s = run(linear_attention, (q, k, v), do)
-            _report(f"linear_attn B8-H16-T16384-D64 {tag}", 4 * nb, 11 * nb, f, s, flush)
+            rows.append(_report(f"linear_attn B8-H16-T16384-D64 {tag}", 4 * nb, 11 * nb, f, s, flush))
         else:
             f, s = run(simple_la, (q, k, v), do)
-            _report(f"simple_la B8-H16-T16384-D64 {tag}", 4 * nb, 11 * nb, f, s, flush)
-    feature_map_config(dev, flush)
-    caller_configs(dev, flush)
-    varlen_config(dev, flush)
+            rows.append(_report(f"simple_la B8-H16-T16384-D64 {tag}", 4 * nb, 11 * nb, f, s, flush))
+    rows.append(feature_map_config(dev, flush))
+    rows += caller_configs(dev, flush, head_dims=True)
+    return rows
 
 
-def caller_configs(dev, flush):
-    """The decoupled operator at the shape of benchmark_decoupled_la.py and the head dims of the layer callers."""
+def caller_configs(dev, flush, head_dims=False):
+    """The decoupled operator at the shape of benchmark_decoupled_la.py (one head against the float64
+    oracle), and with `head_dims` the head dims of the layer callers."""
+    from helpers import np64
+    from oracle import closed_form as cf
     from flash_bla.ops.linear_attn.decoupled import decoupled_la
     from flash_bla.ops.linear_attn.fused import linear_attention
     run = _fwd_and_step
+    rows = []
 
     def leaves(*ts):
         return [t.requires_grad_() for t in ts]
 
-    q, k, v, do = make_inputs(2, 16, 16384, 64, torch.bfloat16, dev)
-    qr, kr, _, _ = make_inputs(2, 16, 16384, 64, torch.bfloat16, dev, seed=7)
-    leaves(q, k, qr, kr, v)
+    T = 16384
+    q, k, v, do = make_inputs(2, 16, T, 64, torch.bfloat16, dev)
+    qr, kr, _, _ = make_inputs(2, 16, T, 64, torch.bfloat16, dev, seed=7)
+    args = leaves(q, k, qr, kr, v)
     nb = q.numel() * 2
-    f, s = run(decoupled_la, (q, k, qr, kr, v), do)
-    _report("decoupled_la B2-H16-T16384-D64 bf16 (benchmark_decoupled_la.py shape)", 6 * nb, 16 * nb, f, s, flush)
-    del q, k, v, do, qr, kr
+    f, s = run(decoupled_la, args, do)
+    s()
+    sl = (slice(1, 2), slice(5, 6))
+    ref = cf.dense_backward(np64(q[sl]), np64(k[sl]), np64(v[sl]), np64(do[sl]), 1.0 / T,
+                            q_rope=np64(qr[sl]), k_rope=np64(kr[sl]))
+    names = ("o", "dq", "dk", "dq_rope", "dk_rope", "dv")
+    got = (f(), q.grad, k.grad, qr.grad, kr.grad, v.grad)
+    par = _one_head_parity([(g[sl], ref[n], None) for g, n in zip(got, names)], names, torch.bfloat16)
+    rows.append(_report("decoupled_la B2-H16-T16384-D64 bf16 (benchmark_decoupled_la.py shape)", 6 * nb, 16 * nb,
+                        f, s, flush, {"parity": par}))
+    del q, k, v, do, qr, kr, args, got
+    if not head_dims:
+        return rows
 
     # head dims of the layer callers: MLLA / RALA blocks (decoupled, D=32: mlla.py:88, rala.py:74),
     # PolaFormer (DK = 2d, DV = d/2: polaformer.py:75-90)
@@ -546,19 +604,25 @@ def caller_configs(dev, flush):
         if dec:
             qr, kr = feats(B, H, T, DK, 3), feats(B, H, T, DK, 4)
             f, s = run(decoupled_la, (q, k, qr, kr, v), do)
-            _report(name, 4 * nqk + 2 * nv, 11 * nqk + 5 * nv, f, s, flush)
+            rows.append(_report(name, 4 * nqk + 2 * nv, 11 * nqk + 5 * nv, f, s, flush))
         else:
             f, s = run(linear_attention, (q, k, v), do)
-            _report(name, 2 * nqk + 2 * nv, 6 * nqk + 5 * nv, f, s, flush)
+            rows.append(_report(name, 2 * nqk + 2 * nv, 6 * nqk + 5 * nv, f, s, flush))
+    return rows
 
 
 def varlen_config(dev, flush):
-    """BASELINE config 3: packed variable-length, 64 sequences U[256, 2048], H=16, bf16."""
+    """BASELINE config 3: packed variable-length, 64 sequences U[256, 2048], H=16, bf16; sequence 17,
+    heads 0-1 against the float64 oracle."""
+    from helpers import np64
+    from oracle import closed_form as cf
     from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
     g = torch.Generator().manual_seed(42)
     lengths = torch.randint(256, 2049, (64,), generator=g)
     cu = torch.cat([torch.zeros(1, dtype=torch.int32), torch.cumsum(lengths, 0).to(torch.int32)]).to(dev)
     total, max_len = int(lengths.sum()), int(lengths.max())
+    bounds = cu.tolist()
+    rows = []
     for D in (64, 128):
         gg = torch.Generator(device=dev).manual_seed(42)
         q = (F.elu(torch.randn(total, 16, D, generator=gg, device=dev)) + 1).bfloat16().requires_grad_()
@@ -574,8 +638,17 @@ def varlen_config(dev, flush):
         def fwd():
             with torch.no_grad():
                 return varlen_linear_attention(q, k, v, cu, max_len)
-        _report(f"C3 varlen 64 seqs U[256,2048] H16 D{D} bf16", 4 * nb, 11 * nb, fwd, step, flush,
-                {"total_tokens": total, "max_seqlen": max_len})
+        step()
+        b, e = bounds[17], bounds[18]
+        head = lambda t: t[b:e, :2].transpose(0, 1)  # noqa: E731
+        ref = cf.dense_backward(*(np64(head(t)) for t in (q, k, v, do)), 1.0 / (e - b))
+        par = _one_head_parity([(head(fwd()), ref["o"], None), (head(q.grad), ref["dq"], ref["dq_mag"]),
+                                (head(k.grad), ref["dk"], ref["dk_mag"]), (head(v.grad), ref["dv"], None)],
+                               ("o", "dq", "dk", "dv"), torch.bfloat16)
+        rows.append(_report(f"C3 varlen 64 seqs U[256,2048] H16 D{D} bf16", 4 * nb, 11 * nb, fwd, step, flush,
+                            {"total_tokens": total, "max_seqlen": max_len, "parity": par}))
+        del q, k, v, do
+    return rows
 
 
 def layer_config(dev, flush):
@@ -585,6 +658,7 @@ def layer_config(dev, flush):
     with the torch formula, and the operator alone."""
     from flash_bla.layers.linfusion import GeneralizedLinearAttention
     from flash_bla.ops.linear_attn.fused import linear_attention
+    rows = []
     for L, C, heads in ((4096, 640, 10), (1024, 1280, 20)):
         torch.manual_seed(42)
         layer = GeneralizedLinearAttention(query_dim=C, heads=heads, dim_head=64).to(dev).half().eval()
@@ -603,101 +677,130 @@ def layer_config(dev, flush):
             err = (layer(x, mode="triton").float() - layer(x, mode="torch").float()).abs().max().item()
             ref = layer(x, mode="torch").float().abs().max().item()
         nb = 4 * q.numel() * 2
-        print(json.dumps({"config": f"C4 LinFusion layer fwd B2-L{L}-C{C}-{heads}x64 fp16",
-                          "layer_ms": round(t_fast[0], 5), "layer_hip_graph_ms": round(t_graph[0], 5),
-                          "hip_graph_equals_eager": graph_equal,
-                          "layer_torch_mode_ms": round(t_torch[0], 5),
-                          "op_ms": round(t_op[0], 5), "op_gbps": round(nb / t_op[0] / 1e6, 1),
-                          "modes_max_abs_diff_over_max": round(err / ref, 6)}), file=sys.stderr, flush=True)
+        rows.append({"config": f"C4 LinFusion layer fwd B2-L{L}-C{C}-{heads}x64 fp16",
+                     "layer_ms": round(t_fast[0], 5), "layer_hip_graph_ms": round(t_graph[0], 5),
+                     "hip_graph_equals_eager": graph_equal,
+                     "layer_torch_mode_ms": round(t_torch[0], 5),
+                     "op_ms": round(t_op[0], 5), "op_alg_bytes": nb, "op_gbps": round(nb / t_op[0] / 1e6, 1),
+                     "op_frac": round(nb / t_op[0] / 1e6 / HBM_PEAK_GBPS, 4),
+                     "parity": {"layer_vs_torch_mode_max_abs_over_max": round(err / ref, 6),
+                                "ok": err / ref <= 2e-3}})
+        print(json.dumps(rows[-1]), file=sys.stderr, flush=True)
+    return rows
 
 
-def reference_tables(dev, flush, md_path=None):
-    """The tables of the reference's three benchmark scripts, columns named as there:
+PROVIDERS6 = ["torch_la_fwd", "flash_bla_fwd", "torch_sdpa_fwd", "torch_la_bwd", "flash_bla_bwd", "torch_sdpa_bwd"]
+# x axis, columns and plot names of the reference's three benchmark scripts
+TABLE_SPECS = {
+    "linear_attn": {"script": "benchmarks/ops/benchmark_linear_attn.py:11-29", "plot_name": "B2-H16-D64",
+                    "dtype": "bf16", "x_name": "T", "x_vals": [1024, 4096, 16384, 32768], "line_vals": PROVIDERS6},
+    "decoupled_la": {"script": "benchmarks/ops/benchmark_decoupled_la.py:11-29", "plot_name": "B2-H16-D64",
+                     "dtype": "bf16", "x_name": "T", "x_vals": [1024, 4096, 16384, 32768], "line_vals": PROVIDERS6},
+    "varlen_linear_attn": {"script": "benchmarks/ops/benchmark_varlen_linear_attn.py:18-44",
+                           "plot_name": "varlen-equal-B8-H16-D64", "dtype": "bf16", "x_name": "max_seqlen",
+                           "x_vals": [256, 1024, 4096],
+                           "line_vals": ["flash_padded_fwd", "varlen_fwd", "flash_padded_fwdbwd", "varlen_fwdbwd"]},
+}
+
+
+def reference_tables(dev, flush, md_path=None, x_vals=None, readme_table=False):
+    """The tables of the reference's three benchmark scripts, x axis and columns named as there:
     benchmarks/ops/benchmark_linear_attn.py (providers torch_la / flash_bla / torch_sdpa, `_fwd` and
-    `_bwd` = forward + backward, T in {1024, 4096, 16384, 32768}; the script runs B2-H16-D64 bf16,
-    the README quotes B8 fp16: both), benchmark_decoupled_la.py:11-62 (B2-H16-D64 bf16) and
-    benchmark_varlen_linear_attn.py:20-86 (8 equal sequences, H16-D64 bf16, the padded dense
-    operator against the packed one, forward and forward + backward).  Flushed medians in ms;
-    gradients are reset before every backward (the scripts let them accumulate in the leaves,
-    which times one more elementwise pass per tensor)."""
+    `_bwd` = forward + backward, T in {1024, 4096, 16384, 32768}, B2-H16-D64 bf16),
+    benchmark_decoupled_la.py:11-62 (same axis and providers) and benchmark_varlen_linear_attn.py:20-86
+    (8 equal sequences, H16-D64 bf16, the padded dense operator against the packed one, forward and
+    forward + backward).  Flushed medians in ms; gradients are reset before every backward (the
+    scripts let them accumulate in the leaves, which times one more elementwise pass per tensor).
+    Returns {table: {script, plot_name, dtype, x_name, x_vals, line_vals, rows}} with one row of
+    `line_vals` times per x value.  `x_vals` replaces every table's x axis (tests use tiny lengths);
+    `readme_table` adds the linear_attn table at the README's B8 fp16."""
     from flash_bla.ops.linear_attn.decoupled import decoupled_la
     from flash_bla.ops.linear_attn.fused import linear_attention
     from flash_bla.ops.linear_attn.naive import naive_decoupled_la, naive_linear_attn
     from flash_bla.ops.linear_attn.varlen import varlen_linear_attention
-    rows = []
+    tables = {}
 
-    def emit(row):
-        rows.append(row)
-        print(json.dumps(row), file=sys.stderr, flush=True)
+    def new_table(name, spec_name, **changes):
+        spec = dict(TABLE_SPECS[spec_name], **changes)
+        if x_vals is not None:
+            spec["x_vals"] = list(x_vals)
+        tables[name] = dict(spec, rows=[])
+        return tables[name]
 
-    def time_providers(row, providers, leaves, do):
-        def bwd_of(fn):
-            def step():
-                for t in leaves:
-                    t.grad = None
-                fn().backward(do)
-            return step
+    def emit(table, name, x, row):
+        table["rows"].append([row[c] for c in table["line_vals"]])
+        print(json.dumps(dict({"table": name, table["x_name"]: x}, **row)), file=sys.stderr, flush=True)
+
+    def fwd_bwd_of(fn, leaves, do):
+        def step():
+            for t in leaves:
+                t.grad = None
+            fn().backward(do)
+        return step
+
+    def time_providers(providers, leaves, do):
+        row = {}
         for name, fn in providers:
             with torch.no_grad():
                 row[name + "_fwd"] = round(do_bench(fn, flush)[0], 4)
-            row[name + "_bwd"] = round(do_bench(bwd_of(fn), flush)[0], 4)
+            row[name + "_bwd"] = round(do_bench(fwd_bwd_of(fn, leaves, do), flush)[0], 4)
+        return row
 
-    lengths = (1024, 4096, 16384, 32768)
-    for B, dtype, tag in ((2, torch.bfloat16, "bf16"), (8, torch.float16, "fp16")):
-        for T in lengths:
+    variants = [("linear_attn", 2, torch.bfloat16, {})]
+    if readme_table:
+        variants.append(("linear_attn_readme_B8_fp16", 8, torch.float16, {"plot_name": "B8-H16-D64", "dtype": "fp16"}))
+    for name, B, dtype, changes in variants:
+        table = new_table(name, "linear_attn", **changes)
+        for T in table["x_vals"]:
             q, k, v, do = make_inputs(B, 16, T, 64, dtype, dev)
             leaves = [t.requires_grad_() for t in (q, k, v)]
-            row = {"table": f"linear_attn B{B}-H16-D64 {tag}", "T": T}
-            time_providers(row, (("torch_la", lambda: naive_linear_attn(q, k, v)),
-                                 ("flash_bla", lambda: linear_attention(q, k, v)),
-                                 ("torch_sdpa", lambda: F.scaled_dot_product_attention(q, k, v))), leaves, do)
-            emit(row)
+            emit(table, name, T, time_providers(
+                (("torch_la", lambda: naive_linear_attn(q, k, v)),
+                 ("flash_bla", lambda: linear_attention(q, k, v)),
+                 ("torch_sdpa", lambda: F.scaled_dot_product_attention(q, k, v))), leaves, do))
             del q, k, v, do, leaves
-    for T in lengths:
+    table = new_table("decoupled_la", "decoupled_la")
+    for T in table["x_vals"]:
         q, k, v, do = make_inputs(2, 16, T, 64, torch.bfloat16, dev)
         qr, kr, _, _ = make_inputs(2, 16, T, 64, torch.bfloat16, dev, seed=7)
         leaves = [t.requires_grad_() for t in (q, k, qr, kr, v)]
-        row = {"table": "decoupled_la B2-H16-D64 bf16", "T": T}
-        time_providers(row, (("torch_la", lambda: naive_decoupled_la(q, k, qr, kr, v)),
-                             ("flash_bla", lambda: decoupled_la(q, k, qr, kr, v)),
-                             ("torch_sdpa", lambda: F.scaled_dot_product_attention(q, k, v))), leaves, do)
-        emit(row)
+        emit(table, "decoupled_la", T, time_providers(
+            (("torch_la", lambda: naive_decoupled_la(q, k, qr, kr, v)),
+             ("flash_bla", lambda: decoupled_la(q, k, qr, kr, v)),
+             ("torch_sdpa", lambda: F.scaled_dot_product_attention(q, k, v))), leaves, do))
         del q, k, v, do, qr, kr, leaves
-    for max_len in (256, 1024, 4096):
+    table = new_table("varlen_linear_attn", "varlen_linear_attn")
+    for max_len in table["x_vals"]:
         cu = (torch.arange(9, dtype=torch.int32) * max_len).to(dev)
         qd, kd, vd, dod = make_inputs(8, 16, max_len, 64, torch.bfloat16, dev)
         qp, kp, vp, dop = (t.transpose(1, 2).reshape(8 * max_len, 16, 64).contiguous() for t in (qd, kd, vd, dod))
         dense, packed = [t.requires_grad_() for t in (qd, kd, vd)], [t.requires_grad_() for t in (qp, kp, vp)]
-
-        def fwdbwd(fn, leaves, do):
-            def step():
-                for t in leaves:
-                    t.grad = None
-                fn().backward(do)
-            return step
         pad = lambda: linear_attention(qd, kd, vd)  # noqa: E731
         var = lambda: varlen_linear_attention(qp, kp, vp, cu, max_len)  # noqa: E731
-        row = {"table": "varlen-equal-B8-H16-D64 bf16", "max_seqlen": max_len}
+        row = {}
         with torch.no_grad():
             row["flash_padded_fwd"] = round(do_bench(pad, flush)[0], 4)
             row["varlen_fwd"] = round(do_bench(var, flush)[0], 4)
-        row["flash_padded_fwdbwd"] = round(do_bench(fwdbwd(pad, dense, dod), flush)[0], 4)
-        row["varlen_fwdbwd"] = round(do_bench(fwdbwd(var, packed, dop), flush)[0], 4)
-        emit(row)
+        row["flash_padded_fwdbwd"] = round(do_bench(fwd_bwd_of(pad, dense, dod), flush)[0], 4)
+        row["varlen_fwdbwd"] = round(do_bench(fwd_bwd_of(var, packed, dop), flush)[0], 4)
+        emit(table, "varlen_linear_attn", max_len, row)
     if md_path:
         with open(md_path, "w") as f:
             f.write("Flushed medians in ms (`_bwd` columns = forward + backward, as in the reference's scripts).\n")
-            table = None
-            for row in rows:
-                cols = [c for c in row if c != "table"]
-                if row["table"] != table:
-                    table = row["table"]
-                    f.write(f"\n**{table}**\n\n| " + " | ".join(cols) + " |\n|" + "---|" * len(cols) + "\n")
-                f.write("| " + " | ".join(str(row[c]) for c in cols) + " |\n")
+            for name, t in tables.items():
+                cols = [t["x_name"]] + t["line_vals"]
+                f.write(f"\n**{name}** ({t['script']}, plot {t['plot_name']}, {t['dtype']})\n\n| "
+                        + " | ".join(cols) + " |\n|" + "---|" * len(cols) + "\n")
+                for x, row in zip(t["x_vals"], t["rows"]):
+                    f.write("| " + " | ".join(str(c) for c in [x] + row) + " |\n")
+    return tables
 
 
 def piecewise_config(dev, flush):
-    """BASELINE config 5: PISA forward, B1-H24-T16384-D128 bf16, 64-token blocks, density 0.25."""
+    """BASELINE config 5: PISA forward, B1-H24-T16384-D128 bf16, 64-token blocks, density 0.25; head 11
+    against the dense float64 oracle evaluated with the kernel's own selection."""
+    from helpers import np64
+    from oracle import piecewise as pw
     from flash_bla.ops.piecewise_attn.kernel import (chunk_reduce_fp32, piecewise_sparse_attention,
                                                      select_blocks)
     g = torch.Generator(device=dev).manual_seed(42)
@@ -713,13 +816,21 @@ def piecewise_config(dev, flush):
     t_all = do_bench(lambda: piecewise_sparse_attention(q, k, v, density=0.25), flush)
     t_red = do_bench(lambda: chunk_reduce_fp32(q, k, v, 64), flush)
     t_att = do_bench(lambda: piecewise_sparse_attention(q, k, v, indices=indices), flush)
-    print(json.dumps({
-        "config": "C5 piecewise fwd B1-H24-T16384-D128 bf16 block64 density0.25",
-        "total_ms": round(t_all[0], 4), "chunk_reduce_ms": round(t_red[0], 4),
-        "chunk_reduce_gbps": round(3 * nb / t_red[0] / 1e6, 1),
-        "chunk_reduce_plus_attention_ms": round(t_att[0], 4),
-        "exact_branch_tflops": round(flops_exact / ((t_att[0] - t_red[0]) * 1e-3) / 1e12, 1),
-        "min_traffic_gbps": round(4 * nb / t_all[0] / 1e6, 1)}), file=sys.stderr, flush=True)
+    o = piecewise_sparse_attention(q, k, v, density=0.25, indices=indices)
+    hd = 11
+    ref = pw.piecewise_forward(np64(q)[0, hd], np64(k)[0, hd], np64(v)[0, hd], indices[0, hd].cpu().numpy(), 64)
+    par = _one_head_parity([(o[0, hd], ref, None)], ("o",), torch.bfloat16)
+    tflops = flops_exact / ((t_att[0] - t_red[0]) * 1e-3) / 1e12
+    row = {"config": "C5 piecewise fwd B1-H24-T16384-D128 bf16 block64 density0.25",
+           "total_ms": round(t_all[0], 4), "chunk_reduce_ms": round(t_red[0], 4),
+           "chunk_reduce_gbps": round(3 * nb / t_red[0] / 1e6, 1),
+           "chunk_reduce_plus_attention_ms": round(t_att[0], 4),
+           "exact_branch_flops": flops_exact, "exact_branch_tflops": round(tflops, 1),
+           "exact_branch_frac_of_mfma_peak": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+           "min_traffic_bytes": 4 * nb, "min_traffic_gbps": round(4 * nb / t_all[0] / 1e6, 1),
+           "parity": par}
+    print(json.dumps(row), file=sys.stderr, flush=True)
+    return row
 
 
 if __name__ == "__main__":
