@@ -49,6 +49,10 @@ static int check_dims(const char* what, int64_t N, int64_t H, int64_t L, int DK,
     set_error("%s: unknown dtype %d", what, dtype);
     return kErrBadArg;
   }
+  if (flags & ~kPublicFlags) {
+    set_error("%s: unknown flag bits 0x%x", what, flags & ~kPublicFlags);
+    return kErrBadArg;
+  }
   if ((flags & kDecoupled) && !(flags & kNormalize)) {
     set_error("%s: FBLA_DECOUPLED requires FBLA_NORMALIZE", what);
     return kErrBadArg;

@@ -7,6 +7,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 namespace fbla {
 
@@ -22,6 +23,9 @@ enum Flags : int {
   kXcdOrder = 256,    // internal (set per launch): packed batches keep a sequence's heads on one XCD
   kInterleave = 512,  // internal (set per launch): the workgroups of a head take interleaved token steps
 };
+// what a caller may pass; the per-launch bits are the plan's alone (set from outside they would change
+// how the kernels walk without changing how the partials are counted)
+constexpr int kPublicFlags = kNormalize | kDecoupled | kDefaultScale | kElu1 | kElu1Grad;
 
 // One problem instance.  Dense: cu == nullptr, N = batch, every sequence has L
 // tokens and tensors are [N,H,L,D].  Packed: cu = int32[N+1] on the device and
@@ -90,6 +94,20 @@ __device__ __forceinline__ float seq_scale(const Prob& p, int len) {
 
 template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
 template <typename T> __device__ __forceinline__ T from_f32(float x) { return (T)x; }
+
+// Integer launch-geometry constants.  A build with -DFBLA_TUNING (make TUNING=1, for sweeps and A/B
+// runs) lets the environment variable `name` replace the default; the shipped library ignores the
+// environment: the kernels' alignment assumptions are only tested with the defaults.
+inline int tuning_knob(const char* name, int dflt, bool zero_ok = false) {
+#ifdef FBLA_TUNING
+  const char* v = getenv(name);
+  if (v && (atoi(v) > 0 || (zero_ok && v[0] == '0'))) return atoi(v);
+#else
+  (void)name;
+  (void)zero_ok;
+#endif
+  return dflt;
+}
 
 inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }

@@ -2342,11 +2342,8 @@ static int cu_count() {
   return n;
 }
 
-// Integer tuning knob, overridable from the environment (FBLA_<NAME>) for sweeps.
-static int knob(const char* name, int dflt) {
-  const char* v = getenv(name);
-  return v && atoi(v) > 0 ? atoi(v) : dflt;
-}
+// Integer tuning constant (environment override only in -DFBLA_TUNING builds).
+static int knob(const char* name, int dflt) { return tuning_knob(name, dflt); }
 
 // Tokens per workgroup for a kernel of which `wgs_per_cu` workgroups fit on a CU:
 // the grid is sized to at most `rounds` full rounds of resident workgroups, with
@@ -2628,7 +2625,7 @@ static int run_rows(const Prob& p, const RowsJob& job, const RowsJob* job2, int 
 // rounds of them).
 static bool small_tiles(int DR, int DC) { return tiled_dim(DR) == 64 && tiled_dim(DC) == 64; }
 static Prob xcd_ordered(const Prob& p, int kernel_bit) {
-  static const int mask = [] { const char* v = getenv("FBLA_XCD_ORDER"); return v ? atoi(v) : 2; }();
+  static const int mask = tuning_knob("FBLA_XCD_ORDER", 2, true);
   Prob r = p;
   if (p.cu && (mask & kernel_bit)) r.flags |= kXcdOrder;
   return r;
@@ -2638,7 +2635,7 @@ static Prob xcd_ordered(const Prob& p, int kernel_bit) {
 // the workgroups of a head take interleaved token steps (bit 0 the state kernel, bit 1 the
 // row-parallel kernels, bit 2 backward pass A).
 static int interleave_mask() {
-  static const int mask = [] { const char* v = getenv("FBLA_ILEAVE"); return v ? atoi(v) : 7; }();
+  static const int mask = tuning_knob("FBLA_ILEAVE", 7, true);
   return mask;
 }
 bool interleaved(const Prob& p, int dtype, int kernel_bit) {

@@ -94,16 +94,14 @@ static bool fold_reduce(const Prob& p, int reduce_nchunks, int DR, int DC) {
   const int64_t rows_nchunks = cdiv64(p.L, mfma::rows_chunk(p, DR, DC));
   const double extra = (double)p.N * p.H * (double)(rows_nchunks - 1) * reduce_nchunks *
                        ((double)p.DK * p.DV + p.DK) * sizeof(float);
-  static const double limit = [] {
-    const char* v = getenv("FBLA_FOLD_MAX_MB");
-    return v && atof(v) > 0 ? atof(v) * 1e6 : 16.0e6;
-  }();
+  static const double limit = tuning_knob("FBLA_FOLD_MAX_MB", 16) * 1e6;
   return extra <= limit;
 }
 
 // the walking order of a packed batch with too many sequences to rank inside every workgroup
 static size_t perm_bytes(const Prob& p) {
-  static const int inline_max = [] { const char* v = getenv("FBLA_RANK_INLINE"); return v ? atoi(v) : kRankInline; }();
+  // (the in-workgroup ranking has LDS for kRankInline lengths)
+  static const int inline_max = std::min(tuning_knob("FBLA_RANK_INLINE", kRankInline, true), kRankInline);
   return (p.cu && p.N > inline_max && p.N >= 2 && p.N <= kRankMax) ? align_up((size_t)p.N * sizeof(int32_t), 256) : 0;
 }
 // Writes the order behind the first `used` bytes of the workspace and returns the problem with it.

@@ -5,8 +5,13 @@ Key blocks of `block_size` tokens are ranked per query block by the product of b
 queries and keys; the top `density` fraction is attended exactly (softmax), every
 other block contributes through its mean key and value sum (zeroth order) plus a
 first-order correction with H = sum_c (K_c - kc_c)^T V_c.  All block statistics
-are kept in fp32 (the reference stores them in the input dtype) and the running
-linear-branch normaliser is rescaled consistently with the running maximum.
+are kept in fp32 (the reference stores them in the input dtype).
+
+Deliberate difference from the reference's kernel: the running normaliser of the linear branch is
+rescaled together with the running maximum.  The Triton kernel rescales its accumulator and its
+exact-branch sum but not that normaliser when the maximum grows between groups of unselected blocks
+(kernel.py:263-276), so with more blocks than one group (its autotuned GROUP_SIZE) its output depends
+on the group size; with one group both agree.  What is computed here is the group-independent value.
 
 Two kernels: fp16 / bf16 inputs with head dims in {64, 128} and 64-token blocks run on the
 MFMA kernel; every other head dim up to 128, every other block size and fp32 inputs run on a
@@ -36,6 +41,13 @@ def fused_chunk_reduce(q, k, v, chunk_size, use_bias=False, p=2):
     Returned in the input dtype like the reference; `chunk_reduce_fp32` keeps fp32."""
     qc, kc, vc, h, bias = chunk_reduce_fp32(q, k, v, chunk_size, use_bias, p)
     return qc.to(k.dtype), kc.to(k.dtype), vc.to(v.dtype), h.to(v.dtype), bias
+
+
+def chunk_reduce(q, k, v, chunk_size):
+    """The block means and value sums alone (kernel.py:131-149): qc, kc `(B,H,N,K)`, vc `(B,H,N,V)`
+    in the input dtype."""
+    qc, kc, vc, _, _ = chunk_reduce_fp32(q, k, v, chunk_size)
+    return qc.to(k.dtype), kc.to(k.dtype), vc.to(v.dtype)
 
 
 def chunk_reduce_fp32(q, k, v, chunk_size, use_bias=False, p=2):

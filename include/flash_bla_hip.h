@@ -115,7 +115,10 @@ int fbla_la_bwd(const void* q, const void* k, const void* v, const void* q_rope,
  * holds one copy until the process ends).  A problem whose fbla_la_workspace_bytes(0, ...)
  * exceeds that returns FBLA_ERR_WORKSPACE.  The call makes no hipMalloc / hipFree and no
  * allocating library call.  All calls on one GPU share the array: calls that overlap on one
- * GPU (two streams, two threads) race; serialise them or use fbla_la_fwd. */
+ * GPU (two streams, two threads) race; serialise them or use fbla_la_fwd.  The first call on a
+ * device looks up the array's address (hipGetSymbolAddress, which may load the code object) and
+ * sets the kernels' LDS attributes: make one eager call per device and problem shape before
+ * recording calls into a HIP graph. */
 #define FBLA_STATIC_SCRATCH_BYTES (16u << 20)
 size_t fbla_static_scratch_bytes(void);
 int fbla_la_fwd_static(const void* q, const void* k, const void* v, const void* q_rope,

@@ -87,7 +87,7 @@ def test_explicit_scale_and_eps(dtype):
     _check_dense("simple", 1, 2, 130, 64, 48, dtype, scale=0.5)
 
 
-@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "*.npz"))), ids=os.path.basename)
+@pytest.mark.parametrize("path", sorted(p for p in glob.glob(os.path.join(GOLDEN, "*.npz")) if not os.path.basename(p).startswith("layer_")), ids=os.path.basename)
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
 def test_golden_fixtures(path, dtype):
     d = np.load(path)

@@ -180,6 +180,44 @@ def test_use_bias_selection_and_errors():
         piecewise_sparse_attention(big, big, big)
 
 
+@pytest.mark.parametrize("dtype,T,K,V,block", [(torch.bfloat16, 1024, 64, 64, 64), (torch.float16, 1500, 128, 128, 64),
+                                               (torch.float32, 700, 48, 40, 32)])
+def test_use_bias_end_to_end(dtype, T, K, V, block):
+    """use_bias=True through the wrapper: the block norms reach the selection (softmax is monotone, so
+    the ranking is that of score + log(norm + 1e-5), kernel.py:172-174,314-318) and the attention runs
+    on that selection."""
+    from flash_bla.ops.piecewise_attn.kernel import (chunk_reduce, chunk_reduce_fp32, piecewise_sparse_attention,
+                                                     select_blocks)
+    q, k, v = _inputs(1, 2, T, K, V, dtype, seed=21)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    scale, density = K ** -0.5, 0.25
+    o = piecewise_sparse_attention(qd, kd, vd, density=density, block_size=block, use_bias=True)
+    qc, kc, vc, h, bias = chunk_reduce_fp32(qd, kd, vd, block, True)
+    NT = qc.shape[-2]
+    assert bias.shape == (1, 2, 1, NT)
+    idx = select_blocks(qc, kc, scale, density, bias)
+    # the wrapper ran on exactly this selection (with use_bias the statistics come from the kernels that
+    # also write the norms, so the comparison keeps the flag)
+    assert torch.equal(o, piecewise_sparse_attention(qd, kd, vd, block_size=block, use_bias=True, indices=idx))
+    for hd in range(2):
+        rq, rk, rv, rhc, _, _ = pw.chunk_reduce(np64(q)[0, hd], np64(k)[0, hd], np64(v)[0, hd], block)
+        # the norms the selection saw
+        want_norm = np.linalg.norm(rhc.reshape(NT, -1), axis=-1)
+        assert max_rel_err(bias[0, hd, 0], want_norm) < 1e-4
+        # the selection against the oracle's, as sets; near ties may differ
+        want = np.sort(pw.select_blocks(rq, rk, scale, density, hc=rhc, use_bias=True), axis=-1)
+        got = idx[0, hd].cpu().numpy()
+        differ = (want != got).any(-1)
+        assert differ.sum() <= max(1, NT // 20), f"{differ.sum()} of {NT} query blocks select differently"
+        # the output on the kernel's own selection against the dense oracle
+        ref = pw.piecewise_forward(np64(q)[0, hd], np64(k)[0, hd], np64(v)[0, hd], got, block, scale)
+        assert_parity(o[0, hd], ref, dtype, f"use_bias head {hd}")
+    # the three-output form of the statistics
+    c3 = chunk_reduce(qd, kd, vd, block)
+    assert [t.dtype for t in c3] == [dtype] * 3
+    assert torch.equal(c3[1], kc.to(dtype)) and torch.equal(c3[2], vc.to(dtype))
+
+
 @pytest.mark.parametrize("NT,K,top_density", [(256, 128, 0.25), (37, 64, 0.3), (1, 64, 1.0), (130, 128, 0.01),
                                               (64, 64, 1.0)])
 @pytest.mark.parametrize("with_bias", [False, True])

@@ -2,6 +2,10 @@
 `mode='triton'` (the HIP operators) must agree with it for the output and the
 input gradient, with the acceptance rule of the reference layers' self-tests
 (flash_bla/utils.py:55-67 with ratio 0.06; layers/linfusion.py:116-141 etc.)."""
+import ast
+import os
+
+import numpy as np
 import pytest
 import torch
 
@@ -67,6 +71,51 @@ def test_state_dict_names_and_shapes_follow_the_reference_modules():
     for name, (module, shapes) in want.items():
         got = {k: tuple(v.shape) for k, v in module.state_dict().items()}
         assert got == shapes, name
+
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+GOLDEN_BLOCKS = {"mlla": MambaLikeLinearAttention, "rala": RALALinearAttention, "focused": FocusedLinearAttention,
+                 "focused_sr2": FocusedLinearAttention, "pola": PolaLinearAttention, "pola_sr2": PolaLinearAttention}
+
+
+def _golden_block(name, device="cpu", dtype=None):
+    """Our block with the constructor arguments and the parameters of the fixture
+    tests/golden/layer_<name>.npz (written by tests/golden/make_layer_golden.py from the reference's
+    own block in mode='torch'), and the fixture's x, dy, y, dx."""
+    data = np.load(os.path.join(GOLDEN, f"layer_{name}.npz"))
+    kwargs = ast.literal_eval(str(data["kwargs"]))
+    state = {k[len("param."):]: torch.from_numpy(data[k]) for k in data.files if k.startswith("param.")}
+    ref_dtype = torch.from_numpy(data["y"]).dtype
+    block = GOLDEN_BLOCKS[name](**kwargs).to(ref_dtype)
+    block.load_state_dict(state, strict=True)   # every name and shape of the reference's state dict
+    block = block.to(device, dtype or ref_dtype).eval()
+    tensors = {k: torch.from_numpy(data[k]).to(device, dtype or ref_dtype) for k in ("x", "dy", "y", "dx")}
+    return block, tensors, tuple(int(v) for v in data["extra"])
+
+
+@pytest.mark.parametrize("name", sorted(GOLDEN_BLOCKS))
+def test_torch_mode_reproduces_the_reference_block(name):
+    """Arithmetic of the blocks against the reference's own modules (RoPE pair layout, RALA's
+    efficiency weighting, the focusing power, the spatial reduction, the polarity split)."""
+    block, t, extra = _golden_block(name)
+    x = t["x"].clone().requires_grad_()
+    y = block(x, *extra, mode="torch")
+    y.backward(t["dy"])
+    tol = 1e-9 if y.dtype == torch.float64 else 1e-5
+    assert (y - t["y"]).abs().max() <= tol * t["y"].abs().max(), name
+    assert (x.grad - t["dx"]).abs().max() <= tol * t["dx"].abs().max(), name
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(GOLDEN_BLOCKS))
+def test_fast_mode_reproduces_the_reference_block(name):
+    """mode='triton' (the HIP operators, fp32) against the reference block's torch-mode output."""
+    block, t, extra = _golden_block(name, "cuda", torch.float32)
+    x = t["x"].clone().requires_grad_()
+    y = block(x, *extra, mode="triton")
+    y.backward(t["dy"])
+    assert (y - t["y"]).abs().max() <= 2e-5 * t["y"].abs().max(), name
+    assert (x.grad - t["dx"]).abs().max() <= 2e-5 * t["dx"].abs().max(), name
 
 
 GPU_CASES = {

@@ -246,6 +246,28 @@ def test_piecewise_chunk_reduce_and_selection():
     assert (np.sort(idx, -1) == np.sort(torch.topk(score, 2, dim=-1).indices.numpy(), -1)).all()
 
 
+@pytest.mark.parametrize("p", [1, 2])
+def test_piecewise_selection_with_bias_ranks_score_plus_log_norm(p):
+    """kernel.py:172-174,314-318: with use_bias the ranking is torch.topk of softmax(score + log(norm + 1e-5)).
+    The softmax is monotone per row, so the selected set must be topk(score + log(norm + 1e-5)), with the
+    norms from torch.norm(p=...) of the flattened chunk matrices: evaluated here with torch on the
+    softmax itself, as the reference's wrapper does."""
+    q, k, v = _pw_inputs(T=64 * 11 + 5, seed=9)
+    qc, kc, vc, hc, H, lens = pw.chunk_reduce(q, k, v, 64)
+    NT = qc.shape[0]
+    scale = 16 ** -0.5
+    idx = pw.select_blocks(qc, kc, scale, 0.3, hc=hc, use_bias=True, p=p)
+    top_k = max(1, int(0.3 * NT))
+    assert idx.shape == (NT, top_k)
+    h_norm = torch.norm(torch.from_numpy(hc).flatten(-2, -1), p=p, dim=-1)
+    score = torch.from_numpy(qc) @ (torch.from_numpy(kc) * scale).T + torch.log(h_norm + 1e-5)[None, :]
+    want = torch.topk(torch.softmax(score, dim=-1), top_k, dim=-1).indices.numpy()
+    assert (np.sort(idx, -1) == np.sort(want, -1)).all()
+    # and the bias changes the selection (otherwise the check above pins nothing about it)
+    plain = pw.select_blocks(qc, kc, scale, 0.3)
+    assert (np.sort(idx, -1) != np.sort(plain, -1)).any()
+
+
 def test_piecewise_first_order_term_is_taylor_expansion():
     # Small scores: exp(s_ij) ~ exp(sb_ic)(1 + s_ij - sb_ic); the first-order term must
     # move the result towards exact attention (a sanity check; the coefficient itself

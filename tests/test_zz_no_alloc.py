@@ -45,6 +45,45 @@ def test_static_forward_equals_workspace_forward_twice(dtype):
         assert_parity(o, cf.dense_forward(np64(q), np64(k), np64(v), 1.0 / T)[0], dtype, "o")
 
 
+def test_static_forward_under_graph_capture():
+    """The use the entry point exists for: after one eager call (which looks up the scratch address and
+    sets the kernels' LDS attributes, neither of which may happen inside a capture) the call is recorded
+    into a HIP graph; every replay on fresh inputs equals fbla_la_fwd bit for bit."""
+    from flash_bla import _hip as hip
+    dev = torch.device("cuda")
+    B, H, T, D = 2, 4, 6000, 64
+    dtype = torch.float16
+    q, k, v, _ = make_qkv((B, H, T, D), (B, H, T, D), dtype, seed=5)
+    qd, kd, vd = (t.to(dev) for t in (q, k, v))
+    L = hip.lib()
+    o = torch.empty_like(vd)
+    s = torch.empty(B, H, D, D, dtype=torch.float32, device=dev)
+    km = torch.empty(B, H, D, dtype=torch.float32, device=dev)
+
+    def call():
+        return L.fbla_la_fwd_static(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), None, None, o.data_ptr(),
+                                    s.data_ptr(), km.data_ptr(), B, H, T, D, D, hip.dtype_code(qd), hip.NORMALIZE,
+                                    1.0 / T, 1e-6, torch.cuda.current_stream().cuda_stream)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        assert call() == 0, L.fbla_last_error()   # eager warm-up on the capturing stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = call()
+    assert rc == 0, L.fbla_last_error()
+    for seed in (11, 12, 13):
+        qn, kn, vn, _ = make_qkv((B, H, T, D), (B, H, T, D), dtype, seed=seed)
+        qd.copy_(qn.to(dev)), kd.copy_(kn.to(dev)), vd.copy_(vn.to(dev))
+        o.zero_(), s.zero_(), km.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        o_ref, s_ref, km_ref = hip.la_fwd(qd, kd, vd, None, None, 1.0 / T, 1e-6, hip.NORMALIZE)
+        torch.cuda.synchronize()
+        assert torch.equal(o, o_ref) and torch.equal(s, s_ref) and torch.equal(km, km_ref), f"replay {seed}"
+
+
 def test_static_forward_rejects_oversized_problem():
     from flash_bla import _hip as hip
     dev = torch.device("cuda")
