@@ -608,7 +608,53 @@ def caller_configs(dev, flush, head_dims=False):
         else:
             f, s = run(linear_attention, (q, k, v), do)
             rows.append(_report(name, 2 * nqk + 2 * nv, 6 * nqk + 5 * nv, f, s, flush))
+    rows.append(polaformer_config(dev, flush))
     return rows
+
+
+def polaformer_config(dev, flush):
+    """PolaFormer's attention core (layers/polaformer.py:89-90) at B8-H16-T4096, head dim 64 (DK = 128, two value
+    halves of 32): the two operator calls that share k against the one-state-pass operator.  Bytes: the tensors
+    the shared-state form has to move (forward q1, q2, k, v, o1, o2; backward q1, q2, k, v, dO, dq1, dq2, dk, dv)."""
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    from flash_bla.ops.linear_attn.paired import paired_linear_attention
+    B, H, T, DK, DV = 8, 16, 4096, 128, 64
+    g = torch.Generator(device=dev).manual_seed(5)
+    feat = lambda: (F.elu(torch.randn(B, H, T, DK, generator=g, device=dev)) + 1).half().requires_grad_()  # noqa: E731
+    q1, q2, k = feat(), feat(), feat()
+    v = torch.randn(B, H, T, DV, generator=g, device=dev).half().requires_grad_()
+    do1, do2 = (torch.randn(B, H, T, DV // 2, generator=g, device=dev).half() for _ in range(2))
+    leaves = (q1, q2, k, v)
+
+    def two_calls():
+        v1, v2 = (t.contiguous() for t in v.chunk(2, dim=-1))
+        return linear_attention(q1, k, v1), linear_attention(q2, k, v2)
+
+    def shared():
+        return paired_linear_attention(q1, q2, k, v)
+
+    def step_of(fn):
+        def step():
+            for t in leaves:
+                t.grad = None
+            torch.autograd.backward(fn(), [do1, do2])
+        return step
+    nqk, nv = q1.numel() * 2, v.numel() * 2
+    fwd_bytes, step_bytes = 3 * nqk + 2 * nv, 3 * nqk + 2 * nv + 4 * nqk + 3 * nv
+    with torch.no_grad():
+        f2, f1 = do_bench(two_calls, flush)[0], do_bench(shared, flush)[0]
+        a, b = two_calls(), shared()
+        same = max((x.float() - y.float()).abs().max().item() / y.float().abs().max().item() for x, y in zip(a, b))
+    s2, s1 = do_bench(step_of(two_calls), flush)[0], do_bench(step_of(shared), flush)[0]
+    row = {"config": "PolaFormer pairings B8-H16-T4096 DK128 DV2x32 fp16",
+           "two_calls_fwd_ms": round(f2, 5), "two_calls_fwd_bwd_ms": round(s2, 5),
+           "fwd_ms": round(f1, 5), "fwd_gbps": round(fwd_bytes / f1 / 1e6, 1),
+           "fwd_frac": round(fwd_bytes / f1 / 1e6 / HBM_PEAK_GBPS, 4),
+           "fwd_bwd_ms": round(s1, 5), "fwd_bwd_gbps": round(step_bytes / s1 / 1e6, 1),
+           "fwd_bwd_frac": round(step_bytes / s1 / 1e6 / HBM_PEAK_GBPS, 4),
+           "parity": {"shared_vs_two_calls_max_abs_over_max": float(f"{same:.2e}"), "ok": same <= 2e-3}}
+    print(json.dumps(row), file=sys.stderr, flush=True)
+    return row
 
 
 def varlen_config(dev, flush):

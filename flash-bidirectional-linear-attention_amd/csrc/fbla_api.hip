@@ -267,6 +267,71 @@ int fbla_la_fwd_static(const void* q, const void* k, const void* v, const void* 
   return run_fwd(what, p, dtype, a, (hipStream_t)stream);
 }
 
+// ---- two queries on shared keys and values ---------------------------------------------------
+size_t fbla_la_pair_workspace_bytes(int pass, int64_t B, int64_t H, int64_t L, int DK, int DV, int dtype) {
+  if (check_dims("fbla_la_pair_workspace_bytes", B, H, L, DK, DV, dtype, kNormalize) != kOk) return 0;
+  Prob p = make_prob(nullptr, B, H, L, B * L, DK, DV, kNormalize, 1.f, 0.f);
+  if (!plan::pair_supported(p, dtype)) return 0;
+  return pass == 0 ? plan::pair_fwd_workspace_bytes(p, dtype) : plan::pair_bwd_workspace_bytes(p, dtype);
+}
+
+int fbla_la_pair_fwd(const void* q1, const void* q2, const void* k, const void* v, void* o1, void* o2, float* s,
+                     float* km, void* workspace, size_t workspace_bytes_, int64_t B, int64_t H, int64_t L, int DK,
+                     int DV, int dtype, float scale, float eps, void* stream) {
+  const char* what = "fbla_la_pair_fwd";
+  int rc = check_dims(what, B, H, L, DK, DV, dtype, kNormalize);
+  if (rc != kOk) return rc;
+  if (B * H * L == 0) return kOk;
+  if (!q1 || !q2 || !k || !v || !o1 || !o2 || !s || !km) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  if (check_aligned(what, {q1, q2, k, v, o1, o2, s, km, workspace}) != kOk) return kErrBadArg;
+  Prob p = make_prob(nullptr, B, H, L, B * L, DK, DV, kNormalize, scale, eps);
+  if (!plan::pair_supported(p, dtype)) {
+    set_error("%s: needs dense fp16 / bf16 tensors with DK, DV/2 multiples of 8 (got DK=%d DV=%d dtype=%d)", what, DK,
+              DV, dtype);
+    return kErrUnsupported;
+  }
+  const size_t need = plan::pair_fwd_workspace_bytes(p, dtype);
+  if (workspace_bytes_ < need || !workspace) {
+    set_error("%s: workspace too small (%zu < %zu bytes)", what, workspace_bytes_, need);
+    return kErrWorkspace;
+  }
+  PairFwdArgs a{{q1, q2}, k, v, {o1, o2}, s, km, workspace, workspace_bytes_};
+  rc = plan::pair_forward(p, dtype, a, (hipStream_t)stream);
+  return rc != kOk ? rc : check_launch(what);
+}
+
+int fbla_la_pair_bwd(const void* q1, const void* q2, const void* k, const void* v, const void* dout1,
+                     const void* dout2, const float* s, const float* km, void* dq1, void* dq2, void* dk, void* dv,
+                     void* workspace, size_t workspace_bytes_, int64_t B, int64_t H, int64_t L, int DK, int DV,
+                     int dtype, float scale, float eps, void* stream) {
+  const char* what = "fbla_la_pair_bwd";
+  int rc = check_dims(what, B, H, L, DK, DV, dtype, kNormalize);
+  if (rc != kOk) return rc;
+  if (B * H * L == 0) return kOk;
+  if (!q1 || !q2 || !k || !v || !dout1 || !dout2 || !s || !km || !dq1 || !dq2 || !dk || !dv) {
+    set_error("%s: null tensor pointer", what);
+    return kErrBadArg;
+  }
+  if (check_aligned(what, {q1, q2, k, v, dout1, dout2, s, km, dq1, dq2, dk, dv, workspace}) != kOk) return kErrBadArg;
+  Prob p = make_prob(nullptr, B, H, L, B * L, DK, DV, kNormalize, scale, eps);
+  if (!plan::pair_supported(p, dtype)) {
+    set_error("%s: needs dense fp16 / bf16 tensors with DK, DV/2 multiples of 8 (got DK=%d DV=%d dtype=%d)", what, DK,
+              DV, dtype);
+    return kErrUnsupported;
+  }
+  const size_t need = plan::pair_bwd_workspace_bytes(p, dtype);
+  if (workspace_bytes_ < need || !workspace) {
+    set_error("%s: workspace too small (%zu < %zu bytes)", what, workspace_bytes_, need);
+    return kErrWorkspace;
+  }
+  PairBwdArgs a{{q1, q2}, k, v, {dout1, dout2}, s, km, {dq1, dq2}, dk, dv, workspace, workspace_bytes_};
+  rc = plan::pair_backward(p, dtype, a, (hipStream_t)stream);
+  return rc != kOk ? rc : check_launch(what);
+}
+
 static int check_cross(const char* what, int64_t Lk, int flags) {
   if (Lk <= 0 || Lk > 0x7fffffffLL / 2) {
     set_error("%s: the number of keys must be positive and fit 32-bit indexing, got %lld", what, (long long)Lk);

@@ -545,6 +545,42 @@ void state_reduce(const Prob& p, const float* partial, int chunk, int nchunks, f
       p, partial, chunk, nchunks, mat, mat_t, vec, blocks_per_head);
 }
 
+// Two queries sharing keys and values: the state's value columns [0, DV/2) serve the first query,
+// [DV/2, DV) the second.  split: lo[nh][r][c] = mat[nh][r][c], hi[nh][r][c] = mat[nh][r][DV/2 + c];
+// join is the inverse for the matrices and adds the two vectors.
+__global__ __launch_bounds__(kThreads) void split_columns_kernel(const float* __restrict__ mat,
+                                                                 float* __restrict__ lo, float* __restrict__ hi,
+                                                                 int DK, int DV) {
+  const int half = DV / 2;
+  const int64_t base = (int64_t)blockIdx.x * DK * DV, hbase = (int64_t)blockIdx.x * DK * half;
+  for (int e = threadIdx.x; e < DK * DV; e += kThreads) {
+    const int r = e / DV, c = e - r * DV;
+    if (c < half) lo[hbase + r * half + c] = mat[base + e];
+    else hi[hbase + r * half + c - half] = mat[base + e];
+  }
+}
+__global__ __launch_bounds__(kThreads) void join_columns_kernel(
+    const float* __restrict__ lo, const float* __restrict__ hi, const float* __restrict__ vec_lo,
+    const float* __restrict__ vec_hi, float* __restrict__ mat, float* __restrict__ vec, int DK, int DV) {
+  const int half = DV / 2;
+  const int64_t base = (int64_t)blockIdx.x * DK * DV, hbase = (int64_t)blockIdx.x * DK * half;
+  for (int e = threadIdx.x; e < DK * DV; e += kThreads) {
+    const int r = e / DV, c = e - r * DV;
+    mat[base + e] = c < half ? lo[hbase + r * half + c] : hi[hbase + r * half + c - half];
+  }
+  if (vec)
+    for (int e = threadIdx.x; e < DK; e += kThreads)
+      vec[(int64_t)blockIdx.x * DK + e] = vec_lo[(int64_t)blockIdx.x * DK + e] + vec_hi[(int64_t)blockIdx.x * DK + e];
+}
+void split_columns(const Prob& p, const float* mat, float* lo, float* hi, hipStream_t st) {
+  split_columns_kernel<<<dim3((unsigned)((int64_t)p.N * p.H)), dim3(kThreads), 0, st>>>(mat, lo, hi, p.DK, p.DV);
+}
+void join_columns(const Prob& p, const float* lo, const float* hi, const float* vec_lo, const float* vec_hi,
+                  float* mat, float* vec, hipStream_t st) {
+  join_columns_kernel<<<dim3((unsigned)((int64_t)p.N * p.H)), dim3(kThreads), 0, st>>>(lo, hi, vec_lo, vec_hi, mat,
+                                                                                       vec, p.DK, p.DV);
+}
+
 void transpose_state(const Prob& p, const float* mat, float* mat_t, hipStream_t st) {
   transpose_state_kernel<<<dim3((unsigned)((int64_t)p.N * p.H)), dim3(kThreads), 0, st>>>(
       mat, mat_t, p.DK, p.DV);

@@ -36,8 +36,33 @@ enum Phase : unsigned {
 };
 unsigned phase_mask();
 
+// Two queries that share keys and values (PolaFormer's same-sign / opposite-sign pairing): the first
+// attends to the value columns [0, DV/2), the second to [DV/2, DV).  o, dout, dq are pairs of
+// [.., DK] / [.., DV/2] tensors; k, v, dk, dv and the state are those of the whole DK x DV problem.
+struct PairFwdArgs {
+  const void *q[2], *k, *v;
+  void* o[2];
+  float* s;   // [N*H, DK, DV]
+  float* km;  // [N*H, DK]
+  void* workspace;
+  size_t workspace_bytes;
+};
+struct PairBwdArgs {
+  const void *q[2], *k, *v, *dout[2];
+  const float* s;
+  const float* km;
+  void *dq[2], *dk, *dv;
+  void* workspace;
+  size_t workspace_bytes;
+};
+
 // The sequence of kernels behind each entry point.
 namespace plan {
+bool pair_supported(const Prob& p, int dtype);
+size_t pair_fwd_workspace_bytes(const Prob& p, int dtype);
+size_t pair_bwd_workspace_bytes(const Prob& p, int dtype);
+int pair_forward(const Prob& p, int dtype, const PairFwdArgs& a, hipStream_t st);
+int pair_backward(const Prob& p, int dtype, const PairBwdArgs& a, hipStream_t st);
 size_t fwd_workspace_bytes(const Prob& p, int dtype);
 size_t bwd_workspace_bytes(const Prob& p, int dtype);
 int forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st);
@@ -52,6 +77,11 @@ void state_partial(const Prob& p, int dtype, const void* kn, const void* v, cons
 void state_reduce(const Prob& p, const float* partial, int chunk, int nchunks, float* mat,
                   float* mat_t, float* vec, hipStream_t st);
 void transpose_state(const Prob& p, const float* mat, float* mat_t, hipStream_t st);
+// p.DV even: the column halves of a [N*H, DK, DV] matrix as two [N*H, DK, DV/2] matrices, and back
+// (join also adds two [N*H, DK] vectors when `vec` is given)
+void split_columns(const Prob& p, const float* mat, float* lo, float* hi, hipStream_t st);
+void join_columns(const Prob& p, const float* lo, const float* hi, const float* vec_lo, const float* vec_hi,
+                  float* mat, float* vec, hipStream_t st);
 void output(const Prob& p, int dtype, const void* qn, const void* qd, const float* S,
             const float* km, void* o, hipStream_t st);
 void bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* dout,

@@ -306,5 +306,103 @@ int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
   return kOk;
 }
 
+// ---- two queries sharing keys and values -------------------------------------------------------
+// forward :  state partials of the whole DK x DV problem -> reduce (S, km) -> column halves S1, S2
+//            -> one row launch with two jobs: o1 = (q1 S1) / (q1 . km + eps), o2 likewise
+// backward:  pass A per query (dq_i, partials of dS_i and dkm_i) -> reduce -> dS = [dS1 | dS2],
+//            dkm = dkm1 + dkm2 -> pass B of the whole problem (dk, dv): k and v are read once per
+//            direction, dk is written once.
+// Dense 16-bit problems whose whole and half shapes the matrix-core kernels cover, with the fused
+// pass A for the half shape; the plain operator with the denominator.
+static Prob half_values(const Prob& p) {
+  Prob h = p;
+  h.DV = p.DV / 2;
+  return h;
+}
+bool pair_supported(const Prob& p, int dtype) {
+  if (p.cu || dtype == kF32 || (p.DV & 1) || (p.flags & ~kNormalize) || !(p.flags & kNormalize)) return false;
+  const Prob h = half_values(p);
+  return mfma::supported(p, dtype) && mfma::supported(h, dtype) && mfma::bwd_a_supported(h, dtype) &&
+         !mfma::pair_mode(h, dtype);
+}
+static size_t half_state_bytes(const Prob& p) { return state_bytes(half_values(p)); }
+// partials | S1 | S2
+size_t pair_fwd_workspace_bytes(const Prob& p, int dtype) {
+  return partial_bytes(p, dtype, fwd_chunk(p, dtype)) + 2 * half_state_bytes(p);
+}
+// partials (half shape) | S1 | S2 | s dS1 | s dS2 | dkm1/L | dkm2/L | s dS | dkm/L
+size_t pair_bwd_workspace_bytes(const Prob& p, int dtype) {
+  const Prob h = half_values(p);
+  return partial_bytes(h, dtype, bwd_chunk(h, dtype)) + 4 * half_state_bytes(p) + 3 * vec_bytes(p) + state_bytes(p);
+}
+
+int pair_forward(const Prob& p, int dtype, const PairFwdArgs& a, hipStream_t st) {
+  if (!pair_supported(p, dtype)) {
+    set_error("two queries on shared keys and values: dense fp16 / bf16 problems with the denominator whose "
+              "whole (DK x DV) and half (DK x DV/2) shapes the matrix-core kernels cover");
+    return kErrUnsupported;
+  }
+  const Prob h = half_values(p);
+  const int chunk = fwd_chunk(p, dtype);
+  const int nchunks = (int)cdiv64(p.L, chunk);
+  char* ws = (char*)a.workspace;
+  float* partial = (float*)ws;
+  ws += partial_bytes(p, dtype, chunk);
+  float* S1 = (float*)ws;
+  ws += half_state_bytes(p);
+  float* S2 = (float*)ws;
+  const bool direct = nchunks == 1;
+  mfma::state(mfma::with_interleave(p, dtype, 1), dtype, a.k, a.v, a.k, partial, chunk, nchunks, st,
+              direct ? a.s : nullptr, direct ? a.km : nullptr);
+  if (!direct)
+    generic::state_reduce(p, partial, mfma::partial_chunk(p, dtype, 1, chunk), nchunks, a.s, nullptr, a.km, st);
+  generic::split_columns(p, a.s, S1, S2, st);
+  mfma::RowsJob j1{a.q[0], a.q[0], S1, h.DV, 1, a.km, nullptr, a.o[0]};
+  mfma::RowsJob j2{a.q[1], a.q[1], S2, h.DV, 1, a.km, nullptr, a.o[1]};
+  return mfma::rows2(mfma::with_interleave(h, dtype, 2), dtype, j1, j2, h.DK, h.DV, st);
+}
+
+int pair_backward(const Prob& p, int dtype, const PairBwdArgs& a, hipStream_t st) {
+  if (!pair_supported(p, dtype)) {
+    set_error("two queries on shared keys and values: dense fp16 / bf16 problems with the denominator whose "
+              "whole (DK x DV) and half (DK x DV/2) shapes the matrix-core kernels cover");
+    return kErrUnsupported;
+  }
+  const Prob h = half_values(p);
+  const int chunk = bwd_chunk(h, dtype);
+  const int nchunks = (int)cdiv64(h.L, chunk);
+  char* ws = (char*)a.workspace;
+  float* partial = (float*)ws;
+  ws += partial_bytes(h, dtype, chunk);
+  float* Sh[2];
+  float* dSh[2];
+  float* dkmh[2];
+  for (int i = 0; i < 2; ++i, ws += half_state_bytes(p)) Sh[i] = (float*)ws;
+  for (int i = 0; i < 2; ++i, ws += half_state_bytes(p)) dSh[i] = (float*)ws;
+  for (int i = 0; i < 2; ++i, ws += vec_bytes(p)) dkmh[i] = (float*)ws;
+  float* dkm = (float*)ws;
+  ws += vec_bytes(p);
+  float* dS = (float*)ws;
+  generic::split_columns(p, a.s, Sh[0], Sh[1], st);
+  const bool direct = nchunks == 1;
+  const int pchunk = mfma::partial_chunk(h, dtype, 4, chunk);
+  for (int i = 0; i < 2; ++i) {  // the partial buffer serves both queries in turn (one stream)
+    int rc = mfma::bwd_a(mfma::with_interleave(h, dtype, 4), dtype, a.q[i], a.q[i], a.dout[i], Sh[i], a.km,
+                         a.dq[i], nullptr, partial, chunk, nchunks, st, direct ? dSh[i] : nullptr,
+                         direct ? dkmh[i] : nullptr);
+    if (rc != kOk) return rc;
+    if (!direct) generic::state_reduce(h, partial, pchunk, nchunks, dSh[i], nullptr, dkmh[i], st);
+  }
+  generic::join_columns(p, dSh[0], dSh[1], dkmh[0], dkmh[1], dS, dkm, st);
+  // dk_t = v_t (s dS)^T + dkm/L, dv_t = k_t (s dS)
+  mfma::RowsJob jk{a.v, nullptr, dS, 1, p.DV, nullptr, dkm, a.dk};
+  mfma::RowsJob jv{a.k, nullptr, dS, p.DV, 1, nullptr, nullptr, a.dv};
+  const Prob pi = mfma::with_interleave(p, dtype, 2);
+  if (p.DK == p.DV) return mfma::rows2(pi, dtype, jk, jv, p.DV, p.DK, st);
+  int rc = mfma::rows(pi, dtype, jk, p.DV, p.DK, st);
+  if (rc == kOk) rc = mfma::rows(pi, dtype, jv, p.DK, p.DV, st);
+  return rc;
+}
+
 }  // namespace plan
 }  // namespace fbla

@@ -31,6 +31,9 @@ _SIGNATURES = {
     "fbla_static_scratch_bytes": (_sz, []),
     "fbla_la_fwd_static": (_i32, [_vp] * 8 + [_i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_la_bwd": (_i32, [_vp] * 14 + [_sz, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
+    "fbla_la_pair_workspace_bytes": (_sz, [_i32, _i64, _i64, _i64, _i32, _i32, _i32]),
+    "fbla_la_pair_fwd": (_i32, [_vp] * 9 + [_sz, _i64, _i64, _i64, _i32, _i32, _i32, _f32, _f32, _vp]),
+    "fbla_la_pair_bwd": (_i32, [_vp] * 13 + [_sz, _i64, _i64, _i64, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_la_cross_workspace_bytes": (_sz, [_i32, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32]),
     "fbla_la_cross_fwd": (_i32, [_vp] * 7 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
     "fbla_la_cross_bwd": (_i32, [_vp] * 10 + [_sz, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _vp]),
@@ -216,6 +219,53 @@ def la_bwd(q, k, v, q_rope, k_rope, do, s, km, scale, eps, flags):
                            _stream(dev))
     _check(rc, "fbla_la_bwd")
     return dq, dk, dv, dqr, dkr
+
+
+def pair_supported(q, v):
+    """Whether the two-query operator covers these shapes (contiguous [B,H,L,DK] / [B,H,L,DV])."""
+    B, H, T, DK = q.shape
+    return bool(q.is_cuda and q.dtype in (torch.float16, torch.bfloat16) and
+                lib().fbla_la_pair_workspace_bytes(0, B, H, T, DK, v.shape[-1], dtype_code(q)))
+
+
+def pair_fwd(q1, q2, k, v, scale, eps):
+    """Two queries on shared keys and values: returns (o1, o2, s, km); o_i are [B,H,L,DV/2]."""
+    _require_gpu(q1, q2, k, v)
+    q1, q2, k, v = _aligned(q1, q2, k, v)
+    L = lib()
+    B, H, T, DK = q1.shape
+    DV = v.shape[-1]
+    code = dtype_code(q1)
+    dev = q1.device
+    o1 = torch.empty(B, H, T, DV // 2, dtype=v.dtype, device=dev)
+    o2 = torch.empty_like(o1)
+    s = torch.empty(B, H, DK, DV, dtype=torch.float32, device=dev)
+    km = torch.empty(B, H, DK, dtype=torch.float32, device=dev)
+    with _on(dev):
+        ws = _workspace(L.fbla_la_pair_workspace_bytes(0, B, H, T, DK, DV, code), dev)
+        rc = L.fbla_la_pair_fwd(_ptr(q1), _ptr(q2), _ptr(k), _ptr(v), _ptr(o1), _ptr(o2), _ptr(s), _ptr(km),
+                                _ptr(ws), ws.numel(), B, H, T, DK, DV, code, float(scale), float(eps), _stream(dev))
+    _check(rc, "fbla_la_pair_fwd")
+    return o1, o2, s, km
+
+
+def pair_bwd(q1, q2, k, v, do1, do2, s, km, scale, eps):
+    """Backward of pair_fwd: returns (dq1, dq2, dk, dv)."""
+    _require_gpu(q1, q2, k, v, do1, do2)
+    q1, q2, k, v, do1, do2, s, km = _aligned(q1, q2, k, v, do1, do2, s, km)
+    L = lib()
+    B, H, T, DK = q1.shape
+    DV = v.shape[-1]
+    code = dtype_code(q1)
+    dev = q1.device
+    dq1, dq2, dk, dv = torch.empty_like(q1), torch.empty_like(q2), torch.empty_like(k), torch.empty_like(v)
+    with _on(dev):
+        ws = _workspace(L.fbla_la_pair_workspace_bytes(1, B, H, T, DK, DV, code), dev)
+        rc = L.fbla_la_pair_bwd(_ptr(q1), _ptr(q2), _ptr(k), _ptr(v), _ptr(do1), _ptr(do2), _ptr(s), _ptr(km),
+                                _ptr(dq1), _ptr(dq2), _ptr(dk), _ptr(dv), _ptr(ws), ws.numel(), B, H, T, DK, DV,
+                                code, float(scale), float(eps), _stream(dev))
+    _check(rc, "fbla_la_pair_bwd")
+    return dq1, dq2, dk, dv
 
 
 def varlen_fwd(q, k, v, cu_seqlens, max_seqlen, scale, eps, extra_flags=0):

@@ -8,7 +8,7 @@ import torch.nn.functional as F
 
 from flash_bla.layers._common import check_mode, merge_heads, split_heads, torch_linear_attention
 from flash_bla.layers._pvt import PvtLinearAttentionBase
-from flash_bla.ops.linear_attn.fused import linear_attention
+from flash_bla.ops.linear_attn.paired import paired_linear_attention
 
 
 class PolaLinearAttention(PvtLinearAttentionBase):
@@ -33,8 +33,11 @@ class PolaLinearAttention(PvtLinearAttentionBase):
         q_same = torch.cat([q_pos, q_neg], dim=-1)
         q_opp = torch.cat([q_neg, q_pos], dim=-1)
         k_both = torch.cat([k_pos, k_neg], dim=-1)
-        v_same, v_opp = (t.contiguous() for t in v.chunk(2, dim=-1))
-        attend = linear_attention if fast else torch_linear_attention
-        out = torch.cat([attend(q_same, k_both, v_same), attend(q_opp, k_both, v_opp)], dim=-1)
+        if fast:  # both pairings on one state pass over the shared keys and values
+            out = torch.cat(paired_linear_attention(q_same, q_opp, k_both, v), dim=-1)
+        else:
+            v_same, v_opp = v.chunk(2, dim=-1)
+            out = torch.cat([torch_linear_attention(q_same, k_both, v_same),
+                             torch_linear_attention(q_opp, k_both, v_opp)], dim=-1)
         out = (merge_heads(out) + self._value_conv(v, N, H, W)) * gate
         return self.proj_drop(self.proj(out))

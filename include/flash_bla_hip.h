@@ -126,6 +126,26 @@ int fbla_la_fwd_static(const void* q, const void* k, const void* v, const void* 
                        int64_t L, int DK, int DV, int dtype, int flags, float scale, float eps,
                        void* stream);
 
+/* Two queries on shared keys and values, dense, with the denominator.  Replaces the two operator
+ * calls of PolaLinearAttention.forward (flash_bla/layers/polaformer.py:89-90:
+ *   x_sim = linear_attention(q_sim, k, v1),  x_opp = linear_attention(q_opp, k, v2)
+ * with v1 | v2 the two halves of the value channels), which read k twice forward and twice
+ * backward and leave the sum of the two dk to autograd.  Here
+ *   S = scale * K^T [v1 | v2]  (one pass over k and v),  km = mean k,
+ *   o1 = (q1 S[:, :DV/2]) / (q1 . km + eps),  o2 = (q2 S[:, DV/2:]) / (q2 . km + eps),
+ * and the backward reads k and v once and writes dk = dk1 + dk2 once.
+ * q1, q2, dq1, dq2, k, dk: [B,H,L,DK]; v, dv: [B,H,L,DV]; o1, o2, dout1, dout2: [B,H,L,DV/2];
+ * s: [B,H,DK,DV], km: [B,H,DK] fp32.  fp16 / bf16, DK and DV/2 multiples of 8 up to 128 (the
+ * workspace query returns 0 for anything else, the calls FBLA_ERR_UNSUPPORTED). */
+size_t fbla_la_pair_workspace_bytes(int pass, int64_t B, int64_t H, int64_t L, int DK, int DV, int dtype);
+int fbla_la_pair_fwd(const void* q1, const void* q2, const void* k, const void* v, void* o1, void* o2,
+                     float* s, float* km, void* workspace, size_t workspace_bytes, int64_t B, int64_t H,
+                     int64_t L, int DK, int DV, int dtype, float scale, float eps, void* stream);
+int fbla_la_pair_bwd(const void* q1, const void* q2, const void* k, const void* v, const void* dout1,
+                     const void* dout2, const float* s, const float* km, void* dq1, void* dq2, void* dk,
+                     void* dv, void* workspace, size_t workspace_bytes, int64_t B, int64_t H, int64_t L,
+                     int DK, int DV, int dtype, float scale, float eps, void* stream);
+
 /* Dense problems with Lk key / value tokens and Lq query tokens per (batch, head), Lk != Lq:
  * q, dq: [B,H,Lq,DK]; k, dk: [B,H,Lk,DK]; v, dv: [B,H,Lk,DV]; o, dout: [B,H,Lq,DV]; km is the mean
  * over the Lk keys.  The reference has no counterpart: its dense kernels take one length from q
