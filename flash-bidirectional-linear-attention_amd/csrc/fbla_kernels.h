@@ -172,8 +172,8 @@ int bwd_a(const Prob& p, int dtype, const void* qn, const void* qd, const void* 
 }  // namespace mfma
 
 namespace mfma32 {
-// fp32 inputs on v_mfma_f32_32x32x2_f32: head dims that are multiples of 4 up to 64, not
-// decoupled.  Called through the mfma:: entry points, which dispatch on the dtype.
+// fp32 inputs on v_mfma_f32_32x32x2_f32: head dims that are multiples of 4 up to 64 (plain and
+// decoupled) or up to 128 (plain).  Called through the mfma:: entry points, which dispatch on the dtype.
 bool supported(const Prob& p);
 void state(const Prob& p, const float* kn, const float* v, const float* kd, float* partial,
            const float* tokscal, int64_t total_rows, int chunk, int nchunks, hipStream_t st, float* fin_mat,
@@ -181,6 +181,15 @@ void state(const Prob& p, const float* kn, const float* v, const float* kd, floa
 int rows(const Prob& p, const mfma::RowsJob& job, const mfma::RowsJob* job2, int dr, int dc, hipStream_t st);
 int bwd_tokens(const Prob& p, const float* qn, const float* qd, const float* dout, const float* S,
                const float* km, float* dqn, float* dqd, float* tokscal, int64_t total_rows, hipStream_t st);
+// Heads with a side above 64 (fbla_mfma32w.hip): tiled 128 x 128, head dims that are multiples of 4 up
+// to 128, the plain operator (not decoupled).  The functions above hand such problems over.
+bool wide(const Prob& p);
+bool wide_supported(const Prob& p);
+void wide_state(const Prob& p, const float* kn, const float* v, float* partial, const float* tokscal,
+                int64_t total_rows, int chunk, int nchunks, hipStream_t st, float* fin_mat, float* fin_vec);
+int wide_rows(const Prob& p, const mfma::RowsJob& job, const mfma::RowsJob* job2, int dr, int dc, hipStream_t st);
+int wide_bwd_tokens(const Prob& p, const float* q, const float* dout, const float* S, const float* km, float* dq,
+                    float* tokscal, int64_t total_rows, hipStream_t st);
 }  // namespace mfma32
 
 // The callers' feature map elu(x) + 1 and its derivative (fbla_feature.hip).

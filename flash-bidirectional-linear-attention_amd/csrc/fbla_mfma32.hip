@@ -1,8 +1,8 @@
-// MFMA kernels for fp32 inputs, heads tiled 64 x 64: head dims that are multiples of 4 (16-byte
-// row pieces) up to 64, smaller ones with zero padding (PAD variants: true row lengths in memory,
+// MFMA kernels for fp32 inputs, heads tiled 64 x 64 (larger heads: fbla_mfma32w.hip): head dims that
+// are multiples of 4 (16-byte row pieces) up to 64, smaller ones with zero padding (PAD variants: true row lengths in memory,
 // missing features read as zero, outputs and state in their true shapes).  Dense and packed
 // layouts, with or without the denominator, plain and decoupled (numerator from the rotary
-// features, denominator from the plain ones); larger heads stay on the shape-generic kernels.  v_mfma_f32_32x32x2_f32 computes in fp32 throughout, so
+// features, denominator from the plain ones).  v_mfma_f32_32x32x2_f32 computes in fp32 throughout, so
 // there is no operand splitting here: A lane l holds A[m = l%32][k = l/32], B lane l
 // holds B[k = l/32][n = l%32], C register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32].
 // One instruction covers two values of the contraction index and takes 64 cycles:
@@ -490,6 +490,7 @@ __global__ __launch_bounds__(kThreads) void rows32_kernel(Prob p, Rows32Job job0
 // host side
 // ===========================================================================
 bool supported(const Prob& p) {
+  if (wide(p)) return wide_supported(p);
   return p.DK >= 4 && p.DV >= 4 && p.DK <= D && p.DV <= D && p.DK % 4 == 0 && p.DV % 4 == 0;
 }
 static bool padded(const Prob& p) { return p.DK != D || p.DV != D; }
@@ -497,6 +498,7 @@ static bool padded(const Prob& p) { return p.DK != D || p.DV != D; }
 void state(const Prob& p, const float* kn, const float* v, const float* kd, float* partial,
            const float* tokscal, int64_t total_rows, int chunk, int nchunks, hipStream_t st, float* fin_mat,
            float* fin_vec) {
+  if (wide(p)) return wide_state(p, kn, v, partial, tokscal, total_rows, chunk, nchunks, st, fin_mat, fin_vec);
   const dim3 grid((unsigned)((int64_t)p.N * p.H * nchunks)), block(kThreads);
   auto go = [&](auto kernel) {
     kernel<<<grid, block, 0, st>>>(p, kn, v, kd, partial, tokscal, tokscal ? total_rows : 0, fin_mat, fin_vec, chunk, nchunks);
@@ -564,6 +566,7 @@ static Rows32Job convert(const mfma::RowsJob& j, int dr, int dc) {
 
 // dr, dc: the contracted and the output head dim of the job (of both jobs when there are two)
 int rows(const Prob& p, const mfma::RowsJob& job, const mfma::RowsJob* job2, int dr, int dc, hipStream_t st) {
+  if (wide(p)) return wide_rows(p, job, job2, dr, dc, st);
   const Rows32Job a = convert(job, dr, dc);
   if (job.xden && job.xden != job.x) return launch_rows<true, false, true>(p, a, nullptr, st);
   if (job.xden) return launch_rows<true, false>(p, a, nullptr, st);
@@ -578,6 +581,7 @@ int rows(const Prob& p, const mfma::RowsJob& job, const mfma::RowsJob* job2, int
 // qd = q and dqd = dq; otherwise qn == qd and dqd is not used)
 int bwd_tokens(const Prob& p, const float* qn, const float* qd, const float* dout, const float* S,
                const float* km, float* dqn, float* dqd, float* tokscal, int64_t total_rows, hipStream_t st) {
+  if (wide(p)) return wide_bwd_tokens(p, qn, dout, S, km, dqn, tokscal, total_rows, st);
   Rows32Job j;
   j.x = dout;
   j.xnum = qn;
