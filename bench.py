@@ -237,11 +237,12 @@ def main():
     ap.add_argument("--no-tables", action="store_true", help="skip the reference's benchmark tables")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the other BASELINE configs (the `configs` list of the JSON line)")
-    ap.add_argument("--only", choices=["c3", "c5", "fm", "callers", "tables"], default=None,
+    ap.add_argument("--only", choices=["c3", "c5", "fm", "callers", "f32", "tables"], default=None,
                     help="profiling aid: time just BASELINE config 3 (packed variable-length, D=64 and "
                          "D=128), config 5 (piecewise attention), the feature map together with the "
-                         "attention (fm) or the decoupled operator and the layer callers' head dims "
-                         "(callers), table on stderr, no headline line")
+                         "attention (fm), the decoupled operator, the layer callers' head dims and PolaFormer's "
+                         "pairings (callers), fp32 inputs (f32), table on stderr, no headline line; tables: the "
+                         "reference's benchmark tables as one JSON object")
     ap.add_argument("--configs", action="store_true",
                     help="add the other operator families (simple_la, bf16, the feature map, the layer callers' "
                          "head dims) to the `configs` list")
@@ -268,6 +269,8 @@ def main():
             feature_map_config(dev, flush)
         elif args.only == "callers":
             caller_configs(dev, flush, head_dims=True)
+        elif args.only == "f32":
+            fp32_config(dev, flush)
         else:
             piecewise_config(dev, flush)
         return
@@ -552,6 +555,7 @@ def other_configs(dev, flush):
             rows.append(_report(f"simple_la B8-H16-T16384-D64 {tag}", 4 * nb, 11 * nb, f, s, flush))
     rows.append(feature_map_config(dev, flush))
     rows += caller_configs(dev, flush, head_dims=True)
+    rows += fp32_config(dev, flush)
     return rows
 
 
@@ -609,6 +613,22 @@ def caller_configs(dev, flush, head_dims=False):
             f, s = run(linear_attention, (q, k, v), do)
             rows.append(_report(name, 2 * nqk + 2 * nv, 6 * nqk + 5 * nv, f, s, flush))
     rows.append(polaformer_config(dev, flush))
+    return rows
+
+
+def fp32_config(dev, flush):
+    """fp32 inputs (the precision the reference's tests use, tests/ops/test_varlen_linear_attn.py:15-18) at
+    B8-H16-T4096: heads of 64 and of 128 on the fp32 matrix instructions."""
+    from flash_bla.ops.linear_attn.fused import linear_attention
+    rows = []
+    for D in (64, 128):
+        q, k, v, do = make_inputs(8, 16, 4096, D, torch.float32, dev)
+        for t in (q, k, v):
+            t.requires_grad_()
+        nb = q.numel() * 4
+        f, s = _fwd_and_step(linear_attention, (q, k, v), do)
+        rows.append(_report(f"linear_attn B8-H16-T4096-D{D} fp32", 4 * nb, 11 * nb, f, s, flush))
+        del q, k, v, do
     return rows
 
 
