@@ -48,8 +48,8 @@ __device__ __forceinline__ f32x16 mma(float a, float b, f32x16 c) {
 // ===========================================================================
 // Lane l = (f = l%32, kb = l/32); wave w = block (bk, bv).  A 16-token tile is eight k-steps; in
 // k-step s the lane holds feature 64 bk + 32 a + f of the key row and 64 bv + 32 b + f of the value
-// row of token 2s + kb (a, b = 0, 1).  All four waves walk the same tiles; two register buffers
-// alternate.
+// row of token 2s + kb (a, b = 0, 1).  All four waves walk the same tiles; two or three register
+// buffers rotate.
 template <bool SCALED, bool PAD>
 __global__ __launch_bounds__(kThreads, 2) void state32w_kernel(
     Prob p, const float* __restrict__ kn, const float* __restrict__ v, float* __restrict__ partial,
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(kThreads, 2) void state32w_kernel(
     Buf b0;
     fetch_checked(b0, t0);
     compute(b0, t0, true);
-  } else {
+  } else if constexpr (SCALED) {  // (the per-row scalars leave registers for two buffers)
     Buf b0, b1;
     fetch(b0, t0);
     while (true) {
@@ -191,6 +191,26 @@ __global__ __launch_bounds__(kThreads, 2) void state32w_kernel(
       if (t0 >= t_end) break;
       fetch(b0, t0 + 16);
       compute(b1, t0, false);
+      t0 += 16;
+      if (t0 >= t_end) break;
+    }
+  } else {
+    // three register buffers in rotation: the rows of two tiles are in flight while one is multiplied
+    // (one tile is 2048 matrix cycles, less than a load takes under load)
+    Buf b0, b1, b2;
+    fetch(b0, t0);
+    fetch(b1, t0 + 16);
+    while (true) {
+      fetch(b2, t0 + 32);
+      compute(b0, t0, false);
+      t0 += 16;
+      if (t0 >= t_end) break;
+      fetch(b0, t0 + 32);
+      compute(b1, t0, false);
+      t0 += 16;
+      if (t0 >= t_end) break;
+      fetch(b1, t0 + 32);
+      compute(b2, t0, false);
       t0 += 16;
       if (t0 >= t_end) break;
     }
