@@ -6,6 +6,8 @@
 //
 // Replaces the Triton kernels of flash_bla/ops/linear_attn/fused.py:26-347,
 // decoupled.py:27-408, varlen.py:30-332 and simple_la/fused.py:26-426.
+#include <algorithm>
+
 #include "fbla_kernels.h"
 
 namespace fbla {
@@ -543,6 +545,77 @@ void state_reduce(const Prob& p, const float* partial, int chunk, int nchunks, f
   const int blocks_per_head = (p.DK * p.DV + p.DK + kThreads - 1) / kThreads;
   state_reduce_kernel<<<dim3((unsigned)((int64_t)p.N * p.H * blocks_per_head)), dim3(kThreads), 0, st>>>(
       p, partial, chunk, nchunks, mat, mat_t, vec, blocks_per_head);
+}
+
+// count matrices [rs][cs] -> [rd][cd]: the common part copied, the rest of the destination zero (widening
+// token rows to the next row length the matrix-core kernels take, and narrowing their results back).
+// Consecutive threads take consecutive destination elements.
+template <typename E>
+__global__ __launch_bounds__(kThreads) void resize_matrices_kernel(const E* __restrict__ src, int64_t rs, int cs,
+                                                                   E* __restrict__ dst, int64_t rd, int cd,
+                                                                   int64_t total) {
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kThreads) {
+    const int64_t row_all = i / cd;
+    const int c = (int)(i - row_all * cd);
+    const int64_t m = row_all / rd, r = row_all - m * rd;
+    dst[i] = (r < rs && c < cs) ? src[(m * rs + r) * cs + c] : E(0);
+  }
+}
+// The same for one matrix of many rows whose number does not change (token tensors): every workgroup takes a
+// span of kResizeSpan consecutive destination elements, thread t the elements t, t + 256, ... of it (whole
+// 128-byte pieces per wave instruction), with one division per thread and the row / column carried along.
+constexpr int kResizePer = 16, kResizeSpan = kThreads * kResizePer;
+template <typename E>
+__global__ __launch_bounds__(kThreads) void resize_rows_kernel(const E* __restrict__ src, int cs, E* __restrict__ dst,
+                                                               int cd, int64_t total) {
+  const int64_t base = (int64_t)blockIdx.x * kResizeSpan;
+  const int64_t row0 = base / cd;  // (uniform: scalar arithmetic)
+  const uint32_t c0 = (uint32_t)(base - row0 * cd) + threadIdx.x;
+  uint32_t rowd = c0 / (uint32_t)cd, c = c0 - rowd * (uint32_t)cd;
+  const uint32_t left = (uint32_t)(total - base < kResizeSpan ? total - base : kResizeSpan);
+  const E* s = src + row0 * cs;
+  E* d = dst + base;
+  E val[kResizePer];
+#pragma unroll
+  for (int u = 0; u < kResizePer; ++u) {
+    const uint32_t off = threadIdx.x + u * kThreads;
+    const bool in = off < left && c < (uint32_t)cs;
+    val[u] = s[in ? (size_t)rowd * cs + c : 0];
+    val[u] = in ? val[u] : E(0);
+    c += kThreads;
+    while (c >= (uint32_t)cd) {
+      c -= cd;
+      ++rowd;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kResizePer; ++u) {
+    const uint32_t off = threadIdx.x + u * kThreads;
+    if (off < left) d[off] = val[u];
+  }
+}
+
+void resize_matrices(const void* src, int64_t rs, int cs, void* dst, int64_t rd, int cd, int64_t count, int elem_bytes,
+                     hipStream_t st) {
+  const int64_t total = count * rd * cd;
+  if (total <= 0) return;
+  if (count == 1 && rs == rd) {
+    const unsigned spans = (unsigned)cdiv64(total, kResizeSpan);
+    if (elem_bytes == 2)
+      resize_rows_kernel<uint16_t><<<dim3(spans), dim3(kThreads), 0, st>>>((const uint16_t*)src, cs, (uint16_t*)dst, cd,
+                                                                          total);
+    else
+      resize_rows_kernel<uint32_t><<<dim3(spans), dim3(kThreads), 0, st>>>((const uint32_t*)src, cs, (uint32_t*)dst, cd,
+                                                                          total);
+    return;
+  }
+  const unsigned grid = (unsigned)std::min<int64_t>(cdiv64(total, kThreads), 1 << 20);
+  if (elem_bytes == 2)
+    resize_matrices_kernel<uint16_t><<<dim3(grid), dim3(kThreads), 0, st>>>((const uint16_t*)src, rs, cs, (uint16_t*)dst,
+                                                                           rd, cd, total);
+  else
+    resize_matrices_kernel<uint32_t><<<dim3(grid), dim3(kThreads), 0, st>>>((const uint32_t*)src, rs, cs, (uint32_t*)dst,
+                                                                           rd, cd, total);
 }
 
 // Two queries sharing keys and values: the state's value columns [0, DV/2) serve the first query,

@@ -77,6 +77,10 @@ void state_partial(const Prob& p, int dtype, const void* kn, const void* v, cons
 void state_reduce(const Prob& p, const float* partial, int chunk, int nchunks, float* mat,
                   float* mat_t, float* vec, hipStream_t st);
 void transpose_state(const Prob& p, const float* mat, float* mat_t, hipStream_t st);
+// `count` matrices of rs x cs elements (2 or 4 bytes each) into matrices of rd x cd: the common part is copied,
+// the rest of the destination is zero
+void resize_matrices(const void* src, int64_t rs, int cs, void* dst, int64_t rd, int cd, int64_t count, int elem_bytes,
+                     hipStream_t st);
 // p.DV even: the column halves of a [N*H, DK, DV] matrix as two [N*H, DK, DV/2] matrices, and back
 // (join also adds two [N*H, DK] vectors when `vec` is given)
 void split_columns(const Prob& p, const float* mat, float* lo, float* hi, hipStream_t st);

@@ -1,7 +1,8 @@
 // The plan: which kernels run, in which order, for each entry point, and how the
 // caller's workspace is carved up.  MFMA kernels are used for the shapes they
-// cover (16-bit inputs with head dims that are multiples of 8 up to 128, fp32 inputs
-// with head dims that are multiples of 4 up to 64); everything else runs on the generic kernels.
+// cover (16-bit inputs with head dims that are multiples of 8 up to 128, fp32 inputs with head dims
+// that are multiples of 4 up to 128, up to 64 for the decoupled operator); other head dims run on
+// them through zero-widened copies, what is left runs on the generic kernels.
 //
 // forward :  state partials -> fixed-order reduce (S, km) -> output rows
 // backward:  S^T -> pass A (dq, partial dS/dkm) -> reduce (s dS, its transpose, dkm/L)
@@ -115,6 +116,64 @@ static Prob with_order(const Prob& p, void* workspace, size_t used, hipStream_t 
   return r;
 }
 
+// ---- head dims between the row lengths the matrix-core kernels take --------------------------
+// 16-bit rows are moved in 16-byte pieces (head dims that are multiples of 8), fp32 rows likewise
+// (multiples of 4).  A problem with another head dim (17 x 13, 100 x 100: shapes of the reference's
+// test matrix, tests/ops/test_varlen_linear_attn.py:15-18) is widened to the next such row length
+// with zeros in workspace copies of its tensors, run on the matrix-core kernels, and its results are
+// narrowed back: zero features add nothing to any sum of the operator, so the results are those of the
+// original problem.  The copies cost two to three tensor passes per tensor; the shape-generic kernels
+// they replace are five to ten times slower than the matrix-core ones.
+static int elem_bytes(int dtype) { return dtype == kF32 ? 4 : 2; }
+static int widened_dim(int d, int dtype) {
+  const int unit = dtype == kF32 ? 4 : 8;
+  return (d + unit - 1) / unit * unit;
+}
+static Prob widened(const Prob& p, int dtype) {
+  Prob w = p;
+  w.DK = widened_dim(p.DK, dtype);
+  w.DV = widened_dim(p.DV, dtype);
+  return w;
+}
+static bool widen(const Prob& p, int dtype) {
+  if (mfma::supported(p, dtype)) return false;
+  const Prob w = widened(p, dtype);
+  return w.DK <= 128 && w.DV <= 128 && mfma::supported(w, dtype);
+}
+// rows of the tensors on the query side / on the key side
+static int64_t query_rows(const Prob& p) { return p.cu ? p.T * p.H : (int64_t)p.N * p.H * p.L; }
+static int64_t key_rows(const Prob& p) { return p.cu ? p.T * p.H : (int64_t)p.N * p.H * (cross(p) ? p.Lk : p.L); }
+static size_t rows_bytes(int64_t rows, int d, int dtype) { return align_up((size_t)rows * d * elem_bytes(dtype), 256); }
+// carves `bytes` out of the workspace
+static void* take(char*& ws, size_t bytes) {
+  void* r = ws;
+  ws += bytes;
+  return r;
+}
+// a widened copy of a token tensor (null stays null)
+static const void* widen_rows(const void* src, int64_t rows, int d, int dw, int dtype, char*& ws, hipStream_t st) {
+  if (!src) return nullptr;
+  void* dst = take(ws, rows_bytes(rows, dw, dtype));
+  generic::resize_matrices(src, rows, d, dst, rows, dw, 1, elem_bytes(dtype), st);
+  return dst;
+}
+
+static size_t widened_fwd_bytes(const Prob& p, int dtype) {
+  const Prob w = widened(p, dtype);
+  const bool dec = p.flags & kDecoupled;
+  return (dec ? 2 : 1) * (rows_bytes(query_rows(p), w.DK, dtype) + rows_bytes(key_rows(p), w.DK, dtype)) +
+         rows_bytes(key_rows(p), w.DV, dtype) + rows_bytes(query_rows(p), w.DV, dtype) + state_bytes(w) + vec_bytes(w) +
+         fwd_workspace_bytes(w, dtype);
+}
+static size_t widened_bwd_bytes(const Prob& p, int dtype) {
+  const Prob w = widened(p, dtype);
+  const bool dec = p.flags & kDecoupled;
+  // inputs q, k, v, dO (+ rotary rows), gradients dq, dk, dv (+ rotary), state, mean key
+  return (dec ? 4 : 2) * (rows_bytes(query_rows(p), w.DK, dtype) + rows_bytes(key_rows(p), w.DK, dtype)) +
+         2 * rows_bytes(key_rows(p), w.DV, dtype) + rows_bytes(query_rows(p), w.DV, dtype) + state_bytes(w) +
+         vec_bytes(w) + bwd_workspace_bytes(w, dtype);
+}
+
 static size_t fwd_used_bytes(const Prob& pc, int dtype) {
   const Prob p = key_side(pc);
   return partial_bytes(p, dtype, fwd_chunk(p, dtype));
@@ -126,18 +185,86 @@ static size_t bwd_used_bytes(const Prob& pc, int dtype) {
 }
 
 // partials | walking order
-size_t fwd_workspace_bytes(const Prob& pc, int dtype) { return fwd_used_bytes(pc, dtype) + perm_bytes(pc); }
+size_t fwd_workspace_bytes(const Prob& pc, int dtype) {
+  if (widen(pc, dtype)) return widened_fwd_bytes(pc, dtype);
+  return fwd_used_bytes(pc, dtype) + perm_bytes(pc);
+}
 
 // partials | S^T | s*dS | (s*dS)^T | dkm/L | per-row scalars | walking order
-size_t bwd_workspace_bytes(const Prob& pc, int dtype) { return bwd_used_bytes(pc, dtype) + perm_bytes(pc); }
+size_t bwd_workspace_bytes(const Prob& pc, int dtype) {
+  if (widen(pc, dtype)) return widened_bwd_bytes(pc, dtype);
+  return bwd_used_bytes(pc, dtype) + perm_bytes(pc);
+}
 
 // Different numbers of queries and keys work for every operator family (the decoupled one too:
 // its rotary and plain rows come in pairs of equal length on either side).
 static int check_cross(const Prob&, int) { return kOk; }
 
+static int widened_forward(const Prob& p, int dtype, const FwdArgs& a, hipStream_t st) {
+  const Prob w = widened(p, dtype);
+  const int64_t qr = query_rows(p), kr = key_rows(p), nh = (int64_t)p.N * p.H;
+  char* ws = (char*)a.workspace;
+  FwdArgs b = a;
+  b.q = widen_rows(a.q, qr, p.DK, w.DK, dtype, ws, st);
+  b.k = widen_rows(a.k, kr, p.DK, w.DK, dtype, ws, st);
+  b.v = widen_rows(a.v, kr, p.DV, w.DV, dtype, ws, st);
+  b.q_rope = widen_rows(a.q_rope, qr, p.DK, w.DK, dtype, ws, st);
+  b.k_rope = widen_rows(a.k_rope, kr, p.DK, w.DK, dtype, ws, st);
+  b.o = take(ws, rows_bytes(qr, w.DV, dtype));
+  b.s = (float*)take(ws, state_bytes(w));
+  b.km = (float*)take(ws, vec_bytes(w));
+  b.workspace = ws;
+  b.workspace_bytes = a.workspace_bytes - (size_t)(ws - (char*)a.workspace);
+  int rc = forward(w, dtype, b, st);
+  if (rc != kOk) return rc;
+  generic::resize_matrices(b.o, qr, w.DV, a.o, qr, p.DV, 1, elem_bytes(dtype), st);
+  generic::resize_matrices(b.s, w.DK, w.DV, a.s, p.DK, p.DV, nh, 4, st);
+  if (a.km) generic::resize_matrices(b.km, 1, w.DK, a.km, 1, p.DK, nh, 4, st);
+  return kOk;
+}
+
+static int widened_backward(const Prob& p, int dtype, const BwdArgs& a, hipStream_t st) {
+  const Prob w = widened(p, dtype);
+  const int64_t qr = query_rows(p), kr = key_rows(p), nh = (int64_t)p.N * p.H;
+  const bool dec = p.flags & kDecoupled;
+  char* ws = (char*)a.workspace;
+  BwdArgs b = a;
+  b.q = widen_rows(a.q, qr, p.DK, w.DK, dtype, ws, st);
+  b.k = widen_rows(a.k, kr, p.DK, w.DK, dtype, ws, st);
+  b.v = widen_rows(a.v, kr, p.DV, w.DV, dtype, ws, st);
+  b.q_rope = widen_rows(a.q_rope, qr, p.DK, w.DK, dtype, ws, st);
+  b.k_rope = widen_rows(a.k_rope, kr, p.DK, w.DK, dtype, ws, st);
+  b.dout = widen_rows(a.dout, qr, p.DV, w.DV, dtype, ws, st);
+  float* sw = (float*)take(ws, state_bytes(w));
+  float* kmw = (float*)take(ws, vec_bytes(w));
+  generic::resize_matrices(a.s, p.DK, p.DV, sw, w.DK, w.DV, nh, 4, st);
+  if (a.km) generic::resize_matrices(a.km, 1, p.DK, kmw, 1, w.DK, nh, 4, st);
+  b.s = sw;
+  b.km = a.km ? kmw : nullptr;
+  b.dq = take(ws, rows_bytes(qr, w.DK, dtype));
+  b.dk = take(ws, rows_bytes(kr, w.DK, dtype));
+  b.dv = take(ws, rows_bytes(kr, w.DV, dtype));
+  b.dq_rope = dec ? take(ws, rows_bytes(qr, w.DK, dtype)) : nullptr;
+  b.dk_rope = dec ? take(ws, rows_bytes(kr, w.DK, dtype)) : nullptr;
+  b.workspace = ws;
+  b.workspace_bytes = a.workspace_bytes - (size_t)(ws - (char*)a.workspace);
+  int rc = backward(w, dtype, b, st);
+  if (rc != kOk) return rc;
+  const int eb = elem_bytes(dtype);
+  generic::resize_matrices(b.dq, qr, w.DK, a.dq, qr, p.DK, 1, eb, st);
+  generic::resize_matrices(b.dk, kr, w.DK, a.dk, kr, p.DK, 1, eb, st);
+  generic::resize_matrices(b.dv, kr, w.DV, a.dv, kr, p.DV, 1, eb, st);
+  if (dec) {
+    generic::resize_matrices(b.dq_rope, qr, w.DK, a.dq_rope, qr, p.DK, 1, eb, st);
+    generic::resize_matrices(b.dk_rope, kr, w.DK, a.dk_rope, kr, p.DK, 1, eb, st);
+  }
+  return kOk;
+}
+
 int forward(const Prob& pc_, int dtype, const FwdArgs& a, hipStream_t st) {
   int rc_cross = check_cross(pc_, dtype);
   if (rc_cross != kOk) return rc_cross;
+  if (widen(pc_, dtype) && phase_mask() == kPhaseAll) return widened_forward(pc_, dtype, a, st);
   const Prob pc = with_order(pc_, a.workspace, fwd_used_bytes(pc_, dtype), st);
   const bool is_cross = cross(pc);
   const Prob p_ = key_side(pc);    // state kernel, reduce
@@ -200,6 +327,7 @@ int forward(const Prob& pc_, int dtype, const FwdArgs& a, hipStream_t st) {
 int backward(const Prob& pc_, int dtype, const BwdArgs& a, hipStream_t st) {
   int rc_cross = check_cross(pc_, dtype);
   if (rc_cross != kOk) return rc_cross;
+  if (widen(pc_, dtype) && phase_mask() == kPhaseAll) return widened_backward(pc_, dtype, a, st);
   if ((pc_.flags & kElu1) && !(pc_.flags & kElu1Grad)) {
     set_error("the feature map on load (FBLA_ELU1_QK) in a backward needs FBLA_ELU1_GRAD as well: dq, dk are then "
               "gradients with respect to the q, k given");

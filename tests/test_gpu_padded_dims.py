@@ -197,3 +197,23 @@ def test_fp32_decoupled(dims):
     """The decoupled operator in fp32 (the MLLA / RALA blocks without autocast)."""
     for i, L in enumerate(LENGTHS + [5000]):
         _check_dense("decoupled", 2, 2, L, dims[0], dims[1], torch.float32, 60 * i + dims[1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32], ids=str)
+@pytest.mark.parametrize("variant,DK,DV", [("linear", 100, 100), ("simple", 17, 13), ("decoupled", 30, 50),
+                                           ("linear", 125, 7), ("linear", 3, 2)])
+def test_head_dims_between_row_lengths_are_widened(variant, DK, DV, dtype):
+    """Head dims that are not multiples of 8 (16-bit) / 4 (fp32) run on the matrix-core kernels through
+    zero-widened workspace copies (the decoupled operator in fp32 only up to 64): same results as the
+    original problem, checked against the float64 oracle like every other shape."""
+    from flash_bla import _hip
+    B, H, L = 2, 3, 333
+    _check_dense(variant, B, H, L, DK, DV, dtype, DK * 7 + DV)
+    # the workspace the library asks for holds the widened copies (the shape-generic path needs far less)
+    code = {torch.float16: _hip.F16, torch.bfloat16: _hip.BF16, torch.float32: _hip.F32}[dtype]
+    flags = _hip.NORMALIZE * (variant != "simple") | _hip.DECOUPLED * (variant == "decoupled")
+    unit = 4 if dtype == torch.float32 else 8
+    widened = (DK % unit or DV % unit) and not (dtype == torch.float32 and variant == "decoupled" and max(DK, DV) > 64)
+    need = _hip.lib().fbla_la_workspace_bytes(0, B, H, L, DK, DV, code, flags)
+    if widened:
+        assert need >= 3 * B * H * L * min(DK, DV) * (4 if dtype == torch.float32 else 2)
