@@ -517,9 +517,27 @@ int fbla_chunk_reduce(const void* q, const void* k, const void* v, float* qc, fl
   return check_launch(what);
 }
 
+// 16-bit inputs, 64-token blocks, head dims other than 64 / 128: the matrix-core kernel runs on copies
+// widened with zeros to 64 / 128 (zero key features leave every score as it is, zero value columns give
+// zero output columns, which are dropped again) instead of the shape-generic kernel, which is about ten
+// times slower.  q | k | v | o | kc | vc | h (widened) | the kernel's own workspace
+static int pw_wide(int d) { return d <= 64 ? 64 : 128; }
+static bool pw_widen(int K, int V, int block, int dtype) {
+  return (dtype == kF16 || dtype == kBF16) && block == 64 && K <= 128 && V <= 128 &&
+         !piecewise::attention_supported(K, V, block, dtype);
+}
+static size_t pw_widened_bytes(int64_t BH, int64_t T, int K, int V) {
+  const int Kw = pw_wide(K), Vw = pw_wide(V);
+  const int64_t NT = (T + 63) / 64;
+  return 2 * align_up((size_t)BH * T * Kw * 2, 256) + 2 * align_up((size_t)BH * T * Vw * 2, 256) +
+         align_up((size_t)BH * NT * Kw * 4, 256) + align_up((size_t)BH * NT * Vw * 4, 256) +
+         align_up((size_t)BH * Kw * Vw * 4, 256) + piecewise::attention_workspace_bytes(BH, T, Kw, Vw);
+}
+
 size_t fbla_piecewise_workspace_bytes(int64_t BH, int64_t T, int K, int V, int block, int dtype) {
   if (check_dims("fbla_piecewise_workspace_bytes", BH, 1, T, K, V, dtype, 0) != kOk) return 0;
   if (piecewise::attention_supported(K, V, block, dtype)) return piecewise::attention_workspace_bytes(BH, T, K, V);
+  if (pw_widen(K, V, block, dtype)) return pw_widened_bytes(BH, T, K, V);
   // the shape-generic kernel needs no workspace; a token size keeps "0 = not supported"
   return piecewise::attention_generic_supported(T, K, V, block, dtype) ? 256 : 0;
 }
@@ -531,7 +549,8 @@ int fbla_piecewise_fwd(const void* q, const void* k, const void* v, const float*
   const char* what = "fbla_piecewise_fwd";
   int rc = check_dims(what, BH, 1, T, K, V, dtype, 0);
   if (rc != kOk) return rc;
-  const bool fast = piecewise::attention_supported(K, V, block, dtype);
+  const bool widen = pw_widen(K, V, block, dtype);
+  const bool fast = widen || piecewise::attention_supported(K, V, block, dtype);
   if (!fast && !piecewise::attention_generic_supported(T, K, V, block, dtype)) {
     set_error("%s: needs head dims in [1,128], a positive block size and block flags that fit LDS "
               "(got K=%d V=%d block=%d dtype=%d T=%lld)", what, K, V, block, dtype, (long long)T);
@@ -553,10 +572,33 @@ int fbla_piecewise_fwd(const void* q, const void* k, const void* v, const float*
     if (rc != kOk) return rc;
     return check_launch(what);
   }
-  const size_t need = piecewise::attention_workspace_bytes(BH, T, K, V);
+  const size_t need = widen ? pw_widened_bytes(BH, T, K, V) : piecewise::attention_workspace_bytes(BH, T, K, V);
   if (workspace_bytes_ < need || !workspace) {
     set_error("%s: workspace too small (%zu < %zu bytes)", what, workspace_bytes_, need);
     return kErrWorkspace;
+  }
+  if (widen) {
+    hipStream_t st = (hipStream_t)stream;
+    const int Kw = pw_wide(K), Vw = pw_wide(V);
+    char* ws = (char*)workspace;
+    auto take = [&](size_t bytes) { void* r = ws; ws += align_up(bytes, 256); return r; };
+    void* qw = take((size_t)BH * T * Kw * 2);
+    void* kw = take((size_t)BH * T * Kw * 2);
+    void* vw = take((size_t)BH * T * Vw * 2);
+    void* ow = take((size_t)BH * T * Vw * 2);
+    float* kcw = (float*)take((size_t)BH * NT * Kw * 4);
+    float* vcw = (float*)take((size_t)BH * NT * Vw * 4);
+    float* hw = (float*)take((size_t)BH * Kw * Vw * 4);
+    generic::resize_matrices(q, BH * T, K, qw, BH * T, Kw, 1, 2, st);
+    generic::resize_matrices(k, BH * T, K, kw, BH * T, Kw, 1, 2, st);
+    generic::resize_matrices(v, BH * T, V, vw, BH * T, Vw, 1, 2, st);
+    generic::resize_matrices(kc, BH * NT, K, kcw, BH * NT, Kw, 1, 4, st);
+    generic::resize_matrices(vc, BH * NT, V, vcw, BH * NT, Vw, 1, 4, st);
+    generic::resize_matrices(h, K, V, hw, Kw, Vw, BH, 4, st);
+    rc = piecewise::attention(qw, kw, vw, kcw, vcw, hw, indices, ow, ws, BH, T, Kw, Vw, NS, scale, dtype, st);
+    if (rc != kOk) return rc;
+    generic::resize_matrices(ow, BH * T, Vw, o, BH * T, V, 1, 2, st);
+    return check_launch(what);
   }
   rc = piecewise::attention(q, k, v, kc, vc, h, indices, o, workspace, BH, T, K, V, NS, scale, dtype,
                             (hipStream_t)stream);

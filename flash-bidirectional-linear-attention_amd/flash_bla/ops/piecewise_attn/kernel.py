@@ -13,9 +13,9 @@ exact-branch sum but not that normaliser when the maximum grows between groups o
 (kernel.py:263-276), so with more blocks than one group (its autotuned GROUP_SIZE) its output depends
 on the group size; with one group both agree.  What is computed here is the group-independent value.
 
-Two kernels: fp16 / bf16 inputs with head dims in {64, 128} and 64-token blocks run on the
-MFMA kernel; every other head dim up to 128, every other block size and fp32 inputs run on a
-shape-generic fp32 kernel (correct, about an order of magnitude slower).
+Two kernels: fp16 / bf16 inputs with 64-token blocks run on the MFMA kernel (head dims other than 64 / 128
+through copies widened with zeros inside the library); other block sizes and fp32 inputs run on a
+shape-generic fp32 kernel (correct, one to two orders of magnitude slower).
 """
 import torch
 

@@ -61,10 +61,13 @@ def _oracle(q, k, v, indices, scale=None, block=64):
     (256, 64, 64, 64, 0.25, torch.float32),     # the MFMA shape in fp32
     (70, 8, 4, 1, 0.05, torch.float32),         # one-token blocks
     (260, 32, 16, 64, 0.25, torch.bfloat16),    # 16-bit head dims that the state kernel pads
+    (700, 96, 80, 64, 0.25, torch.bfloat16),    # 16-bit, 64-token blocks: widened to 128 x 128 for the MFMA kernel
+    (130, 8, 120, 64, 0.4, torch.float16),      # widened to 64 x 128
 ])
 def test_shape_generic_kernel_matches_oracle_and_per_token_evaluation(T, K, V, block, density, dtype):
     """Head dims, block sizes and the dtype outside the MFMA kernel's domain run on the
-    shape-generic kernel: against the float64 closed form and, independently, against the
+    shape-generic kernel (16-bit inputs with 64-token blocks: on the MFMA kernel through copies widened
+    with zeros to 64 / 128): against the float64 closed form and, independently, against the
     per-token C evaluation that follows the reference kernel's phases."""
     from flash_bla.ops.piecewise_attn.kernel import (chunk_reduce_fp32, piecewise_sparse_attention,
                                                      select_blocks)
