@@ -34,7 +34,10 @@ import torch.nn.functional as F  # noqa: E402
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16 matrix peak
 
-CLOCK_RAMP_S = 0.1  # untimed work before the warm-up steps
+# Untimed work before the warm-up steps.  The GPU reaches its steady clocks after 0.15-0.2 s of continuous work: a
+# timed region of 20 steps reads 0.522 ms per step after 0.1 s of work and 0.503 ms after 0.2 s or more, the value every
+# later region of the same process reads.
+CLOCK_RAMP_S = 0.25
 
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "linear_attn_fwd_bwd_B8H16T16384D64_fp16_hbm_traffic.md")
 TRAFFIC_ROW = {"fwd_state": "state_kernel", "fwd_output": "rows_kernel NORM", "bwd_pass_a": "bwd_a_kernel",
