@@ -2388,14 +2388,29 @@ static int whole_state_chunk(const Prob& p) {
   return chunk_for(p, 2, 1, 256, 64, true);
 }
 
+// Dense heads short enough for one workgroup each: the state kernel stores the finished sums itself (no
+// partials, no reduce launch) when that leaves at least a quarter of the CUs with a workgroup.
+// B8-H16-D64 fp16 forward: T=512 21.8 -> 20.3 us, T=1024 28.2 -> 25.9 us, T=2048 41.1 -> 40.7 us; backward
+// pass A loses with it (step as a HIP graph at T=1024 71.1 -> 72.0 us, at T=2048 107 -> 115 us) and keeps its chunks.
+static int whole_sequence_chunk(const Prob& p, int align) {
+  static const int max_len = knob("FBLA_DIRECT_MAX_L", 1024);
+  if (p.cu || p.L > max_len || (int64_t)p.N * p.H * 4 < cu_count()) return 0;
+  return (int)(cdiv64(p.L, align) * align);
+}
+
 int state_chunk(const Prob& p, bool block_stats) {
   static const int per_cu = knob("FBLA_STATE_WGS_PER_CU", 2);
+  if (!block_stats) {
+    const int direct = whole_sequence_chunk(p, 64);
+    if (direct) return direct;
+  }
   const int whole = block_stats && padded(p) ? 0 : whole_state_chunk(p);
   return whole ? whole : chunk_for(p, per_cu, 1, 256, 64, true);
 }
 
 int bwd_a_chunk(const Prob& p) {
   static const int per_cu = knob("FBLA_BWDA_WGS_PER_CU", 2);
+
   // 128 x 128: two workgroups of four waves per CU, steps of 64 tokens
   if (tiled_dim(p.DK) == 128 || tiled_dim(p.DV) == 128) return chunk_for(p, 2, 1, 512, 64, true);
   return chunk_for(p, per_cu, 1, 256, 128, true);
