@@ -517,13 +517,13 @@ int fbla_chunk_reduce(const void* q, const void* k, const void* v, float* qc, fl
   return check_launch(what);
 }
 
-// 16-bit inputs, 64-token blocks, head dims other than 64 / 128: the matrix-core kernel runs on copies
+// 16-bit inputs, blocks of a multiple of 64 tokens, head dims other than 64 / 128: the matrix-core kernel runs on copies
 // widened with zeros to 64 / 128 (zero key features leave every score as it is, zero value columns give
 // zero output columns, which are dropped again) instead of the shape-generic kernel, which is about ten
 // times slower.  q | k | v | o | kc | vc | h (widened) | the kernel's own workspace
 static int pw_wide(int d) { return d <= 64 ? 64 : 128; }
 static bool pw_widen(int K, int V, int block, int dtype) {
-  return (dtype == kF16 || dtype == kBF16) && block == 64 && K <= 128 && V <= 128 &&
+  return (dtype == kF16 || dtype == kBF16) && block >= 64 && block % 64 == 0 && K <= 128 && V <= 128 &&
          !piecewise::attention_supported(K, V, block, dtype);
 }
 static size_t pw_widened_bytes(int64_t BH, int64_t T, int K, int V) {
@@ -595,12 +595,12 @@ int fbla_piecewise_fwd(const void* q, const void* k, const void* v, const float*
     generic::resize_matrices(kc, BH * NT, K, kcw, BH * NT, Kw, 1, 4, st);
     generic::resize_matrices(vc, BH * NT, V, vcw, BH * NT, Vw, 1, 4, st);
     generic::resize_matrices(h, K, V, hw, Kw, Vw, BH, 4, st);
-    rc = piecewise::attention(qw, kw, vw, kcw, vcw, hw, indices, ow, ws, BH, T, Kw, Vw, NS, scale, dtype, st);
+    rc = piecewise::attention(qw, kw, vw, kcw, vcw, hw, indices, ow, ws, BH, T, Kw, Vw, block, NS, scale, dtype, st);
     if (rc != kOk) return rc;
     generic::resize_matrices(ow, BH * T, Vw, o, BH * T, V, 1, 2, st);
     return check_launch(what);
   }
-  rc = piecewise::attention(q, k, v, kc, vc, h, indices, o, workspace, BH, T, K, V, NS, scale, dtype,
+  rc = piecewise::attention(q, k, v, kc, vc, h, indices, o, workspace, BH, T, K, V, block, NS, scale, dtype,
                             (hipStream_t)stream);
   if (rc != kOk) return rc;
   return check_launch(what);

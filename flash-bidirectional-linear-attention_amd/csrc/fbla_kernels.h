@@ -220,7 +220,7 @@ bool attention_supported(int K, int V, int block, int dtype);
 size_t attention_workspace_bytes(int64_t BH, int64_t T, int K, int V);
 int attention(const void* q, const void* k, const void* v, const float* kc, const float* vc,
               const float* h, const int32_t* indices, void* o, void* workspace, int64_t BH, int64_t T,
-              int K, int V, int NS, float scale, int dtype, hipStream_t st);
+              int K, int V, int block, int NS, float scale, int dtype, hipStream_t st);
 // the same operator for every head dim up to 128, every block size and fp32 inputs (fp32 FMAs,
 // no workspace): what `attention` does not cover
 bool attention_generic_supported(int64_t T, int K, int V, int block, int dtype);

@@ -300,7 +300,8 @@ struct Attn32Args {
   const void* r;                 // [BH, T, V] q H per token
   const int32_t* indices;        // [BH, NT, NS]
   void* o;                       // [BH, T, V]
-  int T, NT, NTp, NS;
+  int T, NT, NTp, NS;            // NT blocks of `block` tokens (NTp: padded to a multiple of 64)
+  int block, NTq;                // block: a multiple of 64; NTq query tiles of 64 tokens
   float scale;
 };
 
@@ -334,8 +335,8 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   __shared__ __attribute__((aligned(1024))) unsigned char ring2[LY::kSlot];
   extern __shared__ __attribute__((aligned(16))) unsigned char sel[];
 
-  const int tq = blockIdx.x % a.NT;
-  const int64_t bh = blockIdx.x / a.NT;
+  const int tq = blockIdx.x % a.NTq;
+  const int64_t bh = blockIdx.x / a.NTq;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int qh = wave & 1, kh = wave >> 1;
@@ -361,16 +362,21 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
 
   for (int i = tid; i < a.NTp; i += kThreads) sel[i] = 0;
   __syncthreads();
-  const int32_t* idx = a.indices + (bh * a.NT + tq) * a.NS;
-  // first key row and row count of every selected block (0 rows: an index out of range), kept in
+  // A block of `block` tokens is `tpb` tiles of 64 keys; the 64 queries of this workgroup lie in
+  // query block tq / tpb and share its selection.
+  const int tpb = a.block >> 6, NE = a.NS * tpb;
+  const int32_t* idx = a.indices + (bh * a.NT + tq / tpb) * a.NS;
+  // first key row and row count of every tile of the selected blocks (0 rows: an index out of
+  // range, or a tile past the end of the last block), kept in
   // LDS: the stages below read them with LDS loads, which the tile loads' counter does not see
-  // (the list is padded with empty blocks to a multiple of three, and one more group of three)
+  // (the list is padded with empty tiles to a multiple of three, and one more group of three)
   int2* blk = reinterpret_cast<int2*>(sel + ((a.NTp + 15) & ~15));
-  for (int i = tid; i < (a.NS + 2) / 3 * 3 + 3; i += kThreads) {
-    const int b = i < a.NS ? idx[i] : -1;
+  for (int i = tid; i < (NE + 2) / 3 * 3 + 3; i += kThreads) {
+    const int b = i < NE ? idx[i / tpb] : -1;
     const bool ok = b >= 0 && b < a.NT;
     if (ok) sel[b] = 1;
-    blk[i] = ok ? int2{b * 64, min(64, a.T - b * 64)} : int2{0, 0};
+    const int row0 = b * a.block + 64 * (i % tpb);
+    blk[i] = ok && row0 < a.T ? int2{row0, min(64, a.T - row0)} : int2{0, 0};
   }
 
   // Q^T operand: k-step s covers features 16s + 8kg + i
@@ -556,7 +562,7 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   // Phase 1 is padded to a multiple of three blocks (six stages) and phase 2 to a multiple of
   // three groups (twelve stages), so that the ring slot of every stage is a compile-time
   // constant in loops unrolled by that much; padding stages request and compute nothing.
-  const int NS3 = (a.NS + 2) / 3 * 3, S1 = 2 * NS3;
+  const int NS3 = (NE + 2) / 3 * 3, S1 = 2 * NS3;
   const int NG = (a.NT + 63) / 64;
   // phase 2 by stream position (s >= S1): number of load instructions a wave issues for tile s
   // (0: no such tile), and the request itself
@@ -658,7 +664,8 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   }
 
   // ---- phase 2: unselected blocks through their means / sums (hi + lo 16-bit pairs) ----
-  const int last_len = a.T - (a.NT - 1) * 64;
+  const int last_len = a.T - (a.NT - 1) * a.block;
+  const float full_len = (float)a.block;
   f32x16 stw;
   auto mean_hi_stage = [&](int s, unsigned char* cur, unsigned char* slot_s2) {
     begin_stage(tile_loads(s + 1));
@@ -677,7 +684,7 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
       const unsigned char* selk = sel + c0 + kb;
       const int left = a.NT - c0;  // blocks from c0 on
       softmax(st, pw, [&](int c) { return kb < left - c && !selk[c]; },
-              [&](int c) { return kb == left - 1 - c ? (float)last_len : 64.f; }, yes, yes);
+              [&](int c) { return kb == left - 1 - c ? (float)last_len : full_len; }, yes, yes);
     }
   };
   auto sum_stage = [&](int s, unsigned char* cur, unsigned char* slot_s2) {
@@ -1048,7 +1055,7 @@ int chunk_reduce(const void* q, const void* k, const void* v, float* qc, float* 
 
 bool attention_supported(int K, int V, int block, int dtype) {
   return (dtype == kF16 || dtype == kBF16) && (K == 64 || K == 128) && (V == 64 || V == 128) &&
-         block == 64;
+         block >= 64 && block % 64 == 0;
 }
 
 static int64_t padded_chunks(int64_t T) { return cdiv64(cdiv64(T, 64), 64) * 64; }
@@ -1064,22 +1071,22 @@ template <typename T, int K, int V>
 static int launch_attention(const Attn32Args& a, int64_t BH, hipStream_t st) {
   using LY = Attn32Layout<K, V>;
   // the tile ring is static; dynamic: the selected-block bitmap and the selected blocks' rows
-  const int lds = ((a.NTp + 15) & ~15) + ((a.NS + 2) / 3 * 3 + 3) * 8;
+  const int lds = ((a.NTp + 15) & ~15) + ((a.NS * (a.block / 64) + 2) / 3 * 3 + 3) * 8;
   if (LY::kTiles + lds > 64 * 1024) {
     set_error("piecewise attention: %d key blocks need more LDS than a workgroup has", a.NT);
     return kErrUnsupported;
   }
   auto kernel = attention32_kernel<T, K, V>;
-  kernel<<<dim3((unsigned)(BH * a.NT)), dim3(kThreads), lds, st>>>(a);
+  kernel<<<dim3((unsigned)(BH * a.NTq)), dim3(kThreads), lds, st>>>(a);
   return kOk;
 }
 
 template <typename T>
 static int attention_t(const void* q, const void* k, const void* v, const float* kc, const float* vc,
                        const float* h, const int32_t* indices, void* o, void* workspace, int64_t BH,
-                       int64_t Tn, int K, int V, int NS, float scale, int dtype, hipStream_t st) {
-  const int NT = (int)cdiv64(Tn, 64);
-  const int64_t NTp = padded_chunks(Tn);
+                       int64_t Tn, int K, int V, int block, int NS, float scale, int dtype, hipStream_t st) {
+  const int NT = (int)cdiv64(Tn, block), NTq = (int)cdiv64(Tn, 64);
+  const int64_t NTp = cdiv64(NT, 64) * 64;  // at most padded_chunks(Tn), which sizes the workspace
   char* ws = (char*)workspace;
   T* kc_hi = (T*)ws;
   ws += align_up((size_t)BH * NTp * K * 2, 256);
@@ -1099,7 +1106,7 @@ static int attention_t(const void* q, const void* k, const void* v, const float*
   mfma::RowsJob job{q, nullptr, h, V, 1, nullptr, nullptr, r};
   int rc = mfma::rows(p, dtype, job, K, V, st);
   if (rc != kOk) return rc;
-  Attn32Args a{q, k, v, kc_hi, kc_lo, vc_hi, vc_lo, r, indices, o, (int)Tn, NT, (int)NTp, NS, scale};
+  Attn32Args a{q, k, v, kc_hi, kc_lo, vc_hi, vc_lo, r, indices, o, (int)Tn, NT, (int)NTp, NS, block, NTq, scale};
   if (K == 64 && V == 64) return launch_attention<T, 64, 64>(a, BH, st);
   if (K == 64) return launch_attention<T, 64, 128>(a, BH, st);
   if (V == 64) return launch_attention<T, 128, 64>(a, BH, st);
@@ -1304,10 +1311,10 @@ int attention_generic(const void* q, const void* k, const void* v, const float* 
 
 int attention(const void* q, const void* k, const void* v, const float* kc, const float* vc,
               const float* h, const int32_t* indices, void* o, void* workspace, int64_t BH, int64_t T,
-              int K, int V, int NS, float scale, int dtype, hipStream_t st) {
+              int K, int V, int block, int NS, float scale, int dtype, hipStream_t st) {
   if (dtype == kF16)
-    return attention_t<_Float16>(q, k, v, kc, vc, h, indices, o, workspace, BH, T, K, V, NS, scale, dtype, st);
-  return attention_t<__bf16>(q, k, v, kc, vc, h, indices, o, workspace, BH, T, K, V, NS, scale, dtype, st);
+    return attention_t<_Float16>(q, k, v, kc, vc, h, indices, o, workspace, BH, T, K, V, block, NS, scale, dtype, st);
+  return attention_t<__bf16>(q, k, v, kc, vc, h, indices, o, workspace, BH, T, K, V, block, NS, scale, dtype, st);
 }
 
 }  // namespace piecewise

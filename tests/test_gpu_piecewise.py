@@ -285,6 +285,44 @@ def test_selection_lengths_around_the_unrolled_stream(K, V):
         assert torch.equal(o, o_padded), f"{ns} blocks, padded list"
 
 
+@pytest.mark.parametrize("T,K,V,block,dtype", [
+    (128 * 5 + 16, 128, 128, 128, torch.bfloat16),   # the last block ends inside its first tile
+    (128 * 4 + 100, 64, 64, 128, torch.float16),     # ... inside its second tile
+    (192 * 3 + 70, 64, 128, 192, torch.bfloat16),    # three tiles per block
+    (256 * 3 + 129, 128, 64, 256, torch.float16),    # four tiles per block
+    (128 * 6 + 40, 96, 72, 128, torch.bfloat16),     # widened head dims
+])
+def test_blocks_of_several_tiles(T, K, V, block, dtype):
+    """Blocks of a multiple of 64 tokens run on the MFMA kernel as several 64-key tiles per selected block,
+    the query tiles of one block sharing its selection: every list length from 1 to 5 in random block
+    order (the ragged last block first in one list, so that its empty tiles sit in the middle of the
+    stream), against the float64 closed form and the per-token evaluation; a list padded with -1 gives
+    the result of the unpadded one."""
+    from flash_bla.ops.piecewise_attn.kernel import piecewise_sparse_attention
+    from oracle.piecewise_tokens import pisa_tokens
+    NT = -(-T // block)
+    q, k, v = _inputs(1, 1, T, K, V, dtype, seed=T + block)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    rng = np.random.default_rng(block + K)
+    for ns in range(1, min(NT, 5) + 1):
+        lists = [rng.permutation(NT)[:ns] for _ in range(NT)]
+        lists[0] = np.concatenate([[NT - 1], rng.permutation(NT - 1)[:ns - 1]]).astype(lists[0].dtype)
+        indices = torch.tensor(np.stack(lists), dtype=torch.int32)[None, None].cuda()
+        o = piecewise_sparse_attention(qd, kd, vd, block_size=block, indices=indices)
+        floor = _oracle(q, k, v.abs(), indices, block=block)
+        assert_parity(o, _oracle(q, k, v, indices, block=block), dtype, f"block {block}, {ns} selected", floor)
+        if ns == 2:
+            tok = pisa_tokens(np64(q)[0, 0], np64(k)[0, 0], np64(v)[0, 0], indices[0, 0].cpu().numpy(), block,
+                              K ** -0.5)
+            assert_parity(o[0, 0], tok, dtype, f"per-token evaluation, block {block}", floor[0, 0])
+            padded = torch.full((1, 1, NT, min(ns + 2, NT)), -1, dtype=torch.int32)
+            padded[..., 0] = indices[..., 0].cpu()
+            padded[..., 2] = indices[..., 1].cpu()
+            assert torch.equal(o, piecewise_sparse_attention(qd, kd, vd, block_size=block, indices=padded.cuda()))
+    o_auto = piecewise_sparse_attention(qd, kd, vd, density=0.4, block_size=block)
+    assert torch.isfinite(o_auto.float()).all()
+
+
 @pytest.mark.parametrize("seed", range(3))
 def test_random_piecewise_cases(seed):
     """Seeded random lengths (ragged last blocks, one block, many blocks), head dims, densities
