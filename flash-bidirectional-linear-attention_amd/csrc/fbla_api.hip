@@ -523,21 +523,22 @@ int fbla_chunk_reduce(const void* q, const void* k, const void* v, float* qc, fl
 // times slower.  q | k | v | o | kc | vc | h (widened) | the kernel's own workspace
 static int pw_wide(int d) { return d <= 64 ? 64 : 128; }
 static bool pw_widen(int K, int V, int block, int dtype) {
-  return (dtype == kF16 || dtype == kBF16) && block >= 64 && block % 64 == 0 && K <= 128 && V <= 128 &&
+  return (dtype == kF16 || dtype == kBF16) && piecewise::attention_supported(64, 64, block, dtype) && K <= 128 &&
+         V <= 128 &&
          !piecewise::attention_supported(K, V, block, dtype);
 }
-static size_t pw_widened_bytes(int64_t BH, int64_t T, int K, int V) {
+static size_t pw_widened_bytes(int64_t BH, int64_t T, int K, int V, int block) {
   const int Kw = pw_wide(K), Vw = pw_wide(V);
-  const int64_t NT = (T + 63) / 64;
+  const int64_t NT = (T + block - 1) / block;
   return 2 * align_up((size_t)BH * T * Kw * 2, 256) + 2 * align_up((size_t)BH * T * Vw * 2, 256) +
          align_up((size_t)BH * NT * Kw * 4, 256) + align_up((size_t)BH * NT * Vw * 4, 256) +
-         align_up((size_t)BH * Kw * Vw * 4, 256) + piecewise::attention_workspace_bytes(BH, T, Kw, Vw);
+         align_up((size_t)BH * Kw * Vw * 4, 256) + piecewise::attention_workspace_bytes(BH, T, Kw, Vw, block);
 }
 
 size_t fbla_piecewise_workspace_bytes(int64_t BH, int64_t T, int K, int V, int block, int dtype) {
   if (check_dims("fbla_piecewise_workspace_bytes", BH, 1, T, K, V, dtype, 0) != kOk) return 0;
-  if (piecewise::attention_supported(K, V, block, dtype)) return piecewise::attention_workspace_bytes(BH, T, K, V);
-  if (pw_widen(K, V, block, dtype)) return pw_widened_bytes(BH, T, K, V);
+  if (piecewise::attention_supported(K, V, block, dtype)) return piecewise::attention_workspace_bytes(BH, T, K, V, block);
+  if (pw_widen(K, V, block, dtype)) return pw_widened_bytes(BH, T, K, V, block);
   // the shape-generic kernel needs no workspace; a token size keeps "0 = not supported"
   return piecewise::attention_generic_supported(T, K, V, block, dtype) ? 256 : 0;
 }
@@ -572,7 +573,7 @@ int fbla_piecewise_fwd(const void* q, const void* k, const void* v, const float*
     if (rc != kOk) return rc;
     return check_launch(what);
   }
-  const size_t need = widen ? pw_widened_bytes(BH, T, K, V) : piecewise::attention_workspace_bytes(BH, T, K, V);
+  const size_t need = widen ? pw_widened_bytes(BH, T, K, V, block) : piecewise::attention_workspace_bytes(BH, T, K, V, block);
   if (workspace_bytes_ < need || !workspace) {
     set_error("%s: workspace too small (%zu < %zu bytes)", what, workspace_bytes_, need);
     return kErrWorkspace;

@@ -217,7 +217,7 @@ bool select_blocks_supported(int NT, int K);
 int select_blocks(const float* qc, const float* kc, const float* bias, int32_t* indices, int64_t BH,
                   int NT, int K, int NS, float scale, hipStream_t st);
 bool attention_supported(int K, int V, int block, int dtype);
-size_t attention_workspace_bytes(int64_t BH, int64_t T, int K, int V);
+size_t attention_workspace_bytes(int64_t BH, int64_t T, int K, int V, int block);
 int attention(const void* q, const void* k, const void* v, const float* kc, const float* vc,
               const float* h, const int32_t* indices, void* o, void* workspace, int64_t BH, int64_t T,
               int K, int V, int block, int NS, float scale, int dtype, hipStream_t st);

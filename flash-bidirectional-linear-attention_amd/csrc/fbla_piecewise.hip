@@ -319,7 +319,16 @@ typedef uint32_t u32x2p __attribute__((ext_vector_type(2)));
 // (hi, lo).  Stage s works on tile s in ring slot s % 3 while tile s+1 has landed or is landing
 // and tile s+2 is requested: three tiles of 16 KiB per workgroup instead of two K + V^T pairs,
 // so that three workgroups (three waves per SIMD, at most 168 registers) share a CU.
-template <typename T, int K, int V>
+//
+// Block sizes.  A block of a multiple of 64 tokens is several key tiles in a row, and the query
+// tiles of one block share its selection.  SUB = true: blocks of 16 or 32 tokens.  The 64 queries
+// of the workgroup then belong to 64 / block query blocks with selections of their own: the tile
+// stream of phase 1 serves them one after the other, a key tile is put together from 64 / block
+// selected blocks of the query block it belongs to, and the queries of the other query blocks
+// are masked (waves without a query of that block skip the tile's arithmetic, so the exact
+// branch runs at block / 32 of its speed, at most 1); every query block has its own bitmap of
+// selected blocks for phase 2.
+template <typename T, int K, int V, bool SUB>
 __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) {
   using LY = Attn32Layout<K, V>;
   constexpr int KS = K / 16;                 // k-steps of the score product
@@ -360,23 +369,46 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   const auto vch_rs = descriptor((const T*)a.vc_hi + bh * a.NTp * V, (int64_t)a.NTp * V * 2);
   const auto vcl_rs = descriptor((const T*)a.vc_lo + bh * a.NTp * V, (int64_t)a.NTp * V * 2);
 
-  for (int i = tid; i < a.NTp; i += kThreads) sel[i] = 0;
+  // SUB: query blocks per query tile = selected blocks per key tile, tiles per query block
+  const int lg = 31 - __builtin_clz(a.block);
+  const int sub = SUB ? 64 >> lg : 1, tpj = SUB ? (a.NS + sub - 1) >> (6 - lg) : 0;
+  for (int i = tid; i < sub * a.NTp; i += kThreads) sel[i] = 0;
   __syncthreads();
   // A block of `block` tokens is `tpb` tiles of 64 keys; the 64 queries of this workgroup lie in
   // query block tq / tpb and share its selection.
-  const int tpb = a.block >> 6, NE = a.NS * tpb;
-  const int32_t* idx = a.indices + (bh * a.NT + tq / tpb) * a.NS;
+  const int tpb = SUB ? 1 : a.block >> 6, NE = SUB ? sub * tpj : a.NS * tpb;
+  const int32_t* idx = a.indices + (bh * a.NT + (SUB ? tq * sub : tq / tpb)) * a.NS;
   // first key row and row count of every tile of the selected blocks (0 rows: an index out of
   // range, or a tile past the end of the last block), kept in
   // LDS: the stages below read them with LDS loads, which the tile loads' counter does not see
   // (the list is padded with empty tiles to a multiple of three, and one more group of three)
-  int2* blk = reinterpret_cast<int2*>(sel + ((a.NTp + 15) & ~15));
-  for (int i = tid; i < (NE + 2) / 3 * 3 + 3; i += kThreads) {
-    const int b = i < NE ? idx[i / tpb] : -1;
-    const bool ok = b >= 0 && b < a.NT;
-    if (ok) sel[b] = 1;
-    const int row0 = b * a.block + 64 * (i % tpb);
-    blk[i] = ok && row0 < a.T ? int2{row0, min(64, a.T - row0)} : int2{0, 0};
+  int2* blk = reinterpret_cast<int2*>(sel + ((sub * a.NTp + 15) & ~15));
+  // SUB: first key row of each of the tile's selected blocks, -1: none (list exhausted, index out
+  // of range, or a query block past the end of the sequence)
+  int4* blk4 = reinterpret_cast<int4*>(blk);
+  if constexpr (SUB) {
+    for (int i = tid; i < (NE + 2) / 3 * 3 + 3; i += kThreads) {
+      int r0[4] = {-1, -1, -1, -1};
+      const int j = i / max(tpj, 1), t = i - j * tpj;
+      if (i < NE && tq * sub + j < a.NT)
+        for (int pc = 0; pc < sub; ++pc) {
+          const int e = t * sub + pc;
+          const int b = e < a.NS ? idx[(int64_t)j * a.NS + e] : -1;
+          if (b >= 0 && b < a.NT) {
+            r0[pc] = b << lg;
+            sel[j * a.NTp + b] = 1;
+          }
+        }
+      blk4[i] = int4{r0[0], r0[1], r0[2], r0[3]};
+    }
+  } else {
+    for (int i = tid; i < (NE + 2) / 3 * 3 + 3; i += kThreads) {
+      const int b = i < NE ? idx[i / tpb] : -1;
+      const bool ok = b >= 0 && b < a.NT;
+      if (ok) sel[b] = 1;
+      const int row0 = b * a.block + 64 * (i % tpb);
+      blk[i] = ok && row0 < a.T ? int2{row0, min(64, a.T - row0)} : int2{0, 0};
+    }
   }
 
   // Q^T operand: k-step s covers features 16s + 8kg + i
@@ -436,6 +468,29 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
 #pragma unroll
     for (int j = 0; j < VJ; ++j)
       dma16(rs, tile + (4 * VRW * j + VRW * wave) * VROWB, v_lane_off, (row0 + 4 * VRW * j) * VROWB);
+  };
+  // SUB: a tile put together from up to four selected blocks (a, b, c, d: their first key rows, -1:
+  // none).  The rows of one load instruction (4 or 8) lie in one block; the rows of a missing block
+  // are requested past the end of the tensor and arrive as zeros.
+  struct Tile { int a, b, c, d; };
+  auto source_row = [&](const Tile& t, int R) {  // of tile row R
+    const int pc = R >> lg;
+    const int r0 = pc == 0 ? t.a : pc == 1 ? t.b : pc == 2 ? t.c : t.d;
+    return r0 >= 0 ? r0 + (R & (a.block - 1)) : a.T;
+  };
+  auto dma_pieces_k = [&](unsigned char* tile, const Tile& t) {
+#pragma unroll
+    for (int j = 0; j < KJ; ++j) {
+      const int R = 4 * KRW * j + KRW * wave;
+      dma16(k_rs, tile + R * KROWB, k_lane_off - KRW * wave * KROWB, source_row(t, R) * KROWB);
+    }
+  };
+  auto dma_pieces_v = [&](unsigned char* tile, const Tile& t) {
+#pragma unroll
+    for (int j = 0; j < VJ; ++j) {
+      const int R = 4 * VRW * j + VRW * wave;
+      dma16(v_rs, tile + R * VROWB, v_lane_off - VRW * wave * VROWB, source_row(t, R) * VROWB);
+    }
   };
 
   // per-lane LDS offsets of the operand reads
@@ -599,21 +654,64 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   for (int r = 0; r < 16; ++r) zero16[r] = 0.f;
   const auto none = [](int) { return 0.f; };
 
-  // ---- phase 1: selected blocks, three per iteration (first key row x, row count y of each;
-  // y = 0: no such block, nothing is requested or computed) ----
+  // ---- phase 1: the tiles of the selected blocks, three per iteration (not SUB: first key row a,
+  // row count b of each; an empty tile - no such block - requests and computes nothing) ----
   auto block_info = [&](int i) {
-    const int2 v = blk[i];
-    return int2{__builtin_amdgcn_readfirstlane(v.x), __builtin_amdgcn_readfirstlane(v.y)};
+    if constexpr (SUB) {
+      const int4 v = blk4[i];
+      return Tile{__builtin_amdgcn_readfirstlane(v.x), __builtin_amdgcn_readfirstlane(v.y),
+                  __builtin_amdgcn_readfirstlane(v.z), __builtin_amdgcn_readfirstlane(v.w)};
+    } else {
+      const int2 v = blk[i];
+      return Tile{__builtin_amdgcn_readfirstlane(v.x), __builtin_amdgcn_readfirstlane(v.y), 0, 0};
+    }
   };
-  auto key_compute = [&](const unsigned char* cur, int nrows) {
-    if (nrows == 64) {
+  auto has = [&](const Tile& t) {
+    if constexpr (SUB) return (t.a & t.b & t.c & t.d) >= 0;
+    else return t.b != 0;
+  };
+  auto request_k = [&](unsigned char* slot, const Tile& t) {
+    if constexpr (SUB) dma_pieces_k(slot, t);
+    else dma_tile_k(k_rs, slot, t.a);
+  };
+  auto request_v = [&](unsigned char* slot, const Tile& t) {
+    if constexpr (SUB) dma_pieces_v(slot, t);
+    else dma_tile_v(v_rs, slot, t.a);
+  };
+  // SUB: does tile i belong to a query block with queries in this wave?  (tiles come grouped by
+  // query block, tpj each)
+  auto owner = [&](int i) { return (i >= tpj) + (i >= 2 * tpj) + (i >= 3 * tpj); };
+  auto mine = [&](const Tile& t, int i) {
+    if constexpr (SUB) return has(t) && ((owner(i) << lg) >> 5) == qh;
+    else return has(t);
+  };
+  auto key_compute = [&](const unsigned char* cur, const Tile& t, int i) {
+    if constexpr (SUB) {
+      if (!mine(t, i)) return;
       const f32x16 st = scores(cur, zero16);
-      softmax(st, pw, [](int) { return true; }, none, no, no);
-    } else if (nrows > 0) {
-      const f32x16 st = scores(cur, zero16);
-      int kb = kbase;
-      asm volatile("" : "+v"(kb));  // (keeps the sixteen sums kb + c out of registers across the loop)
-      softmax(st, pw, [&](int c) { return kb < nrows - c; }, none, yes, no);
+      // this wave's 32 keys are two groups of 16 with nA / nB valid rows: two blocks of 16, or the
+      // halves of a block of 32; a lane counts them only if its query lies in the tile's query block
+      const int pa = (32 * kh) >> lg;
+      const int ra = pa == 0 ? t.a : pa == 1 ? t.b : pa == 2 ? t.c : t.d;
+      const int rb = pa == 0 ? t.b : pa == 2 ? t.d : -1;  // (blocks of 16: the wave's second block)
+      const int na = ra >= 0 ? min(a.block, a.T - ra) : 0;
+      const int nb = a.block == 32 ? na - 16 : (rb >= 0 ? min(16, a.T - rb) : 0);
+      const bool own = ((32 * qh + n) >> lg) == owner(i);
+      const int nal = own ? na : 0, nbl = own ? nb : 0;
+      int kg4 = 4 * kg;
+      asm volatile("" : "+v"(kg4));
+      softmax(st, pw, [&](int c) { return c < 16 ? kg4 < nal - c : kg4 < nbl - (c - 16); }, none, yes, no);
+    } else {
+      const int nrows = t.b;
+      if (nrows == 64) {
+        const f32x16 st = scores(cur, zero16);
+        softmax(st, pw, [](int) { return true; }, none, no, no);
+      } else if (nrows > 0) {
+        const f32x16 st = scores(cur, zero16);
+        int kb = kbase;
+        asm volatile("" : "+v"(kb));  // (keeps the sixteen sums kb + c out of registers across the loop)
+        softmax(st, pw, [&](int c) { return kb < nrows - c; }, none, yes, no);
+      }
     }
   };
   // the query operand has arrived before the first tile is requested: a later wait for it would
@@ -622,10 +720,10 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   for (int s = 0; s < KS; ++s) asm volatile("" ::"v"(qop[s]));
   __syncthreads();  // the selected blocks' rows are in LDS
   if (NS3 > 0) {
-    const int2 b0 = block_info(0);
-    if (b0.y) {
-      dma_tile_k(k_rs, ring0, b0.x);
-      dma_tile_v(v_rs, ring1, b0.x);
+    const Tile b0 = block_info(0);
+    if (has(b0)) {
+      request_k(ring0, b0);
+      request_v(ring1, b0);
     }
   } else {
     fetch(S1, ring0);
@@ -633,34 +731,34 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
   }
   for (int i0 = 0; i0 < NS3; i0 += 3) {
     const bool last = i0 + 3 == NS3;  // the tiles after this iteration's are phase 2's first two
-    const int2 b0 = block_info(i0), b1 = block_info(i0 + 1), b2 = block_info(i0 + 2), b3 = block_info(i0 + 3);
-    const int k3 = last ? tile_loads(S1) : (b3.y ? KJ : 0);
+    const Tile b0 = block_info(i0), b1 = block_info(i0 + 1), b2 = block_info(i0 + 2), b3 = block_info(i0 + 3);
+    const int k3 = last ? tile_loads(S1) : (has(b3) ? KJ : 0);
     // K of b0 in slot 0
-    begin_stage(b0.y ? VJ : 0);
-    if (b1.y) dma_tile_k(k_rs, ring2, b1.x);
-    key_compute(ring0, b0.y);
+    begin_stage(has(b0) ? VJ : 0);
+    if (has(b1)) request_k(ring2, b1);
+    key_compute(ring0, b0, i0);
     // V of b0 in slot 1
-    begin_stage(b1.y ? KJ : 0);
-    if (b1.y) dma_tile_v(v_rs, ring0, b1.x);
-    if (b0.y) values(ring1, pw);
+    begin_stage(has(b1) ? KJ : 0);
+    if (has(b1)) request_v(ring0, b1);
+    if (mine(b0, i0)) values(ring1, pw);
     // K of b1 in slot 2
-    begin_stage(b1.y ? VJ : 0);
-    if (b2.y) dma_tile_k(k_rs, ring1, b2.x);
-    key_compute(ring2, b1.y);
+    begin_stage(has(b1) ? VJ : 0);
+    if (has(b2)) request_k(ring1, b2);
+    key_compute(ring2, b1, i0 + 1);
     // V of b1 in slot 0
-    begin_stage(b2.y ? KJ : 0);
-    if (b2.y) dma_tile_v(v_rs, ring2, b2.x);
-    if (b1.y) values(ring0, pw);
+    begin_stage(has(b2) ? KJ : 0);
+    if (has(b2)) request_v(ring2, b2);
+    if (mine(b1, i0 + 1)) values(ring0, pw);
     // K of b2 in slot 1
-    begin_stage(b2.y ? VJ : 0);
+    begin_stage(has(b2) ? VJ : 0);
     if (last) fetch(S1, ring0);
-    else if (b3.y) dma_tile_k(k_rs, ring0, b3.x);
-    key_compute(ring1, b2.y);
+    else if (has(b3)) request_k(ring0, b3);
+    key_compute(ring1, b2, i0 + 2);
     // V of b2 in slot 2
     begin_stage(k3);
     if (last) fetch(S1 + 1, ring1);
-    else if (b3.y) dma_tile_v(v_rs, ring1, b3.x);
-    if (b2.y) values(ring2, pw);
+    else if (has(b3)) request_v(ring1, b3);
+    if (mine(b2, i0 + 2)) values(ring2, pw);
   }
 
   // ---- phase 2: unselected blocks through their means / sums (hi + lo 16-bit pairs) ----
@@ -681,7 +779,8 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
       const f32x16 st = scores(cur, stw);
       int kb = kbase;
       asm volatile("" : "+v"(kb));
-      const unsigned char* selk = sel + c0 + kb;
+      // (SUB: the bitmap of this lane's query block)
+      const unsigned char* selk = sel + (SUB ? ((32 * qh + n) >> lg) * a.NTp : 0) + c0 + kb;
       const int left = a.NT - c0;  // blocks from c0 on
       softmax(st, pw, [&](int c) { return kb < left - c && !selk[c]; },
               [&](int c) { return kb == left - 1 - c ? (float)last_len : full_len; }, yes, yes);
@@ -1055,30 +1154,46 @@ int chunk_reduce(const void* q, const void* k, const void* v, float* qc, float* 
 
 bool attention_supported(int K, int V, int block, int dtype) {
   return (dtype == kF16 || dtype == kBF16) && (K == 64 || K == 128) && (V == 64 || V == 128) &&
-         block >= 64 && block % 64 == 0;
+         (block == 16 || block == 32 || (block >= 64 && block % 64 == 0));
 }
 
-static int64_t padded_chunks(int64_t T) { return cdiv64(cdiv64(T, 64), 64) * 64; }
+static int64_t padded_chunks(int64_t T, int block) { return cdiv64(cdiv64(T, block), 64) * 64; }
 
 // kc_hi | kc_lo | vc_hi | vc_lo | r
-size_t attention_workspace_bytes(int64_t BH, int64_t T, int K, int V) {
-  const int64_t NTp = padded_chunks(T);
+size_t attention_workspace_bytes(int64_t BH, int64_t T, int K, int V, int block) {
+  const int64_t NTp = padded_chunks(T, block);
   return 2 * align_up((size_t)BH * NTp * K * 2, 256) + 2 * align_up((size_t)BH * NTp * V * 2, 256) +
          align_up((size_t)BH * T * V * 2, 256);
 }
 
-template <typename T, int K, int V>
-static int launch_attention(const Attn32Args& a, int64_t BH, hipStream_t st) {
+template <typename T, int K, int V, bool SUB>
+static int launch_attention_variant(const Attn32Args& a, int64_t BH, hipStream_t st) {
   using LY = Attn32Layout<K, V>;
-  // the tile ring is static; dynamic: the selected-block bitmap and the selected blocks' rows
-  const int lds = ((a.NTp + 15) & ~15) + ((a.NS * (a.block / 64) + 2) / 3 * 3 + 3) * 8;
+  // the tile ring is static; dynamic: the selected-block bitmaps and the tile list of phase 1
+  const int sub = SUB ? 64 / a.block : 1;
+  const int tiles = SUB ? sub * ((a.NS + sub - 1) / sub) : a.NS * (a.block / 64);
+  const int lds = ((sub * a.NTp + 15) & ~15) + ((tiles + 2) / 3 * 3 + 3) * (SUB ? 16 : 8);
+  auto kernel = attention32_kernel<T, K, V, SUB>;
   if (LY::kTiles + lds > 64 * 1024) {
-    set_error("piecewise attention: %d key blocks need more LDS than a workgroup has", a.NT);
-    return kErrUnsupported;
+    if (LY::kTiles + lds > 160 * 1024) {
+      set_error("piecewise attention: %d key blocks need more LDS than a workgroup has", a.NT);
+      return kErrUnsupported;
+    }
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) {
+      set_error("piecewise attention: cannot reserve %d bytes of LDS: %s", lds, hipGetErrorString(e));
+      return kErrLaunch;
+    }
   }
-  auto kernel = attention32_kernel<T, K, V>;
   kernel<<<dim3((unsigned)(BH * a.NTq)), dim3(kThreads), lds, st>>>(a);
   return kOk;
+}
+
+template <typename T, int K, int V>
+static int launch_attention(const Attn32Args& a, int64_t BH, hipStream_t st) {
+  return a.block < 64 ? launch_attention_variant<T, K, V, true>(a, BH, st)
+                      : launch_attention_variant<T, K, V, false>(a, BH, st);
 }
 
 template <typename T>
@@ -1086,7 +1201,7 @@ static int attention_t(const void* q, const void* k, const void* v, const float*
                        const float* h, const int32_t* indices, void* o, void* workspace, int64_t BH,
                        int64_t Tn, int K, int V, int block, int NS, float scale, int dtype, hipStream_t st) {
   const int NT = (int)cdiv64(Tn, block), NTq = (int)cdiv64(Tn, 64);
-  const int64_t NTp = cdiv64(NT, 64) * 64;  // at most padded_chunks(Tn), which sizes the workspace
+  const int64_t NTp = padded_chunks(Tn, block);
   char* ws = (char*)workspace;
   T* kc_hi = (T*)ws;
   ws += align_up((size_t)BH * NTp * K * 2, 256);
@@ -1117,7 +1232,7 @@ static int attention_t(const void* q, const void* k, const void* v, const float*
 // shape-generic attention kernel
 // ===========================================================================
 // Every head dim up to 128, every block size, fp16 / bf16 / fp32 inputs: what the MFMA kernel
-// (16-bit, head dims 64 / 128, 64-token blocks) does not cover.  Plain fp32 FMAs, correct
+// (16-bit, head dims 64 / 128, blocks of 16, 32 or a multiple of 64 tokens) does not cover.  Plain fp32 FMAs, correct
 // everywhere and an order of magnitude slower.  One workgroup per (query block, head); the
 // block's queries are handled 64 at a time: four neighbouring lanes share a query, each
 // holding a quarter of the contraction index for the scores (summed with two lane exchanges)

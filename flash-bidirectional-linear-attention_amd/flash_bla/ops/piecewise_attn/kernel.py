@@ -13,9 +13,10 @@ exact-branch sum but not that normaliser when the maximum grows between groups o
 (kernel.py:263-276), so with more blocks than one group (its autotuned GROUP_SIZE) its output depends
 on the group size; with one group both agree.  What is computed here is the group-independent value.
 
-Two kernels: fp16 / bf16 inputs with 64-token blocks run on the MFMA kernel (head dims other than 64 / 128
-through copies widened with zeros inside the library); other block sizes and fp32 inputs run on a
-shape-generic fp32 kernel (correct, one to two orders of magnitude slower).
+Two kernels: fp16 / bf16 inputs with blocks of 16, 32 or a multiple of 64 tokens run on the MFMA kernel
+(head dims other than 64 / 128 through copies widened with zeros inside the library; blocks below 64 at
+block / 64 of the exact branch's speed); other block sizes and fp32 inputs run on a shape-generic fp32
+kernel (correct, one to two orders of magnitude slower).
 """
 import torch
 
@@ -76,8 +77,8 @@ def piecewise_sparse_attention(q, k, v, density=0.1, block_size=64, scale=None, 
     Args:
         q, k: `(B, H, T, K)`; v: `(B, H, T, V)`; fp16, bf16 or fp32, K and V up to 128.
         density: fraction of key blocks attended exactly per query block (at least one).
-        block_size: tokens per block (the MFMA kernel is built for 64; other sizes take the
-            shape-generic kernel).
+        block_size: tokens per block (the MFMA kernel takes 16, 32 and multiples of 64; other
+            sizes take the shape-generic kernel).
         scale: score scale, default `K ** -0.5`.
         use_bias: rank blocks by softmax(score + log(norm of the block's first-order matrix)).
         indices: optional precomputed selection `(B, H, N, top_k)` (not in the reference;

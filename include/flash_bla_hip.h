@@ -239,10 +239,11 @@ size_t fbla_piecewise_workspace_bytes(int64_t BH, int64_t T, int K, int V, int b
  * query block of `block` tokens (indices: int32 [BH, NT, NS], NT = ceil(T / block)), the
  * remaining blocks through their mean key / value sum (zeroth order) and h (first order).
  * kc, vc, h are the fp32 outputs of fbla_chunk_reduce with chunk = block.  fp16 / bf16 with
- * K, V in {64,128} and block = 64 run on the MFMA kernel; every other K, V in [1,128], every
- * other block size and fp32 inputs run on a shape-generic fp32 kernel (same results to
- * rounding, about an order of magnitude slower, no workspace used).  The reference takes the
- * same domain through BK = min(128, next_pow2(K)) (kernel.py:296-308). */
+ * block = 16, 32 or a multiple of 64 run on the MFMA kernel (K, V other than 64 / 128 through
+ * zero-widened copies in the workspace); other block sizes and fp32 inputs run on a shape-generic
+ * fp32 kernel (same results to rounding, one to two orders of magnitude slower, no workspace
+ * used).  The reference takes the same domain through BK = min(128, next_pow2(K))
+ * (kernel.py:296-308). */
 int fbla_piecewise_fwd(const void* q, const void* k, const void* v, const float* kc, const float* vc,
                        const float* h, const int32_t* indices, void* o, void* workspace,
                        size_t workspace_bytes, int64_t BH, int64_t T, int K, int V, int block, int NS,

@@ -55,8 +55,9 @@ def _oracle(q, k, v, indices, scale=None, block=64):
 @pytest.mark.parametrize("T,K,V,block,density,dtype", [
     (200, 16, 8, 32, 0.3, torch.float32),       # small head dims, ragged last block, fp32
     (300, 100, 72, 64, 0.25, torch.float16),    # head dims that are not multiples of 16
-    (257, 64, 64, 16, 0.2, torch.bfloat16),     # the MFMA head dims with another block size
-    (400, 128, 128, 128, 0.5, torch.float16),   # 128-token blocks
+    (257, 64, 64, 16, 0.2, torch.bfloat16),     # 16-token blocks (MFMA kernel, four query blocks per query tile)
+    (400, 128, 128, 128, 0.5, torch.float16),   # 128-token blocks (MFMA kernel, two key tiles per block)
+    (300, 64, 64, 48, 0.3, torch.float16),      # a block size the MFMA kernel does not take
     (333, 24, 40, 50, 0.1, torch.float32),      # nothing a power of two
     (256, 64, 64, 64, 0.25, torch.float32),     # the MFMA shape in fp32
     (70, 8, 4, 1, 0.05, torch.float32),         # one-token blocks
@@ -66,8 +67,8 @@ def _oracle(q, k, v, indices, scale=None, block=64):
 ])
 def test_shape_generic_kernel_matches_oracle_and_per_token_evaluation(T, K, V, block, density, dtype):
     """Head dims, block sizes and the dtype outside the MFMA kernel's domain run on the
-    shape-generic kernel (16-bit inputs with 64-token blocks: on the MFMA kernel through copies widened
-    with zeros to 64 / 128): against the float64 closed form and, independently, against the
+    shape-generic kernel (16-bit inputs with blocks of 16, 32 or a multiple of 64 tokens: on the MFMA kernel,
+    head dims other than 64 / 128 through copies widened with zeros): against the float64 closed form and, independently, against the
     per-token C evaluation that follows the reference kernel's phases."""
     from flash_bla.ops.piecewise_attn.kernel import (chunk_reduce_fp32, piecewise_sparse_attention,
                                                      select_blocks)
@@ -320,6 +321,51 @@ def test_blocks_of_several_tiles(T, K, V, block, dtype):
             padded[..., 2] = indices[..., 1].cpu()
             assert torch.equal(o, piecewise_sparse_attention(qd, kd, vd, block_size=block, indices=padded.cuda()))
     o_auto = piecewise_sparse_attention(qd, kd, vd, density=0.4, block_size=block)
+    assert torch.isfinite(o_auto.float()).all()
+
+
+@pytest.mark.parametrize("T,K,V,block,dtype", [
+    (64 * 5 + 40, 128, 128, 32, torch.bfloat16),   # ragged last block (8 of 32 rows), last query tile with one block
+    (64 * 4 + 50, 64, 64, 16, torch.float16),      # ragged last block (2 of 16 rows)
+    (64 * 3, 64, 128, 32, torch.float16),          # whole tiles
+    (64 * 6 + 17, 128, 64, 16, torch.bfloat16),
+    (64 * 4 + 33, 96, 72, 32, torch.bfloat16),     # widened head dims
+    (20, 64, 64, 16, torch.float16),               # less than one tile
+])
+def test_blocks_smaller_than_a_tile(T, K, V, block, dtype):
+    """Blocks of 16 / 32 tokens run on the MFMA kernel too: a key tile is put together from 64 / block
+    selected blocks of one query block, the queries of the tile's other query blocks are masked.  Every list
+    length from 1 to 7 in random block order (odd lengths leave a tile partly empty; the ragged last block
+    is first in one list), against the float64 closed form and the per-token evaluation; a list padded
+    with -1 in the middle is checked against the oracle of the unpadded one."""
+    from flash_bla.ops.piecewise_attn.kernel import piecewise_sparse_attention
+    from oracle.piecewise_tokens import pisa_tokens
+    NT = -(-T // block)
+    q, k, v = _inputs(1, 2, T, K, V, dtype, seed=T + block)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    rng = np.random.default_rng(block + K + T)
+    for ns in range(1, min(NT, 7) + 1):
+        heads = []
+        for hd in range(2):
+            lists = [rng.permutation(NT)[:ns] for _ in range(NT)]
+            lists[hd] = np.concatenate([[NT - 1], rng.permutation(NT - 1)[:ns - 1]]).astype(lists[0].dtype)
+            heads.append(np.stack(lists))
+        indices = torch.tensor(np.stack(heads), dtype=torch.int32)[None].cuda()
+        o = piecewise_sparse_attention(qd, kd, vd, block_size=block, indices=indices)
+        floor = _oracle(q, k, v.abs(), indices, block=block)
+        assert_parity(o, _oracle(q, k, v, indices, block=block), dtype, f"block {block}, {ns} selected", floor)
+        if ns == 3:
+            tok = pisa_tokens(np64(q)[0, 1], np64(k)[0, 1], np64(v)[0, 1], indices[0, 1].cpu().numpy(), block,
+                              K ** -0.5)
+            assert_parity(o[0, 1], tok, dtype, f"per-token evaluation, block {block}", floor[0, 1])
+            padded = torch.full((1, 2, NT, min(ns + 2, NT)), -1, dtype=torch.int32)
+            padded[..., 0] = indices[..., 0].cpu()
+            padded[..., 2] = indices[..., 1].cpu()
+            padded[..., 3] = indices[..., 2].cpu()
+            # (the holes change which blocks share a tile, hence the order of the sums: not bit-equal)
+            o_padded = piecewise_sparse_attention(qd, kd, vd, block_size=block, indices=padded.cuda())
+            assert_parity(o_padded, _oracle(q, k, v, indices, block=block), dtype, f"block {block}, padded list", floor)
+    o_auto = piecewise_sparse_attention(qd, kd, vd, density=0.3, block_size=block)
     assert torch.isfinite(o_auto.float()).all()
 
 
