@@ -159,6 +159,18 @@ def test_all_blocks_selected_is_softmax_attention(dtype):
     assert_parity(o, ref, dtype, "density 1")
 
 
+def test_many_small_blocks_need_more_than_64k_of_lds():
+    """2048 blocks of 16 tokens, all selected: four bitmaps and a list of 2048 key tiles next to the tile ring
+    take more LDS than a kernel gets by default (the launch raises its limit).  With every block selected
+    the result is softmax attention, evaluated here by torch in fp32 on the GPU."""
+    from flash_bla.ops.piecewise_attn.kernel import piecewise_sparse_attention
+    dtype = torch.float16
+    q, k, v = (t.cuda() for t in _inputs(1, 1, 32768, 64, 64, dtype, seed=9, qk_scale=0.5))
+    o = piecewise_sparse_attention(q, k, v, density=1.0, block_size=16)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
+    assert_parity(o, ref.double().cpu(), dtype, "2048 blocks of 16 tokens, density 1")
+
+
 def test_small_scores_first_order_branch():
     """Small logits: the linear branch carries real weight and the first-order term matters."""
     from flash_bla.ops.piecewise_attn.kernel import chunk_reduce_fp32, piecewise_sparse_attention
