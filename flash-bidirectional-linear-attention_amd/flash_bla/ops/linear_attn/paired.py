@@ -11,6 +11,7 @@ two calls' key gradients) once.  Not in the reference, which runs the two calls 
 from typing import Optional, Tuple
 
 import torch
+import torch.nn.functional as F
 
 from flash_bla import _hip
 from flash_bla.ops._check import check_dense
@@ -52,8 +53,8 @@ def paired_linear_attention(
         scale: factor on the key-value state, default `1 / L`; eps: added to the denominators.
     Returns `(o1, o2)`, each `(B, H, L, V/2)`:
     `linear_attention(q1, k, v[..., :V/2])` and `linear_attention(q2, k, v[..., V/2:])`.
-    fp16 / bf16 with K and V/2 multiples of 8 and as many keys as queries take the shared-state
-    kernels; everything else runs the two operator calls.
+    fp16 / bf16 with as many keys as queries take the shared-state kernels (K and V/2 that are not
+    multiples of 8 through zero-padded copies); everything else runs the two operator calls.
     """
     check_dense("paired_linear_attention", q1, k, v)
     if q2.shape != q1.shape or q2.dtype != q1.dtype or q2.device != q1.device:
@@ -62,7 +63,20 @@ def paired_linear_attention(
         raise ValueError("paired_linear_attention: the value dim must be even")
     if scale is None:
         scale = k.shape[-2] ** -1.0
-    if k.shape[-2] == q1.shape[-2] and _hip.pair_supported(q1, v):
-        return PairedLinearAttnFunction.apply(q1, q2, k, v, scale, eps)
-    v1, v2 = (t.contiguous() for t in v.chunk(2, dim=-1))
-    return linear_attention(q1, k, v1, scale, eps), linear_attention(q2, k, v2, scale, eps)
+    v1, v2 = v.chunk(2, dim=-1)
+    if k.shape[-2] == q1.shape[-2]:
+        if _hip.pair_supported(q1, v):
+            return PairedLinearAttnFunction.apply(q1, q2, k, v, scale, eps)
+        # head dims that are not multiples of 8: zero features up to the next multiple change nothing
+        # (zero key features add nothing to any product, zero value columns give zero output columns)
+        # and keep the one pass over k and v, with its single rounding of dk
+        half = v.shape[-1] // 2
+        kw, hw = -(-q1.shape[-1] // 8) * 8, -(-half // 8) * 8
+        if q1.dtype != torch.float32 and (kw, hw) != (q1.shape[-1], half):
+            widen = lambda t, n: F.pad(t, (0, n - t.shape[-1]))
+            vw = torch.cat([widen(v1, hw), widen(v2, hw)], dim=-1)
+            q1w, q2w, kwide = (widen(t, kw) for t in (q1, q2, k))
+            if _hip.pair_supported(q1w, vw):
+                o1, o2 = PairedLinearAttnFunction.apply(q1w, q2w, kwide, vw, scale, eps)
+                return o1[..., :half], o2[..., :half]
+    return linear_attention(q1, k, v1.contiguous(), scale, eps), linear_attention(q2, k, v2.contiguous(), scale, eps)

@@ -58,8 +58,8 @@ def test_paired_explicit_scale_and_eps():
 
 @pytest.mark.parametrize("case", ["fp32", "fewer_keys", "odd_half"])
 def test_paired_shapes_outside_the_shared_kernels_run_the_two_calls(case):
-    """fp32, another number of keys than queries, halves that are not multiples of 8: same results
-    through two operator calls."""
+    """fp32 and another number of keys than queries run the two operator calls, halves that are not
+    multiples of 8 zero-padded copies on the shared kernels: same results."""
     from flash_bla import _hip
     from flash_bla.ops.linear_attn.paired import paired_linear_attention
     dtype = torch.float32 if case == "fp32" else torch.float16
@@ -76,6 +76,27 @@ def test_paired_shapes_outside_the_shared_kernels_run_the_two_calls(case):
     for o, q, vv in ((o1, q1, v[..., :half]), (o2, q2, v[..., half:])):
         ref = cf.dense_forward(np64(q), np64(k), np64(vv), 1.0 / Lk)[0]
         assert_parity(o, ref, dtype, case)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("B,H,L,DK,DV", [(1, 2, 1500, 100, 128), (3, 4, 15, 100, 26), (1, 1, 400, 17, 10)])
+def test_paired_head_dims_that_are_not_multiples_of_eight(dtype, B, H, L, DK, DV):
+    """Zero-padded copies keep the shared pass over k and v (one rounding of dk instead of the sum of two
+    rounded gradients): outputs and all four gradients against the oracle."""
+    from flash_bla.ops.linear_attn.paired import paired_linear_attention
+    q1, k, v, do, q2 = make_qkv((B, H, L, DK), (B, H, L, DV), dtype, seed=L + DK, n_extra=1)
+    half = DV // 2
+    do1, do2 = do[..., :half].contiguous(), do[..., half:].contiguous()
+    leaves = [t.cuda().requires_grad_() for t in (q1, q2, k, v)]
+    o1, o2 = paired_linear_attention(*leaves)
+    assert o1.shape == (B, H, L, half) and o2.shape == (B, H, L, half)
+    torch.autograd.backward([o1, o2], [do1.cuda(), do2.cuda()])
+    ref = _oracle(q1, q2, k, v, do1, do2, 1.0 / L)
+    assert_parity(o1, ref["o1"], dtype, "o1")
+    assert_parity(o2, ref["o2"], dtype, "o2")
+    for name, leaf in zip(("dq1", "dq2", "dk", "dv"), leaves):
+        assert leaf.grad.shape == leaf.shape
+        assert_parity(leaf.grad, ref[name], dtype, name, ref.get(name + "_mag"))
 
 
 def test_paired_rejects_mismatched_queries():
