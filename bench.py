@@ -32,7 +32,8 @@ import torch  # noqa: E402
 import torch.nn.functional as F  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
-MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 / fp16 matrix peak
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+MFMA_FP32_PEAK_TFLOPS = 157.3  # dense bf16 / fp16 matrix peak
 
 # Untimed work before the warm-up steps.  The GPU reaches its steady clocks after 0.15-0.2 s of continuous work: a
 # timed region of 20 steps reads 0.522 ms per step after 0.1 s of work and 0.503 ms after 0.2 s or more, the value every
@@ -427,7 +428,8 @@ def sweep(dtype, dev, flush):
     return rows
 
 
-def _report(name, nbytes_fwd, nbytes_step, fwd_fn, step_fn, flush, extra=None):
+def _report(name, nbytes_fwd, nbytes_step, fwd_fn, step_fn, flush, extra=None, fp32_flops=None):
+    """fp32_flops = (forward, forward + backward) FLOP: adds the fraction of the fp32 matrix peak."""
     f = do_bench(fwd_fn, flush)
     s = do_bench(step_fn, flush) if step_fn else None
     row = {"config": name, "fwd_ms": round(f[0], 5), "fwd_gbps": round(nbytes_fwd / f[0] / 1e6, 1),
@@ -435,6 +437,11 @@ def _report(name, nbytes_fwd, nbytes_step, fwd_fn, step_fn, flush, extra=None):
     if s:
         row.update({"fwd_bwd_ms": round(s[0], 5), "fwd_bwd_gbps": round(nbytes_step / s[0] / 1e6, 1),
                     "fwd_bwd_frac": round(nbytes_step / s[0] / 1e6 / HBM_PEAK_GBPS, 4)})
+    if fp32_flops:
+        for key, flop, t in (("fwd", fp32_flops[0], f), ("fwd_bwd", fp32_flops[1], s)):
+            if t:
+                row[key + "_tflops"] = round(flop / (t[0] * 1e-3) / 1e12, 1)
+                row[key + "_frac_of_fp32_mfma_peak"] = round(flop / (t[0] * 1e-3) / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4)
     if extra:
         row.update(extra)
     print(json.dumps(row), file=sys.stderr, flush=True)
@@ -631,7 +638,11 @@ def fp32_config(dev, flush):
             t.requires_grad_()
         nb = q.numel() * 4
         f, s = _fwd_and_step(linear_attention, (q, k, v), do)
-        rows.append(_report(f"linear_attn B8-H16-T4096-D{D} fp32", 4 * nb, 11 * nb, f, s, flush))
+        # the fp32 matrix instructions (157.3 TFLOP/s) bound these shapes next to HBM: forward 4 DK DV
+        # FLOP per (token, head), backward about 10 more
+        flop = q.numel() * D
+        rows.append(_report(f"linear_attn B8-H16-T4096-D{D} fp32", 4 * nb, 11 * nb, f, s, flush,
+                            fp32_flops=(4 * flop, 14 * flop)))
         del q, k, v, do
     return rows
 
