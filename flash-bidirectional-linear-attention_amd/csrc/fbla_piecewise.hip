@@ -961,11 +961,12 @@ __global__ __launch_bounds__(kThreads) void select_blocks_kernel(
     if (r0 + row < NT) x = load4(qh + (int64_t)(r0 + row) * Km, c4);
     *reinterpret_cast<f4*>(qs + row * K + 4 * c4) = x;
   }
-  for (int j0 = 0; j0 < NT; j0 += kSelKeys) {
-    // the tile's pieces of this thread are all requested before the first is stored (clamped
-    // addresses instead of branches: a loop of guarded loads waits for every single one)
-    constexpr int NPRE = KT ? kSelKeys * (KT / 4) / kThreads : kSelKeys * 32 / kThreads;
-    f4 pre[NPRE];
+  // the tile's pieces of this thread are all requested before the first is stored (clamped
+  // addresses instead of branches: a loop of guarded loads waits for every single one), and the
+  // next tile's while this one is multiplied
+  constexpr int NPRE = KT ? kSelKeys * (KT / 4) / kThreads : kSelKeys * 32 / kThreads;
+  f4 pre[NPRE];
+  auto request_tile = [&](int j0) {
 #pragma unroll
     for (int u = 0; u < NPRE; ++u) {
       const int e = tid + u * kThreads, row = e / (K / 4), c4 = e % (K / 4);
@@ -973,6 +974,9 @@ __global__ __launch_bounds__(kThreads) void select_blocks_kernel(
       pre[u] = load4(kh + (int64_t)(in ? j0 + row : 0) * Km, in ? c4 : 0);
       if (!in) pre[u] = f4{0.f, 0.f, 0.f, 0.f};
     }
+  };
+  request_tile(0);
+  for (int j0 = 0; j0 < NT; j0 += kSelKeys) {
     __syncthreads();  // previous tile consumed (first trip: nothing to wait for but cheap)
 #pragma unroll
     for (int u = 0; u < NPRE; ++u) {
@@ -980,6 +984,7 @@ __global__ __launch_bounds__(kThreads) void select_blocks_kernel(
       if (e < kSelKeys * (K / 4)) *reinterpret_cast<f4*>(kt + row * KLD + 4 * c4) = pre[u];
     }
     __syncthreads();
+    if (j0 + kSelKeys < NT) request_tile(j0 + kSelKeys);
     float acc[RW];  // rows RW*wave .. +RW-1 against key j0 + lane
 #pragma unroll
     for (int rr = 0; rr < RW; ++rr) acc[rr] = 0.f;
