@@ -33,9 +33,23 @@ __device__ __forceinline__ void map_tensor(const T* __restrict__ x, T* __restric
                                            int64_t vec_step) {
   constexpr int E = Elems<T>::kPerVec;
   const int64_t nvec = n / E;
-  for (int64_t i = first_vec; i < nvec; i += vec_step) {
+  // two vectors per trip, both requested before the first is mapped; the input is read once
+  // (streaming hint), the output is left to the caches for the kernel that follows
+  int64_t i = first_vec;
+  for (; i + vec_step < nvec; i += 2 * vec_step) {
+    union { u32x4 w; T e[E]; } in0, in1, out0, out1;
+    in0.w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + i * E));
+    in1.w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + (i + vec_step) * E));
+#pragma unroll
+    for (int j = 0; j < E; ++j) out0.e[j] = phi(in0.e[j]);
+#pragma unroll
+    for (int j = 0; j < E; ++j) out1.e[j] = phi(in1.e[j]);
+    *reinterpret_cast<u32x4*>(y + i * E) = out0.w;
+    *reinterpret_cast<u32x4*>(y + (i + vec_step) * E) = out1.w;
+  }
+  if (i < nvec) {
     union { u32x4 w; T e[E]; } in, out;
-    in.w = *reinterpret_cast<const u32x4*>(x + i * E);
+    in.w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + i * E));
 #pragma unroll
     for (int j = 0; j < E; ++j) out.e[j] = phi(in.e[j]);
     *reinterpret_cast<u32x4*>(y + i * E) = out.w;
@@ -66,8 +80,8 @@ __global__ __launch_bounds__(kThreads) void elu1_bwd_kernel(const T* __restrict_
   const int64_t first = (int64_t)blockIdx.x * kThreads + threadIdx.x, step = (int64_t)gridDim.x * kThreads;
   for (int64_t i = first; i < nvec; i += step) {
     union { u32x4 w; T e[E]; } xin, gin, out;
-    xin.w = *reinterpret_cast<const u32x4*>(x + i * E);
-    gin.w = *reinterpret_cast<const u32x4*>(g + i * E);
+    xin.w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + i * E));
+    gin.w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(g + i * E));
 #pragma unroll
     for (int j = 0; j < E; ++j) out.e[j] = dphi(xin.e[j], gin.e[j]);
     *reinterpret_cast<u32x4*>(dx + i * E) = out.w;

@@ -40,10 +40,10 @@ __global__ __launch_bounds__(kThreads) void chunk_sums_kernel(
     float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
     int t = 0;
     for (; t + 4 <= n; t += 4) {
-      a0 += to_f32(src[(int64_t)t * D + d]);
-      a1 += to_f32(src[(int64_t)(t + 1) * D + d]);
-      a2 += to_f32(src[(int64_t)(t + 2) * D + d]);
-      a3 += to_f32(src[(int64_t)(t + 3) * D + d]);
+      a0 += to_f32(__builtin_nontemporal_load(src + (int64_t)t * D + d));
+      a1 += to_f32(__builtin_nontemporal_load(src + (int64_t)(t + 1) * D + d));
+      a2 += to_f32(__builtin_nontemporal_load(src + (int64_t)(t + 2) * D + d));
+      a3 += to_f32(__builtin_nontemporal_load(src + (int64_t)(t + 3) * D + d));
     }
     for (; t < n; ++t) a0 += to_f32(src[(int64_t)t * D + d]);
     const float s = (a0 + a1) + (a2 + a3);
@@ -83,7 +83,8 @@ __global__ __launch_bounds__(kThreads) void chunk_sums16_kernel(
 #pragma unroll
     for (int u = 0; u < NLD; ++u) {
       const int row = base + u * RPI + r0;
-      w[u] = row < n ? *reinterpret_cast<const u32x4s*>(src + (int64_t)row * D + ch * 8)
+      // (streaming hint: every row is read once here)
+      w[u] = row < n ? __builtin_nontemporal_load(reinterpret_cast<const u32x4s*>(src + (int64_t)row * D + ch * 8))
                      : u32x4s{0u, 0u, 0u, 0u};
     }
 #pragma unroll
