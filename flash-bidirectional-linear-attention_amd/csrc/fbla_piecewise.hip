@@ -881,13 +881,21 @@ __global__ __launch_bounds__(kThreads, 3) void attention32_kernel(Attn32Args a) 
 }
 
 // kc (fp32 mean) / vc (fp32 sum) -> zero-padded 16-bit hi + lo arrays [BH, NTp, D]
+// (one launch for both statistics: workgroups [0, wgs0) take the keys' means, the rest the values' sums)
 template <typename T>
-__global__ __launch_bounds__(kThreads) void split_hi_lo_kernel(const float* __restrict__ src,
-                                                               T* __restrict__ hi, T* __restrict__ lo,
-                                                               int64_t BH, int NT, int NTp, int D) {
+__global__ __launch_bounds__(kThreads) void split_hi_lo_kernel(const float* __restrict__ src0, T* __restrict__ hi0,
+                                                               T* __restrict__ lo0, int D0,
+                                                               const float* __restrict__ src1, T* __restrict__ hi1,
+                                                               T* __restrict__ lo1, int D1, int64_t BH, int NT,
+                                                               int NTp, int wgs0) {
+  const bool second = (int)blockIdx.x >= wgs0;
+  const float* __restrict__ src = second ? src1 : src0;
+  T* __restrict__ hi = second ? hi1 : hi0;
+  T* __restrict__ lo = second ? lo1 : lo0;
+  const int D = second ? D1 : D0;
+  const int64_t wg = second ? blockIdx.x - wgs0 : blockIdx.x, wgs = second ? gridDim.x - wgs0 : wgs0;
   const int64_t total = BH * NTp * D;
-  for (int64_t e = (int64_t)blockIdx.x * kThreads + threadIdx.x; e < total;
-       e += (int64_t)gridDim.x * kThreads) {
+  for (int64_t e = wg * kThreads + threadIdx.x; e < total; e += wgs * kThreads) {
     const int d = (int)(e % D);
     const int64_t bc = e / D;
     const int c = (int)(bc % NTp);
@@ -1220,8 +1228,8 @@ static int attention_t(const void* q, const void* k, const void* v, const float*
   T* r = (T*)ws;
   const unsigned gk = (unsigned)std::min<int64_t>(cdiv64(BH * NTp * K, kThreads), 4096);
   const unsigned gv = (unsigned)std::min<int64_t>(cdiv64(BH * NTp * V, kThreads), 4096);
-  split_hi_lo_kernel<T><<<dim3(gk), dim3(kThreads), 0, st>>>(kc, kc_hi, kc_lo, BH, NT, (int)NTp, K);
-  split_hi_lo_kernel<T><<<dim3(gv), dim3(kThreads), 0, st>>>(vc, vc_hi, vc_lo, BH, NT, (int)NTp, V);
+  split_hi_lo_kernel<T><<<dim3(gk + gv), dim3(kThreads), 0, st>>>(kc, kc_hi, kc_lo, K, vc, vc_hi, vc_lo, V, BH, NT,
+                                                                  (int)NTp, (int)gk);
   // r_t = q_t H: the row-parallel kernel with M = H
   const Prob p = dense_prob(BH, Tn, K, V);
   mfma::RowsJob job{q, nullptr, h, V, 1, nullptr, nullptr, r};
