@@ -119,9 +119,17 @@ class _Here:
 _HERE = _Here()
 
 
+_one_device = None
+
+
 def _on(device):
-    """Context that makes `device` current for the launch (kernels run on the current device)."""
-    if device.index is None or device.index == torch.cuda.current_device():
+    """Context that makes `device` current for the launch (kernels run on the current device).
+    With a single visible GPU there is nothing to switch (and asking torch for the current device
+    costs 2 us on the host-bound path of small problems)."""
+    global _one_device
+    if _one_device is None:
+        _one_device = torch.cuda.device_count() == 1
+    if _one_device or device.index is None or device.index == torch.cuda.current_device():
         return _HERE
     return torch.cuda.device(device)
 
